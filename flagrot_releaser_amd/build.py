@@ -1,0 +1,86 @@
+"""Builds the gfx950 shared libraries of this package with hipcc (cross-compiles without a GPU).
+
+    python -m flagrot_releaser_amd.build            # all libraries
+    python -m flagrot_releaser_amd.build kernels    # one of: kernels, kivi, mq
+
+Libraries land in flagrot_releaser_amd/lib/ (in-tree, git-ignored).  Counterpart of the reference's
+integrations/vllm_flagrot/csrc/build.sh / build_kivi.sh / build_mq.sh.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+LIBDIR = HERE / "lib"
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+# packed fp32 instructions are disabled for every device translation unit
+COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
+# bit-exact translation units: every fp32 operation rounded on its own
+STRICT = ["-ffp-contract=off", "-fno-fast-math"]
+
+# library -> [(source, extra flags)]
+LIBS = {
+    "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("capi.hip", [])]),
+    "kivi": ("libflagrot_kivi.so", [("kivi.hip", [])]),
+    "mq": ("libflagrot_mq.so", [("mq_prefill.hip", [])]),
+}
+
+
+def lib_path(name: str) -> Path:
+    return LIBDIR / LIBS[name][0]
+
+
+def sources(name: str) -> list:
+    return [CSRC / s for s, _ in LIBS[name][1]] + sorted(CSRC.glob("*.hpp")) + [Path(__file__)]
+
+
+def _compile(args):
+    src, flags, obj = args
+    cmd = [HIPCC, *COMMON, *flags, "-c", str(src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stdout}\n{r.stderr}")
+    return obj
+
+
+def build(name: str, verbose: bool = True) -> Path:
+    out, units = LIBS[name]
+    units = [(CSRC / s, f) for s, f in units if (CSRC / s).exists()]
+    if not units:
+        raise FileNotFoundError(f"no sources for library {name}")
+    LIBDIR.mkdir(exist_ok=True)
+    objdir = LIBDIR / "obj"
+    objdir.mkdir(exist_ok=True)
+    jobs = [(s, f, objdir / (s.stem + ".o")) for s, f in units]
+    with ThreadPoolExecutor(max_workers=min(4, len(jobs))) as ex:
+        objs = list(ex.map(_compile, jobs))
+    target = LIBDIR / out
+    tmp = target.with_suffix(".so.tmp")
+    r = subprocess.run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed for {out}:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, target)
+    if verbose:
+        print(f"built {target}")
+    return target
+
+
+def build_all(verbose: bool = True) -> list:
+    return [build(n, verbose) for n in LIBS if all((CSRC / s).exists() for s, _ in LIBS[n][1])]
+
+
+if __name__ == "__main__":
+    names = sys.argv[1:] or None
+    if names:
+        for n in names:
+            build(n)
+    else:
+        build_all()

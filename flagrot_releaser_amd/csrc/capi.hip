@@ -1,0 +1,176 @@
+// extern "C" surface of libflagrot_kernels.so (declared in include/flagrot_kernels.h): argument checks, the
+// reference's return codes, and dispatch to the launchers of writer.hip / decode.hip.
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/flagrot_kernels.h"
+#include "fr_common.hpp"
+#include "fr_launch.hpp"
+
+namespace fr {
+namespace {
+char g_err[512] = "";
+}
+void set_error(const char* msg) {
+  std::strncpy(g_err, msg, sizeof(g_err) - 1);
+  g_err[sizeof(g_err) - 1] = 0;
+}
+namespace {
+int fail(int code, const char* msg) {
+  set_error(msg);
+  return code;
+}
+int launched(int rc, const char* what) {
+  if (rc == -1) {
+    char buf[400];
+    std::snprintf(buf, sizeof(buf), "%s: %s", what, hipGetErrorString(hipGetLastError()));
+    set_error(buf);
+  } else if (rc == -4) set_error("unknown format / kind");
+  else if (rc == -5) set_error("page size not supported");
+  return rc;
+}
+constexpr int GEN = 1024, GT8 = 2048, HD256 = 4096;
+
+int fmt_of_kind(int kind) {
+  return kind == KIND_KONLY ? FMT_KONLY : kind == KIND_KONLYA ? FMT_KONLYA : kind == KIND_KONLYA2 ? FMT_KONLYA2 : -1;
+}
+bool fmt_int2(int fmt) { return fmt == FMT_INT2A || fmt == FMT_KONLYA2; }
+}  // namespace
+}  // namespace fr
+
+using namespace fr;
+
+extern "C" {
+
+int fr_abi_version(void) { return 9; }
+
+int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
+               const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale,
+               const uint8_t* kmask, const uint8_t* vmask, int rb, int qrot, int vrot, int variant, int stages,
+               float* opart, float* mlpart, int* counter, void* out, long long o_bs, const void* tail,
+               const int* tail_len, const int* tail_idx, long long tail_bs, long long tail_ts, void* stream,
+               int gqa, int kv_start) {
+  if (B <= 0) return 0;
+  if (fmt < FMT_INT4 || fmt > FMT_KONLYA2) return fail(-4, "fr_v2_attn: unknown format");
+  if (variant & HD256) return fail(-8, "fr_v2_attn: head dim 256 is not built");
+  if ((variant & ~(GEN | GT8 | HD256)) != 264 && (variant & ~(GEN | GT8 | HD256)) != 0)
+    return fail(-3, "fr_v2_attn: unsupported variant");
+  if (stages < 1 || stages > 8) return fail(-3, "fr_v2_attn: unsupported stages");
+  if (page != 16) return fail(-5, "fr_v2_attn: page size 16 only");
+  if (gqa <= 0) gqa = 4;
+  if (gqa > 64) return fail(-7, "fr_v2_attn: gqa out of range");
+  if (gqa != 4 && !(variant & GEN)) return fail(-7, "fr_v2_attn: gqa != 4 needs the generalised variant");
+  if (rb != 32 && (qrot || vrot)) return fail(-3, "fr_v2_attn: rotation block 32 only");
+  if (nsplit < 1 || chunk <= 0 || chunk % 16) return fail(-3, "fr_v2_attn: bad split plan");
+  const bool k2 = fmt == FMT_KONLY || fmt == FMT_KONLYA || fmt == FMT_KONLYA2;
+  DecodeParams p{};
+  p.q = q; p.q_bs = q_bs; p.pool = pool; p.block_table = block_table; p.bt_stride = bt_stride; p.seq_lens = seq_lens;
+  p.B = B; p.Hkv = Hkv; p.page = page; p.nsplit = nsplit; p.chunk = chunk; p.qscale = qscale;
+  p.kmask = (!k2 && qrot) ? kmask : nullptr;
+  p.vmask = (!k2 && (vrot || tail != nullptr)) ? vmask : nullptr;
+  p.opart = opart; p.mlpart = mlpart; p.counter = counter;
+  const int gt = ((variant & GEN) && (variant & GT8)) ? 8 : 4;
+  const int ntile = (gqa + 3) / 4, nct = (gqa + gt - 1) / gt;
+  p.counter_div = ntile / nct;
+  p.out = out; p.o_bs = o_bs;
+  p.tail = tail; p.tail_len = tail_len; p.tail_idx = tail_idx; p.tail_bs = tail_bs; p.tail_ts = tail_ts;
+  p.gqa = gqa; p.kv_start = kv_start;
+  return launched(decode_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_attn");
+}
+
+int fr_v2_write(int fmt, const void* kv, long long kv_ts, const long long* slots, int T, int Hkv, int page,
+                const uint8_t* mask, int rb, uint8_t* pool, void* stream, int hd, const float* kmu) {
+  if (T <= 0) return 0;
+  if (hd != 0 && hd != 128 && hd != 256) return fail(-8, "fr_v2_write: head dim 128 | 256");
+  if (rb != 32) return fail(-3, "fr_v2_write: rotation block 32 only");
+  StaticWriteParams p{};
+  p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.T = T; p.Hkv = hd == 256 ? 2 * Hkv : Hkv; p.page = page;
+  p.mask = mask; p.hfull = nullptr; p.kmu = kmu; p.pool = pool;
+  return launched(static_write_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_write");
+}
+
+int fr_v2_occupancy(int fmt, int variant, int stages, int page) {
+  (void)variant; (void)stages;
+  if (page != 16 || fmt < FMT_INT4 || fmt > FMT_KONLYA2) return 0;
+  return decode_occupancy(fmt);
+}
+int fr_v2_chunk_bytes(int fmt, int page) { return page * (fmt_int2(fmt) ? 80 : 144); }
+
+int fr_cb_nsg(void) { return 15; }
+
+int fr_cb_write(const void* kv, long long kv_ts, const long long* slots, int slot_ph, int T, int Hkv, int page, int tg,
+                const float* CT, const float* co, const unsigned* sg, int kind, uint8_t* pool, void* stream, int hd,
+                const float* kmu) {
+  (void)tg; (void)co; (void)sg;
+  if (T <= 0) return 0;
+  if (hd != 0 && hd != 128) return fail(-8, "fr_cb_write: head dim 128 only");
+  K2WriteParams p{};
+  p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.slot_ph = slot_ph; p.T = T; p.Hkv = Hkv; p.page = page;
+  p.CT = CT; p.kmu = kmu; p.pool = pool; p.passes = 3;
+  return launched(k2_write_launch(kind, p, static_cast<hipStream_t>(stream)), "fr_cb_write");
+}
+
+int fr_cb_write3(const void* kv, long long kv_ts, const long long* slots, int slot_ph, int T, int Hkv, int page,
+                 const float* CT, const float* co, const void* C1, const float* beta, const unsigned* sg, int kind,
+                 uint8_t* pool, int nchunk, int nchunk_v, void* stream, const float* kmu) {
+  (void)co; (void)C1; (void)beta; (void)sg;
+  if (T <= 0) return 0;
+  K2WriteParams p{};
+  p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.slot_ph = slot_ph; p.T = T; p.Hkv = Hkv; p.page = page;
+  p.CT = CT; p.kmu = kmu; p.pool = pool;
+  p.passes = (nchunk >= 0 ? 1 : 0) | (nchunk_v >= 0 ? 2 : 0);
+  if (p.passes == 0) return 0;
+  return launched(k2_write_launch(kind, p, static_cast<hipStream_t>(stream)), "fr_cb_write3");
+}
+
+int fr_w3_static_write(const void* kv, long long kv_ts, const long long* slots, int T, int Hkv, int page,
+                       const uint8_t* mask, const uint8_t* hfull, int asym, uint8_t* pool, int path, void* stream,
+                       const float* kmu) {
+  (void)path;
+  if (T <= 0) return 0;
+  if (asym < 0 || asym > 2) return fail(-4, "fr_w3_static_write: asym must be 0, 1 or 2");
+  StaticWriteParams p{};
+  p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.T = T; p.Hkv = Hkv; p.page = page;
+  p.mask = mask; p.hfull = hfull; p.kmu = kmu; p.pool = pool;
+  const int fmt = asym == 0 ? FMT_INT4 : asym == 1 ? FMT_INT4A : FMT_INT2A;
+  return launched(static_write_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_w3_static_write");
+}
+
+int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
+               const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale, const unsigned* sg,
+               int kind, int variant, int stages, float* opart, float* mlpart, int* counter, void* out, long long o_bs,
+               const void* tail, const int* tail_len, const int* tail_idx, long long tail_bs, long long tail_ts,
+               void* stream, int kv_start) {
+  (void)sg;
+  if (B <= 0) return 0;
+  const int fmt = fmt_of_kind(kind);
+  if (fmt < 0) return fail(-4, "fr_cb_attn: kind must be 6 (konly), 10 (konlya) or 11 (konlya2)");
+  if (variant != 0 && variant != 1) return fail(-3, "fr_cb_attn: unsupported variant");
+  return fr_v2_attn(fmt, q, q_bs, pool, block_table, bt_stride, seq_lens, B, Hkv, page, nsplit, chunk, qscale, nullptr,
+                    nullptr, 32, 0, 0, 264, stages, opart, mlpart, counter, out, o_bs, tail, tail_len, tail_idx,
+                    tail_bs, tail_ts, stream, 4, kv_start);
+}
+
+int fr_cb_occupancy(int kind, int variant, int stages, int page) {
+  (void)variant; (void)stages;
+  if (page != 16 || fmt_of_kind(kind) < 0) return 0;
+  return decode_occupancy(fmt_of_kind(kind));
+}
+int fr_cb_chunk_bytes(int kind, int page) { return page * (kind == KIND_KONLYA2 ? 80 : 144); }
+int fr_cb_write_smem(int kind, int tg, int hd) {
+  (void)tg;
+  if (fmt_of_kind(kind) < 0 || (hd != 0 && hd != 128)) return 0;
+  return k2_write_lds_bytes();
+}
+
+const char* fr_last_error(void) { return g_err; }
+
+int fr_head_fwht(const void* x, long long x_ts, void* out, long long o_ts, int T, int H, const uint8_t* flags,
+                 float scale, void* stream, int D) {
+  if (T <= 0) return 0;
+  if (D != 128 && D != 256) return fail(-8, "fr_head_fwht: head dim 128 | 256");
+  return launched(head_fwht_launch(x, x_ts, out, o_ts, T, H, flags, scale, static_cast<hipStream_t>(stream), D),
+                  "fr_head_fwht");
+}
+
+}  // extern "C"

@@ -1,0 +1,397 @@
+"""ctypes front end of libflagrot_kernels.so (gfx950): paged FlagRot KV-cache writers + paged decode attention.
+
+Host-side mirror of the reference plugin's front end (integrations/vllm_flagrot/vllm_flagrot/kernels.py of the
+reference): same function names, argument meaning and error behaviour, so callers written against it
+(`v2_write`, `v2_attn`, `cb_write`, `cb_write3`, `w3_static_write`, `cb_attn`, `head_fwht`, `plan_v2`, `plan_cb`,
+`Workspace`) run unchanged.  PyTorch-ROCm only supplies device memory and the current HIP stream; every launch is
+asynchronous on that stream and allocates nothing.
+
+The shared library is built in-tree by `flagrot_releaser_amd.build` (hipcc, --offload-arch=gfx950).  It is rebuilt on
+first use when it is missing or older than a source (file lock; set FLAGROT_NO_REBUILD=1 to forbid), and a missing
+compiler or a failed build raises: there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+import fcntl
+import math
+import os
+from pathlib import Path
+
+import torch
+
+from . import build as _build
+
+ABI = 9
+D, RB, NG = 128, 32, 4
+V2_FMT = {"int4": 4, "int4a": 5, "konly": 6, "konlya": 7, "int2a": 8, "konlya2": 9}
+INT2_FMTS = ("int2a", "konlya2")
+GEN, GT8, HD256 = 1024, 2048, 4096
+CB_KINDS = {"konly": 6, "konlya": 10, "konlya2": 11}
+K2 = ("konly", "konlya", "konlya2")
+STAGES = 4
+MAX_CHUNK, MAX_SPLITS = 8192, 512
+SEEDS = (0,) + tuple(range(2, 16))
+W3_SPLIT_T = int(os.environ.get("W3_SPLIT_T", "256"))
+
+
+# ------------------------------------------------------------------------------------------------ library
+def _lib_path() -> Path:
+    return Path(os.environ.get("FLAGROT_LIB", _build.lib_path("kernels")))
+
+
+def _stale(lib: Path) -> bool:
+    if not lib.exists():
+        return True
+    if os.environ.get("FLAGROT_NO_REBUILD") or "FLAGROT_LIB" in os.environ:
+        return False
+    t = lib.stat().st_mtime
+    return any(s.exists() and s.stat().st_mtime > t for s in _build.sources("kernels"))
+
+
+_LIB = None
+
+
+def lib():
+    """the loaded library (built first when missing or out of date); raises when it cannot be had."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = _lib_path()
+    if _stale(path):
+        if os.environ.get("FLAGROT_NO_REBUILD"):
+            raise RuntimeError(f"{path} is missing and FLAGROT_NO_REBUILD is set")
+        path.parent.mkdir(parents=True, exist_ok=True)
+        with open(str(path) + ".lock", "w") as lk:
+            fcntl.flock(lk, fcntl.LOCK_EX)
+            try:
+                if _stale(path):
+                    _build.build("kernels", verbose=False)
+            finally:
+                fcntl.flock(lk, fcntl.LOCK_UN)
+    L = ctypes.CDLL(str(path))
+    P, I, LL, F = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong, ctypes.c_float
+    L.fr_abi_version.restype = I
+    if L.fr_abi_version() != ABI:
+        raise RuntimeError(f"libflagrot_kernels ABI {L.fr_abi_version()} != {ABI}: rebuild ({path})")
+    sig = {
+        "fr_v2_attn": [I, P, LL, P, P, I, P, I, I, I, I, I, F, P, P, I, I, I, I, I, P, P, P, P, LL, P, P, P, LL, LL, P,
+                       I, I],
+        "fr_v2_write": [I, P, LL, P, I, I, I, P, I, P, P, I, P],
+        "fr_v2_occupancy": [I, I, I, I],
+        "fr_v2_chunk_bytes": [I, I],
+        "fr_cb_nsg": [],
+        "fr_cb_write": [P, LL, P, I, I, I, I, I, P, P, P, I, P, P, I, P],
+        "fr_cb_write3": [P, LL, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P],
+        "fr_w3_static_write": [P, LL, P, I, I, I, P, P, I, P, I, P, P],
+        "fr_cb_attn": [P, LL, P, P, I, P, I, I, I, I, I, F, P, I, I, I, P, P, P, P, LL, P, P, P, LL, LL, P, I],
+        "fr_cb_occupancy": [I, I, I, I],
+        "fr_cb_chunk_bytes": [I, I],
+        "fr_cb_write_smem": [I, I, I],
+        "fr_head_fwht": [P, LL, P, LL, I, I, P, F, P, I],
+    }
+    for name, args in sig.items():
+        fn = getattr(L, name)
+        fn.argtypes, fn.restype = args, I
+    L.fr_last_error.restype = ctypes.c_char_p
+    _LIB = L
+    return L
+
+
+EXPORTS = ("fr_abi_version", "fr_v2_attn", "fr_v2_write", "fr_v2_occupancy", "fr_v2_chunk_bytes", "fr_cb_nsg",
+           "fr_cb_write", "fr_cb_write3", "fr_w3_static_write", "fr_cb_attn", "fr_cb_occupancy", "fr_cb_chunk_bytes",
+           "fr_cb_write_smem", "fr_last_error", "fr_head_fwht")
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        raise RuntimeError(f"{what}: launch failed (code {rc}, {lib().fr_last_error().decode()})")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+_DEV_IDX: list = []
+
+
+def _stream():
+    """raw hipStream_t of torch's current stream (the device index is cached: one device per process)."""
+    if not _DEV_IDX:
+        _DEV_IDX.append(torch.cuda.current_device())
+    return torch._C._cuda_getCurrentRawStream(_DEV_IDX[0])
+
+
+_SG = None
+
+
+def sign_words():
+    """uint32[15 * 4] sign table argument of the codebook entry points.  The key-only kinds never read it; it is
+    passed as zeros to keep the reference signature."""
+    global _SG
+    if _SG is None:
+        _SG = (ctypes.c_uint * (len(SEEDS) * 4))()
+    return _SG
+
+
+# ------------------------------------------------------------------------------------------------ shapes / variants
+def qtile(G: int, Dh: int = 128) -> int:
+    return 8 if Dh == 128 and 5 <= G <= 8 else 4
+
+
+def v2_variant(fmt: str, G: int = 4, Dh: int = 128) -> int:
+    if G == 4 and Dh == 128 and fmt in ("int4", "int4a", "int2a"):
+        return 264
+    return 264 | GEN | (GT8 if qtile(G, Dh) == 8 else 0) | (HD256 if Dh == 256 else 0)
+
+
+def tile_of(variant: int) -> int:
+    return 8 if (variant & GEN) and (variant & GT8) else 4
+
+
+def vheads(Hkv: int, G: int, Dh: int = 128, fmt: str = "int4") -> int:
+    return Hkv * -(-G // tile_of(v2_variant(fmt, G, Dh)))
+
+
+def v2_chunk_bytes(page: int, Dh: int = 128, fmt: str = "int4") -> int:
+    return page * (80 if fmt in INT2_FMTS else 144) * Dh // 128
+
+
+def cb_chunk_bytes(kind: str, page: int, Dh: int = 128) -> int:
+    return page * (80 if kind in INT2_FMTS else 144) * Dh // 128
+
+
+# ------------------------------------------------------------------------------------------------ split planner
+_NUM_CU = None
+_OCC: dict = {}
+
+
+def _slots(key, occ_fn) -> int:
+    """workgroups resident on the GPU at once: occupancy per CU x CU count."""
+    global _NUM_CU
+    if _NUM_CU is None:
+        _NUM_CU = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    if key not in _OCC:
+        _OCC[key] = max(1, occ_fn())
+    return _OCC[key] * _NUM_CU
+
+
+def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, fixed: int = 512, merge: int = 48):
+    """(nsplit, chunk): chunk a multiple of 64 tokens, <= 8192, nsplit = ceil(Lmax / chunk).  Cost model in
+    token-equivalents: waves of `slots` concurrent workgroups, each costing its chunk + a fixed launch/prologue/merge
+    share, + a per-split merge term."""
+    gran = max(64, page)
+    Lmax = max(1, int(Lmax))
+    if nsplit is not None:
+        chunk = min(MAX_CHUNK, math.ceil(Lmax / nsplit / gran) * gran)
+        return math.ceil(Lmax / chunk), chunk
+    best = None
+    for ns in range(max(1, math.ceil(Lmax / MAX_CHUNK)), min(MAX_SPLITS, math.ceil(Lmax / gran)) + 1):
+        chunk = math.ceil(Lmax / ns / gran) * gran
+        if chunk > MAX_CHUNK:
+            continue
+        nse = math.ceil(Lmax / chunk)
+        if best is not None and nse == best[1]:
+            continue
+        cost = math.ceil(B * HV * nse / slots) * (chunk + fixed) + (merge * nse if nse > 1 else 0)
+        if best is None or cost < best[0] - 1e-9:
+            best = (cost, nse, chunk)
+    return best[1], best[2]
+
+
+def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
+    HV = Hkv * -(-G // 4)                                  # workgroups per (row, split): q tiles of 4 heads
+    s = _slots(("v2", fmt, page), lambda: lib().fr_v2_occupancy(V2_FMT[fmt], v2_variant(fmt, G, Dh), STAGES, page))
+    return plan_splits(B, Lmax, HV, page, s, nsplit)
+
+
+def plan_cb(B, Lmax, Hkv, page, kind, nsplit=None, G=4, Dh=128):
+    if kind in K2 and (G != 4 or Dh != 128):
+        return plan_v2(B, Lmax, Hkv, page, nsplit, fmt=kind, G=G, Dh=Dh)
+    s = _slots(("cb", kind, page), lambda: lib().fr_cb_occupancy(CB_KINDS[kind], 0, STAGES, page))
+    return plan_splits(B, Lmax, Hkv, page, s, nsplit)
+
+
+class Workspace:
+    """split-K partials for up to `parts` (row, kv head / q tile, split) partials of GT q heads x Dh dims, plus the
+    per-(row, kv head / q tile) merge tickets (zeroed once, self-resetting).  Allocate before graph capture."""
+
+    def __init__(self, rows: int, Hkv: int, parts: int, device, GT: int = 4, Dh: int = 128):
+        self.rows, self.parts, self.HV, self.GT, self.Dh = rows, parts, Hkv, GT, Dh
+        self.opart = torch.empty(parts * GT * Dh, device=device, dtype=torch.float32)
+        self.mlpart = torch.empty(parts * GT * 2, device=device, dtype=torch.float32)
+        self.counter = torch.zeros(rows * Hkv, device=device, dtype=torch.int32)
+
+    def fits(self, B, Hkv, nsplit_total, GT=4, Dh=128):
+        return (B <= self.rows and B * Hkv * nsplit_total <= self.parts and Hkv <= self.HV
+                and GT * Dh <= self.GT * self.Dh
+                and B * Hkv * nsplit_total * GT * Dh <= self.parts * self.GT * self.Dh)
+
+
+# ------------------------------------------------------------------------------------------------ launches
+def _kmu(kmu, kv):
+    if kmu is None:
+        return None
+    Hkv, Dh = kv.shape[1] // 2, kv.shape[2]
+    assert kmu.dtype == torch.float32 and kmu.is_contiguous() and tuple(kmu.shape) == (Hkv, Dh) \
+        and kmu.device == kv.device, (kmu.dtype, tuple(kmu.shape), (Hkv, Dh))
+    return kmu.data_ptr()
+
+
+def _rows_ok(kv):
+    """bf16 rows contiguous over (head, dim) and 8-byte aligned (the kernels load 4 elements at a time)."""
+    Dh = kv.shape[2]
+    if kv.stride(2) != 1 or kv.stride(1) != Dh or kv.stride(0) % 4 or kv.data_ptr() % 8:
+        kv = kv.contiguous()
+    return kv
+
+
+def v2_write(kv, slots, mask, rb, pool, page, fmt="int4", kmu=None):
+    """kv bf16 [T, 2*Hkv, Dh] (Dh 128 | 256) -> pool [num_pages, Hkv, chunk] at slots int64 [T] (< 0 skipped);
+    mask uint8 [2*Hkv, Dh/rb] (K rows first); fmt "int4" | "int4a" | "int2a"."""
+    T = kv.shape[0]
+    if T == 0:
+        return
+    Dh = kv.shape[2]
+    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
+    kv = _rows_ok(kv)
+    _check(lib().fr_v2_write(V2_FMT[fmt], kv.data_ptr(), kv.stride(0), slots.data_ptr(), T, kv.shape[1] // 2, page,
+                             mask.data_ptr(), rb, pool.data_ptr(), _stream(), Dh, _kmu(kmu, kv)), "fr_v2_write")
+
+
+def v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kmask=None, vmask=None, rb=32,
+            tail=None, tail_len=None, tail_idx=None, tail_bs=None, tail_ts=None, page=16, fmt="int4", kv_start=0):
+    """q bf16 [B, G*Hkv, Dh] -> out bf16 [B, G*Hkv*Dh].  block_table int32 [B, *] (row stride may be 0), seq_lens int32
+    [B]; tail: bf16 window rows (strides tail_bs / tail_ts elements) with tail_len int32 [B] (+ tail_idx int32 [B]).
+    qscale = softmax scale * log2(e).  kv_start: tokens [0, kv_start) are masked in the paged body."""
+    B, Hq, Dh = q.shape
+    Hkv = pool.shape[1]
+    G = Hq // Hkv
+    assert Hq == G * Hkv and q.stride(2) == 1 and q.stride(1) == Dh and out.stride(1) == 1
+    v = v2_variant(fmt, G, Dh)
+    GT = tile_of(v)
+    assert ws.fits(B, vheads(Hkv, G, Dh, fmt), nsplit + (tail is not None), GT, Dh), "split-K workspace too small"
+    _check(lib().fr_v2_attn(V2_FMT[fmt], q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(),
+                            block_table.stride(0), seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale,
+                            _ptr(kmask), _ptr(vmask), rb, int(kmask is not None), int(vmask is not None), v, STAGES,
+                            ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
+                            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
+                            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), G,
+                            int(kv_start)), "fr_v2_attn")
+
+
+def cb_write(kv, slots, CT, co, kind, pool, page, tg=None, kmu=None):
+    """kv bf16 [T, 2*Hkv, 128] -> pool at slots int64 [T]; CT fp32 [Hkv, 128, 128] = C_q^T, co fp32 [Hkv, 128]."""
+    T = kv.shape[0]
+    if T == 0:
+        return
+    Dh = kv.shape[2]
+    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
+    kv = _rows_ok(kv)
+    if tg is None:
+        tg = 1 if T <= 16 else (2 if T <= 64 or kind not in K2 else 4)
+    _check(lib().fr_cb_write(kv.data_ptr(), kv.stride(0), slots.data_ptr(), 0, T, kv.shape[1] // 2, page, tg,
+                             CT.data_ptr(), co.data_ptr(), sign_words(), CB_KINDS[kind], pool.data_ptr(), _stream(),
+                             Dh, _kmu(kmu, kv)), "fr_cb_write")
+
+
+_SIDE: dict = {}
+
+
+def side_stream(device=None):
+    """second stream of the two-pass writer (one per device, default priority; create before graph capture)."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if dev not in _SIDE:
+        _SIDE[dev] = torch.cuda.Stream(dev)
+    return _SIDE[dev]
+
+
+def w3_nchunk(Hkv, per_cu):
+    global _NUM_CU
+    if _NUM_CU is None:
+        _NUM_CU = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    return max(1, (per_cu * _NUM_CU) // Hkv)
+
+
+def w3_calib(Cq, kappa=None, nd=8):
+    """the reference's writer v3 takes tensor-core screening constants (C1 fp16 [H, 168, 128], aux fp32 [H, 48]).
+    This library's writer evaluates the exact fp32 criterion directly and ignores them; zero tensors of the reference
+    shapes keep callers unchanged."""
+    H = Cq.shape[0]
+    return (torch.zeros(H, 168, 128, dtype=torch.float16, device=Cq.device),
+            torch.zeros(H, 48, dtype=torch.float32, device=Cq.device))
+
+
+def cb_write3(kv, slots, CT, co, C1, beta, kind, pool, page, split=None, kmu=None):
+    """= cb_write (same pool bytes).  split (default: T <= W3_SPLIT_T): key pass on the current stream, value pass on
+    the side stream (fork / join by stream waits, graph capturable), else both in one launch."""
+    T = kv.shape[0]
+    if T == 0:
+        return
+    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
+    assert kv.shape[2] == D, f"writer v3: head dim {D} only (got {kv.shape[2]}; use cb_write)"
+    kv = _rows_ok(kv)
+    slots = slots.contiguous()
+    Hkv = kv.shape[1] // 2
+    L = lib()
+    nk, nv = w3_nchunk(Hkv, 2), w3_nchunk(Hkv, 3)
+    km = _kmu(kmu, kv)
+    args = (kv.data_ptr(), kv.stride(0), slots.data_ptr(), 0, T, Hkv, page, CT.data_ptr(), co.data_ptr(),
+            _ptr(C1), _ptr(beta), sign_words(), CB_KINDS[kind], pool.data_ptr())
+    if split is None:
+        split = T <= W3_SPLIT_T
+    if not split:
+        _check(L.fr_cb_write3(*args, nk, nv, _stream(), km), "fr_cb_write3")
+        return
+    cur = torch.cuda.current_stream()
+    side = side_stream(kv.device)
+    side.wait_stream(cur)
+    _check(L.fr_cb_write3(*args, nk, -1, cur.cuda_stream, km), "fr_cb_write3 (keys)")
+    _check(L.fr_cb_write3(*args, -1, nv, side.cuda_stream, None), "fr_cb_write3 (values)")
+    cur.wait_stream(side)
+
+
+def w3_static_write(kv, slots, mask, hfull, pool, page, fmt="int4", path=0, kmu=None):
+    """= head_fwht(kv, hfull, 1/16) + v2_write(.., mask, rb 32, ..) in one launch (same pool bytes)."""
+    T = kv.shape[0]
+    if T == 0:
+        return
+    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
+    assert kv.shape[2] == D, f"writer v3: head dim {D} only (got {kv.shape[2]}; use v2_write)"
+    kv = _rows_ok(kv)
+    slots = slots.contiguous()
+    _check(lib().fr_w3_static_write(kv.data_ptr(), kv.stride(0), slots.data_ptr(), T, kv.shape[1] // 2, page,
+                                    _ptr(mask), _ptr(hfull), {"int4": 0, "int4a": 1, "int2a": 2}[fmt],
+                                    pool.data_ptr(), path, _stream(), _kmu(kmu, kv)), "fr_w3_static_write")
+
+
+def cb_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kind, tail=None, tail_len=None,
+            tail_idx=None, tail_bs=None, tail_ts=None, page=16, kv_start=0):
+    B, Hq, Dh = q.shape
+    if kind in K2 and (Hq != 4 * pool.shape[1] or Dh != 128):
+        return v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, tail=tail, tail_len=tail_len,
+                       tail_idx=tail_idx, tail_bs=tail_bs, tail_ts=tail_ts, page=page, fmt=kind, kv_start=kv_start)
+    Hkv = Hq // 4
+    assert Hq == 4 * pool.shape[1] and Dh == D, f"codebook {kind}: GQA 4, head dim 128 only"
+    assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
+    assert ws.fits(B, Hkv, nsplit + (tail is not None)), "split-K workspace too small"
+    _check(lib().fr_cb_attn(q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+                            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, sign_words(), CB_KINDS[kind], 0,
+                            STAGES, ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
+                            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
+                            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), int(kv_start)),
+           "fr_cb_attn")
+
+
+def head_fwht(x, flags, scale, out=None):
+    """x bf16 [T, H, Dh] (Dh 128 | 256) -> scale * H_Dh x (unnormalised +-1 Sylvester) for heads with flags[h] != 0,
+    a copy otherwise; out may alias x."""
+    T, H, Dh = x.shape
+    assert x.dtype == torch.bfloat16 and x.stride(2) == 1 and x.stride(1) == Dh
+    if out is None:
+        out = torch.empty(T, H, Dh, dtype=x.dtype, device=x.device)
+    assert out.stride(2) == 1 and out.stride(1) == Dh
+    if T:
+        _check(lib().fr_head_fwht(x.data_ptr(), x.stride(0), out.data_ptr(), out.stride(0), T, H, flags.data_ptr(),
+                                  scale, _stream(), Dh), "fr_head_fwht")
+    return out

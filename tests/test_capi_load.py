@@ -1,0 +1,43 @@
+"""CPU-side checks of the drop-in boundary: the library builds/loads and exports every symbol the header declares
+(no compute calls here: there is no GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b((?:fr|kv|frmq)_[a-z0-9_]+)\s*\(", text)
+
+
+def test_kernels_library_exports_header_symbols():
+    from flagrot_releaser_amd import build, kernels
+    path = build.lib_path("kernels")
+    if not path.exists():
+        build.build("kernels", verbose=False)
+    L = ctypes.CDLL(str(path))
+    names = _declared("flagrot_kernels.h")
+    assert set(names) == set(kernels.EXPORTS)
+    for n in names:
+        assert hasattr(L, n), n
+    L.fr_abi_version.restype = ctypes.c_int
+    assert L.fr_abi_version() == 9
+    assert L.fr_cb_nsg() == 15
+    assert L.fr_v2_chunk_bytes(5, 16) == 2304 and L.fr_v2_chunk_bytes(8, 16) == 1280
+    assert L.fr_cb_chunk_bytes(10, 16) == 2304 and L.fr_cb_chunk_bytes(11, 16) == 1280
+
+
+def test_host_planner_invariants():
+    from flagrot_releaser_amd import kernels as K
+    for B, L in ((1, 1), (1, 2048), (32, 8192), (64, 16384), (3, 33000), (8, 65536)):
+        for slots in (256, 512, 1024):
+            ns, ch = K.plan_splits(B, L, 8, 16, slots)
+            assert ch % 64 == 0 and ch <= K.MAX_CHUNK and ns == -(-L // ch) and ns <= K.MAX_SPLITS
+    assert K.plan_splits(4, 1000, 8, 16, 512, nsplit=3) == (3, 384)
+    assert K.v2_variant("int4a", 4) == 264 and K.tile_of(K.v2_variant("konlya", 8)) == 8
+    assert K.vheads(8, 8, 128, "konlya") == 8 and K.vheads(4, 12, 128, "int4") == 12

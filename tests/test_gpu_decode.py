@@ -1,0 +1,154 @@
+"""GPU parity of paged decode attention through the C ABI against the oracle's dequantise-then-attend reference.
+
+Bar (floating point): |out - ref| <= 2e-3 + 1e-2 * |ref| element-wise, ref = fp64 softmax attention over the pages
+parsed by the oracle's independent layout parser (the cache bytes themselves are written by the HIP writers, whose
+bit-exactness tests/test_gpu_writers.py establishes)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attend as A
+from oracle import pages as PG
+from tests.gpu_util import P, alloc_tables, bits, make_kv, slots_of, spd_calib
+
+pytestmark = pytest.mark.gpu
+LOG2E = 1.4426950408889634
+ATOL, RTOL = 2e-3, 1e-2
+
+
+def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None):
+    from flagrot_releaser_amd import kernels as K
+    g = torch.Generator().manual_seed(seed)
+    B = len(lens)
+    HQ = G * Hkv
+    num_pages = sum((n + P - 1) // P for n in lens) + 7
+    pool = torch.randint(0, 256, (num_pages, Hkv, PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g).to(dev)
+    bt = alloc_tables(lens, num_pages, g)
+    if bt_shared:
+        bt = bt[:1].expand(B, -1)
+        if bt_shared != "stride0":
+            bt = bt.contiguous()
+    mask = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8)
+    if mode == "codebook":
+        Cq, co = spd_calib(Hkv, g)
+        CT, co = Cq.transpose(1, 2).contiguous().to(dev), co.to(dev)
+    for b in range(B if not bt_shared else 1):
+        n = max(lens) if bt_shared else lens[b]
+        if n == 0:
+            continue
+        kv = make_kv(n, Hkv, g, edge=(b == 0)).to(dev)
+        sl = slots_of(bt, b, n).to(dev)
+        if mode == "static":
+            K.v2_write(kv, sl, mask.to(dev), 32, pool, P, fmt=fmt)
+        else:
+            K.cb_write(kv, sl, CT, co, fmt, pool, P)
+    q = (torch.randn(B, HQ, 128, generator=g) * 0.8).bfloat16()
+    scale = 1 / math.sqrt(128)
+    tail = tail_len = tail_idx = None
+    if win is not None:
+        W, R = win
+        tail = torch.randn(R, W, 2 * Hkv, 128, generator=g).bfloat16()
+        tail_idx = torch.randperm(R, generator=g)[:B].int()
+        tail_len = torch.randint(0, W + 1, (B,), generator=g).int()
+    Lmax = max(max(lens), 1)
+    seq = torch.tensor(lens, dtype=torch.int32)
+    ref = A.decode_reference(bits(q), pool.cpu().numpy(), fmt, P, bt.numpy(), lens, scale,
+                             kmask=mask[:Hkv].numpy() if mode == "static" else None,
+                             vmask=mask[Hkv:].numpy() if mode == "static" else None,
+                             tail=None if tail is None else bits(tail),
+                             tail_len=None if tail is None else tail_len.numpy(),
+                             tail_idx=None if tail is None else tail_idx.numpy(), kv_start=kv_start)
+    out = torch.full((B, HQ * 128), float("nan"), dtype=torch.bfloat16, device=dev)
+    if mode == "static":
+        ns, ch = K.plan_v2(B, Lmax, Hkv, P, nsplit=nsplit, fmt=fmt, G=G)
+    else:
+        ns, ch = K.plan_cb(B, Lmax, Hkv, P, fmt, nsplit=nsplit, G=G)
+    gfmt = fmt
+    if mode == "static" or G != 4:
+        HV, GT = K.vheads(Hkv, G, 128, gfmt), K.tile_of(K.v2_variant(gfmt, G, 128))
+    else:
+        HV, GT = Hkv, 4
+    ws = K.Workspace(B, HV, B * HV * (ns + 1), dev, GT, 128)
+    tkw = {}
+    if tail is not None:
+        dt = tail.to(dev)
+        tkw = dict(tail=dt, tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), tail_bs=dt.stride(0), tail_ts=dt.stride(1))
+    dq, dbt, dseq = q.to(dev), bt.to(dev) if bt_shared != "stride0" else bt.to(dev)[:1].expand(B, -1), seq.to(dev)
+    for rep in range(2):      # second call: the self-resetting tickets must be back at zero
+        out.fill_(float("nan"))
+        if mode == "static":
+            K.v2_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, kmask=mask[:Hkv].to(dev),
+                      vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, **tkw)
+        else:
+            K.cb_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start, **tkw)
+        torch.cuda.synchronize()
+        got = out.view(B, HQ, 128).float().cpu().numpy().astype(np.float64)
+        valid = np.array([min(kv_start, lens[b]) < lens[b] or (tail is not None and int(tail_len[b]) > 0) for b in range(B)])
+        assert not np.isnan(got[valid]).any(), (fmt, lens, "NaN in output")
+        err = np.abs(got - ref)[valid]
+        lim = (ATOL + RTOL * np.abs(ref))[valid]
+        assert (err <= lim).all(), (fmt, lens, ns, ch, float(err.max()), float((err / lim).max()))
+    assert int(ws.counter.abs().sum()) == 0
+    return ns, ch
+
+
+LENS = [1, 15, 16, 17, 63, 64, 65, 200, 1000, 3, 511]
+
+
+@pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
+def test_codebook_decode(dev, kind):
+    run_case(dev, "codebook", LENS, kind, seed=1)
+
+
+@pytest.mark.parametrize("fmt", ["int4", "int4a", "int2a"])
+def test_static_decode(dev, fmt):
+    run_case(dev, "static", LENS, fmt, seed=2)
+
+
+@pytest.mark.parametrize("kind", ["konlya", "konlya2"])
+def test_codebook_decode_long_and_splits(dev, kind):
+    run_case(dev, "codebook", [4097, 33, 2500], kind, seed=3, Hkv=2)
+    run_case(dev, "codebook", [700, 120], kind, seed=4, Hkv=2, nsplit=3)
+    run_case(dev, "codebook", [700, 120], kind, seed=5, Hkv=2, nsplit=1)
+
+
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
+                                      ("static", "int4a"), ("static", "int4"), ("static", "int2a")])
+def test_window_and_kv_start(dev, mode, fmt):
+    run_case(dev, mode, [300, 5, 0, 64, 37], fmt, win=(132, 7), seed=6, Hkv=2, kv_start=4)
+    run_case(dev, mode, [300, 5, 17], fmt, win=(32, 4), seed=7, Hkv=2, kv_start=16)
+    run_case(dev, mode, [90, 40], fmt, seed=8, Hkv=2, kv_start=37)
+
+
+@pytest.mark.parametrize("shared", ["copy", "stride0"])
+def test_shared_block_table_row(dev, shared):
+    run_case(dev, "codebook", [100, 37, 64], "konlya", bt_shared=shared, seed=9, Hkv=2)
+    if shared == "copy":
+        run_case(dev, "static", [100, 37, 64], "int4a", bt_shared=shared, seed=10, Hkv=2)
+
+
+@pytest.mark.parametrize("G,Hkv", [(8, 8), (5, 8), (12, 4), (6, 2), (1, 4)])
+def test_gqa_groups(dev, G, Hkv):
+    run_case(dev, "codebook", [130, 31, 700], "konlya", seed=11, G=G, Hkv=Hkv, win=(40, 5), kv_start=4)
+    run_case(dev, "static", [130, 31, 700], "int4a", seed=12, G=G, Hkv=Hkv)
+    run_case(dev, "codebook", [130, 31], "konlya2", seed=13, G=G, Hkv=Hkv)
+
+
+def test_decode_error_codes(dev):
+    from flagrot_releaser_amd import kernels as K
+    L = K.lib()
+    z = torch.zeros(1024, dtype=torch.uint8, device=dev)
+    zp = z.data_ptr()
+    base = [zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, None, None, 32, 0, 0, 264, 4, zp, zp, zp, zp, 512, None, None,
+            None, 0, 0, None]
+    assert L.fr_v2_attn(99, *base, 4, 0) == -4
+    bad_page = list(base); bad_page[8] = 32
+    assert L.fr_v2_attn(5, *bad_page, 4, 0) == -5
+    assert L.fr_v2_attn(5, *base, 8, 0) == -7            # gqa 8 without the generalised variant bits
+    hd = list(base); hd[17] = 264 | 1024 | 4096
+    assert L.fr_v2_attn(5, *hd, 4, 0) == -8
+    assert L.fr_cb_attn(zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, K.sign_words(), 3, 0, 4, zp, zp, zp, zp, 512, None,
+                        None, None, 0, 0, None, 0) == -4
+    assert L.fr_v2_attn(5, *(base[:6] + [0] + base[7:]), 4, 0) == 0     # B = 0: nothing to do
