@@ -55,50 +55,51 @@ DEVI void wave_lds_sync() {
 
 // ---------------------------------------------------------------------------------------------- code unpacking
 // A 32-bit word of eight 4-bit fields f0..f7 (or, INT2, the 2-bit fields at bit 4 n of a pre-shifted word) becomes
-// four fp16 pairs (f0,f4) (f1,f5) (f2,f6) (f3,f7) with value = OFF[pair] + field.
+// four fp16 pairs (f0,f4) (f1,f5) (f2,f6) (f3,f7): the field is or-ed into the mantissa of 1024.0 (exact), then
+// -(1024 + zero point) is added with one packed fp16 add, which is exact too: the pairs hold code - zero point.
+DEVI uint32_t pk_add(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, as_h2(a) + as_h2(b));
+}
 template <int QM> struct Unpack;
 template <> struct Unpack<QM_ASYM4> {
-  static constexpr float OFF[4] = {1024.f, 64.f, 4.f, 64.f};
-  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
-    x[0] = (w & 0x000F000Fu) | 0x64006400u;
-    x[1] = (w & 0x00F000F0u) | 0x54005400u;
-    x[2] = (w & 0x0F000F00u) | 0x44004400u;
-    x[3] = ((w >> 8) & 0x00F000F0u) | 0x54005400u;
+  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], uint32_t (&x)[4]) {
+    x[0] = pk_add((w & 0x000F000Fu) | 0x64006400u, nz[0]);
+    x[1] = pk_add(((w >> 4) & 0x000F000Fu) | 0x64006400u, nz[1]);
+    x[2] = pk_add(((w >> 8) & 0x000F000Fu) | 0x64006400u, nz[2]);
+    x[3] = pk_add(((w >> 12) & 0x000F000Fu) | 0x64006400u, nz[3]);
   }
 };
 template <> struct Unpack<QM_ASYM2> {
-  static constexpr float OFF[4] = {1024.f, 256.f, 4.f, 256.f};
-  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {  // fields at bits 0, 2, 8, 10 (+16) of w
-    x[0] = (w & 0x00030003u) | 0x64006400u;
-    x[1] = (w & 0x000C000Cu) | 0x5C005C00u;
-    x[2] = (w & 0x03000300u) | 0x44004400u;
-    x[3] = ((w >> 8) & 0x000C000Cu) | 0x5C005C00u;
+  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], uint32_t (&x)[4]) {  // fields at bits 0, 2, 8, 10 (+16)
+    x[0] = pk_add((w & 0x00030003u) | 0x64006400u, nz[0]);
+    x[1] = pk_add(((w >> 2) & 0x00030003u) | 0x64006400u, nz[1]);
+    x[2] = pk_add(((w >> 8) & 0x00030003u) | 0x64006400u, nz[2]);
+    x[3] = pk_add(((w >> 10) & 0x00030003u) | 0x64006400u, nz[3]);
   }
 };
-template <> struct Unpack<QM_SYM4> {  // sign-magnitude bytes s0000mmm -> exact signed fp16, no offset
-  static constexpr float OFF[4] = {0.f, 0.f, 0.f, 0.f};
+template <> struct Unpack<QM_SYM4> {  // sign-magnitude bytes s0000mmm -> exact signed fp16
   static DEVI uint32_t pair(uint32_t bytes02) {  // bytes at bits 0..7 and 16..23
-    const uint32_t m = (bytes02 & 0x00070007u) | 0x64006400u;
-    const half2_t v = as_h2(m) - as_h2(0x64006400u);
-    return __builtin_bit_cast(uint32_t, v) ^ ((bytes02 & 0x00800080u) << 8);
+    const uint32_t m = pk_add((bytes02 & 0x00070007u) | 0x64006400u, 0xE400E400u);
+    return m ^ ((bytes02 & 0x00800080u) << 8);
   }
-  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
+  static DEVI void run(uint32_t w, const uint32_t (&)[4], uint32_t (&x)[4]) {
     const uint32_t a = w & 0x87878787u;                                   // A_i in byte i
     const uint32_t b = ((w << 4) | (w >> 28)) & 0x87878787u;              // B_i in byte i
     x[0] = pair(a); x[1] = pair(b); x[2] = pair(a >> 8); x[3] = pair(b >> 8);
   }
 };
+// fp16 pattern of -(1024 + z)
+DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
 constexpr int NWAVE = 4;
 constexpr int QV_BYTES = 3 * 4 * 16 * 16;          // [variant][head][tg][j][8 fp16]
-constexpr int QC_FLOATS = 3 * 4 * 4 * 2;           // [variant][head][group] (offset sum, plain sum)
 constexpr int PB_BYTES = 2 * 4 * 4 * 16;           // per wave: [c8][group][head][8 fp16]
+constexpr int ZB_BYTES = 2 * 4 * 16;               // per wave: [c8][group][8 fp16] = -(1024 + zero point) per token
 
 struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
-  alignas(16) float qc[QC_FLOATS];
   alignas(16) uint8_t pb[NWAVE][PB_BYTES];
-  alignas(16) float cc[NWAVE][4][4];                // per wave: offset / zero-point sums [head][group]
+  alignas(16) uint8_t zb[NWAVE][ZB_BYTES];
   alignas(16) float o[NWAVE][4][128];
   float m[NWAVE][4], l[NWAVE][4];
   int last;
@@ -108,7 +109,8 @@ struct Smem {
 DEVI int kslot(int isB, int i) { return 2 * (2 * (i & 1) + isB) + (i >> 1); }
 DEVI int vslot(int r8) { return 2 * (r8 & 3) + (r8 >> 2); }
 
-// Rotates the q tile three ways and stores it (times qscale) as fp16 in code-word order; also the per-group sums.
+// Rotates the q tile three ways and stores it as fp16 in code-word order (the identity variant of a bf16 query is
+// exact in fp16; qscale is applied to the fp32 score).
 template <int QM, bool K2>
 DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
   const int w = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
@@ -118,8 +120,7 @@ DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
     const uint16_t* qr = static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
                          (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 4 * l32;
     const uint2 raw = *reinterpret_cast<const uint2*>(qr);
-    x[0] = bf16_lo(raw.x) * p.qscale; x[1] = bf16_hi(raw.x) * p.qscale;
-    x[2] = bf16_lo(raw.y) * p.qscale; x[3] = bf16_hi(raw.y) * p.qscale;
+    x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
   }
   const int g = l32 >> 3;
   // half 0: variants 0 (identity, or the static kmask rotation) and 1 (H32); half 1: variant 2 (H128)
@@ -140,23 +141,11 @@ DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
     }
-    float so = 0.f, ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int d = 4 * l32 + i, r = d & 31;
       const int isB = r >> 4, tg = (r & 15) >> 2, ii = r & 3;
-      const _Float16 hv = static_cast<_Float16>(v[i]);
-      const int slot = kslot(isB, ii);
-      reinterpret_cast<_Float16*>(S.qv)[(((var * 4 + w) * 4 + tg) * 4 + g) * 8 + slot] = hv;
-      const float hf = static_cast<float>(hv);
-      so += hf * Unpack<QM>::OFF[slot >> 1];
-      ss += hf;
-    }
-    so += hx(so, 1); so += hx(so, 2); so += hx(so, 4);
-    ss += hx(ss, 1); ss += hx(ss, 2); ss += hx(ss, 4);
-    if ((l32 & 7) == 0) {
-      S.qc[((var * 4 + w) * 4 + g) * 2 + 0] = so;
-      S.qc[((var * 4 + w) * 4 + g) * 2 + 1] = ss;
+      reinterpret_cast<_Float16*>(S.qv)[(((var * 4 + w) * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i]);
     }
   }
 }
@@ -192,11 +181,11 @@ DEVI void load_page(PageRegs<QM>& r, const uint8_t* chunk, int lane) {
 struct WaveState {
   float m[4], l[4];
   float acc[4][4];   // [head][entry word] of the lane's V^T entry
-  float cc[4];       // [head] running sum of p' * (offset + zero point) of the lane's (token, group) role
 };
 
 template <int QM, bool K2, int P>
-DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, int wave, int tok0, int lo, int hi) {
+DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, int wave, int tok0, int lo, int hi,
+                       float qscale) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   const int t = lane >> 2, tg = lane & 3;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
@@ -206,8 +195,10 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     uint32_t x[4];
-    if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[j >> 1] >> 4) : r.kc[j >> 1], x);
-    else Unpack<QM>::run(r.kc[j], x);
+    const uint32_t nz1 = negz16(kw[j] & ZM) * 0x00010001u;
+    const uint32_t nz[4] = {nz1, nz1, nz1, nz1};
+    if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[j >> 1] >> 4) : r.kc[j >> 1], nz, x);
+    else Unpack<QM>::run(r.kc[j], nz, x);
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
     const float s = f16_value(kw[j] & 0x7FFFu);
     const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + (var * 16 + tg) * 4 + j;   // + head * 16
@@ -221,16 +212,6 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
       part[h] += s * a;
     }
   }
-  if constexpr (QM != QM_SYM4) {  // remove offsets and zero point of group tg (one group per lane of the quad)
-    const uint32_t w = tg == 0 ? kw[0] : tg == 1 ? kw[1] : tg == 2 ? kw[2] : kw[3];
-    const int var = K2 ? (full ? 2 : static_cast<int>(w >> 15)) : 0;
-    const float s = f16_value(w & 0x7FFFu), z = static_cast<float>(w & ZM);
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const float2 c = *reinterpret_cast<const float2*>(&S.qc[((var * 4 + h) * 4 + tg) * 2]);
-      part[h] -= s * (c.x + z * c.y);
-    }
-  }
   const int tok = tok0 + t;
   const bool valid = tok >= lo && tok < hi;
   float p[4];
@@ -239,7 +220,7 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
     float sc = part[h];
     sc += dpp_xor1(sc);
     sc += dpp_xor2(sc);
-    sc = valid ? sc : -INFINITY;
+    sc = valid ? sc * qscale : -INFINITY;
     const float mx = wave_max_over_tokens(sc);
     const float mn = fmaxf(st.m[h], mx);
     const float alpha = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
@@ -248,19 +229,16 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
     st.l[h] = st.l[h] * alpha + wave_sum_over_tokens(p[h]);   // one lane per token: the exchange keeps the quarter
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha;
-    st.cc[h] *= alpha;
   }
-  // ---- p' = p * V scale of (token, group tg), fp16, into the wave's LDS strip in V^T token order
+  // ---- p' = p * V scale of (token, group tg) as fp16, and -(1024 + zero point), into the wave's LDS strips in
+  //      V^T token order
   {
     const float sv = f16_value(r.vs & 0x7FFFu);
-    const float oz = Unpack<QM>::OFF[t & 3] + static_cast<float>(r.vs & ZM);
-    _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + (((t >> 3) * 4 + tg) * 4) * 8 + vslot(t & 7);
+    const int so = ((t >> 3) * 4 + tg) * 8 + vslot(t & 7);
+    _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + 4 * (so & ~7) + (so & 7);
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const _Float16 ph = valid ? static_cast<_Float16>(p[h] * sv) : static_cast<_Float16>(0.f);
-      pb[h * 8] = ph;
-      if constexpr (QM != QM_SYM4) st.cc[h] += static_cast<float>(ph) * oz;
-    }
+    for (int h = 0; h < 4; ++h) pb[h * 8] = valid ? static_cast<_Float16>(p[h] * sv) : static_cast<_Float16>(0.f);
+    if constexpr (QM != QM_SYM4) reinterpret_cast<uint16_t*>(S.zb[wave])[so] = static_cast<uint16_t>(negz16(r.vs & ZM));
   }
   wave_lds_sync();
   // ---- value phase: lane = V^T entry (w = lane >> 4, gid, c8 = lane & 1)
@@ -270,11 +248,18 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
     uint4 pa[4], pc[4];
 #pragma unroll
     for (int h = 0; h < 4; ++h) { pa[h] = pp[g0 * 4 + h]; pc[h] = pp[(2 + g0) * 4 + h]; }
+    uint4 za = make_uint4(0, 0, 0, 0), zc = za;
+    if constexpr (QM != QM_SYM4) {
+      const uint4* zp = reinterpret_cast<const uint4*>(S.zb[wave]) + c8 * 4;
+      za = zp[g0]; zc = zp[2 + g0];
+    }
 #pragma unroll
     for (int sub = 0; sub < 4; ++sub) {
       uint32_t x[4];
-      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[sub >> 1] >> 4) : r.vc[sub >> 1], x);
-      else Unpack<QM>::run(r.vc[sub], x);
+      const uint4 zz = sub < 2 ? za : zc;
+      const uint32_t nz[4] = {zz.x, zz.y, zz.z, zz.w};
+      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[sub >> 1] >> 4) : r.vc[sub >> 1], nz, x);
+      else Unpack<QM>::run(r.vc[sub], nz, x);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const uint4 pq = sub < 2 ? pa[h] : pc[h];
@@ -346,7 +331,7 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     WaveState st;
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      st.m[h] = -INFINITY; st.l[h] = 0.f; st.cc[h] = 0.f;
+      st.m[h] = -INFINITY; st.l[h] = 0.f;
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] = 0.f;
     }
@@ -361,7 +346,7 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
       for (; pg < pg1; pg += NWAVE) {
         const int pn = pg + NWAVE;
         if (pn < pg1) load_page<QM, P>(nxt, p.pool + (static_cast<long long>(bt[pn]) * p.Hkv + kvh) * L::CHUNK, lane);
-        process_page<QM, K2, P>(S, st, cur, lane, wave, pg * P, lo, hi);
+        process_page<QM, K2, P>(S, st, cur, lane, wave, pg * P, lo, hi, p.qscale);
         cur = nxt;
       }
     }
@@ -370,14 +355,11 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     for (int h = 0; h < 4; ++h) {
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
-      float c = st.cc[h];   // lanes with the same quarter tg hold group tg
-      c += swz_xor<4>(c); c += swz_xor<8>(c); c += swz_xor<16>(c); c += xor32(c);
-      if (lane < 4) S.cc[wave][h][lane] = c;
       if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = st.l[h]; }
     }
     __syncthreads();
     {
-      const int wq = lane >> 4, gid = (lane >> 1) & 7, g0 = lane >> 5;
+      const int wq = lane >> 4, gid = (lane >> 1) & 7;
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         float M = fmaxf(fmaxf(S.m[0][h], S.m[1][h]), fmaxf(S.m[2][h], S.m[3][h]));
@@ -386,8 +368,7 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
 #pragma unroll
           for (int sub = 0; sub < 4; ++sub) {
             const int d = 64 * (sub >> 1) + 16 * wq + gid + 8 * (sub & 1);
-            const float cc = S.cc[wave][h][2 * (sub >> 1) + g0];
-            S.o[wave][h][d] = f * (st.acc[h][sub] - cc);
+            S.o[wave][h][d] = f * st.acc[h][sub];
           }
         }
       }
