@@ -1,0 +1,206 @@
+"""Headline benchmark: paged FlagRot decode attention on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2]
+
+A step is one decode layer-step: one launch of the paged decode attention (through the C ABI of
+libflagrot_kernels.so) over the whole batch, on a synthetic cache that is already resident in HBM.  Successive steps
+cycle through several distinct copies of the cache so that no page is served from the last-level cache.
+
+Workloads (BASELINE.json configs):
+  int4  configs[1]: INT4 FlagRot (key-only 2x2 codebook, kind konlya), Llama-3.1-8B GQA shape 32q/8kv, d=128,
+        batch 32, context 8192, page 16, randomly permuted page table.                       [default, headline]
+  int2  configs[2]: INT2 FlagRot (kind konlya2) with static key centring, 4 sink + 128 window BF16 tokens,
+        batch 64, context 16384.
+Prints ONE JSON line: value = achieved GB/s of page bytes (the reference's convention: B * L * Hkv * bytes per token),
+with `roofline` (HBM, measured with events on the launch stream) and `cpu_baseline` (the numpy oracle's
+dequantise-then-attend path, timed on the host on configs[0]'s shape).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+LOG2E = 1.4426950408889634
+PEAK_HBM_GBPS = 8000.0
+P, HKV, G, DH = 16, 8, 4, 128
+
+
+def synth_kv(T, g, dev, torch, outliers=4, gain=8.0, mu=None):
+    """K ~ N(0,1) with `outliers` channels per head x gain and per-token norms ~ lognormal(0, 0.5); V ~ N(0,1)."""
+    kv = torch.randn(T, 2 * HKV, DH, generator=g, device=dev)
+    for h in range(HKV):
+        ch = torch.randint(0, DH, (outliers,), generator=g, device=dev)
+        kv[:, h, ch] *= gain
+    kv[:, :HKV] *= torch.exp(0.5 * torch.randn(T, 1, 1, generator=g, device=dev))
+    if mu is not None:
+        kv[:, :HKV] += mu[None]
+    return kv.bfloat16()
+
+
+def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192):
+    """fills one pool with B sequences of L tokens through the selecting writer; returns pool, block table, calib."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    npages = B * ((L + P - 1) // P)
+    pool = torch.zeros(npages + 16, HKV, K.cb_chunk_bytes(kind, P), dtype=torch.uint8, device=dev)
+    perm = torch.randperm(npages + 16, generator=g, device=dev)[:npages].int()
+    bt = perm.view(B, -1).contiguous()
+    w = 0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)
+    CT = torch.diag_embed(w).contiguous()                      # C_q = diag(w) (symmetric: C^T = C)
+    co = w.contiguous()
+    t0 = time.perf_counter()
+    for b in range(B):
+        for s in range(0, L, chunk_tokens):
+            n = min(chunk_tokens, L - s)
+            kv = synth_kv(n, g, dev, torch, mu=kmu)
+            pos = torch.arange(s, s + n, device=dev)
+            slots = bt[b].long()[pos // P] * P + pos % P
+            K.cb_write(kv, slots, CT, co, kind, pool, P, kmu=kmu)
+    torch.cuda.synchronize()
+    return pool, bt, CT, co, time.perf_counter() - t0
+
+
+def cpu_baseline(torch, K, dev):
+    """the oracle's decode path (page parse + dequantise + inverse transforms + fp64 softmax attention) on
+    configs[0]'s shape: batch 1, context 2048, 32q/8kv; the cache bytes come from the HIP writer."""
+    import numpy as np
+    from oracle import attend as A
+    kind, L = "konly", 2048
+    pool, bt, CT, co, _ = build_cache(torch, K, dev, kind, 1, L, seed=0)
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, G * HKV, DH, generator=g).bfloat16()
+    qb = q.view(torch.int16).numpy().view(np.uint16)
+    hp, hbt = pool.cpu().numpy(), bt.cpu().numpy()
+    ts = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        A.decode_reference(qb, hp, kind, P, hbt, [L], 1 / math.sqrt(DH))
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts[1:])[len(ts[1:]) // 2]
+    nbytes = L * HKV * 144
+    try:
+        from threadpoolctl import threadpool_info
+        cores = max([i.get("num_threads", 1) for i in threadpool_info()] + [1])
+    except Exception:
+        cores = 1
+    return {"value": round(nbytes / t / 1e9, 6), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"numpy oracle decode_reference, B=1 L={L} 32q/8kv INT4 (konly) pages = {nbytes} page bytes, "
+                      f"median of 3 after 1 warm-up: {t * 1e6:.0f} us per layer-step; host has {os.cpu_count()} cpus"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="int4", choices=["int4", "int2"])
+    ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU (every (sequence, KV head) is independent; see DESIGN.md "
+              "for how it shards); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from flagrot_releaser_amd import kernels as K
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    K.lib()
+    if args.workload == "int4":
+        kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144
+        name = "configs[1]: INT4 FlagRot konlya paged decode, Llama-3.1-8B GQA 32q/8kv d=128, B=32 L=8192 page=16"
+    else:
+        kind, B, L, S, W, cell = "konlya2", 64, 16384, 4, 128, 80
+        name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
+                "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
+    g = torch.Generator(device=dev).manual_seed(1)
+    kmu = None
+    if args.workload == "int2":
+        kmu = (2.0 * torch.randn(HKV, DH, generator=g, device=dev)).contiguous()
+    pool, bt, CT, co, fill_s = build_cache(torch, K, dev, kind, B, L, seed=1, kmu=kmu)
+    pool_bytes = pool.numel()
+    ncopy = max(1, min(8, int(6e9 // pool_bytes)))
+    pools = [pool] + [pool.clone() for _ in range(ncopy - 1)]
+    q = torch.randn(B, G * HKV, DH, generator=g, device=dev).bfloat16()
+    out = torch.zeros(B, G * HKV * DH, dtype=torch.bfloat16, device=dev)
+    T = S + W
+    tkw = {}
+    Lpages = L - W if T else L                      # the newest W tokens live in the BF16 ring, not in pages
+    seq = torch.full((B,), Lpages, dtype=torch.int32, device=dev)
+    if T:
+        ring = torch.randn(B + 1, T, 2 * HKV, DH, generator=g, device=dev).bfloat16()
+        tkw = dict(tail=ring, tail_len=torch.full((B,), T, dtype=torch.int32, device=dev),
+                   tail_idx=torch.arange(B, dtype=torch.int32, device=dev), tail_bs=ring.stride(0),
+                   tail_ts=ring.stride(1), kv_start=S)
+    ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None)
+    ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
+    scale = LOG2E / math.sqrt(DH)
+
+    def step(i):
+        K.cb_attn(q, pools[i % ncopy], bt, seq, out, ns, ch, ws, scale, kind, **tkw)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(args.steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
+    total_ms = ev[0].elapsed_time(ev[-1])
+    ms_per_step = total_ms / args.steps
+    page_bytes = B * (Lpages - S) * HKV * cell
+    tail_bytes = B * T * 2 * HKV * DH * 2
+    alg_bytes = page_bytes + tail_bytes
+    gbps = alg_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
+    kv_new = synth_kv(B, g, dev, torch, mu=kmu)
+    slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
+    for _ in range(3):
+        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
+    e1.record()
+    torch.cuda.synchronize()
+    writer_us = e0.elapsed_time(e1) / 20 * 1e3
+
+    res = {
+        "metric": "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "us_per_layer_step": round(ms_per_step * 1e3, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 codes, fp16 products, f32 accumulate",
+        "data": "synthetic", "config": {"workload": name, "nsplit": ns, "chunk": ch, "cache_copies_cycled": ncopy,
+                                         "sink": S, "window": W},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(ms_per_step * 1e3, 2),
+                     "median_launch_us": round(per[len(per) // 2] * 1e3, 2), "min_launch_us": round(per[0] * 1e3, 2)},
+        "writer": {"decode_step_us": round(writer_us, 2), "decode_step_tokens": B,
+                   "prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * L,
+                   "note": "prefill_fill_s includes synthetic input generation"},
+        "host_wall_s": round(wall, 4),
+    }
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline(torch, K, dev)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -93,8 +93,8 @@ DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
 constexpr int NWAVE = 4;
 constexpr int QV_BYTES = 3 * 4 * 16 * 16;          // [variant][head][tg][j][8 fp16]
-constexpr int PB_BYTES = 2 * 4 * 4 * 16;           // per wave: [c8][group][head][8 fp16]
-constexpr int ZB_BYTES = 2 * 4 * 16;               // per wave: [c8][group][8 fp16] = -(1024 + zero point) per token
+constexpr int PB_BYTES = 4 * 2 * 4 * 4 * 16;       // per wave: [page][c8][group][head][8 fp16]
+constexpr int ZB_BYTES = 4 * 2 * 4 * 16;           // per wave: [page][c8][group][8 fp16] = -(1024 + zero point)
 
 struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
@@ -150,107 +150,165 @@ DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
   }
 }
 
-template <int QM> struct PageRegs {
-  uint32_t kc[QM == QM_ASYM2 ? 2 : 4];
-  uint32_t vc[QM == QM_ASYM2 ? 2 : 4];
+// One wave iteration covers 4 consecutive pages = 64 tokens.  Key phase: lane = token (page lane >> 4, position
+// lane & 15).  Value phase: lane = V^T entry `lane` of each of the 4 pages in turn.
+template <int QM> struct KRegs {
+  static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;   // code words per 16-byte / 8-byte quarter row
+  uint32_t kc[4][NW];       // [quarter tg][word]
   uint2 ks;                 // the token's 4 K scale words
-  uint32_t vs, vs0;         // V scale word of (token, group = quarter), of (token, group 0)
+  uint32_t vs[4];           // the token's 4 V scale words (one per group)
+};
+template <int QM> struct VRegs {
+  static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;
+  uint32_t vc[4][NW];       // [page][entry word]
 };
 
 template <int QM, int P>
-DEVI void load_page(PageRegs<QM>& r, const uint8_t* chunk, int lane) {
+DEVI void load_k(KRegs<QM>& r, const uint8_t* chunk, int pos) {
   using L = Lay<QM, P>;
-  const int t = lane >> 2, tg = lane & 3;
   if constexpr (QM == QM_ASYM2) {
-    const uint2 k = *reinterpret_cast<const uint2*>(chunk + L::K_OFF + 32 * (t ^ ((t >> 1) & 2)) + 8 * tg);
-    r.kc[0] = k.x; r.kc[1] = k.y;
-    const uint2 v = *reinterpret_cast<const uint2*>(chunk + L::V_OFF + 8 * lane);
-    r.vc[0] = v.x; r.vc[1] = v.y;
+    const uint8_t* row = chunk + L::K_OFF + 32 * (pos ^ ((pos >> 1) & 2));
+#pragma unroll
+    for (int tg = 0; tg < 4; ++tg) {
+      const uint2 k = *reinterpret_cast<const uint2*>(row + 8 * tg);
+      r.kc[tg][0] = k.x; r.kc[tg][1] = k.y;
+    }
   } else {
-    const uint4 k = *reinterpret_cast<const uint4*>(chunk + L::K_OFF + 64 * t + 16 * tg);
-    r.kc[0] = k.x; r.kc[1] = k.y; r.kc[2] = k.z; r.kc[3] = k.w;
-    const uint4 v = *reinterpret_cast<const uint4*>(chunk + L::V_OFF + 16 * lane);
-    r.vc[0] = v.x; r.vc[1] = v.y; r.vc[2] = v.z; r.vc[3] = v.w;
+    const uint8_t* row = chunk + L::K_OFF + 64 * pos;
+#pragma unroll
+    for (int tg = 0; tg < 4; ++tg) {
+      const uint4 k = *reinterpret_cast<const uint4*>(row + 16 * tg);
+      r.kc[tg][0] = k.x; r.kc[tg][1] = k.y; r.kc[tg][2] = k.z; r.kc[tg][3] = k.w;
+    }
   }
-  r.ks = *reinterpret_cast<const uint2*>(chunk + L::KS_OFF + 8 * t);
-  const int vo = L::VS_OFF + (8 * (t >> 3) + vs_slot8(t)) * 2;
-  r.vs = *reinterpret_cast<const uint16_t*>(chunk + vo + tg * P * 2);
-  r.vs0 = *reinterpret_cast<const uint16_t*>(chunk + vo);
+  r.ks = *reinterpret_cast<const uint2*>(chunk + L::KS_OFF + 8 * pos);
+  const uint8_t* vo = chunk + L::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) r.vs[g] = *reinterpret_cast<const uint16_t*>(vo + g * P * 2);
+}
+
+template <int QM, int P>
+DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
+  using L = Lay<QM, P>;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if constexpr (QM == QM_ASYM2) {
+      const uint2 v = *reinterpret_cast<const uint2*>(chunk[k] + L::V_OFF + 8 * lane);
+      r.vc[k][0] = v.x; r.vc[k][1] = v.y;
+    } else {
+      const uint4 v = *reinterpret_cast<const uint4*>(chunk[k] + L::V_OFF + 16 * lane);
+      r.vc[k][0] = v.x; r.vc[k][1] = v.y; r.vc[k][2] = v.z; r.vc[k][3] = v.w;
+    }
+  }
 }
 
 struct WaveState {
-  float m[4], l[4];
-  float acc[4][4];   // [head][entry word] of the lane's V^T entry
+  float m[4];        // running maximum per head (wave uniform)
+  float l[4];        // this lane's share of the running sum per head
+  float acc[4][4];   // [head][entry word] of the lane's V^T entries
 };
 
-template <int QM, bool K2, int P>
-DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, int wave, int tok0, int lo, int hi,
-                       float qscale) {
+DEVI float wave_max64(float v) {
+  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
+  return wave_max_over_tokens(v);
+}
+DEVI float wave_sum64(float v) {
+  v += dpp_xor1(v); v += dpp_xor2(v);
+  return wave_sum_over_tokens(v);
+}
+
+// scores of the lane's token against the 4 q heads (log2 domain, unmasked)
+template <int QM, bool K2>
+DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
-  const int t = lane >> 2, tg = lane & 3;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
-  const bool full = K2 && (r.vs0 & 0x8000u);
-  float part[4] = {0.f, 0.f, 0.f, 0.f};
-  // ---- key phase
+  const bool full = K2 && (r.vs[0] & 0x8000u);
+  float a[4][4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    uint32_t x[4];
     const uint32_t nz1 = negz16(kw[j] & ZM) * 0x00010001u;
     const uint32_t nz[4] = {nz1, nz1, nz1, nz1};
-    if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[j >> 1] >> 4) : r.kc[j >> 1], nz, x);
-    else Unpack<QM>::run(r.kc[j], nz, x);
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
-    const float s = f16_value(kw[j] & 0x7FFFu);
-    const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + (var * 16 + tg) * 4 + j;   // + head * 16
+    const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + var * 64 + j;   // + head * 16 + tg * 4
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const uint4 qq = qp[h * 16];
-      float a = dot2(x[0], qq.x, 0.f);
-      a = dot2(x[1], qq.y, a);
-      a = dot2(x[2], qq.z, a);
-      a = dot2(x[3], qq.w, a);
-      part[h] += s * a;
+    for (int tg = 0; tg < 4; ++tg) {
+      uint32_t x[4];
+      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], nz, x);
+      else Unpack<QM>::run(r.kc[tg][j], nz, x);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const uint4 qq = qp[h * 16 + tg * 4];
+        float v = tg == 0 ? 0.f : a[j][h];
+        v = dot2(x[0], qq.x, v);
+        v = dot2(x[1], qq.y, v);
+        v = dot2(x[2], qq.z, v);
+        v = dot2(x[3], qq.w, v);
+        a[j][h] = v;
+      }
     }
   }
-  const int tok = tok0 + t;
-  const bool valid = tok >= lo && tok < hi;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    float v = f16_value(kw[0] & 0x7FFFu) * a[0][h];
+#pragma unroll
+    for (int j = 1; j < 4; ++j) v += f16_value(kw[j] & 0x7FFFu) * a[j][h];
+    sc[h] = v * qscale;
+  }
+}
+
+// online softmax step for 64 tokens: the running maximum is only re-reduced over the wave when some lane beats it
+template <int QM>
+DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], bool valid, int lane, int wave) {
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  bool beat = false;
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    sc[h] = valid ? sc[h] : -INFINITY;
+    beat |= sc[h] > st.m[h];
+  }
+  if (__any(beat)) {
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const float mn = fmaxf(st.m[h], wave_max64(sc[h]));
+      const float alpha = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
+      st.m[h] = mn;
+      st.l[h] *= alpha;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha;
+    }
+  }
+  const int pi = lane >> 4, pos = lane & 15;
   float p[4];
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
-    float sc = part[h];
-    sc += dpp_xor1(sc);
-    sc += dpp_xor2(sc);
-    sc = valid ? sc * qscale : -INFINITY;
-    const float mx = wave_max_over_tokens(sc);
-    const float mn = fmaxf(st.m[h], mx);
-    const float alpha = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
-    p[h] = valid ? fexp2(sc - mn) : 0.f;
-    st.m[h] = mn;
-    st.l[h] = st.l[h] * alpha + wave_sum_over_tokens(p[h]);   // one lane per token: the exchange keeps the quarter
-#pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha;
+    p[h] = valid ? fexp2(sc[h] - st.m[h]) : 0.f;
+    st.l[h] += p[h];
   }
-  // ---- p' = p * V scale of (token, group tg) as fp16, and -(1024 + zero point), into the wave's LDS strips in
-  //      V^T token order
-  {
-    const float sv = f16_value(r.vs & 0x7FFFu);
-    const int so = ((t >> 3) * 4 + tg) * 8 + vslot(t & 7);
-    _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + 4 * (so & ~7) + (so & 7);
+  // p' = p * V scale per group as fp16, and -(1024 + zero point), in V^T token order of the token's page
+  const int so = (pi * 2 + (pos >> 3)) * 32 + vslot(pos & 7);           // + group * 8
+  _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + 4 * (so & ~7) + (so & 7);
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb[wave]) + so;
 #pragma unroll
-    for (int h = 0; h < 4; ++h) pb[h * 8] = valid ? static_cast<_Float16>(p[h] * sv) : static_cast<_Float16>(0.f);
-    if constexpr (QM != QM_SYM4) reinterpret_cast<uint16_t*>(S.zb[wave])[so] = static_cast<uint16_t>(negz16(r.vs & ZM));
+  for (int g = 0; g < 4; ++g) {
+    const float sv = f16_value(r.vs[g] & 0x7FFFu);
+#pragma unroll
+    for (int h = 0; h < 4; ++h) pb[(g * 4 + h) * 8] = valid ? static_cast<_Float16>(p[h] * sv) : static_cast<_Float16>(0.f);
+    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<uint16_t>(negz16(r.vs[g] & ZM));
   }
-  wave_lds_sync();
-  // ---- value phase: lane = V^T entry (w = lane >> 4, gid, c8 = lane & 1)
-  {
-    const int c8 = lane & 1, g0 = lane >> 5;
-    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + (c8 * 4) * 4;   // + group * 4 + head
+}
+
+template <int QM>
+DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
+  const int c8 = lane & 1, g0 = lane >> 5;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + ((k * 2 + c8) * 4) * 4;   // + group * 4 + head
     uint4 pa[4], pc[4];
 #pragma unroll
     for (int h = 0; h < 4; ++h) { pa[h] = pp[g0 * 4 + h]; pc[h] = pp[(2 + g0) * 4 + h]; }
     uint4 za = make_uint4(0, 0, 0, 0), zc = za;
     if constexpr (QM != QM_SYM4) {
-      const uint4* zp = reinterpret_cast<const uint4*>(S.zb[wave]) + c8 * 4;
+      const uint4* zp = reinterpret_cast<const uint4*>(S.zb[wave]) + (k * 2 + c8) * 4;
       za = zp[g0]; zc = zp[2 + g0];
     }
 #pragma unroll
@@ -258,8 +316,8 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
       uint32_t x[4];
       const uint4 zz = sub < 2 ? za : zc;
       const uint32_t nz[4] = {zz.x, zz.y, zz.z, zz.w};
-      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[sub >> 1] >> 4) : r.vc[sub >> 1], nz, x);
-      else Unpack<QM>::run(r.vc[sub], nz, x);
+      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], nz, x);
+      else Unpack<QM>::run(r.vc[k][sub], nz, x);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const uint4 pq = sub < 2 ? pa[h] : pc[h];
@@ -272,7 +330,6 @@ DEVI void process_page(Smem& S, WaveState& st, const PageRegs<QM>& r, int lane, 
       }
     }
   }
-  wave_lds_sync();
 }
 
 // BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
@@ -340,14 +397,43 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
       __syncthreads();
       const int pg0 = lo / P, pg1 = (hi + P - 1) / P;
       const int* bt = p.block_table + static_cast<long long>(b) * p.bt_stride;
-      PageRegs<QM> cur, nxt;
-      int pg = pg0 + wave;
-      if (pg < pg1) load_page<QM, P>(cur, p.pool + (static_cast<long long>(bt[pg]) * p.Hkv + kvh) * L::CHUNK, lane);
-      for (; pg < pg1; pg += NWAVE) {
-        const int pn = pg + NWAVE;
-        if (pn < pg1) load_page<QM, P>(nxt, p.pool + (static_cast<long long>(bt[pn]) * p.Hkv + kvh) * L::CHUNK, lane);
-        process_page<QM, K2, P>(S, st, cur, lane, wave, pg * P, lo, hi, p.qscale);
+      const int pi = lane >> 4, pos = lane & 15;
+      auto chunk_of = [&](int pg) {   // pages past the range read the last page of the range; their tokens are masked
+        return p.pool + (static_cast<long long>(bt[min(pg, pg1 - 1)]) * p.Hkv + kvh) * L::CHUNK;
+      };
+      KRegs<QM> cur, nxt;
+      int q4 = pg0 + 4 * wave;       // first page of this wave's current quad
+      const uint8_t* mine = chunk_of(q4 + pi);
+      if (q4 < pg1) load_k<QM, P>(cur, mine, pos);
+      for (; q4 < pg1; q4 += 4 * NWAVE) {
+        VRegs<QM> vr;
+        {
+          const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
+          const uint8_t* ch[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const uint32_t lo32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp), 16 * k);
+            const uint32_t hi32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp >> 32), 16 * k);
+            ch[k] = reinterpret_cast<const uint8_t*>((static_cast<unsigned long long>(hi32) << 32) | lo32);
+          }
+          load_v<QM, P>(vr, ch, lane);
+        }
+        const int qn = q4 + 4 * NWAVE;
+        const uint8_t* mine_n = mine;
+        if (qn < pg1) {
+          mine_n = chunk_of(qn + pi);
+          load_k<QM, P>(nxt, mine_n, pos);
+        }
+        const int tok = (q4 + pi) * P + pos;
+        const bool valid = tok >= lo && tok < hi;
+        float sc[4];
+        key_phase<QM, K2>(S, cur, p.qscale, sc);
+        softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
+        wave_lds_sync();
+        value_phase<QM>(S, st, vr, lane, wave);
+        wave_lds_sync();
         cur = nxt;
+        mine = mine_n;
       }
     }
     // ---- fold the wave: entry pairs (c8 = 0 / 1), offset sums per (head, group)
@@ -355,7 +441,8 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     for (int h = 0; h < 4; ++h) {
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
-      if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = st.l[h]; }
+      const float lsum = wave_sum64(st.l[h]);
+      if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = lsum; }
     }
     __syncthreads();
     {
@@ -423,21 +510,29 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     }
   }
   if (nparts > 1) {
+    // Partials cross workgroups (and XCDs, each with its own L2) through device-scope relaxed atomic stores / loads,
+    // which are write-through / read-through; a device-scope fence here would write back and invalidate the whole
+    // L2 once per workgroup.  Order: stores acknowledged (workgroup release = wait for the store counter), barrier,
+    // ticket; the last arriver reads after its ticket returned.
     float* op = p.opart + part_id * 512 + oh * 128 + 2 * lane;
-    *reinterpret_cast<float2*>(op) = make_float2(po[0], po[1]);
-    if (lane == 0) *reinterpret_cast<float2*>(p.mlpart + part_id * 8 + 2 * oh) = make_float2(pm, pl);
-    __threadfence();
+    __hip_atomic_store(op, po[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(op + 1, po[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) {
+      __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh, pm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh + 1, pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     const int tpc = p.counter_div;                               // q tiles that share one counter slot
     int* ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
     if (threadIdx.x == 0) {
-      const int prev = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      const int prev = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       S.last = prev == tpc * nparts - 1;
       if (S.last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!S.last) return;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
   // ---- final merge (last arriving workgroup, or the only one): all tiles of this counter slot
   const int tpc = nparts > 1 ? p.counter_div : 1;
@@ -447,15 +542,15 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     if (nparts > 1) {
       const long long base = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tt) * nparts;
       M = -INFINITY;
-      for (int s = 0; s < nparts; ++s) M = fmaxf(M, p.mlpart[(base + s) * 8 + 2 * oh]);
+      for (int s = 0; s < nparts; ++s) M = fmaxf(M, __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
       Lsum = 0.f; o0 = 0.f; o1 = 0.f;
       for (int s = 0; s < nparts; ++s) {
-        const float ms = p.mlpart[(base + s) * 8 + 2 * oh];
-        const float ls = p.mlpart[(base + s) * 8 + 2 * oh + 1];
+        const float ms = __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float ls = __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const float f = ms == -INFINITY ? 0.f : fexp2(ms - M);
         Lsum += f * ls;
-        o0 += f * p.opart[(base + s) * 512 + oh * 128 + 2 * lane];
-        o1 += f * p.opart[(base + s) * 512 + oh * 128 + 2 * lane + 1];
+        o0 += f * __hip_atomic_load(p.opart + (base + s) * 512 + oh * 128 + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        o1 += f * __hip_atomic_load(p.opart + (base + s) * 512 + oh * 128 + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
     const float inv = Lsum > 0.f ? 1.f / Lsum : 0.f;
