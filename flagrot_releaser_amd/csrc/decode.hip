@@ -61,40 +61,53 @@ DEVI uint32_t pk_add(uint32_t a, uint32_t b) {
   return __builtin_bit_cast(uint32_t, as_h2(a) + as_h2(b));
 }
 template <int QM> struct Unpack;
+// MAGIC (the fp16 pattern of 1024.0 twice) is kept in a register the compiler cannot constant-fold, so that
+// (w & mask) | MAGIC is a single v_and_or_b32 (one literal per instruction).
+struct Consts { uint32_t magic; };
+DEVI Consts make_consts() {
+  Consts c;
+  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(c.magic));
+  return c;
+}
 template <> struct Unpack<QM_ASYM4> {
-  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], uint32_t (&x)[4]) {
-    x[0] = pk_add((w & 0x000F000Fu) | 0x64006400u, nz[0]);
-    x[1] = pk_add(((w >> 4) & 0x000F000Fu) | 0x64006400u, nz[1]);
-    x[2] = pk_add(((w >> 8) & 0x000F000Fu) | 0x64006400u, nz[2]);
-    x[3] = pk_add(((w >> 12) & 0x000F000Fu) | 0x64006400u, nz[3]);
+  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], const Consts& c, uint32_t (&x)[4]) {
+    x[0] = pk_add((w & 0x000F000Fu) | c.magic, nz[0]);
+    x[1] = pk_add(((w >> 4) & 0x000F000Fu) | c.magic, nz[1]);
+    x[2] = pk_add(((w >> 8) & 0x000F000Fu) | c.magic, nz[2]);
+    x[3] = pk_add(((w >> 12) & 0x000F000Fu) | c.magic, nz[3]);
   }
 };
 template <> struct Unpack<QM_ASYM2> {
-  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], uint32_t (&x)[4]) {  // fields at bits 0, 2, 8, 10 (+16)
-    x[0] = pk_add((w & 0x00030003u) | 0x64006400u, nz[0]);
-    x[1] = pk_add(((w >> 2) & 0x00030003u) | 0x64006400u, nz[1]);
-    x[2] = pk_add(((w >> 8) & 0x00030003u) | 0x64006400u, nz[2]);
-    x[3] = pk_add(((w >> 10) & 0x00030003u) | 0x64006400u, nz[3]);
+  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], const Consts& c, uint32_t (&x)[4]) {  // fields at bits 0, 2, 8, 10 (+16)
+    x[0] = pk_add((w & 0x00030003u) | c.magic, nz[0]);
+    x[1] = pk_add(((w >> 2) & 0x00030003u) | c.magic, nz[1]);
+    x[2] = pk_add(((w >> 8) & 0x00030003u) | c.magic, nz[2]);
+    x[3] = pk_add(((w >> 10) & 0x00030003u) | c.magic, nz[3]);
   }
 };
 template <> struct Unpack<QM_SYM4> {  // sign-magnitude bytes s0000mmm -> exact signed fp16
-  static DEVI uint32_t pair(uint32_t bytes02) {  // bytes at bits 0..7 and 16..23
-    const uint32_t m = pk_add((bytes02 & 0x00070007u) | 0x64006400u, 0xE400E400u);
+  static DEVI uint32_t pair(uint32_t bytes02, const Consts& c) {  // bytes at bits 0..7 and 16..23
+    const uint32_t m = pk_add((bytes02 & 0x00070007u) | c.magic, 0xE400E400u);
     return m ^ ((bytes02 & 0x00800080u) << 8);
   }
-  static DEVI void run(uint32_t w, const uint32_t (&)[4], uint32_t (&x)[4]) {
+  static DEVI void run(uint32_t w, const uint32_t (&)[4], const Consts& c, uint32_t (&x)[4]) {
     const uint32_t a = w & 0x87878787u;                                   // A_i in byte i
     const uint32_t b = ((w << 4) | (w >> 28)) & 0x87878787u;              // B_i in byte i
-    x[0] = pair(a); x[1] = pair(b); x[2] = pair(a >> 8); x[3] = pair(b >> 8);
+    x[0] = pair(a, c); x[1] = pair(b, c); x[2] = pair(a >> 8, c); x[3] = pair(b >> 8, c);
   }
 };
 // fp16 pattern of -(1024 + z)
 DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
 constexpr int NWAVE = 4;
-constexpr int QV_BYTES = 3 * 4 * 16 * 16;          // [variant][head][tg][j][8 fp16]
-constexpr int PB_BYTES = 4 * 2 * 4 * 4 * 16;       // per wave: [page][c8][group][head][8 fp16]
-constexpr int ZB_BYTES = 4 * 2 * 4 * 16;           // per wave: [page][c8][group][8 fp16] = -(1024 + zero point)
+// LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per variant /
+// per row group) start in different banks.
+constexpr int QV_VSTRIDE = 65;                     // uint4 per variant: 64 + 1 pad
+constexpr int QV_BYTES = 3 * QV_VSTRIDE * 16;      // [variant][head][tg][j][8 fp16]
+constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (page, c8): 16 + 1 pad
+constexpr int PB_BYTES = 8 * PB_RSTRIDE * 16;      // per wave: [page][c8][group][head][8 fp16]
+constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
+constexpr int ZB_BYTES = 8 * ZB_RSTRIDE * 16;      // per wave: [page][c8][group][8 fp16] = -(1024 + zero point)
 
 struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
@@ -145,9 +158,18 @@ DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
     for (int i = 0; i < 4; ++i) {
       const int d = 4 * l32 + i, r = d & 31;
       const int isB = r >> 4, tg = (r & 15) >> 2, ii = r & 3;
-      reinterpret_cast<_Float16*>(S.qv)[(((var * 4 + w) * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i]);
+      reinterpret_cast<_Float16*>(S.qv)[(var * QV_VSTRIDE + (w * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i]);
     }
   }
+}
+
+// Page loads are forced into the global address space: a generic (flat) load also counts on the LDS counter, so
+// every wait for an LDS read would wait for the page data in flight as well.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T> DEVI T gload(const uint8_t* p) {
+  typedef const __attribute__((address_space(1))) T* gp;
+  return *(gp)(p);
 }
 
 // One wave iteration covers 4 consecutive pages = 64 tokens.  Key phase: lane = token (page lane >> 4, position
@@ -170,21 +192,21 @@ DEVI void load_k(KRegs<QM>& r, const uint8_t* chunk, int pos) {
     const uint8_t* row = chunk + L::K_OFF + 32 * (pos ^ ((pos >> 1) & 2));
 #pragma unroll
     for (int tg = 0; tg < 4; ++tg) {
-      const uint2 k = *reinterpret_cast<const uint2*>(row + 8 * tg);
+      const u32x2 k = gload<u32x2>(row + 8 * tg);
       r.kc[tg][0] = k.x; r.kc[tg][1] = k.y;
     }
   } else {
     const uint8_t* row = chunk + L::K_OFF + 64 * pos;
 #pragma unroll
     for (int tg = 0; tg < 4; ++tg) {
-      const uint4 k = *reinterpret_cast<const uint4*>(row + 16 * tg);
+      const u32x4 k = gload<u32x4>(row + 16 * tg);
       r.kc[tg][0] = k.x; r.kc[tg][1] = k.y; r.kc[tg][2] = k.z; r.kc[tg][3] = k.w;
     }
   }
-  r.ks = *reinterpret_cast<const uint2*>(chunk + L::KS_OFF + 8 * pos);
+  { const u32x2 t2 = gload<u32x2>(chunk + L::KS_OFF + 8 * pos); r.ks = make_uint2(t2.x, t2.y); }
   const uint8_t* vo = chunk + L::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) r.vs[g] = *reinterpret_cast<const uint16_t*>(vo + g * P * 2);
+  for (int g = 0; g < 4; ++g) r.vs[g] = gload<uint16_t>(vo + g * P * 2);
 }
 
 template <int QM, int P>
@@ -193,10 +215,10 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     if constexpr (QM == QM_ASYM2) {
-      const uint2 v = *reinterpret_cast<const uint2*>(chunk[k] + L::V_OFF + 8 * lane);
+      const u32x2 v = gload<u32x2>(chunk[k] + L::V_OFF + 8 * lane);
       r.vc[k][0] = v.x; r.vc[k][1] = v.y;
     } else {
-      const uint4 v = *reinterpret_cast<const uint4*>(chunk[k] + L::V_OFF + 16 * lane);
+      const u32x4 v = gload<u32x4>(chunk[k] + L::V_OFF + 16 * lane);
       r.vc[k][0] = v.x; r.vc[k][1] = v.y; r.vc[k][2] = v.z; r.vc[k][3] = v.w;
     }
   }
@@ -219,40 +241,38 @@ DEVI float wave_sum64(float v) {
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
 template <int QM, bool K2>
-DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
+DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, const Consts& cst, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
   const bool full = K2 && (r.vs[0] & 0x8000u);
-  float a[4][4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) sc[h] = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const uint32_t nz1 = negz16(kw[j] & ZM) * 0x00010001u;
     const uint32_t nz[4] = {nz1, nz1, nz1, nz1};
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
-    const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + var * 64 + j;   // + head * 16 + tg * 4
+    const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + var * QV_VSTRIDE + j;   // + head * 16 + tg * 4
+    float a[4];
 #pragma unroll
     for (int tg = 0; tg < 4; ++tg) {
       uint32_t x[4];
-      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], nz, x);
-      else Unpack<QM>::run(r.kc[tg][j], nz, x);
+      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], nz, cst, x);
+      else Unpack<QM>::run(r.kc[tg][j], nz, cst, x);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const uint4 qq = qp[h * 16 + tg * 4];
-        float v = tg == 0 ? 0.f : a[j][h];
+        float v = tg == 0 ? 0.f : a[h];
         v = dot2(x[0], qq.x, v);
         v = dot2(x[1], qq.y, v);
         v = dot2(x[2], qq.z, v);
         v = dot2(x[3], qq.w, v);
-        a[j][h] = v;
+        a[h] = v;
       }
     }
-  }
+    const float sj = f16_value(kw[j] & 0x7FFFu) * qscale;
 #pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    float v = f16_value(kw[0] & 0x7FFFu) * a[0][h];
-#pragma unroll
-    for (int j = 1; j < 4; ++j) v += f16_value(kw[j] & 0x7FFFu) * a[j][h];
-    sc[h] = v * qscale;
+    for (int h = 0; h < 4; ++h) sc[h] += sj * a[h];
   }
 }
 
@@ -285,9 +305,9 @@ DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[
     st.l[h] += p[h];
   }
   // p' = p * V scale per group as fp16, and -(1024 + zero point), in V^T token order of the token's page
-  const int so = (pi * 2 + (pos >> 3)) * 32 + vslot(pos & 7);           // + group * 8
-  _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + 4 * (so & ~7) + (so & 7);
-  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb[wave]) + so;
+  const int rg = pi * 2 + (pos >> 3), sl = vslot(pos & 7);
+  _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb[wave]) + rg * ZB_RSTRIDE * 8 + sl;      // + group * 8
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const float sv = f16_value(r.vs[g] & 0x7FFFu);
@@ -298,35 +318,35 @@ DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[
 }
 
 template <int QM>
-DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
+DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave, const Consts& cst) {
   const int c8 = lane & 1, g0 = lane >> 5;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + ((k * 2 + c8) * 4) * 4;   // + group * 4 + head
-    uint4 pa[4], pc[4];
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + (k * 2 + c8) * PB_RSTRIDE;   // + group * 4 + head
 #pragma unroll
-    for (int h = 0; h < 4; ++h) { pa[h] = pp[g0 * 4 + h]; pc[h] = pp[(2 + g0) * 4 + h]; }
-    uint4 za = make_uint4(0, 0, 0, 0), zc = za;
-    if constexpr (QM != QM_SYM4) {
-      const uint4* zp = reinterpret_cast<const uint4*>(S.zb[wave]) + (k * 2 + c8) * 4;
-      za = zp[g0]; zc = zp[2 + g0];
-    }
+    for (int half = 0; half < 2; ++half) {      // entry words 0, 1 belong to group g0, words 2, 3 to group 2 + g0
+      const int g = 2 * half + g0;
+      uint4 pq[4];
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
-      uint32_t x[4];
-      const uint4 zz = sub < 2 ? za : zc;
+      for (int h = 0; h < 4; ++h) pq[h] = pp[g * 4 + h];
+      uint4 zz = make_uint4(0, 0, 0, 0);
+      if constexpr (QM != QM_SYM4) zz = (reinterpret_cast<const uint4*>(S.zb[wave]) + (k * 2 + c8) * ZB_RSTRIDE)[g];
       const uint32_t nz[4] = {zz.x, zz.y, zz.z, zz.w};
-      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], nz, x);
-      else Unpack<QM>::run(r.vc[k][sub], nz, x);
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const uint4 pq = sub < 2 ? pa[h] : pc[h];
-        float a = st.acc[h][sub];
-        a = dot2(x[0], pq.x, a);
-        a = dot2(x[1], pq.y, a);
-        a = dot2(x[2], pq.z, a);
-        a = dot2(x[3], pq.w, a);
-        st.acc[h][sub] = a;
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int sub = 2 * half + s2;
+        uint32_t x[4];
+        if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], nz, cst, x);
+        else Unpack<QM>::run(r.vc[k][sub], nz, cst, x);
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          float a = st.acc[h][sub];
+          a = dot2(x[0], pq[h].x, a);
+          a = dot2(x[1], pq[h].y, a);
+          a = dot2(x[2], pq[h].z, a);
+          a = dot2(x[3], pq[h].w, a);
+          st.acc[h][sub] = a;
+        }
       }
     }
   }
@@ -398,15 +418,18 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
       const int pg0 = lo / P, pg1 = (hi + P - 1) / P;
       const int* bt = p.block_table + static_cast<long long>(b) * p.bt_stride;
       const int pi = lane >> 4, pos = lane & 15;
+      typedef const __attribute__((address_space(1))) uint8_t* gptr;
+      const gptr pool = (gptr)p.pool;
       auto chunk_of = [&](int pg) {   // pages past the range read the last page of the range; their tokens are masked
-        return p.pool + (static_cast<long long>(bt[min(pg, pg1 - 1)]) * p.Hkv + kvh) * L::CHUNK;
+        return (const uint8_t*)(pool + (static_cast<long long>(bt[min(pg, pg1 - 1)]) * p.Hkv + kvh) * L::CHUNK);
       };
-      KRegs<QM> cur, nxt;
+      KRegs<QM> cur;
+      const Consts cst = make_consts();
       int q4 = pg0 + 4 * wave;       // first page of this wave's current quad
       const uint8_t* mine = chunk_of(q4 + pi);
       if (q4 < pg1) load_k<QM, P>(cur, mine, pos);
       for (; q4 < pg1; q4 += 4 * NWAVE) {
-        VRegs<QM> vr;
+        VRegs<QM> vr;                // this quad's V^T entries: in flight during the key phase
         {
           const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
           const uint8_t* ch[4];
@@ -418,22 +441,19 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
           }
           load_v<QM, P>(vr, ch, lane);
         }
-        const int qn = q4 + 4 * NWAVE;
-        const uint8_t* mine_n = mine;
-        if (qn < pg1) {
-          mine_n = chunk_of(qn + pi);
-          load_k<QM, P>(nxt, mine_n, pos);
-        }
         const int tok = (q4 + pi) * P + pos;
         const bool valid = tok >= lo && tok < hi;
         float sc[4];
-        key_phase<QM, K2>(S, cur, p.qscale, sc);
+        key_phase<QM, K2>(S, cur, p.qscale, cst, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
+        const int qn = q4 + 4 * NWAVE;   // the key registers are free: the next quad's keys fly during the value phase
+        if (qn < pg1) {
+          mine = chunk_of(qn + pi);
+          load_k<QM, P>(cur, mine, pos);
+        }
         wave_lds_sync();
-        value_phase<QM>(S, st, vr, lane, wave);
+        value_phase<QM>(S, st, vr, lane, wave, cst);
         wave_lds_sync();
-        cur = nxt;
-        mine = mine_n;
       }
     }
     // ---- fold the wave: entry pairs (c8 = 0 / 1), offset sums per (head, group)
