@@ -181,6 +181,12 @@ def main():
     torch.cuda.synchronize()
     writer_us = e0.elapsed_time(e1) / 20 * 1e3
 
+    traffic = None
+    try:   # measured with rocprofv3 --pmc (see profiles/k_decode_*_flagrot.txt); not measurable from inside this process
+        with open(os.path.join(ROOT, "profiles", "decode_traffic.json")) as f:
+            traffic = json.load(f).get(args.workload, {}).get("traffic_bytes")
+    except OSError:
+        pass
     res = {
         "metric": "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -189,7 +195,7 @@ def main():
         "data": "synthetic", "config": {"workload": name, "nsplit": ns, "chunk": ch, "cache_copies_cycled": ncopy,
                                          "sink": S, "window": W},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": None,
+                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": traffic,
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(ms_per_step * 1e3, 2),
                      "median_launch_us": round(per[len(per) // 2] * 1e3, 2), "min_launch_us": round(per[0] * 1e3, 2)},
         "writer": {"decode_step_us": round(writer_us, 2), "decode_step_tokens": B,

@@ -614,9 +614,7 @@ int launch_qm(const DecodeParams& p, hipStream_t st) {
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
 
-}  // namespace
-
-int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) {
+int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
   switch (fmt) {
     case FMT_INT4: return launch_qm<QM_SYM4, false>(p, st);
     case FMT_INT4A: return launch_qm<QM_ASYM4, false>(p, st);
@@ -628,9 +626,36 @@ int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) {
   return -4;
 }
 
+template <int QM, bool K2>
+int occupancy_qm() {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(&k_decode<QM, K2, 16>), 256, 0) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    return 2;
+  }
+  return n;
+}
+
+}  // namespace
+
+int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) { return decode_dispatch(fmt, p, st); }
+
+// resident workgroups per CU the host split planner may count on (queried once per format)
 int decode_occupancy(int fmt) {
-  (void)fmt;
-  return 2;   // resident workgroups per CU the split planner may count on
+  static int cache[16] = {0};
+  if (fmt < 0 || fmt >= 16) return 0;
+  if (cache[fmt] == 0) {
+    switch (fmt) {
+      case FMT_INT4: cache[fmt] = occupancy_qm<QM_SYM4, false>(); break;
+      case FMT_INT4A: cache[fmt] = occupancy_qm<QM_ASYM4, false>(); break;
+      case FMT_INT2A: cache[fmt] = occupancy_qm<QM_ASYM2, false>(); break;
+      case FMT_KONLY: cache[fmt] = occupancy_qm<QM_SYM4, true>(); break;
+      case FMT_KONLYA: cache[fmt] = occupancy_qm<QM_ASYM4, true>(); break;
+      case FMT_KONLYA2: cache[fmt] = occupancy_qm<QM_ASYM2, true>(); break;
+      default: return 0;
+    }
+  }
+  return cache[fmt];
 }
 
 }  // namespace fr
