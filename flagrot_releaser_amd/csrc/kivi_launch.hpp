@@ -1,0 +1,18 @@
+// Launcher prototypes shared by the translation units of libflagrot_kivi.so (head dim 128, FP16 scale / min).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace frkv {
+
+int v_write_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
+                   int ident, const int* vfix, hipStream_t st);
+int k_encode_launch(const void* src, long long src_rs, const void* src2, long long src2_rs, const long long* sidx,
+                    const long long* dslot, int N, int Hkv, const float* qs, const float* lz, int NQ, float qsc,
+                    uint8_t* pool, int ident, const int* kfix, hipStream_t st);
+int dequant_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nvalid, int Hkv, int fp32, void* ok, void* ov,
+                   hipStream_t st);
+int lse_merge_launch(const void* oa, const float* la, long long la_hs, const void* ob, const float* lb, long long lb_hs,
+                     void* out, long long out_rs, int na, int H, int D, hipStream_t st);
+
+}  // namespace frkv

@@ -32,6 +32,22 @@ def test_kernels_library_exports_header_symbols():
     assert L.fr_cb_chunk_bytes(10, 16) == 2304 and L.fr_cb_chunk_bytes(11, 16) == 1280
 
 
+def test_kivi_library_exports_header_symbols():
+    from flagrot_releaser_amd import build, kivi
+    path = build.lib_path("kivi")
+    if not path.exists():
+        build.build("kivi", verbose=False)
+    L = ctypes.CDLL(str(path))
+    names = _declared("flagrot_kivi.h")
+    assert set(names) == set(kivi.EXPORTS)
+    for n in names:
+        assert hasattr(L, n), n
+    L.kv_abi_version.restype = ctypes.c_int
+    assert L.kv_abi_version() == 9
+    assert L.kv_chunk_bytes(128) == 1552 and L.kv_chunk_bytes8(128) == 1280
+    assert kivi.plan(16, 32768, 8, sms=256) == (24, 1376) and kivi.plan(1, 100, 8, sms=256)[1] == 256
+
+
 def test_host_planner_invariants():
     from flagrot_releaser_amd import kernels as K
     for B, L in ((1, 1), (1, 2048), (32, 8192), (64, 16384), (3, 33000), (8, 65536)):

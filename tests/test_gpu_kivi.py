@@ -1,0 +1,362 @@
+"""GPU parity of libflagrot_kivi.so (through the C-ABI, via flagrot_releaser_amd.kivi) against oracle/kivi.py.
+
+Bars:
+  writers    codes and meta bit-equal to the oracle GIVEN the flags the kernel stored; a stored choice may differ from
+             the oracle's fp64 choice only where the fp64 decision margin is below 1e-3 relative (the reference
+             accumulates the selection errors in fp32 in a thread-dependent order and its own test accepts 2 %
+             mismatches, integrations/vllm_flagrot/tests/test_kivi.py:139-140); `ident` and `fix` modes are bit-pinned
+             on the whole pool;
+  attention  |out - ref| <= 1e-2 max|ref| against fp64 attention over the oracle's dequantised pages + BF16 tail
+             (the reference's bar, tests/test_kivi.py:243);
+  dequant    fp32 within 2e-6 max|ref| of the fp64 oracle; bf16 = round of it within one ulp;
+  lse_merge  bf16 patterns equal to the oracle's, up to one ulp on at most 0.1 % (library exp).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kivi as OK
+from oracle import quant as Q
+from tests.gpu_util import bits
+
+pytestmark = pytest.mark.gpu
+D, PAGE = 128, 16
+CB = OK.chunk_bytes(D)
+
+
+def _kv(T, Hkv, g, shift=2.0):
+    """rows with per-channel offsets (what makes rotated bases win or lose per group) and a few outlier channels."""
+    mu = torch.randn(2 * Hkv, D, generator=g) * shift
+    x = mu[None] + torch.randn(T, 2 * Hkv, D, generator=g) * (0.3 + torch.rand(2 * Hkv, D, generator=g))
+    x[:, :, 5] *= 6
+    if T >= 8:
+        x[3] = 0.0
+        x[4, :, 32:64] = 1.25
+        x[5] *= 1e-4
+        x[6] *= 200
+    return x.bfloat16()
+
+
+def _calib(Hkv, NQ, g):
+    qs = (torch.randn(Hkv, NQ, D, generator=g) * 0.4).contiguous()
+    lz = (3.0 + torch.rand(Hkv, NQ, generator=g) * 4).contiguous()
+    co = (torch.rand(Hkv, D, generator=g) + 0.1).contiguous()
+    return qs, lz, co
+
+
+def _stored_value_flags(pool_np):
+    _, _, _, vm, vf = OK.parse_chunks(pool_np, D)
+    return (vm[..., 0] >> 15).astype(bool), vf.astype(bool)          # [np, H, 16, NV], [np, H, 16]
+
+
+@pytest.mark.parametrize("seed,T,Hkv", [(0, 64, 2), (1, 333, 8), (2, 1, 1)])
+def test_v_write_given_flags(dev, seed, T, Hkv):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(seed)
+    kv = _kv(T, Hkv, g)
+    _, _, co = _calib(Hkv, 8, g)
+    npg = (T + 15) // 16 + 2
+    slots = torch.randperm(npg * 16, generator=g)[:T].long()
+    if T > 10:
+        slots[7] = -1
+    init = torch.randint(0, 256, (npg, Hkv, CB), generator=g, dtype=torch.uint8)
+    pool = init.to(dev)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, pool, Hkv, D)
+    torch.cuda.synchronize()
+    got = pool.cpu().numpy()
+    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy())
+    sH, sF = _stored_value_flags(got)
+    useH = np.zeros((T, Hkv, 4), bool)
+    useF = np.zeros((T, Hkv), bool)
+    for t, s in enumerate(slots.tolist()):
+        if s >= 0:
+            useH[t], useF[t] = sH[s // 16, :, s % 16], sF[s // 16, :, s % 16]
+    codes, meta, vf = OK.v_stored(enc, useH, useF)
+    want = init.numpy().copy()
+    OK.pack_values(want, slots.numpy(), codes, meta, vf)
+    assert np.array_equal(got, want), "value codes / meta differ from the oracle given the stored flags"
+    live = (slots.numpy() >= 0)
+    badF = (useF != enc["useF"]) & live[:, None]
+    assert (enc["marginF"][badF] < 1e-3).all(), enc["marginF"][badF]
+    badH = (useH != enc["useH"]) & ~useF[..., None] & ~enc["useF"][..., None] & live[:, None, None]
+    assert (enc["marginH"][badH] < 1e-3).all(), enc["marginH"][badH]
+    assert badF.mean() < 0.02 and badH.mean() < 0.02
+    if T > 32:
+        assert useH.any() and (~useH).any()
+
+
+@pytest.mark.parametrize("mode", ["ident", "fix"])
+def test_v_write_pinned_modes(dev, mode):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(5)
+    T, Hkv = 200, 4
+    kv = _kv(T, Hkv, g)
+    _, _, co = _calib(Hkv, 8, g)
+    npg = 14
+    slots = torch.randperm(npg * 16, generator=g)[:T].long()
+    fix = torch.tensor([0b0101, 1 << 16, 0b1111, 0], dtype=torch.int32)
+    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, pool, Hkv, D, ident=mode == "ident",
+               fix=fix.to(dev) if mode == "fix" else None)
+    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy(), ident=mode == "ident", fix=fix.numpy() if mode == "fix" else None)
+    want = np.zeros((npg, Hkv, CB), np.uint8)
+    OK.pack_values(want, slots.numpy(), *OK.v_stored(enc))
+    assert np.array_equal(pool.cpu().numpy(), want)
+
+
+def _groups(NG, Hkv, g, ragged=True):
+    """NG groups of 32 tokens from two source tensors; returns kv rows, src2 rows, sidx, dslot, valid."""
+    rows = _kv(NG * 32 + 5, Hkv, g)
+    rows2 = _kv(40, Hkv, g, shift=1.0)
+    sidx = torch.arange(NG * 32).reshape(NG, 32).long() + 5
+    if ragged and NG >= 3:
+        sidx[1, 20:] = -1                      # a short group
+        sidx[2, :8] = -(torch.arange(8) + 2)   # rows 0..7 of the second source
+    pages = torch.randperm(2 * NG + 3, generator=g)[:2 * NG].reshape(NG, 2)
+    dslot = (pages[:, :, None] * 16 + torch.arange(16)[None, None]).reshape(NG, 32).long()
+    return rows, rows2, sidx, dslot
+
+
+def _group_rows(rows, rows2, sidx_row, Hkv):
+    xb = np.zeros((32, Hkv, D), np.uint16)
+    rb, rb2 = bits(rows), bits(rows2)
+    for t, r in enumerate(sidx_row.tolist()):
+        if r >= 0:
+            xb[t] = rb[r, :Hkv]
+        elif r <= -2:
+            xb[t] = rb2[-r - 2, :Hkv]
+    return xb, (sidx_row.numpy() != -1)
+
+
+def _stored_key_flags(pool_np, dslot_row, h):
+    pg0 = int(dslot_row[0]) // 16
+    pg1 = int(dslot_row[16]) // 16
+    _, km, *_ = OK.parse_chunks(pool_np[[pg0, pg1]][:, h:h + 1], D)
+    s = km[:, 0, :, :, 0].reshape(-1)                                 # 128 channel scales, cell-major
+    return (s[:4] >> 15).astype(bool), bool(s[4] >> 15)
+
+
+@pytest.mark.parametrize("seed,NG,Hkv,NQ", [(0, 4, 2, 64), (1, 6, 8, 37), (2, 1, 1, 8)])
+def test_k_encode_given_flags(dev, seed, NG, Hkv, NQ):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(seed)
+    rows, rows2, sidx, dslot = _groups(NG, Hkv, g)
+    qs, lz, _ = _calib(Hkv, NQ, g)
+    qsc = 1 / math.sqrt(D)
+    npg = 2 * NG + 3
+    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
+    KV.k_encode(rows.to(dev), sidx.to(dev), dslot.to(dev), qs.to(dev), lz.to(dev), qsc, pool, Hkv, D, src2=rows2.to(dev))
+    torch.cuda.synchronize()
+    got = pool.cpu().numpy()
+    want = np.zeros_like(got)
+    nbad = ntot = 0
+    seenH = set()
+    for n in range(NG):
+        xb, valid = _group_rows(rows, rows2, sidx[n], Hkv)
+        for h in range(Hkv):
+            enc = OK.k_encode_group(xb[:, h], valid, qs[h].numpy(), lz[h].numpy(), qsc)
+            uH, uF = _stored_key_flags(got, dslot[n].numpy(), h)
+            codes, meta = OK.k_stored(enc, uH, uF)
+            OK.pack_key_group(want, h, dslot[n].numpy(), valid, codes, meta)
+            if uF != enc["useF"]:
+                assert enc["marginF"] < 1e-3, (n, h, enc["marginF"])
+                nbad += 1
+            if not uF and not enc["useF"]:
+                d = uH != enc["useH"]
+                assert (enc["marginH"][d] < 1e-3).all(), (n, h, enc["marginH"][d])
+                nbad += int(d.sum())
+                seenH.update(uH.tolist())
+            ntot += 5
+    assert np.array_equal(got, want), "key codes / meta differ from the oracle given the stored flags"
+    assert nbad <= max(1, 0.02 * ntot)
+    if NG * Hkv >= 8:
+        assert seenH == {True, False}
+
+
+@pytest.mark.parametrize("mode", ["ident", "fix"])
+def test_k_encode_pinned_modes_keep_value_fields(dev, mode):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(9)
+    NG, Hkv = 5, 4
+    rows, rows2, sidx, dslot = _groups(NG, Hkv, g)
+    qs, lz, co = _calib(Hkv, 16, g)
+    fix = torch.tensor([0b0011, 1 << 16, 0b1000, 0], dtype=torch.int32)
+    npg = 2 * NG + 3
+    init = torch.randint(0, 256, (npg, Hkv, CB), generator=g, dtype=torch.uint8)
+    pool = init.to(dev)
+    KV.k_encode(rows.to(dev), sidx.to(dev), dslot.to(dev), qs.to(dev), lz.to(dev), 0.1, pool, Hkv, D, src2=rows2.to(dev),
+                ident=mode == "ident", fix=fix.to(dev) if mode == "fix" else None)
+    want = init.numpy().copy()
+    for n in range(NG):
+        xb, valid = _group_rows(rows, rows2, sidx[n], Hkv)
+        for h in range(Hkv):
+            enc = OK.k_encode_group(xb[:, h], valid, qs[h].numpy(), lz[h].numpy(), 0.1, ident=mode == "ident",
+                                    fix=int(fix[h]) if mode == "fix" else None)
+            OK.pack_key_group(want, h, dslot[n].numpy(), valid, *OK.k_stored(enc))
+    assert np.array_equal(pool.cpu().numpy(), want)       # value fields and unused pages keep their bytes
+
+
+def _filled_cache(dev, lens, Hkv, g, tail_T=0):
+    """pages of B sequences written by the GPU writers (whole groups), block table, and the fp64 K / V the oracle
+    reads back from the same bytes."""
+    from flagrot_releaser_amd import kivi as KV
+    B = len(lens)
+    ngs = [-(-n // 32) for n in lens]
+    npg = 2 * sum(ngs) + 1
+    perm = torch.randperm(npg, generator=g)
+    bt = torch.zeros(B, 2 * max(ngs), dtype=torch.int32)
+    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
+    qs, lz, co = _calib(Hkv, 24, g)
+    o = 0
+    Ks, Vs = [], []
+    for b in range(B):
+        n = ngs[b] * 32
+        bt[b, :2 * ngs[b]] = perm[o:o + 2 * ngs[b]].int()
+        o += 2 * ngs[b]
+        kv = _kv(n, Hkv, g).to(dev)
+        slots = (bt[b].long()[torch.arange(n) // 16] * 16 + torch.arange(n) % 16)
+        KV.v_write(kv, slots.to(dev), co.to(dev), None, pool, Hkv, D)
+        sidx = torch.arange(n).reshape(-1, 32).long()
+        KV.k_encode(kv, sidx.to(dev), slots.reshape(-1, 32).to(dev), qs.to(dev), lz.to(dev), 1 / math.sqrt(D), pool, Hkv, D)
+    torch.cuda.synchronize()
+    pnp = pool.cpu().numpy()
+    for b in range(B):
+        k, v = OK.dequant_groups(pnp[bt[b, :2 * ngs[b]].numpy()], D)
+        Ks.append(k)
+        Vs.append(v)
+    return pool, bt, Ks, Vs
+
+
+def _ref_attn(q, K, V, kv_start, cached, tailK, tailV, G, scale):
+    """fp64 softmax attention of one sequence: q [Hq, D]; K, V [n, Hkv, D]; rows [kv_start, cached) + tail rows."""
+    Hq = q.shape[0]
+    out = np.zeros((Hq, D))
+    for hq in range(Hq):
+        h = hq // G
+        k = np.concatenate([K[kv_start:cached, h], tailK[:, h]])
+        v = np.concatenate([V[kv_start:cached, h], tailV[:, h]])
+        if len(k) == 0:
+            continue
+        s = (k @ q[hq]) * scale
+        p = np.exp(s - s.max())
+        out[hq] = (p / p.sum()) @ v
+    return out
+
+
+CASES = [
+    # lens, Hkv, G, kv_start, nsplit / chunk (None: plan), tail lengths
+    ([96], 1, 1, 0, (1, 256), [0]),
+    ([512, 300, 64], 2, 4, 0, (2, 256), [5, 0, 17]),
+    ([1000, 32], 2, 8, 64, (4, 256), [31, 1]),
+    ([700], 1, 5, 0, (3, 256), [0]),
+    ([2048, 1500], 8, 4, 32, None, [40, 128]),
+    ([40, 40], 2, 2, 64, (1, 256), [3, 0]),       # nothing left in the pages: tail only (and one empty sequence)
+]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_attn_against_fp64(dev, case):
+    from flagrot_releaser_amd import kivi as KV
+    lens, Hkv, G, kv_start, split, tails = CASES[case]
+    g = torch.Generator().manual_seed(100 + case)
+    B, Hq = len(lens), Hkv * G
+    pool, bt, Ks, Vs = _filled_cache(dev, lens, Hkv, g)
+    T = 128
+    R = B + 1
+    ring = (torch.randn((R + 1) * T, 2 * Hkv, D, generator=g) * 1.5).bfloat16()
+    tail_idx = torch.randperm(R + 1, generator=g)[:B].int()
+    tail_len = torch.tensor(tails, dtype=torch.int32)
+    cached = torch.tensor(lens, dtype=torch.int32)
+    q = (torch.randn(B, Hq, D, generator=g) * 1.2).bfloat16()
+    ns, chunk = split if split is not None else KV.plan(B, max(lens), Hkv)
+    assert ns * chunk >= max(lens)
+    ws = KV.Workspace(B * Hkv * (ns + 1), G, D, dev)
+    outbuf = torch.full((B, Hq * D + 64), 7.0, dtype=torch.bfloat16, device=dev)       # padded row stride
+    out = outbuf[:, :Hq * D]
+    scale = 1 / math.sqrt(D)
+    args = (q.to(dev), pool, bt.to(dev), cached.to(dev), out, ns, chunk, ws, scale * math.log2(math.e), kv_start, G)
+    kw = dict(ring=ring.to(dev), tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), T=T)
+    ringf = Q.bf16_to_f32(bits(ring)).astype(np.float64).reshape(R + 1, T, 2 * Hkv, D)
+    qf = Q.bf16_to_f32(bits(q)).astype(np.float64)
+    for rep in range(2):
+        KV.attn(*args, **kw)
+        torch.cuda.synchronize()
+        got = Q.bf16_to_f32(bits(out.contiguous())).astype(np.float64).reshape(B, Hq, D)
+        for b in range(B):
+            tb = ringf[int(tail_idx[b]), :tails[b]]
+            ref = _ref_attn(qf[b], Ks[b], Vs[b], min(kv_start, lens[b]), lens[b], tb[:, :Hkv], tb[:, Hkv:], G, scale)
+            if min(kv_start, lens[b]) >= lens[b] and tails[b] == 0:
+                assert not got[b].any()
+                continue
+            tol = 1e-2 * np.abs(ref).max() + 1e-6
+            assert np.abs(got[b] - ref).max() <= tol, (case, rep, b, np.abs(got[b] - ref).max(), tol)
+    assert (outbuf[:, Hq * D:] == 7.0).all()
+
+
+def test_attn_without_tail_and_rejects(dev):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(7)
+    Hkv, G = 2, 4
+    pool, bt, Ks, Vs = _filled_cache(dev, [320], Hkv, g)
+    q = torch.randn(1, Hkv * G, D, generator=g).bfloat16()
+    out = torch.empty(1, Hkv * G * D, dtype=torch.bfloat16, device=dev)
+    ws = KV.Workspace(Hkv * 3, G, D, dev)
+    cached = torch.tensor([300], dtype=torch.int32, device=dev)             # a partly read last group
+    KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 256, ws, math.log2(math.e) / math.sqrt(D), 0, G)
+    torch.cuda.synchronize()
+    none = np.zeros((0, Hkv, D))
+    ref = _ref_attn(Q.bf16_to_f32(bits(q)).astype(np.float64)[0], Ks[0], Vs[0], 0, 300, none, none, G, 1 / math.sqrt(D))
+    got = Q.bf16_to_f32(bits(out)).astype(np.float64).reshape(Hkv * G, D)
+    assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
+    with pytest.raises(RuntimeError, match="chunk"):
+        KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 100, ws, 0.1, 0, G)
+    with pytest.raises(RuntimeError, match="FP8"):
+        KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 256, ws, 0.1, 0, G, f8=True)
+    with pytest.raises(RuntimeError, match="M is not built"):
+        KV.v_write(torch.zeros(1, 2 * Hkv, D, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
+                   torch.ones(Hkv, D, device=dev), torch.ones(Hkv, D, D, device=dev), pool, Hkv, D)
+
+
+def test_dequant_and_torch_parser(dev):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(11)
+    Hkv = 4
+    pool, bt, Ks, Vs = _filled_cache(dev, [416], Hkv, g)
+    row = bt[0].contiguous().to(dev)
+    for a, n in ((0, 416), (40, 300), (64, 65)):
+        k32, v32 = KV.dequant_cuda(pool, row, a, n, Hkv, D, dtype=torch.float32)
+        kb, vb = KV.dequant_cuda(pool, row, a, n, Hkv, D)
+        kt, vt = KV.dequant(pool, row, a, n, Hkv, D)
+        torch.cuda.synchronize()
+        for got, gotb, gott, ref in ((k32, kb, kt, Ks[0][a:n]), (v32, vb, vt, Vs[0][a:n])):
+            assert got.shape == ref.shape == gotb.shape == gott.shape
+            sc = np.abs(ref).max()
+            assert np.abs(got.cpu().numpy() - ref).max() <= 2e-6 * sc
+            assert np.abs(gott.cpu().numpy() - ref).max() <= 2e-6 * sc
+            assert (gotb.float().cpu() - got.cpu()).abs().max() <= 2 ** -8 * sc
+            back = got.bfloat16()
+            assert ((gotb.view(torch.int16).int() - back.view(torch.int16).int()).abs() <= 1).all()
+
+
+def test_lse_merge(dev):
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(3)
+    n, H = 37, 6
+    oa = torch.randn(n, H, D, generator=g).bfloat16()
+    ob = torch.randn(n, H, D, generator=g).bfloat16()
+    la = torch.randn(H, n, generator=g) * 3
+    lb = torch.randn(H, n, generator=g) * 3
+    la[0, 3] = float("inf")                 # read as -inf: b alone
+    lb[1, 4] = float("-inf")
+    lb[2, 5] = la[2, 5]
+    outbuf = torch.zeros(n, H * D + 32, dtype=torch.bfloat16, device=dev)
+    out = outbuf.as_strided((n, H, D), (H * D + 32, D, 1))
+    KV.lse_merge(oa.to(dev), la.to(dev), ob.to(dev), lb.to(dev), out)
+    torch.cuda.synchronize()
+    want = OK.lse_merge(bits(oa), la.numpy(), bits(ob), lb.numpy())
+    got = bits(out.contiguous())
+    d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 1e-3
+    assert np.array_equal(got[3, 0], bits(ob)[3, 0]) and np.array_equal(got[4, 1], bits(oa)[4, 1])
