@@ -1,6 +1,6 @@
 """Headline benchmark: paged FlagRot decode attention on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2|kivi]
 
 A step is one decode layer-step: one launch of the paged decode attention (through the C ABI of
 libflagrot_kernels.so) over the whole batch, on a synthetic cache that is already resident in HBM.  Successive steps
@@ -11,6 +11,8 @@ Workloads (BASELINE.json configs):
         batch 32, context 8192, page 16, randomly permuted page table.                       [default, headline]
   int2  configs[2]: INT2 FlagRot (kind konlya2) with static key centring, 4 sink + 128 window BF16 tokens,
         batch 64, context 16384.
+  kivi  configs[3]: KIVI-style FlagRot INT2 (keys per channel over 32-token groups, values per token), 128-token
+        BF16 residual, Qwen-32B shape 64q/8kv, d=128, batch 16, context 32768 (libflagrot_kivi.so).
 Prints ONE JSON line: value = achieved GB/s of page bytes (the reference's convention: B * L * Hkv * bytes per token),
 with `roofline` (HBM, measured with events on the launch stream) and `cpu_baseline` (the numpy oracle's
 dequantise-then-attend path, timed on the host on configs[0]'s shape).
@@ -95,12 +97,97 @@ def cpu_baseline(torch, K, dev):
                       f"median of 3 after 1 warm-up: {t * 1e6:.0f} us per layer-step; host has {os.cpu_count()} cpus"}
 
 
+def main_kivi(args, torch, dev):
+    """configs[3] through libflagrot_kivi.so: fill by the value writer + key group encoder, time kv_attn."""
+    from flagrot_releaser_amd import kivi as KV
+    KV.lib()
+    B, L, Gq, W, NQ, outl, gain = 16, 32768, 8, 128, 64, 8, 12.0
+    name = ("configs[3]: KIVI-style FlagRot INT2 paged decode (per-channel keys over 32-token groups, per-token values), "
+            "128-token BF16 residual, Qwen-32B GQA 64q/8kv d=128, B=16 L=32768 page=16")
+    CB = KV.chunk_bytes(DH)
+    g = torch.Generator(device=dev).manual_seed(3)
+    Lp = L - W
+    npages = B * (Lp // P)
+    pool = torch.zeros(npages + 16, HKV, CB, dtype=torch.uint8, device=dev)
+    bt = torch.randperm(npages + 16, generator=g, device=dev)[:npages].int().view(B, -1).contiguous()
+    co = (0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)).contiguous()
+    qs = torch.randn(HKV, NQ, DH, generator=g, device=dev).contiguous()
+    lz = torch.full((HKV, NQ), 6.0, device=dev)
+    t0 = time.perf_counter()
+    for b in range(B):
+        for s0 in range(0, Lp, 8192):
+            n = min(8192, Lp - s0)
+            kv = synth_kv(n, g, dev, torch, outliers=outl, gain=gain)
+            pos = torch.arange(s0, s0 + n, device=dev)
+            slots = bt[b].long()[pos // P] * P + pos % P
+            KV.v_write(kv, slots, co, None, pool, HKV, DH)
+            KV.k_encode(kv, torch.arange(n, device=dev).view(-1, 32), slots.view(-1, 32).contiguous(), qs, lz,
+                        1 / math.sqrt(DH), pool, HKV, DH)
+    torch.cuda.synchronize()
+    fill_s = time.perf_counter() - t0
+    ncopy = max(1, min(8, int(6e9 // pool.numel())))
+    pools = [pool] + [pool.clone() for _ in range(ncopy - 1)]
+    q = torch.randn(B, Gq * HKV, DH, generator=g, device=dev).bfloat16()
+    out = torch.zeros(B, Gq * HKV * DH, dtype=torch.bfloat16, device=dev)
+    ring = torch.randn((B + 1) * W, 2 * HKV, DH, generator=g, device=dev).bfloat16()
+    tail_len = torch.full((B,), W, dtype=torch.int32, device=dev)
+    tail_idx = torch.arange(B, dtype=torch.int32, device=dev)
+    cached = torch.full((B,), Lp, dtype=torch.int32, device=dev)
+    ns, ch = KV.plan(B, Lp, HKV)
+    if args.nsplit:
+        ns = args.nsplit
+        ch = -(-Lp // ns // 32) * 32
+        ns = -(-Lp // ch)
+    ws = KV.Workspace(B * HKV * (ns + 1), Gq, DH, dev)
+    scale = LOG2E / math.sqrt(DH)
+
+    def step(i):
+        KV.attn(q, pools[i % ncopy], bt, cached, out, ns, ch, ws, scale, 0, Gq, ring=ring, tail_len=tail_len,
+                tail_idx=tail_idx, T=W)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    ev[0].record()
+    for i in range(args.steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
+    ms_per_step = ev[0].elapsed_time(ev[-1]) / args.steps
+    alg_bytes = B * Lp * HKV * (CB // P) + B * W * 2 * HKV * DH * 2
+    gbps = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "decode_traffic.json")) as f:
+            traffic = json.load(f).get("kivi", {}).get("traffic_bytes")
+    except OSError:
+        pass
+    res = {
+        "metric": "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "us_per_layer_step": round(ms_per_step * 1e3, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 codes, f32 products and accumulate",
+        "data": "synthetic", "config": {"workload": name, "nsplit": ns, "chunk": ch, "cache_copies_cycled": ncopy,
+                                         "sink": 0, "window": W},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": traffic,
+                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(ms_per_step * 1e3, 2),
+                     "median_launch_us": round(per[len(per) // 2] * 1e3, 2), "min_launch_us": round(per[0] * 1e3, 2),
+                     "note": "one step = kv_attn = the split kernel + the merge kernel"},
+        "writer": {"prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * Lp,
+                   "note": "value writer + key group encoder (64 calibration queries), includes synthetic input generation"},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="int4", choices=["int4", "int2"])
+    ap.add_argument("--workload", default="int4", choices=["int4", "int2", "kivi"])
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -114,6 +201,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.workload == "kivi":
+        return main_kivi(args, torch, dev)
     K.lib()
     if args.workload == "int4":
         kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144

@@ -19,13 +19,11 @@
 // kernels/csrc/attn_codebook_attn.cuh:2093-2126 (per-(token, group) variant selection), attn_merge.cuh:23-84.
 #include "fr_common.hpp"
 #include "fr_launch.hpp"
+#include "fr_unpack.hpp"
 
 namespace fr {
 namespace {
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-DEVI half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 DEVI float dot2(uint32_t a, uint32_t b, float c) { return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), c, false); }
 DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -52,52 +50,6 @@ DEVI void wave_lds_sync() {
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
-
-// ---------------------------------------------------------------------------------------------- code unpacking
-// A 32-bit word of eight 4-bit fields f0..f7 (or, INT2, the 2-bit fields at bit 4 n of a pre-shifted word) becomes
-// four fp16 pairs (f0,f4) (f1,f5) (f2,f6) (f3,f7): the field is or-ed into the mantissa of 1024.0 (exact), then
-// -(1024 + zero point) is added with one packed fp16 add, which is exact too: the pairs hold code - zero point.
-DEVI uint32_t pk_add(uint32_t a, uint32_t b) {
-  return __builtin_bit_cast(uint32_t, as_h2(a) + as_h2(b));
-}
-template <int QM> struct Unpack;
-// MAGIC (the fp16 pattern of 1024.0 twice) is kept in a register the compiler cannot constant-fold, so that
-// (w & mask) | MAGIC is a single v_and_or_b32 (one literal per instruction).
-struct Consts { uint32_t magic; };
-DEVI Consts make_consts() {
-  Consts c;
-  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(c.magic));
-  return c;
-}
-template <> struct Unpack<QM_ASYM4> {
-  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], const Consts& c, uint32_t (&x)[4]) {
-    x[0] = pk_add((w & 0x000F000Fu) | c.magic, nz[0]);
-    x[1] = pk_add(((w >> 4) & 0x000F000Fu) | c.magic, nz[1]);
-    x[2] = pk_add(((w >> 8) & 0x000F000Fu) | c.magic, nz[2]);
-    x[3] = pk_add(((w >> 12) & 0x000F000Fu) | c.magic, nz[3]);
-  }
-};
-template <> struct Unpack<QM_ASYM2> {
-  static DEVI void run(uint32_t w, const uint32_t (&nz)[4], const Consts& c, uint32_t (&x)[4]) {  // fields at bits 0, 2, 8, 10 (+16)
-    x[0] = pk_add((w & 0x00030003u) | c.magic, nz[0]);
-    x[1] = pk_add(((w >> 2) & 0x00030003u) | c.magic, nz[1]);
-    x[2] = pk_add(((w >> 8) & 0x00030003u) | c.magic, nz[2]);
-    x[3] = pk_add(((w >> 10) & 0x00030003u) | c.magic, nz[3]);
-  }
-};
-template <> struct Unpack<QM_SYM4> {  // sign-magnitude bytes s0000mmm -> exact signed fp16
-  static DEVI uint32_t pair(uint32_t bytes02, const Consts& c) {  // bytes at bits 0..7 and 16..23
-    const uint32_t m = pk_add((bytes02 & 0x00070007u) | c.magic, 0xE400E400u);
-    return m ^ ((bytes02 & 0x00800080u) << 8);
-  }
-  static DEVI void run(uint32_t w, const uint32_t (&)[4], const Consts& c, uint32_t (&x)[4]) {
-    const uint32_t a = w & 0x87878787u;                                   // A_i in byte i
-    const uint32_t b = ((w << 4) | (w >> 28)) & 0x87878787u;              // B_i in byte i
-    x[0] = pair(a, c); x[1] = pair(b, c); x[2] = pair(a >> 8, c); x[3] = pair(b >> 8, c);
-  }
-};
-// fp16 pattern of -(1024 + z)
-DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
 constexpr int NWAVE = 4;
 // LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per variant /

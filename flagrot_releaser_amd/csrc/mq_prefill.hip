@@ -1,0 +1,619 @@
+// Prefix-cached multi-query prefill attention straight from FlagRot INT4 / INT2 pages for gfx950 (wave64, MFMA), and the
+// extern "C" surface of libflagrot_mq.so (declared in include/flagrot_mq.h).
+//
+// Workgroup = (work item, KV head): a q tile of ROWS = 32 x waves rows (row r = token r / G, q head h G + r % G) against
+// the item's 64-key blocks.  Per block the workgroup turns the four page chunks into two fp16 tiles in LDS,
+//   K  [64 keys][128]  (code - zero point) * scale, one rounding; elements in code-word order, rows permuted so that
+//                      the score accumulators come out in the V^T token order;
+//   V^T [128 dims][64] eight-token runs exactly as the page stores them;
+// and every wavefront runs v_mfma_f32_32x32x16_f16 transposed: S^T = K q^T (lane = one query row, 32 keys in
+// registers: the softmax needs one cross-lane step), P^T straight from the accumulators as the B operand of
+// O^T = V^T P^T.  Key-only pages (per-token H32 / H128 flags): the query tile is kept in three rotations and the K
+// operand is zero-masked per (token, group) for each, so keys are never transformed.
+// Causal rule: key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext), j < nk.
+// Partials (unnormalised O, running maximum in log2 units, sum) per (item, KV head, row); k_merge combines the items
+// of a tile.  Semantics follow integrations/vllm_flagrot/csrc/mq_prefill.cu:345-498 (k_mq), :716-772 (merge),
+// :789-823 (q preparation), :1350-1465 (BF16 window gather / sink merge), :1469-1601 (C ABI).
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/flagrot_mq.h"
+#include "fr_common.hpp"
+#include "fr_unpack.hpp"
+
+namespace frmq {
+using namespace fr;
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int D = 128, PAGE = 16, BN = 64, TILE_INTS = 9, ITEM_INTS = 4;
+constexpr int KROW = 272;                    // bytes per K tile row: 256 + 16 pad
+constexpr int VROW = 144;                    // bytes per V^T tile row: 128 + 16 pad
+constexpr int KT_BYTES = BN * KROW, VT_BYTES = D * VROW;
+constexpr int QROW = 264;                    // bytes per staged q row (natural order)
+
+struct Smem {
+  alignas(16) uint8_t kt[KT_BYTES];
+  alignas(16) uint8_t vt[VT_BYTES];
+  alignas(16) uint32_t vsc[4][8][4];         // per (group, run): scale pairs (t0,t4) (t1,t5) (t2,t6) (t3,t7)
+  alignas(16) uint32_t vnz[4][8][4];         // per (group, run): -(1024 + zero point) pairs
+  uint32_t kflag[BN];                        // per K tile row: bits 0-3 H32 per group, bit 4 whole head
+};
+static_assert(128 * QROW <= KT_BYTES + VT_BYTES, "q staging aliases the tiles");
+
+struct Params {
+  const uint16_t* q;
+  const uint8_t* pool;
+  long long page_stride;
+  const int* bt;
+  long long bt_stride;
+  const int* tiles;
+  const int* items;
+  int Hkv, G, shift, kmin;
+  float* opart;
+  float* ml;
+};
+
+char g_err[512] = "";
+
+template <typename T> DEVI T gload(const void* p) {
+  return *reinterpret_cast<const __attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p));
+}
+DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+DEVI half8 as_h8(u32x4 v) { return __builtin_bit_cast(half8, v); }
+DEVI uint32_t pack_h2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+DEVI uint32_t pack_h2_rn(float a, float b) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// token (0..31 inside a 32-key tile) -> K tile row, and accumulator index -> token
+DEVI int krow_of_token(int tk) {
+  const int run = tk >> 3, t8 = tk & 7, e = 2 * (t8 & 3) + (t8 >> 2);
+  return 16 * (run >> 1) + 8 * (e >> 2) + 4 * (run & 1) + (e & 3);
+}
+DEVI constexpr int token_of_acc(int i, int hh) {   // accumulator i of the lane half hh
+  const int s = i >> 3, e = i & 7;
+  const int t8 = (e >> 1) + 4 * (e & 1);           // run order t0 t4 t1 t5 t2 t6 t3 t7
+  return 8 * (2 * s + hh) + t8;
+}
+
+template <int QM> struct Fmt {
+  static constexpr int CB = QM == QM_ASYM2 ? 32 : 64;
+  static constexpr int V_OFF = CB * PAGE, KS_OFF = 2 * CB * PAGE, VS_OFF = KS_OFF + 8 * PAGE, CHUNK = VS_OFF + 8 * PAGE;
+  static constexpr uint32_t ZM = QM == QM_ASYM2 ? 3u : 15u;
+};
+
+// ------------------------------------------------------------------------------------------------ tile converters
+template <int QM, bool K2, int NT>
+DEVI void convert_k(Smem& S, const Params& p, const int* bt, int h, int kb, int kend, const Consts& cst) {
+  using F = Fmt<QM>;
+  for (int idx = threadIdx.x; idx < 256; idx += NT) {
+    const int tk = idx >> 2, tg = idx & 3;
+    const int j = kb * BN + tk;
+    const int row = 32 * (tk >> 5) + krow_of_token(tk & 31);
+    u32x4* dst = reinterpret_cast<u32x4*>(S.kt + row * KROW);
+    if (j >= kend) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) dst[4 * g + tg] = u32x4{0u, 0u, 0u, 0u};
+      if (K2 && tg == 0) S.kflag[row] = 0;
+      continue;
+    }
+    const uint8_t* ch = p.pool + static_cast<long long>(bt[j >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+    const int pos = j & 15;
+    uint32_t w[4];
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 c = gload<u32x2>(ch + 32 * (pos ^ ((pos >> 1) & 2)) + 8 * tg);
+      w[0] = c.x; w[1] = c.x >> 4; w[2] = c.y; w[3] = c.y >> 4;
+    } else {
+      const u32x4 c = gload<u32x4>(ch + 64 * pos + 16 * tg);
+      w[0] = c.x; w[1] = c.y; w[2] = c.z; w[3] = c.w;
+    }
+    const u32x2 sw = gload<u32x2>(ch + F::KS_OFF + 8 * pos);
+    const uint32_t s16[4] = {sw.x & 0xFFFFu, sw.x >> 16, sw.y & 0xFFFFu, sw.y >> 16};
+    uint32_t fl = 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
+      const uint32_t nz[4] = {z, z, z, z};
+      uint32_t x[4];
+      Unpack<QM>::run(w[g], nz, cst, x);
+      dst[4 * g + tg] = u32x4{pk_mul(x[0], sc), pk_mul(x[1], sc), pk_mul(x[2], sc), pk_mul(x[3], sc)};
+      fl |= (s16[g] >> 15) << g;
+    }
+    if (K2 && tg == 0) {
+      const uint32_t vw = gload<uint16_t>(ch + F::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2);
+      const uint32_t ff = vw >> 15;
+      S.kflag[row] = ff ? 16u : fl;
+    }
+  }
+}
+
+// per (group, run) scale / zero point pairs in the run order; tokens at or beyond kend get scale 0
+template <int QM, int NT>
+DEVI void v_tables(Smem& S, const Params& p, const int* bt, int h, int kb, int kend) {
+  using F = Fmt<QM>;
+  for (int idx = threadIdx.x; idx < 32; idx += NT) {
+    const int g = idx >> 3, run = idx & 7;
+    const int j0 = kb * BN + 8 * run;
+    u32x4 sc = {0u, 0u, 0u, 0u}, nz = {0u, 0u, 0u, 0u};
+    if (j0 < kend) {
+      const uint8_t* ch = p.pool + static_cast<long long>(bt[j0 >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+      const u32x4 w = gload<u32x4>(ch + F::VS_OFF + (g * PAGE + 8 * (run & 1)) * 2);   // t0 t2 | t4 t6 | t1 t3 | t5 t7
+      const uint32_t t[8] = {w.x & 0xFFFFu, w.z & 0xFFFFu, w.x >> 16, w.z >> 16, w.y & 0xFFFFu, w.w & 0xFFFFu, w.y >> 16, w.w >> 16};
+      uint32_t s[8], z[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        s[k] = j0 + k < kend ? (t[k] & 0x7FFFu) : 0u;
+        z[k] = negz16(t[k] & F::ZM);
+      }
+      sc = u32x4{s[0] | (s[4] << 16), s[1] | (s[5] << 16), s[2] | (s[6] << 16), s[3] | (s[7] << 16)};
+      nz = u32x4{z[0] | (z[4] << 16), z[1] | (z[5] << 16), z[2] | (z[6] << 16), z[3] | (z[7] << 16)};
+    }
+    *reinterpret_cast<u32x4*>(S.vsc[g][run]) = sc;
+    *reinterpret_cast<u32x4*>(S.vnz[g][run]) = nz;
+  }
+}
+
+template <int QM, int NT>
+DEVI void convert_v(Smem& S, const Params& p, const int* bt, int h, int kb, int kend, const Consts& cst) {
+  using F = Fmt<QM>;
+  for (int idx = threadIdx.x; idx < 256; idx += NT) {
+    const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, run = 2 * pgi + c8;
+    const int j0 = kb * BN + PAGE * pgi;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    const bool live = j0 < kend;
+    if (live) {
+      const uint8_t* ch = p.pool + static_cast<long long>(bt[j0 >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+      if constexpr (QM == QM_ASYM2) {
+        const u32x2 c = gload<u32x2>(ch + F::V_OFF + (e * 2 + c8) * 8);
+        w[0] = c.x; w[1] = c.x >> 4; w[2] = c.y; w[3] = c.y >> 4;
+      } else {
+        const u32x4 c = gload<u32x4>(ch + F::V_OFF + (e * 2 + c8) * 16);
+        w[0] = c.x; w[1] = c.y; w[2] = c.z; w[3] = c.w;
+      }
+    }
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      const int d = 64 * (sub >> 1) + 16 * (e >> 3) + 8 * (sub & 1) + (e & 7), g = d >> 5;
+      const u32x4 sc = *reinterpret_cast<const u32x4*>(S.vsc[g][run]);
+      const u32x4 z = *reinterpret_cast<const u32x4*>(S.vnz[g][run]);
+      const uint32_t nz[4] = {z.x, z.y, z.z, z.w};
+      uint32_t x[4];
+      Unpack<QM>::run(w[sub], nz, cst, x);
+      *reinterpret_cast<u32x4*>(S.vt + d * VROW + 16 * run) =
+          u32x4{pk_mul(x[0], sc.x), pk_mul(x[1], sc.y), pk_mul(x[2], sc.z), pk_mul(x[3], sc.w)};
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ main kernel
+template <int QM, bool K2, int NW>
+__global__ void __launch_bounds__(64 * NW) k_mq(const Params p) {
+  constexpr int NT = 64 * NW, ROWS = 32 * NW, NVAR = K2 ? 3 : 1;
+  extern __shared__ __align__(16) uint8_t lds[];
+  Smem& S = *reinterpret_cast<Smem*>(lds);
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int item = blockIdx.x, h = blockIdx.y;
+  const int* it = p.items + ITEM_INTS * item;
+  const int* tl = p.tiles + TILE_INTS * it[0];
+  const int req = tl[0], crow0 = tl[1], ntok = tl[3], pos0 = tl[4], nk = tl[5], ext = tl[8];
+  const int G = p.G, Hq = p.Hkv * G, TQ = ROWS / G;
+  const int* bt = p.bt + static_cast<long long>(req) * p.bt_stride;
+  const int kend = min(min(nk, it[2] * BN), max(pos0 + ntok - p.shift, ext + 1));
+  const int kb0 = it[1];
+  const int kb1 = kend > kb0 * BN ? (kend + BN - 1) / BN : kb0;
+  const Consts cst = make_consts();
+
+  // this lane's query row
+  const int r = 32 * wv + l32, rt = r / G;
+  const bool rvalid = r < TQ * G && rt < ntok;
+  const int lim = rvalid ? min(kend - 1, max(pos0 + rt - p.shift, ext)) : -1;   // last visible key
+
+  // q fragments: stage each rotation of the tile in LDS (natural order), then gather in code-word order
+  u32x4 qf[NVAR][8];
+#pragma unroll
+  for (int var = 0; var < NVAR; ++var) {
+    if (var) __syncthreads();
+    for (int row = tid >> 5; row < ROWS; row += NT / 32) {
+      const int t = row / G, lq = tid & 31;
+      float x[4] = {0.f, 0.f, 0.f, 0.f};
+      if (row < TQ * G && t < ntok) {
+        const u32x2 raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
+        x[0] = f16_value(raw.x & 0xFFFFu); x[1] = f16_value(raw.x >> 16);
+        x[2] = f16_value(raw.y & 0xFFFFu); x[3] = f16_value(raw.y >> 16);
+      }
+      if (var == 1) fwht<32>(x, lq);
+      if (var == 2) fwht<128>(x, lq);
+      *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = u32x2{pack_h2_rn(x[0], x[1]), pack_h2_rn(x[2], x[3])};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int dA = 32 * (s >> 1) + 4 * (2 * (s & 1) + hh);
+      const u32x2 a = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * dA);
+      const u32x2 b = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * (dA + 16));
+      // (A0 A1)(A2 A3), (B0 B1)(B2 B3) -> (A0 A2)(B0 B2)(A1 A3)(B1 B3)
+      qf[var][s] = u32x4{(a.x & 0xFFFFu) | (a.y << 16), (b.x & 0xFFFFu) | (b.y << 16),
+                         (a.x >> 16) | (a.y & 0xFFFF0000u), (b.x >> 16) | (b.y & 0xFFFF0000u)};
+    }
+  }
+
+  f32x16 o[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float mrow = -INFINITY, lrow = 0.f;
+
+  for (int kb = kb0; kb < kb1; ++kb) {
+    __syncthreads();                                   // the tiles (or the q staging) are no longer read
+    convert_k<QM, K2, NT>(S, p, bt, h, kb, kend, cst);
+    v_tables<QM, NT>(S, p, bt, h, kb, kend);
+    __syncthreads();
+    convert_v<QM, NT>(S, p, bt, h, kb, kend, cst);
+    __syncthreads();
+
+    // S^T = K q^T: two 32-key tiles, eight 16-element steps
+    f32x16 sacc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[kt][i] = 0.f;
+      const uint8_t* krow = S.kt + (32 * kt + l32) * KROW + 16 * hh;
+      if constexpr (K2) {
+        const uint32_t fl = S.kflag[32 * kt + l32];
+        const bool anyF = __any(fl & 16u), anyI = __any((fl & 16u) == 0u);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
+          const u32x4 zero = {0u, 0u, 0u, 0u};
+          const bool isF = fl & 16u, isH = (fl >> (s >> 1)) & 1u;
+          if (anyI) {
+            if (__any(!isF && !isH)) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8((!isF && !isH) ? a : zero), as_h8(qf[0][s]), sacc[kt], 0, 0, 0);
+            if (__any(isH)) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(isH ? a : zero), as_h8(qf[NVAR > 1 ? 1 : 0][s]), sacc[kt], 0, 0, 0);
+          }
+          if (anyF) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(isF ? a : zero), as_h8(qf[NVAR > 2 ? 2 : 0][s]), sacc[kt], 0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
+          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(qf[0][s]), sacc[kt], 0, 0, 0);
+        }
+      }
+    }
+    // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys)
+    const int jb = kb * BN;
+    const bool full = __all(rvalid && jb + BN - 1 <= lim) && jb >= p.kmin;
+    if (!full) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = jb + 32 * kt + token_of_acc(i, hh);
+          if (!(j <= lim && j >= p.kmin)) sacc[kt][i] = -INFINITY;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mnew = fmaxf(mrow, mx);
+    const float base = mnew == -INFINITY ? 0.f : mnew;
+    const float alpha = fexp2(mrow - base);
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sacc[kt][i] = fexp2(sacc[kt][i] - base);
+        sum += sacc[kt][i];
+      }
+    lrow = lrow * alpha + sum;
+    if (!__all(mnew == mrow)) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+    mrow = mnew;
+    // O^T += V^T P^T
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const u32x4 pb = {pack_h2_rn(sacc[kt][8 * s], sacc[kt][8 * s + 1]), pack_h2_rn(sacc[kt][8 * s + 2], sacc[kt][8 * s + 3]),
+                          pack_h2_rn(sacc[kt][8 * s + 4], sacc[kt][8 * s + 5]), pack_h2_rn(sacc[kt][8 * s + 6], sacc[kt][8 * s + 7])};
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(S.vt + (32 * db + l32) * VROW + 16 * (4 * kt + 2 * s + hh));
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(pb), o[db], 0, 0, 0);
+        }
+      }
+  }
+  // partials
+  const float l = lrow + __shfl_xor(lrow, 32, 64);
+  if (rvalid) {
+    const long long base = (static_cast<long long>(item) * p.Hkv + h) * ROWS + r;
+    float* op = p.opart + base * D;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<float4*>(op + 32 * db + 8 * q4 + 4 * hh) =
+            make_float4(o[db][4 * q4], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]);
+    if (hh == 0) *reinterpret_cast<float2*>(p.ml + base * 2) = make_float2(mrow, l);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ merge of a tile's items
+__global__ void __launch_bounds__(256) k_merge(const int* __restrict__ tiles, const float* __restrict__ opart,
+                                               const float* __restrict__ ml, int Hkv, int G, int rows, void* out,
+                                               long long o_ts, int out_fp32, float* lse, long long lse_ts) {
+  const int* tl = tiles + TILE_INTS * blockIdx.x;
+  const int h = blockIdx.y;
+  const int crow0 = tl[1], orow0 = tl[2], ntok = tl[3], item0 = tl[6], nitem = tl[7];
+  const int l32 = threadIdx.x & 31;
+  const int r = blockIdx.z * 8 + (threadIdx.x >> 5);
+  const int TQ = rows / G, Hq = Hkv * G, t = r / G;
+  if (r >= TQ * G || t >= ntok) return;
+  const int hq = h * G + r % G;
+  const long long b0 = (static_cast<long long>(item0) * Hkv + h) * rows + r, bs = static_cast<long long>(Hkv) * rows;
+  float M = -INFINITY;
+  for (int s = 0; s < nitem; ++s) M = fmaxf(M, ml[2 * (b0 + s * bs)]);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float L = 0.f;
+  if (M != -INFINITY) {
+    for (int s = 0; s < nitem; ++s) {
+      const long long b = b0 + s * bs;
+      const float2 v = *reinterpret_cast<const float2*>(ml + 2 * b);
+      if (v.x == -INFINITY) continue;
+      const float w = fexp2(v.x - M);
+      L += w * v.y;
+      const float4 x = *reinterpret_cast<const float4*>(opart + b * D + 4 * l32);
+      acc.x += w * x.x; acc.y += w * x.y; acc.z += w * x.z; acc.w += w * x.w;
+    }
+    const float inv = 1.f / L;
+    acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+  }
+  if (out_fp32) {
+    *reinterpret_cast<float4*>(static_cast<float*>(out) + (static_cast<long long>(crow0 + t) * Hq + hq) * D + 4 * l32) = acc;
+  } else {
+    uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(orow0 + t) * o_ts + hq * D + 4 * l32;
+    *reinterpret_cast<uint2*>(dst) = make_uint2(bf16_rn(acc.x) | (bf16_rn(acc.y) << 16), bf16_rn(acc.z) | (bf16_rn(acc.w) << 16));
+  }
+  if (lse != nullptr && l32 == 0)
+    lse[hq * lse_ts + crow0 + t] = M == -INFINITY ? -INFINITY : (M + log2f(L)) * 0.6931471805599453f;
+}
+
+// ------------------------------------------------------------------------------------------------ q preparation
+// one half wave per (row, q head): whole-head unnormalised H128 / 8 when kfull[kv head], then orthonormal H32 on the
+// kmask[kv head] groups, times qscale, rounded to fp16 (every operation in fp32, rounded on its own)
+__global__ void __launch_bounds__(256) k_prep(const void* q, int q_fp32, long long q_ts, const int* idx, int m, int Hq, int G,
+                                              const uint8_t* kfull, const uint8_t* kmask, float qscale, uint16_t* q16) {
+  const long long w = (static_cast<long long>(blockIdx.x) * 256 + threadIdx.x) >> 5;
+  const int l32 = threadIdx.x & 31;
+  if (w >= static_cast<long long>(m) * Hq) return;
+  const int t = static_cast<int>(w / Hq), hq = static_cast<int>(w % Hq), hk = hq / G;
+  const long long row = idx != nullptr ? idx[t] : t;
+  float x[4];
+  if (q_fp32) {
+    const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(q) + row * q_ts + hq * D + 4 * l32);
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+  } else {
+    const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(q) + row * q_ts + hq * D + 4 * l32);
+    x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
+  }
+  if (kfull != nullptr && kfull[hk]) {
+    butterflies<128>(x, l32);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] *= 0.125f;
+  }
+  if (kmask != nullptr) {
+    float y[4] = {x[0], x[1], x[2], x[3]};
+    fwht<32>(y, l32);
+    if (kmask[hk * 4 + (l32 >> 3)]) { x[0] = y[0]; x[1] = y[1]; x[2] = y[2]; x[3] = y[3]; }
+  }
+  const float a = x[0] * qscale, b = x[1] * qscale, c = x[2] * qscale, d = x[3] * qscale;
+  *reinterpret_cast<uint2*>(q16 + (static_cast<long long>(t) * Hq + hq) * D + 4 * l32) =
+      make_uint2(f16_bits_rn(a) | (f16_bits_rn(b) << 16), f16_bits_rn(c) | (f16_bits_rn(d) << 16));
+}
+
+// ------------------------------------------------------------------------------------------------ BF16 window / sink parts
+__global__ void __launch_bounds__(128) k_win_gather(const long long* map, const uint16_t* sinkb, const uint16_t* preb,
+                                                    const uint16_t* kch, long long k_ts, const uint16_t* vch,
+                                                    long long v_ts, int Hkv, uint16_t* kw, uint16_t* vw) {
+  const int d = blockIdx.x;
+  const long long code = map[d];
+  const int kind = static_cast<int>(code >> 32);
+  const long long row = code & 0xffffffffLL;
+  const int nvec = Hkv * D / 8;
+  const uint4 *ks, *vs;
+  if (kind == 2) {
+    ks = reinterpret_cast<const uint4*>(kch + row * k_ts);
+    vs = reinterpret_cast<const uint4*>(vch + row * v_ts);
+  } else {
+    const uint16_t* b = (kind == 0 ? sinkb : preb) + row * 2LL * Hkv * D;
+    ks = reinterpret_cast<const uint4*>(b);
+    vs = reinterpret_cast<const uint4*>(b + Hkv * D);
+  }
+  uint4* kd = reinterpret_cast<uint4*>(kw + static_cast<long long>(d) * Hkv * D);
+  uint4* vd = reinterpret_cast<uint4*>(vw + static_cast<long long>(d) * Hkv * D);
+  for (int i = threadIdx.x; i < nvec; i += 128) { kd[i] = ks[i]; vd[i] = vs[i]; }
+}
+
+// per (compact row, q head) half wave: page part (fp32 o, natural-log lse) + window part (bf16 o, lse) + sink part
+// (keys j < min(S, len), j <= pos - W; fp32 softmax over bf16 rows) merged by LSE -> bf16 output row idx[c]
+__global__ void __launch_bounds__(256) k_bf_merge(int m, int Hq, int Hkv, const uint16_t* q, long long q_ts,
+                                                  const long long* idx, const float* o_p, const float* lse_p,
+                                                  const uint16_t* o_w, const float* lse_w, const uint16_t* sk,
+                                                  const long long* row_req, const long long* row_pos,
+                                                  const long long* sk_len, int S, int W, float scale, uint16_t* out,
+                                                  long long o_ts) {
+  const int c = blockIdx.x, hq = blockIdx.y * 8 + (threadIdx.x >> 5), l32 = threadIdx.x & 31;
+  if (hq >= Hq) return;
+  const int G = Hq / Hkv, kvh = hq / G;
+  const long long brow = idx[c];
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, M = -INFINITY, L = 0.f;
+  {
+    const float l = lse_p[static_cast<long long>(hq) * m + c];
+    if (l != -INFINITY && l != INFINITY && l == l) {
+      const float4 v = *reinterpret_cast<const float4*>(o_p + (static_cast<long long>(c) * Hq + hq) * D + 4 * l32);
+      acc[0] = v.x; acc[1] = v.y; acc[2] = v.z; acc[3] = v.w;
+      M = l; L = 1.f;
+    }
+  }
+  auto merge = [&](float l, const float (&x)[4]) {
+    if (l == -INFINITY || l == INFINITY) return;
+    const float nm = fmaxf(M, l);
+    const float a = M == -INFINITY ? 0.f : expf(M - nm), b = expf(l - nm);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = acc[e] * a + x[e] * b;
+    L = L * a + b;
+    M = nm;
+  };
+  if (o_w != nullptr) {
+    const uint2 raw = *reinterpret_cast<const uint2*>(o_w + (static_cast<long long>(c) * Hq + hq) * D + 4 * l32);
+    const float x[4] = {bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)};
+    merge(lse_w[static_cast<long long>(hq) * m + c], x);
+  }
+  if (sk != nullptr) {
+    const long long rq = row_req[c], lim = row_pos[c] - W, nsk = sk_len[rq];
+    const uint2 qr = *reinterpret_cast<const uint2*>(q + brow * q_ts + static_cast<long long>(hq) * D + 4 * l32);
+    const float qv[4] = {bf16_lo(qr.x), bf16_hi(qr.x), bf16_lo(qr.y), bf16_hi(qr.y)};
+    float sm = -INFINITY, sl = 0.f, so[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < S; ++j) {
+      if (j >= nsk || j > lim) break;
+      const uint16_t* kr = sk + ((rq * S + j) * 2LL * Hkv + kvh) * D + 4 * l32;
+      const uint2 kk = *reinterpret_cast<const uint2*>(kr);
+      const uint2 vv = *reinterpret_cast<const uint2*>(kr + static_cast<long long>(Hkv) * D);
+      float dot = qv[0] * bf16_lo(kk.x) + qv[1] * bf16_hi(kk.x) + qv[2] * bf16_lo(kk.y) + qv[3] * bf16_hi(kk.y);
+#pragma unroll
+      for (int o = 16; o >= 1; o >>= 1) dot += hx(dot, o);
+      const float s = dot * scale, nm = fmaxf(sm, s);
+      const float a = sm == -INFINITY ? 0.f : expf(sm - nm), b = expf(s - nm);
+      so[0] = so[0] * a + bf16_lo(vv.x) * b; so[1] = so[1] * a + bf16_hi(vv.x) * b;
+      so[2] = so[2] * a + bf16_lo(vv.y) * b; so[3] = so[3] * a + bf16_hi(vv.y) * b;
+      sl = sl * a + b;
+      sm = nm;
+    }
+    if (sm != -INFINITY) {
+      const float inv = 1.f / sl;
+      const float x[4] = {so[0] * inv, so[1] * inv, so[2] * inv, so[3] * inv};
+      merge(sm + logf(sl), x);
+    }
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  *reinterpret_cast<uint2*>(out + brow * o_ts + static_cast<long long>(hq) * D + 4 * l32) =
+      make_uint2(bf16_rn(acc[0] * inv) | (bf16_rn(acc[1] * inv) << 16), bf16_rn(acc[2] * inv) | (bf16_rn(acc[3] * inv) << 16));
+}
+
+template <int QM, bool K2, int NW> int launch_mq(const Params& p, int nitems, hipStream_t st) {
+  static bool attr = false;
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_mq<QM, K2, NW>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(sizeof(Smem))) != hipSuccess) return -1;
+    attr = true;
+  }
+  hipLaunchKernelGGL((k_mq<QM, K2, NW>), dim3(nitems, p.Hkv), dim3(64 * NW), sizeof(Smem), st, p);
+  return hipPeekAtLastError() == hipSuccess ? 0 : -1;
+}
+
+int done(int rc, const char* what) {
+  if (rc == -1) std::snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(hipGetLastError()));
+  return rc;
+}
+int bad(int rc, const char* msg) {
+  std::strncpy(g_err, msg, sizeof(g_err) - 1);
+  return rc;
+}
+
+}  // namespace
+}  // namespace frmq
+
+using namespace frmq;
+
+extern "C" {
+
+int frmq_abi_version(void) { return 7; }
+const char* frmq_last_error(void) { return g_err; }
+int frmq_smem_bytes(void) { return static_cast<int>(sizeof(Smem)); }
+
+int frmq_prep_q(const void* q, int q_fp32, long long q_ts, const int* idx, int m, int Hq, int G, const uint8_t* kfull,
+                const uint8_t* kmask, float qscale, void* q16, int Dh, void* stream) {
+  if (m <= 0) return 0;
+  if (Dh != D) return bad(-4, "frmq_prep_q: head dim 128 only");
+  const long long hw = static_cast<long long>(m) * Hq;
+  hipLaunchKernelGGL(k_prep, dim3(static_cast<unsigned>((hw + 7) / 8)), dim3(256), 0, static_cast<hipStream_t>(stream), q,
+                     q_fp32, q_ts, idx, m, Hq, G, kfull, kmask, qscale, static_cast<uint16_t*>(q16));
+  return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_prep_q");
+}
+
+int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const int* bt, long long bt_stride,
+              const int* tiles, const int* items, int nitems, int Hkv, int G, int shift, int konly, float* opart,
+              float* ml, int kernel, int Dh, void* stream, int kmin) {
+  if (nitems <= 0) return 0;
+  const int rows = kernel == 1 ? 64 : 128;
+  if (G < 1 || G > rows) return bad(-3, "frmq_attn: G out of range");
+  if (Dh != D) return bad(-4, "frmq_attn: head dim 128 only");
+  if (kernel < 1 || kernel > 3) return bad(-2, "frmq_attn: kernel must be 1, 2 or 3");
+  Params p{};
+  p.q = static_cast<const uint16_t*>(q16); p.pool = pool; p.page_stride = page_stride; p.bt = bt; p.bt_stride = bt_stride;
+  p.tiles = tiles; p.items = items; p.Hkv = Hkv; p.G = G; p.shift = shift; p.kmin = kmin; p.opart = opart; p.ml = ml;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool k2 = konly & 1, i2 = konly & 2;
+  int rc;
+  if (rows == 64) {
+    rc = i2 ? (k2 ? launch_mq<QM_ASYM2, true, 2>(p, nitems, st) : launch_mq<QM_ASYM2, false, 2>(p, nitems, st))
+            : (k2 ? launch_mq<QM_ASYM4, true, 2>(p, nitems, st) : launch_mq<QM_ASYM4, false, 2>(p, nitems, st));
+  } else {
+    rc = i2 ? (k2 ? launch_mq<QM_ASYM2, true, 4>(p, nitems, st) : launch_mq<QM_ASYM2, false, 4>(p, nitems, st))
+            : (k2 ? launch_mq<QM_ASYM4, true, 4>(p, nitems, st) : launch_mq<QM_ASYM4, false, 4>(p, nitems, st));
+  }
+  return done(rc, "frmq_attn");
+}
+
+int frmq_merge(const int* tiles, int ntiles, const float* opart, const float* ml, int Hkv, int G, int rows, void* out,
+               long long o_ts, int out_fp32, float* lse, long long lse_ts, int Dh, void* stream) {
+  if (ntiles <= 0) return 0;
+  if (Dh != D) return bad(-4, "frmq_merge: head dim 128 only");
+  hipLaunchKernelGGL(k_merge, dim3(ntiles, Hkv, (rows + 7) / 8), dim3(256), 0, static_cast<hipStream_t>(stream), tiles, opart,
+                     ml, Hkv, G, rows, out, o_ts, out_fp32, lse, lse_ts);
+  return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_merge");
+}
+
+int frmq_win_gather(const long long* map, int nk, const void* sinkb, const void* preb, const void* kch, long long k_ts,
+                    const void* vch, long long v_ts, int Hkv, void* kw, void* vw, int Dh, void* stream) {
+  if (nk <= 0) return 0;
+  if (Dh != D) return bad(-4, "frmq_win_gather: head dim 128 only");
+  using U = uint16_t;
+  hipLaunchKernelGGL(k_win_gather, dim3(nk), dim3(128), 0, static_cast<hipStream_t>(stream), map, static_cast<const U*>(sinkb),
+                     static_cast<const U*>(preb), static_cast<const U*>(kch), k_ts, static_cast<const U*>(vch), v_ts, Hkv,
+                     static_cast<U*>(kw), static_cast<U*>(vw));
+  return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_win_gather");
+}
+
+int frmq_bf_merge(int m, int Hq, int Hkv, const void* q, long long q_ts, const long long* idx, const float* o_p,
+                  const float* lse_p, const void* o_w, const float* lse_w, const void* sk, const long long* row_req,
+                  const long long* row_pos, const long long* sk_len, int S, int W, float scale, void* out, long long o_ts,
+                  int Dh, void* stream) {
+  if (m <= 0) return 0;
+  if (Dh != D) return bad(-4, "frmq_bf_merge: head dim 128 only");
+  using U = uint16_t;
+  hipLaunchKernelGGL(k_bf_merge, dim3(m, (Hq + 7) / 8), dim3(256), 0, static_cast<hipStream_t>(stream), m, Hq, Hkv,
+                     static_cast<const U*>(q), q_ts, idx, o_p, lse_p, static_cast<const U*>(o_w), lse_w,
+                     static_cast<const U*>(sk), row_req, row_pos, sk_len, S, W, scale, static_cast<U*>(out), o_ts);
+  return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_bf_merge");
+}
+
+}  // extern "C"

@@ -48,6 +48,21 @@ def test_kivi_library_exports_header_symbols():
     assert kivi.plan(16, 32768, 8, sms=256) == (24, 1376) and kivi.plan(1, 100, 8, sms=256)[1] == 256
 
 
+def test_mq_library_exports_header_symbols():
+    from flagrot_releaser_amd import build, prefill_mq
+    path = build.lib_path("mq")
+    if not path.exists():
+        build.build("mq", verbose=False)
+    L = ctypes.CDLL(str(path))
+    names = _declared("flagrot_mq.h")
+    assert set(names) == set(prefill_mq.EXPORTS)
+    for n in names:
+        assert hasattr(L, n), n
+    L.frmq_abi_version.restype = ctypes.c_int
+    assert L.frmq_abi_version() == 7
+    assert 0 < L.frmq_smem_bytes() <= 160 * 1024
+
+
 def test_host_planner_invariants():
     from flagrot_releaser_amd import kernels as K
     for B, L in ((1, 1), (1, 2048), (32, 8192), (64, 16384), (3, 33000), (8, 65536)):
