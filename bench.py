@@ -1,6 +1,6 @@
 """Headline benchmark: paged FlagRot decode attention on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2|kivi]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2|kivi|mq]
 
 A step is one decode layer-step: one launch of the paged decode attention (through the C ABI of
 libflagrot_kernels.so) over the whole batch, on a synthetic cache that is already resident in HBM.  Successive steps
@@ -13,6 +13,9 @@ Workloads (BASELINE.json configs):
         batch 64, context 16384.
   kivi  configs[3]: KIVI-style FlagRot INT2 (keys per channel over 32-token groups, values per token), 128-token
         BF16 residual, Qwen-32B shape 64q/8kv, d=128, batch 16, context 32768 (libflagrot_kivi.so).
+  mq    configs[4]: prefix-cached multi-query prefill over INT4 pages (libflagrot_mq.so, the MFMA path): 4 requests x
+        512 new tokens over a 16384-token cached prefix, Qwen-32B shape 64q/8kv, d=128; --mq-fmt konlya | int4a.
+        value = TFLOP/s of the attention (4 x 128 flops per visible (row, key) pair), roofline bound "mfma".
 Prints ONE JSON line: value = achieved GB/s of page bytes (the reference's convention: B * L * Hkv * bytes per token),
 with `roofline` (HBM, measured with events on the launch stream) and `cpu_baseline` (the numpy oracle's
 dequantise-then-attend path, timed on the host on configs[0]'s shape).
@@ -182,12 +185,82 @@ def main_kivi(args, torch, dev):
     print(json.dumps(res))
 
 
+def main_mq(args, torch, dev):
+    """configs[4] through libflagrot_mq.so: one step = frmq_prep_q + frmq_attn + frmq_merge of one layer."""
+    from flagrot_releaser_amd import kernels as K
+    from flagrot_releaser_amd import prefill_mq as MQ
+    MQ.lib()
+    R, NQ, PRE, Gq = 4, 512, 16384, 8
+    L = PRE + NQ
+    fmt = args.mq_fmt
+    k2 = fmt == "konlya"
+    name = (f"configs[4]: multi-query prefill over INT4 FlagRot pages ({fmt}), Qwen-32B GQA 64q/8kv d=128, {R} requests x "
+            f"{NQ} new tokens over a {PRE}-token cached prefix (L={L}), page=16, causal inside the chunk")
+    g = torch.Generator(device=dev).manual_seed(4)
+    npg = (L + P - 1) // P
+    pool = torch.zeros(R * npg + 16, HKV, 144 * P, dtype=torch.uint8, device=dev)
+    bt = torch.randperm(R * npg + 16, generator=g, device=dev)[:R * npg].int().view(R, npg).contiguous()
+    w = 0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)
+    CT, co = torch.diag_embed(w).contiguous(), w.contiguous()
+    kmask = (torch.rand(HKV, 4, generator=g, device=dev) < 0.5).to(torch.uint8)
+    mask = torch.cat([kmask, torch.zeros_like(kmask)]).contiguous()
+    for r in range(R):
+        for s0 in range(0, L, 8192):
+            n = min(8192, L - s0)
+            kv = synth_kv(n, g, dev, torch)
+            pos = torch.arange(s0, s0 + n, device=dev)
+            slots = bt[r].long()[pos // P] * P + pos % P
+            if k2:
+                K.cb_write(kv, slots, CT, co, fmt, pool, P)
+            else:
+                K.w3_static_write(kv, slots, mask, None, pool, P, fmt=fmt)
+    torch.cuda.synchronize()
+    reqs = [(r, r * NQ, (r + 1) * NQ, L, PRE) for r in range(R)]
+    plan = MQ.build_plan(reqs, Gq, HKV, 0, dev)
+    q = (2.0 * torch.randn(R * NQ, Gq * HKV, DH, generator=g, device=dev)).bfloat16()
+    out = torch.zeros(R * NQ, Gq * HKV * DH, dtype=torch.bfloat16, device=dev)
+    scale = LOG2E / math.sqrt(DH)
+
+    def step(i):
+        q16 = MQ.prep_q(q, scale, Gq, plan.idx, None, None if k2 else kmask)
+        opart, ml = MQ.attn(q16, pool, bt, plan, Gq, 0, k2, False)
+        MQ.merge(plan, opart, ml, Gq, out=out)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    ev[0].record()
+    for i in range(args.steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
+    ms_per_step = ev[0].elapsed_time(ev[-1]) / args.steps
+    pairs = R * Gq * HKV * sum(PRE + t + 1 for t in range(NQ))
+    flops = 4.0 * DH * pairs
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    res = {
+        "metric": "multi-query prefill attention over INT4 pages: achieved TFLOP/s per layer (ms per layer alongside)",
+        "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 operands, f32 accumulate", "data": "synthetic",
+        "config": {"workload": name, "tiles": plan.ntiles, "items": plan.nitems, "rows_per_tile": plan.rows},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(tflops / 2500.0, 4), "traffic": None, "algorithmic_flops_per_launch": flops,
+                     "avg_launch_us": round(ms_per_step * 1e3, 1), "median_launch_us": round(per[len(per) // 2] * 1e3, 1),
+                     "note": "one step = frmq_prep_q + frmq_attn + frmq_merge; the attention kernel dominates"},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="int4", choices=["int4", "int2", "kivi"])
+    ap.add_argument("--workload", default="int4", choices=["int4", "int2", "kivi", "mq"])
+    ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -203,6 +276,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "kivi":
         return main_kivi(args, torch, dev)
+    if args.workload == "mq":
+        return main_mq(args, torch, dev)
     K.lib()
     if args.workload == "int4":
         kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144

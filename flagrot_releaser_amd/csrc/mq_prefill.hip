@@ -35,6 +35,7 @@ constexpr int KROW = 272;                    // bytes per K tile row: 256 + 16 p
 constexpr int VROW = 144;                    // bytes per V^T tile row: 128 + 16 pad
 constexpr int KT_BYTES = BN * KROW, VT_BYTES = D * VROW;
 constexpr int QROW = 264;                    // bytes per staged q row (natural order)
+constexpr int PG_CACHE = 1024;               // page ids kept in LDS (256 blocks of 64 keys)
 
 struct Smem {
   alignas(16) uint8_t kt[KT_BYTES];
@@ -42,6 +43,7 @@ struct Smem {
   alignas(16) uint32_t vsc[4][8][4];         // per (group, run): scale pairs (t0,t4) (t1,t5) (t2,t6) (t3,t7)
   alignas(16) uint32_t vnz[4][8][4];         // per (group, run): -(1024 + zero point) pairs
   uint32_t kflag[BN];                        // per K tile row: bits 0-3 H32 per group, bit 4 whole head
+  int pages[PG_CACHE];                       // page ids of the blocks [cb, cb + PG_CACHE / 4) of the item
 };
 static_assert(128 * QROW <= KT_BYTES + VT_BYTES, "q staging aliases the tiles");
 
@@ -92,10 +94,66 @@ template <int QM> struct Fmt {
 };
 
 // ------------------------------------------------------------------------------------------------ tile converters
+// The raw page words of a 64-key block are fetched into registers one block ahead (load_raw) and turned into the
+// fp16 tiles after the previous block's matrix work (convert_k, v_tables, convert_v).
+template <int NT> struct Raw {
+  static constexpr int NI = 256 / NT;
+  u32x4 kc[NI];      // K code words of (token, tg): INT4 four groups, INT2 two words in .x .y
+  u32x2 ks[NI];      // the token's four K scale words
+  uint32_t vf[NI];   // the token's group-0 V scale word (whole-head flag of key-only pages)
+  u32x4 vc[NI];      // V^T entry (e, c8) of a page
+  u32x4 vs;          // threads < 32: V scale words of (group, run)
+};
+
 template <int QM, bool K2, int NT>
-DEVI void convert_k(Smem& S, const Params& p, const int* bt, int h, int kb, int kend, const Consts& cst) {
+DEVI void load_raw(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, int kend) {   // pg[0] = first page of block kb
   using F = Fmt<QM>;
-  for (int idx = threadIdx.x; idx < 256; idx += NT) {
+#pragma unroll
+  for (int it = 0; it < Raw<NT>::NI; ++it) {
+    const int idx = threadIdx.x + it * NT;
+    {
+      const int tk = idx >> 2, tg = idx & 3, j = kb * BN + tk;
+      if (j < kend) {
+        const uint8_t* ch = p.pool + static_cast<long long>(pg[tk >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+        const int pos = j & 15;
+        if constexpr (QM == QM_ASYM2) {
+          const u32x2 c = gload<u32x2>(ch + 32 * (pos ^ ((pos >> 1) & 2)) + 8 * tg);
+          R.kc[it] = u32x4{c.x, c.y, 0u, 0u};
+        } else {
+          R.kc[it] = gload<u32x4>(ch + 64 * pos + 16 * tg);
+        }
+        R.ks[it] = gload<u32x2>(ch + F::KS_OFF + 8 * pos);
+        if constexpr (K2) R.vf[it] = gload<uint16_t>(ch + F::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2);
+      }
+    }
+    {
+      const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, j0 = kb * BN + PAGE * pgi;
+      if (j0 < kend) {
+        const uint8_t* ch = p.pool + static_cast<long long>(pg[pgi]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+        if constexpr (QM == QM_ASYM2) {
+          const u32x2 c = gload<u32x2>(ch + F::V_OFF + (e * 2 + c8) * 8);
+          R.vc[it] = u32x4{c.x, c.y, 0u, 0u};
+        } else {
+          R.vc[it] = gload<u32x4>(ch + F::V_OFF + (e * 2 + c8) * 16);
+        }
+      }
+    }
+  }
+  if (threadIdx.x < 32) {
+    const int g = threadIdx.x >> 3, run = threadIdx.x & 7, j0 = kb * BN + 8 * run;
+    if (j0 < kend) {
+      const uint8_t* ch = p.pool + static_cast<long long>(pg[run >> 1]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+      R.vs = gload<u32x4>(ch + F::VS_OFF + (g * PAGE + 8 * (run & 1)) * 2);   // t0 t2 | t4 t6 | t1 t3 | t5 t7
+    }
+  }
+}
+
+template <int QM, bool K2, int NT>
+DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
+  using F = Fmt<QM>;
+#pragma unroll
+  for (int it = 0; it < Raw<NT>::NI; ++it) {
+    const int idx = threadIdx.x + it * NT;
     const int tk = idx >> 2, tg = idx & 3;
     const int j = kb * BN + tk;
     const int row = 32 * (tk >> 5) + krow_of_token(tk & 31);
@@ -106,17 +164,13 @@ DEVI void convert_k(Smem& S, const Params& p, const int* bt, int h, int kb, int 
       if (K2 && tg == 0) S.kflag[row] = 0;
       continue;
     }
-    const uint8_t* ch = p.pool + static_cast<long long>(bt[j >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
-    const int pos = j & 15;
     uint32_t w[4];
     if constexpr (QM == QM_ASYM2) {
-      const u32x2 c = gload<u32x2>(ch + 32 * (pos ^ ((pos >> 1) & 2)) + 8 * tg);
-      w[0] = c.x; w[1] = c.x >> 4; w[2] = c.y; w[3] = c.y >> 4;
+      w[0] = R.kc[it].x; w[1] = R.kc[it].x >> 4; w[2] = R.kc[it].y; w[3] = R.kc[it].y >> 4;
     } else {
-      const u32x4 c = gload<u32x4>(ch + 64 * pos + 16 * tg);
-      w[0] = c.x; w[1] = c.y; w[2] = c.z; w[3] = c.w;
+      w[0] = R.kc[it].x; w[1] = R.kc[it].y; w[2] = R.kc[it].z; w[3] = R.kc[it].w;
     }
-    const u32x2 sw = gload<u32x2>(ch + F::KS_OFF + 8 * pos);
+    const u32x2 sw = R.ks[it];
     const uint32_t s16[4] = {sw.x & 0xFFFFu, sw.x >> 16, sw.y & 0xFFFFu, sw.y >> 16};
     uint32_t fl = 0;
 #pragma unroll
@@ -128,25 +182,20 @@ DEVI void convert_k(Smem& S, const Params& p, const int* bt, int h, int kb, int 
       dst[4 * g + tg] = u32x4{pk_mul(x[0], sc), pk_mul(x[1], sc), pk_mul(x[2], sc), pk_mul(x[3], sc)};
       fl |= (s16[g] >> 15) << g;
     }
-    if (K2 && tg == 0) {
-      const uint32_t vw = gload<uint16_t>(ch + F::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2);
-      const uint32_t ff = vw >> 15;
-      S.kflag[row] = ff ? 16u : fl;
-    }
+    if (K2 && tg == 0) S.kflag[row] = (R.vf[it] >> 15) ? 16u : fl;
   }
 }
 
 // per (group, run) scale / zero point pairs in the run order; tokens at or beyond kend get scale 0
 template <int QM, int NT>
-DEVI void v_tables(Smem& S, const Params& p, const int* bt, int h, int kb, int kend) {
+DEVI void v_tables(Smem& S, const Raw<NT>& R, int kb, int kend) {
   using F = Fmt<QM>;
-  for (int idx = threadIdx.x; idx < 32; idx += NT) {
-    const int g = idx >> 3, run = idx & 7;
+  if (threadIdx.x < 32) {
+    const int g = threadIdx.x >> 3, run = threadIdx.x & 7;
     const int j0 = kb * BN + 8 * run;
     u32x4 sc = {0u, 0u, 0u, 0u}, nz = {0u, 0u, 0u, 0u};
     if (j0 < kend) {
-      const uint8_t* ch = p.pool + static_cast<long long>(bt[j0 >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
-      const u32x4 w = gload<u32x4>(ch + F::VS_OFF + (g * PAGE + 8 * (run & 1)) * 2);   // t0 t2 | t4 t6 | t1 t3 | t5 t7
+      const u32x4 w = R.vs;
       const uint32_t t[8] = {w.x & 0xFFFFu, w.z & 0xFFFFu, w.x >> 16, w.z >> 16, w.y & 0xFFFFu, w.w & 0xFFFFu, w.y >> 16, w.w >> 16};
       uint32_t s[8], z[8];
 #pragma unroll
@@ -163,21 +212,18 @@ DEVI void v_tables(Smem& S, const Params& p, const int* bt, int h, int kb, int k
 }
 
 template <int QM, int NT>
-DEVI void convert_v(Smem& S, const Params& p, const int* bt, int h, int kb, int kend, const Consts& cst) {
-  using F = Fmt<QM>;
-  for (int idx = threadIdx.x; idx < 256; idx += NT) {
+DEVI void convert_v(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
+#pragma unroll
+  for (int it = 0; it < Raw<NT>::NI; ++it) {
+    const int idx = threadIdx.x + it * NT;
     const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, run = 2 * pgi + c8;
     const int j0 = kb * BN + PAGE * pgi;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
-    const bool live = j0 < kend;
-    if (live) {
-      const uint8_t* ch = p.pool + static_cast<long long>(bt[j0 >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+    if (j0 < kend) {
       if constexpr (QM == QM_ASYM2) {
-        const u32x2 c = gload<u32x2>(ch + F::V_OFF + (e * 2 + c8) * 8);
-        w[0] = c.x; w[1] = c.x >> 4; w[2] = c.y; w[3] = c.y >> 4;
+        w[0] = R.vc[it].x; w[1] = R.vc[it].x >> 4; w[2] = R.vc[it].y; w[3] = R.vc[it].y >> 4;
       } else {
-        const u32x4 c = gload<u32x4>(ch + F::V_OFF + (e * 2 + c8) * 16);
-        w[0] = c.x; w[1] = c.y; w[2] = c.z; w[3] = c.w;
+        w[0] = R.vc[it].x; w[1] = R.vc[it].y; w[2] = R.vc[it].z; w[3] = R.vc[it].w;
       }
     }
 #pragma unroll
@@ -196,7 +242,7 @@ DEVI void convert_v(Smem& S, const Params& p, const int* bt, int h, int kb, int 
 
 // ------------------------------------------------------------------------------------------------ main kernel
 template <int QM, bool K2, int NW>
-__global__ void __launch_bounds__(64 * NW) k_mq(const Params p) {
+__global__ void __launch_bounds__(64 * NW, K2 ? 1 : 2) k_mq(const Params p) {
   constexpr int NT = 64 * NW, ROWS = 32 * NW, NVAR = K2 ? 3 : 1;
   extern __shared__ __align__(16) uint8_t lds[];
   Smem& S = *reinterpret_cast<Smem*>(lds);
@@ -216,6 +262,16 @@ __global__ void __launch_bounds__(64 * NW) k_mq(const Params p) {
   const int r = 32 * wv + l32, rt = r / G;
   const bool rvalid = r < TQ * G && rt < ntok;
   const int lim = rvalid ? min(kend - 1, max(pos0 + rt - p.shift, ext)) : -1;   // last visible key
+
+  // page ids of the first blocks (published by the barriers of the q staging below)
+  int cb = kb0;
+  auto fill_pages = [&]() {
+    for (int i = tid; i < PG_CACHE; i += NT) {
+      const int pgx = 4 * cb + i;
+      S.pages[i] = pgx * PAGE < kend ? bt[pgx] : 0;
+    }
+  };
+  fill_pages();
 
   // q fragments: stage each rotation of the tile in LDS (natural order), then gather in code-word order
   u32x4 qf[NVAR][8];
@@ -253,14 +309,21 @@ __global__ void __launch_bounds__(64 * NW) k_mq(const Params p) {
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float mrow = -INFINITY, lrow = 0.f;
 
-  for (int kb = kb0; kb < kb1; ++kb) {
+  Raw<NT> rawA, rawB;
+  if (kb0 < kb1) load_raw<QM, K2, NT>(rawA, p, S.pages, h, kb0, kend);
+  if (kb0 + 1 < kb1) load_raw<QM, K2, NT>(rawB, p, S.pages + 4, h, kb0 + 1, kend);
+  auto block_step = [&](Raw<NT>& raw, int kb) {
     __syncthreads();                                   // the tiles (or the q staging) are no longer read
-    convert_k<QM, K2, NT>(S, p, bt, h, kb, kend, cst);
-    v_tables<QM, NT>(S, p, bt, h, kb, kend);
+    convert_k<QM, K2, NT>(S, raw, kb, kend, cst);
+    v_tables<QM, NT>(S, raw, kb, kend);
+    if (kb + 2 < kb1 && kb + 2 >= cb + PG_CACHE / 4) {   // the next fetch leaves the cached window: slide it
+      cb = kb + 2;
+      fill_pages();
+    }
     __syncthreads();
-    convert_v<QM, NT>(S, p, bt, h, kb, kend, cst);
+    convert_v<QM, NT>(S, raw, kb, kend, cst);
     __syncthreads();
-
+    if (kb + 2 < kb1) load_raw<QM, K2, NT>(raw, p, S.pages + 4 * (kb + 2 - cb), h, kb + 2, kend);   // two blocks ahead
     // S^T = K q^T: two 32-key tiles, eight 16-element steps
     f32x16 sacc[2];
 #pragma unroll
@@ -340,6 +403,10 @@ __global__ void __launch_bounds__(64 * NW) k_mq(const Params p) {
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(pb), o[db], 0, 0, 0);
         }
       }
+  };
+  for (int kb = kb0; kb < kb1; kb += 2) {
+    block_step(rawA, kb);
+    if (kb + 1 < kb1) block_step(rawB, kb + 1);
   }
   // partials
   const float l = lrow + __shfl_xor(lrow, 32, 64);
