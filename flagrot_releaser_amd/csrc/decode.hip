@@ -27,29 +27,6 @@ namespace {
 DEVI float dot2(uint32_t a, uint32_t b, float c) { return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), c, false); }
 DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-DEVI float dpp_xor1(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
-}
-DEVI float dpp_xor2(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
-}
-template <int X> DEVI float swz_xor(float v) {  // xor 4 / 8 / 16 inside a 32-lane half
-  return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (X << 10) | 0x1F));
-}
-DEVI float xor32(float v) { return __shfl_xor(v, 32, 64); }
-DEVI float wave_max_over_tokens(float v) {  // lanes of a quad already agree
-  v = fmaxf(v, swz_xor<4>(v)); v = fmaxf(v, swz_xor<8>(v)); v = fmaxf(v, swz_xor<16>(v));
-  return fmaxf(v, xor32(v));
-}
-DEVI float wave_sum_over_tokens(float v) {
-  v += swz_xor<4>(v); v += swz_xor<8>(v); v += swz_xor<16>(v);
-  return v + xor32(v);
-}
-DEVI void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 constexpr int NWAVE = 4;
 // LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per variant /
@@ -182,14 +159,6 @@ struct WaveState {
   float acc[4][4];   // [head][entry word] of the lane's V^T entries
 };
 
-DEVI float wave_max64(float v) {
-  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
-  return wave_max_over_tokens(v);
-}
-DEVI float wave_sum64(float v) {
-  v += dpp_xor1(v); v += dpp_xor2(v);
-  return wave_sum_over_tokens(v);
-}
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
 template <int QM, bool K2>

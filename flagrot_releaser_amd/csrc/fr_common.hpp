@@ -138,6 +138,40 @@ DEVI uint32_t quant_group(const float (&y)[4], float (&q)[4], float (&deq)[4]) {
   else return quant_asym<QM == QM_ASYM4 ? 4 : 2, WANT_DEQ>(y, q, deq);
 }
 
+// ---------------------------------------------------------------------------------------------- wave reductions
+// xor 1 / 2 by DPP quad permutes, xor 4 / 8 / 16 by ds_swizzle, xor 32 by a wave shuffle
+DEVI float dpp_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+DEVI float dpp_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+}
+template <int X> DEVI float swz_xor(float v) {  // xor 4 / 8 / 16 inside a 32-lane half
+  return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (X << 10) | 0x1F));
+}
+DEVI float xor32(float v) { return __shfl_xor(v, 32, 64); }
+DEVI float wave_max_over_tokens(float v) {  // lanes of a quad already agree
+  v = fmaxf(v, swz_xor<4>(v)); v = fmaxf(v, swz_xor<8>(v)); v = fmaxf(v, swz_xor<16>(v));
+  return fmaxf(v, xor32(v));
+}
+DEVI float wave_sum_over_tokens(float v) {
+  v += swz_xor<4>(v); v += swz_xor<8>(v); v += swz_xor<16>(v);
+  return v + xor32(v);
+}
+DEVI float wave_max64(float v) {
+  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
+  return wave_max_over_tokens(v);
+}
+DEVI float wave_sum64(float v) {
+  v += dpp_xor1(v); v += dpp_xor2(v);
+  return wave_sum_over_tokens(v);
+}
+DEVI void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // ---------------------------------------------------------------------------------------------- page layout
 template <int QM, int P> struct Lay {
   static constexpr int CB = QM == QM_ASYM2 ? 32 : 64;  // code bytes per (token, K or V row)

@@ -14,5 +14,10 @@ int dequant_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nvali
                    hipStream_t st);
 int lse_merge_launch(const void* oa, const float* la, long long la_hs, const void* ob, const float* lb, long long lb_hs,
                      void* out, long long out_rs, int na, int H, int D, hipStream_t st);
+// splits [0, NS) over the pages and split NS over the BF16 ring rows (kivi_decode.hip): partials per (sequence, KV head,
+// split): opart fp32 [.., G, 128] unnormalised, ml fp32 [.., G, 2] = (maximum in log2 units, sum)
+int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
+                       const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
+                       const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, hipStream_t st);
 
 }  // namespace frkv

@@ -24,11 +24,6 @@ DEVI int kv_code(float x, float mn, float s) {
   return static_cast<int>(rintf(q));
 }
 DEVI float kv_rec(int code, float mn, float s) { return static_cast<float>(code) * s + mn; }
-DEVI void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 template <int C> DEVI void to_basis(float (&y)[4], int l32) {   // candidate 0 identity, 1 H32, 2 H128
   if (C == 1) fwht<32>(y, l32);
   if (C == 2) fwht<128>(y, l32);
