@@ -2,15 +2,17 @@
 //
 // One workgroup (4 wavefronts) per (KV head x q tile of 4 heads, split, sequence).  A wavefront streams whole pages
 // (16 tokens x one KV head = one contiguous 2304 / 1280 byte chunk) with 128-bit loads:
-//   key phase    lane = (token, quarter): 16 B of the token's code row = 8 elements of each 32-group.  The codes are
-//                turned into fp16 pairs by mask-and-or with an exponent pattern (value = offset + code, exact) and
-//                contracted with the query by v_dot2_f32_f16.  The query is rotated three ways once per workgroup
+//   key phase    lane = token: its code row, 8 elements of each 32-group per 16-byte quarter.  A code field masked in
+//                place is an fp16 denormal (value code * 2^(position - 24), exact) and is contracted with the query by
+//                v_dot2_f32_f16; the powers of two ride on the query operand and the scale.  The query is rotated three ways once per workgroup
 //                (identity, H32 per group, H128) and kept in LDS in the code words' element order; every lane fetches
 //                the variant its token / group flags ask for, so selection costs no arithmetic.  The exponent offsets
 //                and the zero points are removed with per-(variant, head, group) query sums.
 //   softmax      exp2-domain online softmax per wavefront; p * V-scale is written to LDS as fp16 in V^T token order.
-//   value phase  lane = one 16-byte V^T entry (4 dims x 8 tokens): the same unpacking, contracted with p * scale over
-//                the tokens; offsets / zero points are removed once per workgroup from running per-group sums.
+//   value phase  lane = one 16-byte V^T entry (4 dims x 8 tokens): a code field masked in place is an fp16 denormal
+//                (value code * 2^(position - 24), exact), contracted with p * scale over the tokens by v_dot2; the
+//                powers of two ride on the p * scale operand and one final multiply, the zero points leave through
+//                sum p * scale * zero point, contracted once per (page half, group, head) from the same LDS strips.
 // The four wavefronts are merged through LDS; splits through the caller's workspace with a ticket counter (the last
 // arriving workgroup of a (sequence, KV head) merges, normalises, optionally rotates back, and stores bf16).
 // The BF16 sink / window rows are one more split handled by an extra workgroup of the same grid.
@@ -36,12 +38,13 @@ constexpr int QV_BYTES = 3 * QV_VSTRIDE * 16;      // [variant][head][tg][j][8 f
 constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (page, c8): 16 + 1 pad
 constexpr int PB_BYTES = 8 * PB_RSTRIDE * 16;      // per wave: [page][c8][group][head][8 fp16]
 constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
-constexpr int ZB_BYTES = 8 * ZB_RSTRIDE * 16;      // per wave: [page][c8][group][8 fp16] = -(1024 + zero point)
+constexpr int ZB_BYTES = 8 * ZB_RSTRIDE * 16;      // per wave: [page][c8][group][8 fp16] = zero point (x 2^SH for odd tokens)
 
 struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
   alignas(16) uint8_t pb[NWAVE][PB_BYTES];
   alignas(16) uint8_t zb[NWAVE][ZB_BYTES];
+  alignas(16) float qsum[3][4][4];                   // [variant][group][head]: sum of the group's (fp16) query elements
   alignas(16) float o[NWAVE][4][128];
   float m[NWAVE][4], l[NWAVE][4];
   int last;
@@ -52,7 +55,7 @@ DEVI int kslot(int isB, int i) { return 2 * (2 * (i & 1) + isB) + (i >> 1); }
 DEVI int vslot(int r8) { return 2 * (r8 & 3) + (r8 >> 2); }
 
 // Rotates the q tile three ways and stores it as fp16 in code-word order (the identity variant of a bf16 query is
-// exact in fp16; qscale is applied to the fp32 score).
+// exact in fp16; qscale is applied to the fp32 score), with the sums per 32-group that remove the key zero points.
 template <int QM, bool K2>
 DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
   const int w = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
@@ -83,12 +86,18 @@ DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
     }
+    // the B elements of a code word are unpacked with the factor 2^SH (UnpackD): their query slots carry 2^-SH
+    const float fold = ((l32 >> 2) & 1) ? 1.f / static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
+    float qs = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int d = 4 * l32 + i, r = d & 31;
       const int isB = r >> 4, tg = (r & 15) >> 2, ii = r & 3;
-      reinterpret_cast<_Float16*>(S.qv)[(var * QV_VSTRIDE + (w * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i]);
+      qs += static_cast<float>(static_cast<_Float16>(v[i]));
+      reinterpret_cast<_Float16*>(S.qv)[(var * QV_VSTRIDE + (w * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i] * fold);
     }
+    qs += hx(qs, 1); qs += hx(qs, 2); qs += hx(qs, 4);
+    if ((l32 & 7) == 0) S.qsum[var][g][w] = qs;
   }
 }
 
@@ -156,13 +165,14 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
 struct WaveState {
   float m[4];        // running maximum per head (wave uniform)
   float l[4];        // this lane's share of the running sum per head
-  float acc[4][4];   // [head][entry word] of the lane's V^T entries
+  float acc[4][4];   // [head][entry word] of the lane's V^T entries: 2^-24 sum p' code (zero points not yet removed)
+  float z[2];        // lane = (page, half, group, head pair): its share of sum p' zero point, heads 2 hp and 2 hp + 1
 };
 
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
 template <int QM, bool K2>
-DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, const Consts& cst, float (&sc)[4]) {
+DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
   const bool full = K2 && (r.vs[0] & 0x8000u);
@@ -170,16 +180,14 @@ DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, const Const
   for (int h = 0; h < 4; ++h) sc[h] = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const uint32_t nz1 = negz16(kw[j] & ZM) * 0x00010001u;
-    const uint32_t nz[4] = {nz1, nz1, nz1, nz1};
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
     const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + var * QV_VSTRIDE + j;   // + head * 16 + tg * 4
     float a[4];
 #pragma unroll
     for (int tg = 0; tg < 4; ++tg) {
       uint32_t x[4];
-      if constexpr (QM == QM_ASYM2) Unpack<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], nz, cst, x);
-      else Unpack<QM>::run(r.kc[tg][j], nz, cst, x);
+      if constexpr (QM == QM_ASYM2) UnpackD<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], x);
+      else UnpackD<QM>::run(r.kc[tg][j], x);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const uint4 qq = qp[h * 16 + tg * 4];
@@ -191,9 +199,16 @@ DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, const Const
         a[h] = v;
       }
     }
+    // a = 2^-24 sum code q: score += scale (2^24 a - zero point * sum q)
     const float sj = f16_value(kw[j] & 0x7FFFu) * qscale;
+    const float sj24 = sj * 16777216.f;
+    if constexpr (ZM != 0) {
+      const float4 qs = *reinterpret_cast<const float4*>(&S.qsum[var][j][0]);
+      const float sz = -sj * static_cast<float>(kw[j] & ZM);
+      sc[0] += sz * qs.x; sc[1] += sz * qs.y; sc[2] += sz * qs.z; sc[3] += sz * qs.w;
+    }
 #pragma unroll
-    for (int h = 0; h < 4; ++h) sc[h] += sj * a[h];
+    for (int h = 0; h < 4; ++h) sc[h] += sj24 * a[h];
   }
 }
 
@@ -216,6 +231,7 @@ DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[
       st.l[h] *= alpha;
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha;
+      if ((lane & 1) == (h >> 1)) st.z[h & 1] *= alpha;
     }
   }
   const int pi = lane >> 4, pos = lane & 15;
@@ -225,21 +241,24 @@ DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[
     p[h] = valid ? fexp2(sc[h] - st.m[h]) : 0.f;
     st.l[h] += p[h];
   }
-  // p' = p * V scale per group as fp16, and -(1024 + zero point), in V^T token order of the token's page
+  // p' = p * V scale per group as fp16 and the zero points (fp16 integers), in V^T token order of the token's page.
+  // Odd tokens are unpacked with the factor 2^SH (UnpackD): their p' carries 2^-SH and their zero point 2^SH.
   const int rg = pi * 2 + (pos >> 3), sl = vslot(pos & 7);
   _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
-  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb[wave]) + rg * ZB_RSTRIDE * 8 + sl;      // + group * 8
+  _Float16* zb = reinterpret_cast<_Float16*>(S.zb[wave]) + rg * ZB_RSTRIDE * 8 + sl;     // + group * 8
+  const float fold = (pos & 1) ? 1.f / static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
+  const float unfold = (pos & 1) ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const float sv = f16_value(r.vs[g] & 0x7FFFu);
+    const float svf = valid ? f16_value(r.vs[g] & 0x7FFFu) * fold : 0.f;     // unwritten slots may hold any pattern
 #pragma unroll
-    for (int h = 0; h < 4; ++h) pb[(g * 4 + h) * 8] = valid ? static_cast<_Float16>(p[h] * sv) : static_cast<_Float16>(0.f);
-    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<uint16_t>(negz16(r.vs[g] & ZM));
+    for (int h = 0; h < 4; ++h) pb[(g * 4 + h) * 8] = static_cast<_Float16>(p[h] * svf);
+    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<_Float16>(static_cast<float>(r.vs[g] & ZM) * unfold);
   }
 }
 
 template <int QM>
-DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave, const Consts& cst) {
+DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
   const int c8 = lane & 1, g0 = lane >> 5;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -250,15 +269,12 @@ DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane
       uint4 pq[4];
 #pragma unroll
       for (int h = 0; h < 4; ++h) pq[h] = pp[g * 4 + h];
-      uint4 zz = make_uint4(0, 0, 0, 0);
-      if constexpr (QM != QM_SYM4) zz = (reinterpret_cast<const uint4*>(S.zb[wave]) + (k * 2 + c8) * ZB_RSTRIDE)[g];
-      const uint32_t nz[4] = {zz.x, zz.y, zz.z, zz.w};
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const int sub = 2 * half + s2;
         uint32_t x[4];
-        if constexpr (QM == QM_ASYM2) Unpack<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], nz, cst, x);
-        else Unpack<QM>::run(r.vc[k][sub], nz, cst, x);
+        if constexpr (QM == QM_ASYM2) UnpackD<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], x);
+        else UnpackD<QM>::run(r.vc[k][sub], x);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
           float a = st.acc[h][sub];
@@ -269,6 +285,18 @@ DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane
           st.acc[h][sub] = a;
         }
       }
+    }
+  }
+  if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (page, page half, group, head pair)
+    const int rg = lane >> 3, g = (lane >> 1) & 3, hp = lane & 1;
+    const uint4 zq = (reinterpret_cast<const uint4*>(S.zb[wave]) + rg * ZB_RSTRIDE)[g];
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const uint4 pq = pp[e];
+      float a = st.z[e];
+      a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
+      st.z[e] = a;
     }
   }
 }
@@ -333,6 +361,7 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] = 0.f;
     }
+    st.z[0] = st.z[1] = 0.f;
     if (lo < hi) {   // uniform over the workgroup
       q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
@@ -345,7 +374,6 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
         return (const uint8_t*)(pool + (static_cast<long long>(bt[min(pg, pg1 - 1)]) * p.Hkv + kvh) * L::CHUNK);
       };
       KRegs<QM> cur;
-      const Consts cst = make_consts();
       int q4 = pg0 + 4 * wave;       // first page of this wave's current quad
       const uint8_t* mine = chunk_of(q4 + pi);
       if (q4 < pg1) load_k<QM, P>(cur, mine, pos);
@@ -365,7 +393,7 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
         const int tok = (q4 + pi) * P + pos;
         const bool valid = tok >= lo && tok < hi;
         float sc[4];
-        key_phase<QM, K2>(S, cur, p.qscale, cst, sc);
+        key_phase<QM, K2>(S, cur, p.qscale, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
         const int qn = q4 + 4 * NWAVE;   // the key registers are free: the next quad's keys fly during the value phase
         if (qn < pg1) {
@@ -373,15 +401,30 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
           load_k<QM, P>(cur, mine, pos);
         }
         wave_lds_sync();
-        value_phase<QM>(S, st, vr, lane, wave, cst);
+        value_phase<QM>(S, st, vr, lane, wave);
         wave_lds_sync();
       }
     }
-    // ---- fold the wave: entry pairs (c8 = 0 / 1), offset sums per (head, group)
+    // ---- fold the wave: zero-point sums per (head, group) through the wave's strip, entry pairs (c8 = 0 / 1),
+    //      codes -> values: 2^24 acc - sum p' zero point
+    if constexpr (QM != QM_SYM4) {
+      float z0 = st.z[0], z1 = st.z[1];
+      z0 += swz_xor<8>(z0); z1 += swz_xor<8>(z1);
+      z0 += swz_xor<16>(z0); z1 += swz_xor<16>(z1);
+      z0 += xor32(z0); z1 += xor32(z1);
+      float* zs = reinterpret_cast<float*>(S.pb[wave]);          // [head][group]; the strips are dead by now
+      if (lane < 8) { zs[(2 * (lane & 1)) * 4 + (lane >> 1)] = z0; zs[(2 * (lane & 1) + 1) * 4 + (lane >> 1)] = z1; }
+      wave_lds_sync();
+    }
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
+      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] = (st.acc[h][s4] + dpp_xor1(st.acc[h][s4])) * 16777216.f;
+      if constexpr (QM != QM_SYM4) {
+        const float* zs = reinterpret_cast<const float*>(S.pb[wave]) + h * 4 + (lane >> 5);
+        const float z01 = zs[0], z23 = zs[2];
+        st.acc[h][0] -= z01; st.acc[h][1] -= z01; st.acc[h][2] -= z23; st.acc[h][3] -= z23;
+      }
       const float lsum = wave_sum64(st.l[h]);
       if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = lsum; }
     }

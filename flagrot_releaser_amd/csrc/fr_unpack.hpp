@@ -50,6 +50,35 @@ template <> struct Unpack<QM_SYM4> {  // sign-magnitude bytes s0000mmm -> exact 
     x[0] = pair(a, c); x[1] = pair(b, c); x[2] = pair(a >> 8, c); x[3] = pair(b >> 8, c);
   }
 };
+// Denormal form: a code field masked IN PLACE inside the low 10 bits of an fp16 half is a denormal whose value is
+// code * 2^(position - 24), exactly; v_dot2_f32_f16 takes denormal inputs at full precision.  The four pairs come out as
+// (f0,f4) (f1,f5) (f2,f6) (f3,f7) like above, but pairs 1 and 3 carry the factor 2^SH (SH = field width) and every pair the
+// factor 2^-24: the other operand of the contraction is pre-scaled by 2^-SH in those slots, the sum by 2^24, and the zero
+// point is removed through sums of that other operand (sum(c - z) q = sum c q - z sum q).
+template <int QM> struct UnpackD;
+template <> struct UnpackD<QM_ASYM4> {
+  static constexpr int SH = 4;
+  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
+    const uint32_t t = w >> 8;
+    x[0] = w & 0x000F000Fu; x[1] = w & 0x00F000F0u; x[2] = t & 0x000F000Fu; x[3] = t & 0x00F000F0u;
+  }
+};
+template <> struct UnpackD<QM_ASYM2> {   // fields at bits 0, 2, 8, 10 (+16) of the (pre-shifted) word
+  static constexpr int SH = 2;
+  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
+    const uint32_t t = w >> 8;
+    x[0] = w & 0x00030003u; x[1] = w & 0x000C000Cu; x[2] = t & 0x00030003u; x[3] = t & 0x000C000Cu;
+  }
+};
+template <> struct UnpackD<QM_SYM4> {    // sign-magnitude bytes s0000mmm -> signed denormals (no extra factor)
+  static constexpr int SH = 0;
+  static DEVI uint32_t pair(uint32_t bytes02) { return (bytes02 & 0x00070007u) | ((bytes02 & 0x00800080u) << 8); }
+  static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
+    const uint32_t a = w & 0x87878787u;                                   // A_i in byte i
+    const uint32_t b = ((w << 4) | (w >> 28)) & 0x87878787u;              // B_i in byte i
+    x[0] = pair(a); x[1] = pair(b); x[2] = pair(a >> 8); x[3] = pair(b >> 8);
+  }
+};
 // fp16 pattern of -(1024 + z)
 DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
