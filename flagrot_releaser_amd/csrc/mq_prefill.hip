@@ -8,8 +8,9 @@
 //   V^T [128 dims][64] eight-token runs exactly as the page stores them;
 // and every wavefront runs v_mfma_f32_32x32x16_f16 transposed: S^T = K q^T (lane = one query row, 32 keys in
 // registers: the softmax needs one cross-lane step), P^T straight from the accumulators as the B operand of
-// O^T = V^T P^T.  Key-only pages (per-token H32 / H128 flags): the query tile is kept in three rotations and the K
-// operand is zero-masked per (token, group) for each, so keys are never transformed.
+// O^T = V^T P^T.  Key-only pages (per-token H32 / H128 flags): the conversion applies the token's inverse transform to
+// the fp16 pairs in registers (packed butterflies, the quad of a token exchanging by DPP) before the tile is stored, so
+// the matrix part is the same for every format.
 // Causal rule: key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext), j < nk.
 // Partials (unnormalised O, running maximum in log2 units, sum) per (item, KV head, row); k_merge combines the items
 // of a tile.  Semantics follow integrations/vllm_flagrot/csrc/mq_prefill.cu:345-498 (k_mq), :716-772 (merge),
@@ -42,7 +43,6 @@ struct Smem {
   alignas(16) uint8_t vt[VT_BYTES];
   alignas(16) uint32_t vsc[4][8][4];         // per (group, run): scale pairs (t0,t4) (t1,t5) (t2,t6) (t3,t7)
   alignas(16) uint32_t vnz[4][8][4];         // per (group, run): -(1024 + zero point) pairs
-  uint32_t kflag[BN];                        // per K tile row: bits 0-3 H32 per group, bit 4 whole head
   int pages[PG_CACHE];                       // page ids of the blocks [cb, cb + PG_CACHE / 4) of the item
 };
 static_assert(128 * QROW <= KT_BYTES + VT_BYTES, "q staging aliases the tiles");
@@ -92,6 +92,41 @@ template <int QM> struct Fmt {
   static constexpr int V_OFF = CB * PAGE, KS_OFF = 2 * CB * PAGE, VS_OFF = KS_OFF + 8 * PAGE, CHUNK = VS_OFF + 8 * PAGE;
   static constexpr uint32_t ZM = QM == QM_ASYM2 ? 3u : 15u;
 };
+
+// ------------------------------------------------------------------------------------------------ key-only pages
+// Inverse transform of one token's keys while they are fp16 pairs in registers.  A thread holds, per 32-group, the 8
+// elements d = 4 tg + i (A_i) and 16 + 4 tg + i (B_i) as (A0 A2) (B0 B2) (A1 A3) (B1 B3); the four threads of a quad
+// (tg = lane & 3) hold the group.  Index bits of d: bit 0 = registers 0,1 <-> 2,3; bit 1 = low <-> high half; bits 2,3 =
+// the quad lanes (DPP); bit 4 = registers 0 <-> 1, 2 <-> 3; the two group bits of the whole-head transform = registers of
+// different groups.  The five stages inside a group run on the integers code - zero point (exact in fp16), then the
+// group scale times an exact power of two (2^-2 per group, 2^-3 whole head) is applied, then the two whole-head stages;
+// the remaining 2^-0.5 is one multiply at the end.
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+DEVI h2_t h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+DEVI uint32_t u2(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
+DEVI void bfly(uint32_t& a, uint32_t& b) {
+  const h2_t x = h2(a), y = h2(b);
+  a = u2(x + y); b = u2(x - y);
+}
+DEVI uint32_t bfly_halves(uint32_t a) {                       // (lo, hi) -> (lo + hi, lo - hi)
+  const uint32_t sw = (a >> 16) | (a << 16);
+  const h2_t sg = h2(0xBC003C00u);                            // (1, -1)
+  return u2(__builtin_elementwise_fma(h2(a), sg, h2(sw)));
+}
+template <int CTRL> DEVI uint32_t bfly_lanes(uint32_t a, uint32_t sgn) {   // sgn = (1,1) on the lower lane, (-1,-1) on the upper
+  const uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(a), CTRL, 0xF, 0xF, true));
+  return u2(__builtin_elementwise_fma(h2(a), h2(sgn), h2(o)));
+}
+DEVI void h32_group(uint32_t (&x)[4], uint32_t sgn1, uint32_t sgn2) {
+  bfly(x[0], x[2]); bfly(x[1], x[3]);                          // d bit 0
+#pragma unroll
+  for (int r = 0; r < 4; ++r) x[r] = bfly_halves(x[r]);        // d bit 1
+#pragma unroll
+  for (int r = 0; r < 4; ++r) x[r] = bfly_lanes<0xB1>(x[r], sgn1);   // d bit 2: quad lanes xor 1
+#pragma unroll
+  for (int r = 0; r < 4; ++r) x[r] = bfly_lanes<0x4E>(x[r], sgn2);   // d bit 3: quad lanes xor 2
+  bfly(x[0], x[1]); bfly(x[2], x[3]);                          // d bit 4
+}
 
 // ------------------------------------------------------------------------------------------------ tile converters
 // The raw page words of a 64-key block are fetched into registers one block ahead (load_raw) and turned into the
@@ -161,7 +196,6 @@ DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
     if (j >= kend) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) dst[4 * g + tg] = u32x4{0u, 0u, 0u, 0u};
-      if (K2 && tg == 0) S.kflag[row] = 0;
       continue;
     }
     uint32_t w[4];
@@ -172,17 +206,59 @@ DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
     }
     const u32x2 sw = R.ks[it];
     const uint32_t s16[4] = {sw.x & 0xFFFFu, sw.x >> 16, sw.y & 0xFFFFu, sw.y >> 16};
-    uint32_t fl = 0;
+    if constexpr (!K2) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
-      const uint32_t nz[4] = {z, z, z, z};
-      uint32_t x[4];
-      Unpack<QM>::run(w[g], nz, cst, x);
-      dst[4 * g + tg] = u32x4{pk_mul(x[0], sc), pk_mul(x[1], sc), pk_mul(x[2], sc), pk_mul(x[3], sc)};
-      fl |= (s16[g] >> 15) << g;
+      for (int g = 0; g < 4; ++g) {
+        const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
+        const uint32_t nz[4] = {z, z, z, z};
+        uint32_t x[4];
+        Unpack<QM>::run(w[g], nz, cst, x);
+        dst[4 * g + tg] = u32x4{pk_mul(x[0], sc), pk_mul(x[1], sc), pk_mul(x[2], sc), pk_mul(x[3], sc)};
+      }
+    } else {
+      // key-only pages: the token's flags select identity / H32 per group / whole-head H128 (the quad of a token agrees)
+      const bool ff = (R.vf[it] >> 15) & 1u;
+      const uint32_t sgn1 = (tg & 1) ? 0xBC00BC00u : 0x3C003C00u, sgn2 = (tg & 2) ? 0xBC00BC00u : 0x3C003C00u;
+      uint32_t x[4][4], y[4][4];
+      bool rot[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        rot[g] = ff || ((s16[g] >> 15) & 1u);
+        const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
+        const uint32_t pre = ff ? 0x30003000u : 0x34003400u;                                 // 2^-3, 2^-2 (exact)
+        const uint32_t sce = pk_mul(sc, pre);
+        const uint32_t nz[4] = {z, z, z, z};
+        uint32_t c[4];
+        Unpack<QM>::run(w[g], nz, cst, c);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { x[g][r] = pk_mul(c[r], sc); y[g][r] = c[r]; }
+        h32_group(y[g], sgn1, sgn2);              // on the integers code - zero point: exact (|sum| <= 32 * 15)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[g][r] = pk_mul(y[g][r], sce);
+      }
+      if (__any(ff)) {                                           // the two group bits of the whole-head transform
+        uint32_t f[4][4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) f[g][r] = y[g][r];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { bfly(f[0][r], f[1][r]); bfly(f[2][r], f[3][r]); }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { bfly(f[0][r], f[2][r]); bfly(f[1][r], f[3][r]); }
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) y[g][r] = ff ? f[g][r] : y[g][r];
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x4 v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = rot[g] ? pk_mul(y[g][r], 0x39A839A8u) : x[g][r];   // 2^-0.5
+        dst[4 * g + tg] = v;
+      }
     }
-    if (K2 && tg == 0) S.kflag[row] = (R.vf[it] >> 15) ? 16u : fl;
   }
 }
 
@@ -240,10 +316,79 @@ DEVI void convert_v(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
   }
 }
 
+// ------------------------------------------------------------------------------------------------ one 64-key block
+// scores, mask, online softmax and values of the wavefront's 32 rows against the tiles in LDS
+DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
+                       bool rvalid, int kmin, int l32, int hh) {
+  // S^T = K q^T: two 32-key tiles, eight 16-element steps
+  f32x16 sacc[2];
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[kt][i] = 0.f;
+    const uint8_t* krow = S.kt + (32 * kt + l32) * KROW + 16 * hh;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
+      sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(qf[s]), sacc[kt], 0, 0, 0);
+    }
+  }
+  // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys)
+  const int jb = kb * BN;
+  const bool full = __all(rvalid && jb + BN - 1 <= lim) && jb >= kmin;
+  if (!full) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = jb + 32 * kt + token_of_acc(i, hh);
+        if (!(j <= lim && j >= kmin)) sacc[kt][i] = -INFINITY;
+      }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float mnew = fmaxf(mrow, mx);
+  const float base = mnew == -INFINITY ? 0.f : mnew;
+  const float alpha = fexp2(mrow - base);
+  float sum = 0.f;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sacc[kt][i] = fexp2(sacc[kt][i] - base);
+      sum += sacc[kt][i];
+    }
+  lrow = lrow * alpha + sum;
+  if (!__all(mnew == mrow)) {
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+  }
+  mrow = mnew;
+  // O^T += V^T P^T
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const u32x4 pb = {pack_h2_rn(sacc[kt][8 * s], sacc[kt][8 * s + 1]), pack_h2_rn(sacc[kt][8 * s + 2], sacc[kt][8 * s + 3]),
+                        pack_h2_rn(sacc[kt][8 * s + 4], sacc[kt][8 * s + 5]), pack_h2_rn(sacc[kt][8 * s + 6], sacc[kt][8 * s + 7])};
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(S.vt + (32 * db + l32) * VROW + 16 * (4 * kt + 2 * s + hh));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(pb), o[db], 0, 0, 0);
+      }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ main kernel
 template <int QM, bool K2, int NW>
-__global__ void __launch_bounds__(64 * NW, K2 ? 1 : 2) k_mq(const Params p) {
-  constexpr int NT = 64 * NW, ROWS = 32 * NW, NVAR = K2 ? 3 : 1;
+__global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
+  constexpr int NT = 64 * NW, ROWS = 32 * NW;
   extern __shared__ __align__(16) uint8_t lds[];
   Smem& S = *reinterpret_cast<Smem*>(lds);
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
@@ -273,33 +418,23 @@ __global__ void __launch_bounds__(64 * NW, K2 ? 1 : 2) k_mq(const Params p) {
   };
   fill_pages();
 
-  // q fragments: stage each rotation of the tile in LDS (natural order), then gather in code-word order
-  u32x4 qf[NVAR][8];
+  // q fragments: the tile through LDS (natural order), gathered in code-word order
+  u32x4 qf[8];
+  for (int row = tid >> 5; row < ROWS; row += NT / 32) {
+    const int t = row / G, lq = tid & 31;
+    u32x2 raw = {0u, 0u};
+    if (row < TQ * G && t < ntok) raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
+    *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = raw;
+  }
+  __syncthreads();
 #pragma unroll
-  for (int var = 0; var < NVAR; ++var) {
-    if (var) __syncthreads();
-    for (int row = tid >> 5; row < ROWS; row += NT / 32) {
-      const int t = row / G, lq = tid & 31;
-      float x[4] = {0.f, 0.f, 0.f, 0.f};
-      if (row < TQ * G && t < ntok) {
-        const u32x2 raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
-        x[0] = f16_value(raw.x & 0xFFFFu); x[1] = f16_value(raw.x >> 16);
-        x[2] = f16_value(raw.y & 0xFFFFu); x[3] = f16_value(raw.y >> 16);
-      }
-      if (var == 1) fwht<32>(x, lq);
-      if (var == 2) fwht<128>(x, lq);
-      *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = u32x2{pack_h2_rn(x[0], x[1]), pack_h2_rn(x[2], x[3])};
-    }
-    __syncthreads();
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const int dA = 32 * (s >> 1) + 4 * (2 * (s & 1) + hh);
-      const u32x2 a = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * dA);
-      const u32x2 b = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * (dA + 16));
-      // (A0 A1)(A2 A3), (B0 B1)(B2 B3) -> (A0 A2)(B0 B2)(A1 A3)(B1 B3)
-      qf[var][s] = u32x4{(a.x & 0xFFFFu) | (a.y << 16), (b.x & 0xFFFFu) | (b.y << 16),
-                         (a.x >> 16) | (a.y & 0xFFFF0000u), (b.x >> 16) | (b.y & 0xFFFF0000u)};
-    }
+  for (int s = 0; s < 8; ++s) {
+    const int dA = 32 * (s >> 1) + 4 * (2 * (s & 1) + hh);
+    const u32x2 a = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * dA);
+    const u32x2 b = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * (dA + 16));
+    // (A0 A1)(A2 A3), (B0 B1)(B2 B3) -> (A0 A2)(B0 B2)(A1 A3)(B1 B3)
+    qf[s] = u32x4{(a.x & 0xFFFFu) | (a.y << 16), (b.x & 0xFFFFu) | (b.y << 16),
+                  (a.x >> 16) | (a.y & 0xFFFF0000u), (b.x >> 16) | (b.y & 0xFFFF0000u)};
   }
 
   f32x16 o[4];
@@ -324,85 +459,7 @@ __global__ void __launch_bounds__(64 * NW, K2 ? 1 : 2) k_mq(const Params p) {
     convert_v<QM, NT>(S, raw, kb, kend, cst);
     __syncthreads();
     if (kb + 2 < kb1) load_raw<QM, K2, NT>(raw, p, S.pages + 4 * (kb + 2 - cb), h, kb + 2, kend);   // two blocks ahead
-    // S^T = K q^T: two 32-key tiles, eight 16-element steps
-    f32x16 sacc[2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[kt][i] = 0.f;
-      const uint8_t* krow = S.kt + (32 * kt + l32) * KROW + 16 * hh;
-      if constexpr (K2) {
-        const uint32_t fl = S.kflag[32 * kt + l32];
-        const bool anyF = __any(fl & 16u), anyI = __any((fl & 16u) == 0u);
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
-          const u32x4 zero = {0u, 0u, 0u, 0u};
-          const bool isF = fl & 16u, isH = (fl >> (s >> 1)) & 1u;
-          if (anyI) {
-            if (__any(!isF && !isH)) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8((!isF && !isH) ? a : zero), as_h8(qf[0][s]), sacc[kt], 0, 0, 0);
-            if (__any(isH)) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(isH ? a : zero), as_h8(qf[NVAR > 1 ? 1 : 0][s]), sacc[kt], 0, 0, 0);
-          }
-          if (anyF) sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(isF ? a : zero), as_h8(qf[NVAR > 2 ? 2 : 0][s]), sacc[kt], 0, 0, 0);
-        }
-      } else {
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
-          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(qf[0][s]), sacc[kt], 0, 0, 0);
-        }
-      }
-    }
-    // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys)
-    const int jb = kb * BN;
-    const bool full = __all(rvalid && jb + BN - 1 <= lim) && jb >= p.kmin;
-    if (!full) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int j = jb + 32 * kt + token_of_acc(i, hh);
-          if (!(j <= lim && j >= p.kmin)) sacc[kt][i] = -INFINITY;
-        }
-    }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mnew = fmaxf(mrow, mx);
-    const float base = mnew == -INFINITY ? 0.f : mnew;
-    const float alpha = fexp2(mrow - base);
-    float sum = 0.f;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        sacc[kt][i] = fexp2(sacc[kt][i] - base);
-        sum += sacc[kt][i];
-      }
-    lrow = lrow * alpha + sum;
-    if (!__all(mnew == mrow)) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-    }
-    mrow = mnew;
-    // O^T += V^T P^T
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const u32x4 pb = {pack_h2_rn(sacc[kt][8 * s], sacc[kt][8 * s + 1]), pack_h2_rn(sacc[kt][8 * s + 2], sacc[kt][8 * s + 3]),
-                          pack_h2_rn(sacc[kt][8 * s + 4], sacc[kt][8 * s + 5]), pack_h2_rn(sacc[kt][8 * s + 6], sacc[kt][8 * s + 7])};
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(S.vt + (32 * db + l32) * VROW + 16 * (4 * kt + 2 * s + hh));
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(pb), o[db], 0, 0, 0);
-        }
-      }
+    attend_block(S, qf, o, mrow, lrow, kb, lim, rvalid, p.kmin, l32, hh);
   };
   for (int kb = kb0; kb < kb1; kb += 2) {
     block_step(rawA, kb);
