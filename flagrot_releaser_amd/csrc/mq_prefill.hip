@@ -320,18 +320,38 @@ DEVI void convert_v(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
 // scores, mask, online softmax and values of the wavefront's 32 rows against the tiles in LDS
 DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
                        bool rvalid, int kmin, int l32, int hh) {
-  // S^T = K q^T: two 32-key tiles, eight 16-element steps
+  // S^T = K q^T: two 32-key tiles (two independent accumulator chains), eight 16-element steps; the K operands of four
+  // steps are requested ahead, and the scheduler is told to keep the reads that far in front of the matrix instructions
   f32x16 sacc[2];
 #pragma unroll
-  for (int kt = 0; kt < 2; ++kt) {
+  for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[kt][i] = 0.f;
-    const uint8_t* krow = S.kt + (32 * kt + l32) * KROW + 16 * hh;
+  {
+    const uint8_t* k0 = S.kt + l32 * KROW + 16 * hh;
+    const uint8_t* k1 = k0 + 32 * KROW;
+    u32x4 a0[8], a1[8];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      a0[s] = *reinterpret_cast<const u32x4*>(k0 + 64 * (s >> 1) + 32 * (s & 1));
+      a1[s] = *reinterpret_cast<const u32x4*>(k1 + 64 * (s >> 1) + 32 * (s & 1));
+    }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const u32x4 a = *reinterpret_cast<const u32x4*>(krow + 64 * (s >> 1) + 32 * (s & 1));
-      sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(qf[s]), sacc[kt], 0, 0, 0);
+      if (s + 4 < 8) {
+        a0[s + 4] = *reinterpret_cast<const u32x4*>(k0 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+        a1[s + 4] = *reinterpret_cast<const u32x4*>(k1 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+      }
+      sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a0[s]), as_h8(qf[s]), sacc[0], 0, 0, 0);
+      sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a1[s]), as_h8(qf[s]), sacc[1], 0, 0, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // 8 LDS reads
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     // 2 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // 2 LDS reads
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
   }
   // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys)
   const int jb = kb * BN;
@@ -370,19 +390,37 @@ DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], floa
       for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
   }
   mrow = mnew;
-  // O^T += V^T P^T
+  // O^T += V^T P^T: four independent accumulator chains (the 32-dim blocks); V^T operands requested two steps ahead
+  {
+    u32x4 pb[4], va[4][4];
 #pragma unroll
-  for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const u32x4 pb = {pack_h2_rn(sacc[kt][8 * s], sacc[kt][8 * s + 1]), pack_h2_rn(sacc[kt][8 * s + 2], sacc[kt][8 * s + 3]),
-                        pack_h2_rn(sacc[kt][8 * s + 4], sacc[kt][8 * s + 5]), pack_h2_rn(sacc[kt][8 * s + 6], sacc[kt][8 * s + 7])};
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(S.vt + (32 * db + l32) * VROW + 16 * (4 * kt + 2 * s + hh));
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a), as_h8(pb), o[db], 0, 0, 0);
-      }
+    for (int ks = 0; ks < 4; ++ks) {      // ks = 2 kt + s
+      const int kt = ks >> 1, s2 = ks & 1;
+      pb[ks] = u32x4{pack_h2_rn(sacc[kt][8 * s2], sacc[kt][8 * s2 + 1]), pack_h2_rn(sacc[kt][8 * s2 + 2], sacc[kt][8 * s2 + 3]),
+                     pack_h2_rn(sacc[kt][8 * s2 + 4], sacc[kt][8 * s2 + 5]), pack_h2_rn(sacc[kt][8 * s2 + 6], sacc[kt][8 * s2 + 7])};
     }
+    const uint8_t* v0 = S.vt + l32 * VROW + 16 * hh;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) va[ks][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * ks);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks + 2 < 4) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db) va[ks + 2][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * (ks + 2));
+      }
+#pragma unroll
+      for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(va[ks][db]), as_h8(pb[ks]), o[db], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 1);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ main kernel
