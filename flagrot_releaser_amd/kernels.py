@@ -395,3 +395,144 @@ def head_fwht(x, flags, scale, out=None):
         _check(lib().fr_head_fwht(x.data_ptr(), x.stride(0), out.data_ptr(), out.stride(0), T, H, flags.data_ptr(),
                                   scale, _stream(), Dh), "fr_head_fwht")
     return out
+
+
+# ------------------------------------------------------------------------------------------------ torch page parsers
+# Host-side readers of the page bytes (any device, no library call): what the plugin's PyTorch prefill path and tests use
+# to look inside a cache.  Mirrors parse_int4_pages / parse_int2_pages / parse_pages / dequant_v2_pages / hadamard /
+# dequant_cb_pages of the reference front end (vllm_flagrot/kernels.py:591-765); the key-only 2x2 kinds only.
+_MAPS: dict = {}
+
+
+def _layout_maps(fmt: str, page: int, device):
+    """gather maps of one 128-d chunk: for every (token, K|V, dim) the byte holding its code and the bit position, and
+    for every (token, K|V, group) the byte offset of its 16-bit scale word.  INT4 symmetric additionally: byte / bit of
+    the sign and of the 3-bit magnitude."""
+    key = (fmt, page, str(device))
+    if key in _MAPS:
+        return _MAPS[key]
+    P = page
+    int2, sym = fmt in INT2_FMTS, fmt in ("int4", "konly")
+    cb = 32 if int2 else 64
+    t = torch.arange(P).view(P, 1)
+    d = torch.arange(128).view(1, 128)
+    g, r = d // 32, d % 32
+    isB, tg, i = r // 16, (r % 16) // 4, r % 4
+    # V^T entry of a dim and position of a token inside it
+    e = ((d % 64) // 16) * 8 + d % 8
+    sub = 2 * (d // 64) + (d % 16) // 8
+    c8, ii, odd = t // 8, (t % 8) // 2, t % 2
+    if int2:
+        kbyte = 32 * (t ^ ((t >> 1) & 2)) + 8 * tg + 4 * (g // 2) + i
+        kshift = 4 * (g % 2) + 2 * isB + 0 * t
+        vbyte = cb * P + (e * (P // 8) + c8) * 8 + 4 * (d // 64) + ii
+        vshift = 4 * ((d % 16) // 8) + 2 * odd
+        maps = dict(byte=torch.stack([kbyte, vbyte], 1), shift=torch.stack([kshift.expand(P, 128), vshift], 1))
+    else:
+        kbyte = 64 * t + 16 * tg + 4 * g + i
+        vbyte = cb * P + (e * (P // 8) + c8) * 16 + 4 * sub + ii
+        if not sym:
+            kshift = (4 * isB).expand(P, 128)
+            vshift = (4 * odd).expand(P, 128)
+            maps = dict(byte=torch.stack([kbyte, vbyte], 1), shift=torch.stack([kshift, vshift], 1))
+        else:
+            # A element: sign bit 7, magnitude bits 0-2 of its byte; B element: sign bit 3 of its byte, magnitude bits
+            # 4-6 of the byte (k + 3) % 4 of the same word
+            kB = isB.expand(P, 128).bool()
+            vB = odd.expand(P, 128).bool()
+            kmagb = torch.where(kB, 64 * t + 16 * tg + 4 * g + (i + 3) % 4, kbyte)
+            vmagb = torch.where(vB, cb * P + (e * (P // 8) + c8) * 16 + 4 * sub + (ii + 3) % 4, vbyte)
+            B2 = torch.stack([kB, vB], 1)
+            maps = dict(byte=torch.stack([kbyte, vbyte], 1), magbyte=torch.stack([kmagb, vmagb], 1),
+                        signbit=torch.where(B2, 3, 7), magshift=torch.where(B2, 4, 0))
+    gg = torch.arange(4).view(1, 4)
+    slot8 = torch.where(t % 2 == 1, 4 + (t % 8) // 2, (t % 8) // 2)
+    ks = 2 * cb * P + 8 * t + 2 * gg
+    vs = 2 * cb * P + 8 * P + (gg * P + 8 * (t // 8) + slot8) * 2
+    maps["scale"] = torch.stack([ks, vs], 1)                                        # [P, 2, 4] byte offsets
+    maps = {k: v.to(device) for k, v in maps.items()}
+    _MAPS[key] = maps
+    return maps
+
+
+def parse_pages(chunks, page, fmt, Dh=128):
+    """chunks uint8 [Np, H, >= chunk bytes] of a static format ("int4" | "int4a" | "int2a") or key-only kind ("konly" |
+    "konlya" | "konlya2") -> codes int16 [Np, H, P, 2, Dh] (K then V, stored coordinates, zero point already subtracted
+    for the asymmetric formats), scale magnitudes fp32 [Np, H, P, 2, Dh / 32] (the word read as FP16 without its sign
+    bit), raw scale words int16 [Np, H, P, 2, Dh / 32] (zero point in the low bits, flags in the sign bits).
+    Dh 256: the chunk is two 128-d half chunks (dims 0-127, then 128-255)."""
+    Np, H = chunks.shape[:2]
+    if Dh == 256:
+        half = (80 if fmt in INT2_FMTS else 144) * page
+        c, m, sb = parse_pages(chunks[..., :2 * half].reshape(Np, 2 * H, half), page, fmt)
+        join = lambda x: x.reshape(Np, H, 2, page, 2, x.shape[-1]).permute(0, 1, 3, 4, 2, 5).reshape(Np, H, page, 2, -1)  # noqa: E731
+        return join(c), join(m), join(sb)
+    assert Dh == 128
+    mp = _layout_maps(fmt, page, chunks.device)
+    by = chunks.to(torch.int16)
+    if "shift" in mp:
+        width = 3 if fmt in INT2_FMTS else 15
+        codes = (by[..., mp["byte"]] >> mp["shift"]) & width
+    else:
+        sign = (by[..., mp["byte"]] >> mp["signbit"]) & 1
+        mag = (by[..., mp["magbyte"]] >> mp["magshift"]) & 7
+        codes = torch.where(sign == 1, -mag, mag)
+    so = mp["scale"]
+    lo, hi = chunks[..., so].to(torch.int32), chunks[..., so + 1].to(torch.int32)
+    word = lo | (hi << 8)
+    sbits = torch.where(word >= 32768, word - 65536, word).to(torch.int16)              # [Np, H, P, 2, 4]
+    mag = (sbits & 0x7FFF).view(torch.float16).float()
+    if fmt not in ("int4", "konly"):
+        zmask = 3 if fmt in INT2_FMTS else 15
+        codes = codes - (sbits & zmask).repeat_interleave(RB, -1)
+    return codes.to(torch.int16), mag, sbits
+
+
+def parse_int4_pages(chunks, page, asym=False, Dh=128):
+    return parse_pages(chunks, page, "int4a" if asym else "int4", Dh)
+
+
+def parse_int2_pages(chunks, page, Dh=128):
+    return parse_pages(chunks, page, "int2a", Dh)
+
+
+def dequant_v2_pages(chunks, page, dtype=torch.bfloat16, fmt="int4", Dh=128):
+    """static pages -> K, V [Np, P, H, Dh] in the STORED (rotated) basis: codes times the group's scale magnitude."""
+    codes, mag, _ = parse_pages(chunks, page, fmt, Dh)
+    x = codes.float().reshape(*codes.shape[:-1], Dh // RB, RB) * mag[..., None]
+    x = x.reshape(codes.shape).to(dtype)
+    return x[..., 0, :].transpose(1, 2), x[..., 1, :].transpose(1, 2)
+
+
+_HM: dict = {}
+
+
+def hadamard(n, device, dtype=torch.float32):
+    """orthonormal Sylvester-Hadamard matrix (symmetric)."""
+    key = (n, str(device), dtype)
+    if key not in _HM:
+        h = torch.ones(1, 1, dtype=torch.float64)
+        while h.shape[0] < n:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        _HM[key] = (h / math.sqrt(n)).to(device=device, dtype=dtype)
+    return _HM[key]
+
+
+def dequant_cb_pages(chunks, page, kind, dtype=torch.bfloat16, Dh=128):
+    """key-only 2x2 pages -> K, V [Np, P, H, Dh]: keys in the ORIGINAL basis (H32 on the groups whose K scale word has
+    its sign bit set, whole-head H_Dh when the token's group-0 V scale word has), values as stored."""
+    if kind not in K2:
+        raise NotImplementedError(f"codebook kind {kind}: only the key-only 2x2 kinds are built")
+    Np, H = chunks.shape[:2]
+    codes, mag, sbits = parse_pages(chunks, page, kind, Dh)
+    ng = Dh // RB
+    dev = chunks.device
+    x = codes.float().reshape(*codes.shape[:-1], ng, RB) * mag[..., None]                # [Np, H, P, 2, ng, 32]
+    whole = sbits[..., 1, 0] < 0                                                         # [Np, H, P]
+    local = sbits[..., 0, :] < 0                                                         # [Np, H, P, ng]
+    k = x[..., 0, :, :]
+    kl = torch.where(local[..., None], k @ hadamard(RB, dev), k).reshape(Np, H, page, Dh)
+    kf = k.reshape(Np, H, page, Dh) @ hadamard(Dh, dev)
+    k = torch.where(whole[..., None], kf, kl).to(dtype)
+    v = x[..., 1, :, :].reshape(Np, H, page, Dh).to(dtype)
+    return k.transpose(1, 2), v.transpose(1, 2)
