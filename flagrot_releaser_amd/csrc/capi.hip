@@ -1,5 +1,6 @@
 // extern "C" surface of libflagrot_kernels.so (declared in include/flagrot_kernels.h): argument checks, the
 // reference's return codes, and dispatch to the launchers of writer.hip / decode.hip.
+#include <cstdlib>
 #include <cstdio>
 #include <cstring>
 
@@ -40,6 +41,18 @@ bool fmt_int2(int fmt) { return fmt == FMT_INT2A || fmt == FMT_KONLYA2; }
 
 using namespace fr;
 
+namespace {
+int device_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t pr;
+    n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) ? pr.multiProcessorCount : 256;
+  }
+  return n;
+}
+}  // namespace
+
 extern "C" {
 
 int fr_abi_version(void) { return 9; }
@@ -75,6 +88,20 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   p.out = out; p.o_bs = o_bs;
   p.tail = tail; p.tail_len = tail_len; p.tail_idx = tail_idx; p.tail_bs = tail_bs; p.tail_ts = tail_ts;
   p.gqa = gqa; p.kv_start = kv_start;
+  // Two launch shapes.  (a) The split plan fills the CUs at most once with long chunks: one large workgroup per CU, each
+  // owning its chunk, its wavefronts drawing quads of pages from a counter in LDS.  (b) Otherwise workgroups of 4
+  // wavefronts, and where the slot's counter word can hold both (one q tile per slot, tickets above the draw bits) the
+  // body workgroups of a (sequence, KV head, q tile) share its whole page range and draw quads from the slot's
+  // counter: the split plan then only says how many workgroups there are.  FLAGROT_DECODE_STATIC=1 keeps fixed
+  // ranges, FLAGROT_WG_WAVES=4 | 12 forces a workgroup size.
+  const int nparts = nsplit + (tail != nullptr ? 1 : 0);
+  static const bool force_static = getenv("FLAGROT_DECODE_STATIC") != nullptr && getenv("FLAGROT_DECODE_STATIC")[0] == '1';
+  static const int env_waves = getenv("FLAGROT_WG_WAVES") != nullptr ? atoi(getenv("FLAGROT_WG_WAVES")) : 0;
+  const long long wgs = static_cast<long long>(B) * Hkv * ntile * nsplit;
+  const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && wgs <= device_cus());
+  const bool can_draw = !force_static && counter != nullptr && p.counter_div == 1 && nparts <= 1023;
+  p.wg_waves = big ? decode_waves(1 << 30) : 4;
+  p.dyn = (can_draw && (!big || env_waves > 4)) ? 1 : 0;
   return launched(decode_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_attn");
 }
 
@@ -92,7 +119,7 @@ int fr_v2_write(int fmt, const void* kv, long long kv_ts, const long long* slots
 int fr_v2_occupancy(int fmt, int variant, int stages, int page) {
   (void)variant; (void)stages;
   if (page != 16 || fmt < FMT_INT4 || fmt > FMT_KONLYA2) return 0;
-  return decode_occupancy(fmt);
+  return decode_occupancy(fmt, 4);
 }
 int fr_v2_chunk_bytes(int fmt, int page) { return page * (fmt_int2(fmt) ? 80 : 144); }
 
@@ -154,7 +181,7 @@ int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* bl
 int fr_cb_occupancy(int kind, int variant, int stages, int page) {
   (void)variant; (void)stages;
   if (page != 16 || fmt_of_kind(kind) < 0) return 0;
-  return decode_occupancy(fmt_of_kind(kind));
+  return decode_occupancy(fmt_of_kind(kind), 4);
 }
 int fr_cb_chunk_bytes(int kind, int page) { return page * (kind == KIND_KONLYA2 ? 80 : 144); }
 int fr_cb_write_smem(int kind, int tg, int hd) {

@@ -1,7 +1,9 @@
 // Paged split-K GQA decode attention over FlagRot INT4 / INT2 pages for gfx950 (wave64, no matrix cores).
 //
-// One workgroup (4 wavefronts) per (KV head x q tile of 4 heads, split, sequence).  A wavefront streams whole pages
-// (16 tokens x one KV head = one contiguous 2304 / 1280 byte chunk) with 128-bit loads:
+// One workgroup (16 wavefronts = a whole CU's register file, or 4 for short chunks) per (KV head x q tile of 4 heads,
+// split, sequence).  Its wavefronts draw quads of 4 pages from a counter in LDS, so they finish together whatever
+// share of the issue slots each one got.  A wavefront streams whole pages (16 tokens x one KV head = one contiguous
+// 2304 / 1280 byte chunk) with 128-bit loads:
 //   key phase    lane = token: its code row, 8 elements of each 32-group per 16-byte quarter.  A code field masked in
 //                place is an fp16 denormal (value code * 2^(position - 24), exact) and is contracted with the query by
 //                v_dot2_f32_f16; the powers of two ride on the query operand and the scale.  The query is rotated three ways once per workgroup
@@ -13,7 +15,7 @@
 //                (value code * 2^(position - 24), exact), contracted with p * scale over the tokens by v_dot2; the
 //                powers of two ride on the p * scale operand and one final multiply, the zero points leave through
 //                sum p * scale * zero point, contracted once per (page half, group, head) from the same LDS strips.
-// The four wavefronts are merged through LDS; splits through the caller's workspace with a ticket counter (the last
+// The wavefronts are merged through LDS; splits through the caller's workspace with a ticket counter (the last
 // arriving workgroup of a (sequence, KV head) merges, normalises, optionally rotates back, and stores bf16).
 // The BF16 sink / window rows are one more split handled by an extra workgroup of the same grid.
 //
@@ -30,7 +32,6 @@ DEVI float dot2(uint32_t a, uint32_t b, float c) { return __builtin_amdgcn_fdot2
 DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 
-constexpr int NWAVE = 4;
 // LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per variant /
 // per row group) start in different banks.
 constexpr int QV_VSTRIDE = 65;                     // uint4 per variant: 64 + 1 pad
@@ -39,15 +40,26 @@ constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (page,
 constexpr int PB_BYTES = 8 * PB_RSTRIDE * 16;      // per wave: [page][c8][group][head][8 fp16]
 constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
 constexpr int ZB_BYTES = 8 * ZB_RSTRIDE * 16;      // per wave: [page][c8][group][8 fp16] = zero point (x 2^SH for odd tokens)
+constexpr int STRIP_BYTES = PB_BYTES + ZB_BYTES;   // per wave
+constexpr int DRAW_BATCH = 2;                      // quads per draw from the shared (device-scope) counter
+constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
+constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
 
+template <int NW>
 struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
-  alignas(16) uint8_t pb[NWAVE][PB_BYTES];
-  alignas(16) uint8_t zb[NWAVE][ZB_BYTES];
+  // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
+  alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
   alignas(16) float qsum[3][4][4];                   // [variant][group][head]: sum of the group's (fp16) query elements
-  alignas(16) float o[NWAVE][4][128];
-  float m[NWAVE][4], l[NWAVE][4];
+  float m[NW][4], l[NW][4];
+  int btc[BT_CACHE];
+  int next;                                          // next quad of 4 pages nobody has taken yet
   int last;
+  DEVI uint8_t* pb(int w) { return work + w * STRIP_BYTES; }
+  DEVI const uint8_t* pb(int w) const { return work + w * STRIP_BYTES; }
+  DEVI uint8_t* zb(int w) { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI const uint8_t* zb(int w) const { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI float* o(int w, int h) { return reinterpret_cast<float*>(work) + (w * 4 + h) * 128; }
 };
 
 // slot of element (isB, i) of a K word / of token r8 of a V word inside the 8-fp16 operand vector
@@ -56,8 +68,8 @@ DEVI int vslot(int r8) { return 2 * (r8 & 3) + (r8 >> 2); }
 
 // Rotates the q tile three ways and stores it as fp16 in code-word order (the identity variant of a bf16 query is
 // exact in fp16; qscale is applied to the fp32 score), with the sums per 32-group that remove the key zero points.
-template <int QM, bool K2>
-DEVI void q_prologue(Smem& S, const DecodeParams& p, int b, int kvh, int tile) {
+template <int QM, bool K2, class SM>
+DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {   // wavefronts 0..3: one head each
   const int w = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
   const int hq = tile * 4 + w;                       // head inside the GQA group
   float x[4] = {0.f, 0.f, 0.f, 0.f};
@@ -171,13 +183,13 @@ struct WaveState {
 
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
-template <int QM, bool K2>
-DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
+template <int QM, bool K2, class SM>
+DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float sc0, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
   const bool full = K2 && (r.vs[0] & 0x8000u);
 #pragma unroll
-  for (int h = 0; h < 4; ++h) sc[h] = 0.f;
+  for (int h = 0; h < 4; ++h) sc[h] = sc0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
@@ -191,8 +203,9 @@ DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const uint4 qq = qp[h * 16 + tg * 4];
-        float v = tg == 0 ? 0.f : a[h];
-        v = dot2(x[0], qq.x, v);
+        float v;
+        if (tg == 0) asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(v) : "v"(x[0]), "v"(qq.x));   // no register clear
+        else v = dot2(x[0], qq.x, a[h]);
         v = dot2(x[1], qq.y, v);
         v = dot2(x[2], qq.z, v);
         v = dot2(x[3], qq.w, v);
@@ -213,8 +226,8 @@ DEVI void key_phase(const Smem& S, const KRegs<QM>& r, float qscale, float (&sc)
 }
 
 // online softmax step for 64 tokens: the running maximum is only re-reduced over the wave when some lane beats it
-template <int QM>
-DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], bool valid, int lane, int wave) {
+template <int QM, class SM>
+DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], bool valid, int lane, int wave) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   bool beat = false;
 #pragma unroll
@@ -238,31 +251,37 @@ DEVI void softmax_phase(Smem& S, WaveState& st, const KRegs<QM>& r, float (&sc)[
   float p[4];
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
-    p[h] = valid ? fexp2(sc[h] - st.m[h]) : 0.f;
+    p[h] = fexp2(sc[h] - st.m[h]);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
     st.l[h] += p[h];
   }
-  // p' = p * V scale per group as fp16 and the zero points (fp16 integers), in V^T token order of the token's page.
-  // Odd tokens are unpacked with the factor 2^SH (UnpackD): their p' carries 2^-SH and their zero point 2^SH.
+  // p' = p * V scale per group as fp16 (packed fp16 products of head pairs) and the zero points, in V^T token order
+  // of the token's page.  Odd tokens are unpacked with the factor 2^SH (UnpackD): their scores were lowered by SH
+  // (p carries 2^-SH), their zero point is raised by 2^SH; zero points are fp16 denormals like the codes.
   const int rg = pi * 2 + (pos >> 3), sl = vslot(pos & 7);
-  _Float16* pb = reinterpret_cast<_Float16*>(S.pb[wave]) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
-  _Float16* zb = reinterpret_cast<_Float16*>(S.zb[wave]) + rg * ZB_RSTRIDE * 8 + sl;     // + group * 8
-  const float fold = (pos & 1) ? 1.f / static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
-  const float unfold = (pos & 1) ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
+  uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + rg * ZB_RSTRIDE * 8 + sl;     // + group * 8
+  const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[0], p[1]));
+  const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[2], p[3]));
+  const uint32_t keep = valid ? 0x7FFF7FFFu : 0u;        // unwritten slots may hold any pattern
+  const int zsh = (pos & 1) ? UnpackD<QM>::SH : 0;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const float svf = valid ? f16_value(r.vs[g] & 0x7FFFu) * fold : 0.f;     // unwritten slots may hold any pattern
-#pragma unroll
-    for (int h = 0; h < 4; ++h) pb[(g * 4 + h) * 8] = static_cast<_Float16>(p[h] * svf);
-    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<_Float16>(static_cast<float>(r.vs[g] & ZM) * unfold);
+    const uint32_t sv2 = (r.vs[g] * 0x10001u) & keep;
+    const uint32_t x01 = pk_mul(p01, sv2), x23 = pk_mul(p23, sv2);
+    pb[(g * 4 + 0) * 8] = static_cast<uint16_t>(x01);
+    pb[(g * 4 + 1) * 8] = static_cast<uint16_t>(x01 >> 16);
+    pb[(g * 4 + 2) * 8] = static_cast<uint16_t>(x23);
+    pb[(g * 4 + 3) * 8] = static_cast<uint16_t>(x23 >> 16);
+    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<uint16_t>((r.vs[g] & ZM) << zsh);
   }
 }
 
-template <int QM>
-DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
+template <int QM, class SM>
+DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
   const int c8 = lane & 1, g0 = lane >> 5;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + (k * 2 + c8) * PB_RSTRIDE;   // + group * 4 + head
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + (k * 2 + c8) * PB_RSTRIDE;   // + group * 4 + head
 #pragma unroll
     for (int half = 0; half < 2; ++half) {      // entry words 0, 1 belong to group g0, words 2, 3 to group 2 + g0
       const int g = 2 * half + g0;
@@ -289,8 +308,8 @@ DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane
   }
   if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (page, page half, group, head pair)
     const int rg = lane >> 3, g = (lane >> 1) & 3, hp = lane & 1;
-    const uint4 zq = (reinterpret_cast<const uint4*>(S.zb[wave]) + rg * ZB_RSTRIDE)[g];
-    const uint4* pp = reinterpret_cast<const uint4*>(S.pb[wave]) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
+    const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const uint4 pq = pp[e];
@@ -302,6 +321,7 @@ DEVI void value_phase(const Smem& S, WaveState& st, const VRegs<QM>& r, int lane
 }
 
 // BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
+template <int NW>
 DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&m)[4], float (&l)[4], float (&o)[4][2]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = p.tail_len[b];
@@ -320,7 +340,7 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&
     }
     m[h] = -INFINITY; l[h] = 0.f; o[h][0] = o[h][1] = 0.f;
   }
-  for (int t = wave; t < n; t += NWAVE) {
+  for (int t = wave; t < n; t += NW) {
     const uint16_t* tr = base + static_cast<long long>(t) * p.tail_ts;
     const uint32_t kr = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
     const uint32_t vr = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
@@ -340,20 +360,28 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&
   }
 }
 
-template <int QM, bool K2, int P>
-__global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile, int nparts) {
+template <int QM, bool K2, int P, int NW>
+__global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW == 16 ? 4 : 3) : (K2 ? 4 : 1)) k_decode(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
-  __shared__ Smem S;
+  __shared__ Smem<NW> S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile;
-  const int split = blockIdx.y, b = blockIdx.z;
+  // Workgroups are dispatched in linear order and the CU's arbiter favours the older wavefronts: the splits of one
+  // sequence are spread over the whole dispatch order (split slowest) so that every sequence gets the same mix.
+  const int lin = blockIdx.z * gridDim.y + blockIdx.y;
+  const int split = lin / p.B, b = lin % p.B;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
   const int len = p.seq_lens[b];
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
+  const bool act = wave < 4;      // the 256 threads that own the workgroup's 4 x 128 outputs
 
+  // the (sequence, KV head, q tile)'s counter slot: merge ticket, and in the dynamic mode the quad draw counter
+  const int tpc = p.counter_div;                                 // q tiles that share one counter slot
+  int* const ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
+  const bool dyn = p.dyn != 0;    // the body workgroups of a (sequence, KV head, q tile) draw quads from one counter
   if (!is_tail) {
-    const int lo = max(split * p.chunk, min(p.kv_start, len));
-    const int hi = min(len, (split + 1) * p.chunk);
+    const int lo = dyn ? min(p.kv_start, len) : max(split * p.chunk, min(p.kv_start, len));
+    const int hi = dyn ? len : min(len, (split + 1) * p.chunk);
     WaveState st;
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
@@ -363,21 +391,53 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     }
     st.z[0] = st.z[1] = 0.f;
     if (lo < hi) {   // uniform over the workgroup
-      q_prologue<QM, K2>(S, p, b, kvh, tile);
-      __syncthreads();
       const int pg0 = lo / P, pg1 = (hi + P - 1) / P;
       const int* bt = p.block_table + static_cast<long long>(b) * p.bt_stride;
+      // quads beyond a wave's first one are drawn: from S.next (the workgroup owns a range) or from the slot's draw
+      // counter (all body wavefronts of the slot share the range); a draw is made a whole iteration before its use
+      auto draw = [&]() {
+        int t = 0;
+        if (lane == 0)
+          t = dyn ? (__hip_atomic_fetch_add(ctr, DRAW_BATCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & DRAW_MASK) : atomicAdd(&S.next, 1);
+        return t;
+      };
+      int take = 0;
+      if (dyn) take = draw();        // the first round trip to the device-scope counter hides behind the prologue
+      for (int i = threadIdx.x; i < min(pg1 - pg0, BT_CACHE); i += 64 * NW) S.btc[i] = bt[pg0 + i];
+      if (threadIdx.x == 0) S.next = NW;
+      if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
+      __syncthreads();
+      const int nquad = (pg1 - pg0 + 3) >> 2;
       const int pi = lane >> 4, pos = lane & 15;
+      // odd tokens: the B fields of a V^T word come out of the unpacking with the factor 2^SH, so their scores are
+      // lowered by SH (log2 domain) and their share of the softmax sum is raised again at the end
+      const float sc0 = (pos & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
       typedef const __attribute__((address_space(1))) uint8_t* gptr;
       const gptr pool = (gptr)p.pool;
-      auto chunk_of = [&](int pg) {   // pages past the range read the last page of the range; their tokens are masked
-        return (const uint8_t*)(pool + (static_cast<long long>(bt[min(pg, pg1 - 1)]) * p.Hkv + kvh) * L::CHUNK);
+      auto chunk_of = [&](int quad) {   // pages past the range read the last page of the range; their tokens are masked
+        const int i = min(4 * quad + pi, pg1 - pg0 - 1);
+        const int page = i < BT_CACHE ? S.btc[i] : bt[pg0 + i];
+        return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
       };
+      __builtin_amdgcn_s_setprio(1);
       KRegs<QM> cur;
-      int q4 = pg0 + 4 * wave;       // first page of this wave's current quad
-      const uint8_t* mine = chunk_of(q4 + pi);
-      if (q4 < pg1) load_k<QM, P>(cur, mine, pos);
-      for (; q4 < pg1; q4 += 4 * NWAVE) {
+      // this wave's current quad of 4 pages: the first one by position
+      const int nworker = dyn ? p.nsplit * NW : 0;
+      int qi = dyn ? split * NW + wave : wave;
+      const uint8_t* mine = chunk_of(qi);
+      if (qi < nquad) load_k<QM, P>(cur, mine, pos);
+      if (!dyn) take = draw();
+      int more = 0, nextq = 0;       // quads left of the batch drawn last (the shared counter hands out DRAW_BATCH at a time)
+      while (qi < nquad) {
+        // the next quad: read where the keys of this one are awaited anyway (every older memory operation is then
+        // complete), the following draw goes out ahead of this iteration's loads
+        int qn;
+        if (more > 0) { qn = nextq++; --more; }
+        else {
+          qn = __builtin_amdgcn_readfirstlane(take) + nworker;
+          take = draw();
+          if (dyn) { nextq = qn + 1; more = DRAW_BATCH - 1; }
+        }
         VRegs<QM> vr;                // this quad's V^T entries: in flight during the key phase
         {
           const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
@@ -390,56 +450,66 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
           }
           load_v<QM, P>(vr, ch, lane);
         }
-        const int tok = (q4 + pi) * P + pos;
+        const int tok = (pg0 + 4 * qi + pi) * P + pos;
         const bool valid = tok >= lo && tok < hi;
         float sc[4];
-        key_phase<QM, K2>(S, cur, p.qscale, sc);
+        key_phase<QM, K2>(S, cur, p.qscale, sc0, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
-        const int qn = q4 + 4 * NWAVE;   // the key registers are free: the next quad's keys fly during the value phase
-        if (qn < pg1) {
-          mine = chunk_of(qn + pi);
+        if (qn < nquad) {            // the key registers are free: the next quad's keys fly during the value phase
+          mine = chunk_of(qn);
           load_k<QM, P>(cur, mine, pos);
+          // once the counter has run dry, the wavefronts that still hold a quad go first: they all end together
+          if (qn + NW >= nquad) __builtin_amdgcn_s_setprio(3);
+        } else {
+          __builtin_amdgcn_s_setprio(0);
         }
         wave_lds_sync();
         value_phase<QM>(S, st, vr, lane, wave);
         wave_lds_sync();
+        qi = qn;
       }
     }
     // ---- fold the wave: zero-point sums per (head, group) through the wave's strip, entry pairs (c8 = 0 / 1),
-    //      codes -> values: 2^24 acc - sum p' zero point
+    //      codes -> values: 2^24 (acc - sum p' zero point)
     if constexpr (QM != QM_SYM4) {
       float z0 = st.z[0], z1 = st.z[1];
       z0 += swz_xor<8>(z0); z1 += swz_xor<8>(z1);
       z0 += swz_xor<16>(z0); z1 += swz_xor<16>(z1);
       z0 += xor32(z0); z1 += xor32(z1);
-      float* zs = reinterpret_cast<float*>(S.pb[wave]);          // [head][group]; the strips are dead by now
+      float* zs = reinterpret_cast<float*>(S.pb(wave));          // [head][group]; the strips are dead by now
       if (lane < 8) { zs[(2 * (lane & 1)) * 4 + (lane >> 1)] = z0; zs[(2 * (lane & 1) + 1) * 4 + (lane >> 1)] = z1; }
       wave_lds_sync();
     }
+    const float unfold = (lane & 1) ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;   // lane & 1 = token parity
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] = (st.acc[h][s4] + dpp_xor1(st.acc[h][s4])) * 16777216.f;
+      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
       if constexpr (QM != QM_SYM4) {
-        const float* zs = reinterpret_cast<const float*>(S.pb[wave]) + h * 4 + (lane >> 5);
+        const float* zs = reinterpret_cast<const float*>(S.pb(wave)) + h * 4 + (lane >> 5);
         const float z01 = zs[0], z23 = zs[2];
         st.acc[h][0] -= z01; st.acc[h][1] -= z01; st.acc[h][2] -= z23; st.acc[h][3] -= z23;
       }
-      const float lsum = wave_sum64(st.l[h]);
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= 16777216.f;
+      const float lsum = wave_sum64(st.l[h] * unfold);
       if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = lsum; }
     }
-    __syncthreads();
+    __syncthreads();     // every wave is done with its strip: the partial outputs may overwrite them
     {
       const int wq = lane >> 4, gid = (lane >> 1) & 7;
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
-        float M = fmaxf(fmaxf(S.m[0][h], S.m[1][h]), fmaxf(S.m[2][h], S.m[3][h]));
+        float M = S.m[0][h];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][h]);
         const float f = st.m[h] == -INFINITY ? 0.f : fexp2(st.m[h] - M);
         if ((lane & 1) == 0) {
+          float* o = S.o(wave, h);
 #pragma unroll
           for (int sub = 0; sub < 4; ++sub) {
             const int d = 64 * (sub >> 1) + 16 * wq + gid + 8 * (sub & 1);
-            S.o[wave][h][d] = f * st.acc[h][sub];
+            o[d] = f * st.acc[h][sub];
           }
         }
       }
@@ -447,45 +517,52 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     __syncthreads();
   } else {
     float m[4], l[4], o[4][2];
-    tail_partial(p, b, kvh, tile, m, l, o);
+    tail_partial<NW>(p, b, kvh, tile, m, l, o);
 #pragma unroll
     for (int h = 0; h < 4; ++h)
       if (lane == 0) { S.m[wave][h] = m[h]; S.l[wave][h] = l[h]; }
     __syncthreads();
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      const float M = fmaxf(fmaxf(S.m[0][h], S.m[1][h]), fmaxf(S.m[2][h], S.m[3][h]));
+      float M = S.m[0][h];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][h]);
       const float f = m[h] == -INFINITY ? 0.f : fexp2(m[h] - M);
-      S.o[wave][h][2 * lane] = f * o[h][0];
-      S.o[wave][h][2 * lane + 1] = f * o[h][1];
+      float* so = S.o(wave, h);
+      so[2 * lane] = f * o[h][0];
+      so[2 * lane + 1] = f * o[h][1];
     }
     __syncthreads();
   }
-  // ---- workgroup partial: (o[4][128] relative to M, M, L)
-  float po[2], pm, pl;
-  const int oh = threadIdx.x >> 6;   // head of this thread's two outputs
-  {
-    const float M = fmaxf(fmaxf(S.m[0][oh], S.m[1][oh]), fmaxf(S.m[2][oh], S.m[3][oh]));
+  // ---- workgroup partial: (o[4][128] relative to M, M, L); thread = (head, 2 dims) for the first 4 wavefronts
+  float po[2] = {0.f, 0.f}, pm = -INFINITY, pl = 0.f;
+  const int oh = wave & 3;           // head of this thread's two outputs
+  if (act) {
+    float M = S.m[0][oh];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][oh]);
     float Lsum = 0.f;
 #pragma unroll
-    for (int w = 0; w < NWAVE; ++w) Lsum += S.m[w][oh] == -INFINITY ? 0.f : fexp2(S.m[w][oh] - M) * S.l[w][oh];
+    for (int w = 0; w < NW; ++w) Lsum += S.m[w][oh] == -INFINITY ? 0.f : fexp2(S.m[w][oh] - M) * S.l[w][oh];
     pm = M; pl = Lsum;
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int d = 2 * lane + e;
-      po[e] = (S.o[0][oh][d] + S.o[1][oh][d]) + (S.o[2][oh][d] + S.o[3][oh][d]);
+    for (int w = 0; w < NW; ++w) {
+      const float2 v = *reinterpret_cast<const float2*>(S.o(w, oh) + 2 * lane);
+      po[0] += v.x; po[1] += v.y;
     }
-    if (is_tail && p.vmask != nullptr) {  // the merged sum is rotated back once: bring the tail into the stored basis
-      __syncthreads();
-      S.o[0][oh][2 * lane] = po[0]; S.o[0][oh][2 * lane + 1] = po[1];
-      __syncthreads();
+  }
+  if (is_tail && p.vmask != nullptr) {  // the merged sum is rotated back once: bring the tail into the stored basis
+    __syncthreads();
+    if (act) { S.o(0, oh)[2 * lane] = po[0]; S.o(0, oh)[2 * lane + 1] = po[1]; }
+    __syncthreads();
+    if (act) {
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         const int d = 2 * lane + e, g = d >> 5;
         if (p.vmask[kvh * 4 + g]) {
           float a = 0.f;
           for (int k = 0; k < 32; ++k) {
-            const float v = S.o[0][oh][32 * g + k];
+            const float v = S.o(0, oh)[32 * g + k];
             a += (__builtin_popcount(d & k & 31) & 1) ? -v : v;
           }
           po[e] = a * kC32;
@@ -498,32 +575,34 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     // which are write-through / read-through; a device-scope fence here would write back and invalidate the whole
     // L2 once per workgroup.  Order: stores acknowledged (workgroup release = wait for the store counter), barrier,
     // ticket; the last arriver reads after its ticket returned.
-    float* op = p.opart + part_id * 512 + oh * 128 + 2 * lane;
-    __hip_atomic_store(op, po[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(op + 1, po[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (lane == 0) {
-      __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh, pm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh + 1, pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (act) {
+      float* op = p.opart + part_id * 512 + oh * 128 + 2 * lane;
+      __hip_atomic_store(op, po[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(op + 1, po[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) {
+        __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh, pm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh + 1, pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    const int tpc = p.counter_div;                               // q tiles that share one counter slot
-    int* ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
-    if (threadIdx.x == 0) {
-      const int prev = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      S.last = prev == tpc * nparts - 1;
+    if (threadIdx.x == 0) {    // every draw of this workgroup precedes its ticket: the last arriver may clear the slot
+      const int prev = __hip_atomic_fetch_add(ctr, dyn ? DRAW_MASK + 1 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      S.last = (dyn ? static_cast<int>(static_cast<unsigned>(prev) >> DRAW_BITS) : prev) == tpc * nparts - 1;
       if (S.last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!S.last) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  } else if (dyn && threadIdx.x == 0) {
+    __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // the only workgroup of the slot
   }
   // ---- final merge (last arriving workgroup, or the only one): all tiles of this counter slot
-  const int tpc = nparts > 1 ? p.counter_div : 1;
+  const int ntt = nparts > 1 ? tpc : 1;
   const int tile0 = nparts > 1 ? (tile / tpc) * tpc : tile;
-  for (int tt = tile0; tt < tile0 + tpc; ++tt) {
+  for (int tt = tile0; tt < tile0 + ntt; ++tt) {
     float M = pm, Lsum = pl, o0 = po[0], o1 = po[1];
-    if (nparts > 1) {
+    if (nparts > 1 && act) {
       const long long base = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tt) * nparts;
       M = -INFINITY;
       for (int s = 0; s < nparts; ++s) M = fmaxf(M, __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
@@ -541,31 +620,42 @@ __global__ void __launch_bounds__(256) k_decode(const DecodeParams p, int ntile,
     o0 *= inv; o1 *= inv;
     if (p.vmask != nullptr) {
       __syncthreads();
-      S.o[0][oh][2 * lane] = o0; S.o[0][oh][2 * lane + 1] = o1;
+      if (act) { S.o(0, oh)[2 * lane] = o0; S.o(0, oh)[2 * lane + 1] = o1; }
       __syncthreads();
       float r[2] = {o0, o1};
+      if (act) {
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int d = 2 * lane + e, g = d >> 5;
-        if (p.vmask[kvh * 4 + g]) {
-          float a = 0.f;
-          for (int k = 0; k < 32; ++k) {
-            const float v = S.o[0][oh][32 * g + k];
-            a += (__builtin_popcount(d & k & 31) & 1) ? -v : v;
+        for (int e = 0; e < 2; ++e) {
+          const int d = 2 * lane + e, g = d >> 5;
+          if (p.vmask[kvh * 4 + g]) {
+            float a = 0.f;
+            for (int k = 0; k < 32; ++k) {
+              const float v = S.o(0, oh)[32 * g + k];
+              a += (__builtin_popcount(d & k & 31) & 1) ? -v : v;
+            }
+            r[e] = a * kC32;
           }
-          r[e] = a * kC32;
         }
       }
       o0 = r[0]; o1 = r[1];
     }
     const int hq = tt * 4 + oh;
-    if (hq < p.gqa) {
+    if (act && hq < p.gqa) {
       uint16_t* orow = static_cast<uint16_t*>(p.out) + static_cast<long long>(b) * p.o_bs +
                        (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 2 * lane;
       *reinterpret_cast<uint32_t*>(orow) = bf16_rn(o0) | (bf16_rn(o1) << 16);
     }
   }
 }
+
+// Wavefronts per workgroup: 16 (one workgroup fills a CU: 4 wavefronts per SIMD at 128 registers) when every wavefront
+// has at least two quads of pages to draw, else 4.
+#ifndef FR_BIGW
+#define FR_BIGW 12
+#endif
+constexpr int BIGW = FR_BIGW;   // wavefronts of the large workgroup: 12 leave 168 registers per lane, 16 leave 128
+constexpr int BIG_CHUNK = 2048;   // tokens per split from which the large workgroup pays: >= 2 quads per wavefront
+inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? BIGW : 4; }
 
 template <int QM, bool K2>
 int launch_qm(const DecodeParams& p, hipStream_t st) {
@@ -574,7 +664,8 @@ int launch_qm(const DecodeParams& p, hipStream_t st) {
   const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
-  hipLaunchKernelGGL((k_decode<QM, K2, 16>), grid, dim3(256), 0, st, p, ntile, nparts);
+  if (p.wg_waves == BIGW) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW>), grid, dim3(64 * BIGW), 0, st, p, ntile, nparts);
+  else hipLaunchKernelGGL((k_decode<QM, K2, 16, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -591,11 +682,12 @@ int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
 }
 
 template <int QM, bool K2>
-int occupancy_qm() {
+int occupancy_qm(int waves) {
   int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(&k_decode<QM, K2, 16>), 256, 0) != hipSuccess || n < 1) {
+  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * waves, 0) != hipSuccess || n < 1) {
     (void)hipGetLastError();
-    return 2;
+    return waves > 4 ? 1 : 2;
   }
   return n;
 }
@@ -603,23 +695,27 @@ int occupancy_qm() {
 }  // namespace
 
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) { return decode_dispatch(fmt, p, st); }
+int decode_waves(int chunk_tokens) { return waves_for(chunk_tokens); }
+int decode_big_chunk() { return BIG_CHUNK; }
 
-// resident workgroups per CU the host split planner may count on (queried once per format)
-int decode_occupancy(int fmt) {
-  static int cache[16] = {0};
+// resident workgroups per CU the host split planner may count on (queried once per format and workgroup size)
+int decode_occupancy(int fmt, int waves) {
+  static int cache[16][2] = {{0}};
   if (fmt < 0 || fmt >= 16) return 0;
-  if (cache[fmt] == 0) {
+  const int wi = waves > 4 ? 1 : 0;
+  waves = wi ? BIGW : 4;
+  if (cache[fmt][wi] == 0) {
     switch (fmt) {
-      case FMT_INT4: cache[fmt] = occupancy_qm<QM_SYM4, false>(); break;
-      case FMT_INT4A: cache[fmt] = occupancy_qm<QM_ASYM4, false>(); break;
-      case FMT_INT2A: cache[fmt] = occupancy_qm<QM_ASYM2, false>(); break;
-      case FMT_KONLY: cache[fmt] = occupancy_qm<QM_SYM4, true>(); break;
-      case FMT_KONLYA: cache[fmt] = occupancy_qm<QM_ASYM4, true>(); break;
-      case FMT_KONLYA2: cache[fmt] = occupancy_qm<QM_ASYM2, true>(); break;
+      case FMT_INT4: cache[fmt][wi] = occupancy_qm<QM_SYM4, false>(waves); break;
+      case FMT_INT4A: cache[fmt][wi] = occupancy_qm<QM_ASYM4, false>(waves); break;
+      case FMT_INT2A: cache[fmt][wi] = occupancy_qm<QM_ASYM2, false>(waves); break;
+      case FMT_KONLY: cache[fmt][wi] = occupancy_qm<QM_SYM4, true>(waves); break;
+      case FMT_KONLYA: cache[fmt][wi] = occupancy_qm<QM_ASYM4, true>(waves); break;
+      case FMT_KONLYA2: cache[fmt][wi] = occupancy_qm<QM_ASYM2, true>(waves); break;
       default: return 0;
     }
   }
-  return cache[fmt];
+  return cache[fmt][wi];
 }
 
 }  // namespace fr

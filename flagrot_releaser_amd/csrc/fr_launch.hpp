@@ -57,9 +57,14 @@ struct DecodeParams {
   long long tail_bs, tail_ts;
   int gqa;
   int kv_start;
+  int dyn;                 // 1: the nsplit body workgroups of a (sequence, KV head, q tile) share its whole page range and
+                           //    draw quads of 4 pages from the slot's counter; 0: split s owns tokens [s, s + 1) * chunk
+  int wg_waves;            // wavefronts per workgroup: 4, or the large workgroup that fills a CU
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
-int decode_occupancy(int fmt);
+int decode_occupancy(int fmt, int waves);   // resident workgroups per CU of the 4- or 16-wavefront kernel
+int decode_big_chunk();                     // tokens per split from which the large workgroup is worth launching
+int decode_waves(int chunk_tokens);          // wavefronts per workgroup the launcher picks for a split of that many tokens
 
 void set_error(const char* msg);
 

@@ -176,40 +176,46 @@ def _slots(key, occ_fn) -> int:
     return _OCC[key] * _NUM_CU
 
 
-def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, fixed: int = 512, merge: int = 48):
-    """(nsplit, chunk): chunk a multiple of 64 tokens, <= 8192, nsplit = ceil(Lmax / chunk).  Cost model in
-    token-equivalents: waves of `slots` concurrent workgroups, each costing its chunk + a fixed launch/prologue/merge
-    share, + a per-split merge term."""
+BIG_CHUNK = 2048          # tokens per split from which the library launches one large workgroup per CU
+
+
+def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, ncu: int = None):
+    """(nsplit, chunk) for B sequences x HV (KV head, q tile) pairs: chunk a multiple of 64 tokens, <= 8192,
+    nsplit = ceil(Lmax / chunk).  Mirrors the two launch shapes of the library: when the pairs alone nearly fill the
+    CUs with chunks of >= 2048 tokens, one large workgroup per CU (nsplit = CUs // pairs); otherwise workgroups of 4
+    wavefronts that share a pair's page range, `slots` (= CUs x resident workgroups) of them in one round."""
     gran = max(64, page)
     Lmax = max(1, int(Lmax))
-    if nsplit is not None:
-        chunk = min(MAX_CHUNK, math.ceil(Lmax / nsplit / gran) * gran)
+    ncu = ncu or max(1, slots // 4)
+
+    def plan(ns):
+        ns = max(1, min(MAX_SPLITS, ns, math.ceil(Lmax / gran)))
+        ns = max(ns, math.ceil(Lmax / MAX_CHUNK))
+        chunk = min(MAX_CHUNK, math.ceil(Lmax / ns / gran) * gran)
         return math.ceil(Lmax / chunk), chunk
-    best = None
-    for ns in range(max(1, math.ceil(Lmax / MAX_CHUNK)), min(MAX_SPLITS, math.ceil(Lmax / gran)) + 1):
-        chunk = math.ceil(Lmax / ns / gran) * gran
-        if chunk > MAX_CHUNK:
-            continue
-        nse = math.ceil(Lmax / chunk)
-        if best is not None and nse == best[1]:
-            continue
-        cost = math.ceil(B * HV * nse / slots) * (chunk + fixed) + (merge * nse if nse > 1 else 0)
-        if best is None or cost < best[0] - 1e-9:
-            best = (cost, nse, chunk)
-    return best[1], best[2]
+
+    if nsplit is not None:
+        return plan(nsplit)
+    pairs = B * HV
+    if pairs <= ncu:
+        ns, chunk = plan(ncu // pairs)
+        if chunk >= BIG_CHUNK and pairs * ns >= 0.85 * ncu and pairs * ns <= ncu:
+            return ns, chunk
+    quads = math.ceil(Lmax / 64)
+    return plan(min(max(1, slots // pairs), max(1, quads // 8)))     # >= 2 quads per wavefront
 
 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
     HV = Hkv * -(-G // 4)                                  # workgroups per (row, split): q tiles of 4 heads
     s = _slots(("v2", fmt, page), lambda: lib().fr_v2_occupancy(V2_FMT[fmt], v2_variant(fmt, G, Dh), STAGES, page))
-    return plan_splits(B, Lmax, HV, page, s, nsplit)
+    return plan_splits(B, Lmax, HV, page, s, nsplit, ncu=_NUM_CU)
 
 
 def plan_cb(B, Lmax, Hkv, page, kind, nsplit=None, G=4, Dh=128):
     if kind in K2 and (G != 4 or Dh != 128):
         return plan_v2(B, Lmax, Hkv, page, nsplit, fmt=kind, G=G, Dh=Dh)
     s = _slots(("cb", kind, page), lambda: lib().fr_cb_occupancy(CB_KINDS[kind], 0, STAGES, page))
-    return plan_splits(B, Lmax, Hkv, page, s, nsplit)
+    return plan_splits(B, Lmax, Hkv, page, s, nsplit, ncu=_NUM_CU)
 
 
 class Workspace:

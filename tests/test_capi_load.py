@@ -70,5 +70,10 @@ def test_host_planner_invariants():
             ns, ch = K.plan_splits(B, L, 8, 16, slots)
             assert ch % 64 == 0 and ch <= K.MAX_CHUNK and ns == -(-L // ch) and ns <= K.MAX_SPLITS
     assert K.plan_splits(4, 1000, 8, 16, 512, nsplit=3) == (3, 384)
+    # pairs that fill the CUs with long chunks: one large workgroup each; else one round of shared-range workgroups
+    assert K.plan_splits(32, 8192, 8, 16, 1024, ncu=256) == (1, 8192)
+    assert K.plan_splits(8, 32768, 8, 16, 1024, ncu=256) == (4, 8192)
+    assert K.plan_splits(64, 16256, 8, 16, 1024, ncu=256) == (2, 8128)
+    assert K.plan_splits(2, 4097, 8, 16, 1024, ncu=256) == (8, 576)
     assert K.v2_variant("int4a", 4) == 264 and K.tile_of(K.v2_variant("konlya", 8)) == 8
     assert K.vheads(8, 8, 128, "konlya") == 8 and K.vheads(4, 12, 128, "int4") == 12
