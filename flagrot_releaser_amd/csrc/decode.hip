@@ -235,18 +235,25 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
     sc[h] = valid ? sc[h] : -INFINITY;
     beat |= sc[h] > st.m[h];
   }
-  if (__any(beat)) {
+  // The state is multiplied every time (by 1 unless the maxima moved): modifying it only inside the rare branch makes
+  // the compiler keep two copies of all its registers and move them on the common path.
+  float alpha[4] = {1.f, 1.f, 1.f, 1.f};
+  if (__builtin_expect(__any(beat), 0)) {   // rare after the first quads
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
       const float mn = fmaxf(st.m[h], wave_max64(sc[h]));
-      const float alpha = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
+      alpha[h] = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
       st.m[h] = mn;
-      st.l[h] *= alpha;
-#pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha;
-      if ((lane & 1) == (h >> 1)) st.z[h & 1] *= alpha;
     }
   }
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    st.l[h] *= alpha[h];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha[h];
+  }
+  st.z[0] *= (lane & 1) ? alpha[2] : alpha[0];
+  st.z[1] *= (lane & 1) ? alpha[3] : alpha[1];
   const int pi = lane >> 4, pos = lane & 15;
   float p[4];
 #pragma unroll
