@@ -26,7 +26,11 @@ int fr_abi_version(void);
  * o_bs); kmask / vmask uint8 [Hkv, 4] or null (honoured if qrot / if vrot or tail); tail bf16
  * [rows, W, 2*Hkv, 128] (strides tail_bs / tail_ts elements) + tail_len int32 [B] (+ tail_idx int32 [B]) or null.
  * nsplit counts the body splits; with a tail the workspace must hold B*Hkv*ceil(gqa/GT)*(nsplit+1) partials of
- * GT*128 floats (GT = 8 when variant has bits 1024|2048, else 4); counter zeroed once by the caller. */
+ * GT*128 floats (GT = 8 when variant has bits 1024|2048, else 4); counter int32 [B*Hkv*ceil(gqa/GT)] zeroed once by the
+ * caller (merge tickets and, when the body workgroups of a sequence share its page range, their page draws; the last
+ * arriving workgroup leaves the word at 0).  If B*Hkv*ceil(gqa/4)*nsplit fits the CUs and chunk >= 2048, split s owns
+ * tokens [s, s+1)*chunk and one large workgroup per CU runs it; otherwise nsplit only counts the workgroups per
+ * (sequence, KV head, q tile); nsplit*chunk must cover the longest sequence either way. */
 int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
                const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale,
                const uint8_t* kmask, const uint8_t* vmask, int rb, int qrot, int vrot, int variant, int stages,
@@ -39,7 +43,8 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
 int fr_v2_write(int fmt, const void* kv, long long kv_ts, const long long* slots, int T, int Hkv, int page,
                 const uint8_t* mask, int rb, uint8_t* pool, void* stream, int hd, const float* kmu);
 
-/* flagrot_capi.cu:79-80.  Resident workgroups per CU (for the host split planner); bytes per (page, head) chunk. */
+/* flagrot_capi.cu:79-80.  Resident 4-wavefront workgroups per CU (for the host split planner); bytes per (page, head)
+ * chunk. */
 int fr_v2_occupancy(int fmt, int variant, int stages, int page);
 int fr_v2_chunk_bytes(int fmt, int page);
 
