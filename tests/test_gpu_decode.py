@@ -133,6 +133,17 @@ def test_window_and_kv_start(dev, mode, fmt):
     run_case(dev, mode, [90, 40], fmt, seed=8, Hkv=2, kv_start=37)
 
 
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
+                                      ("static", "int4a"), ("static", "int2a")])
+def test_large_workgroup_shape(dev, mode, fmt):
+    """chunks of >= 2048 tokens on few (sequence, head) pairs: one 12-wavefront workgroup per split, quads drawn from
+    a counter in LDS (the other tests run the 4-wavefront shapes); with splits, tail rows, kv_start and a q tile pair."""
+    ns, ch = run_case(dev, mode, [2300, 2100], fmt, seed=20, Hkv=2, nsplit=1)
+    assert (ns, ch) == (1, 2304)
+    run_case(dev, mode, [4500, 2049, 70], fmt, seed=21, Hkv=2, nsplit=2, win=(40, 5), kv_start=4)
+    run_case(dev, mode, [2200], fmt, seed=22, Hkv=1, G=8, nsplit=1)
+
+
 @pytest.mark.parametrize("shared", ["copy", "stride0"])
 def test_shared_block_table_row(dev, shared):
     run_case(dev, "codebook", [100, 37, 64], "konlya", bt_shared=shared, seed=9, Hkv=2)
