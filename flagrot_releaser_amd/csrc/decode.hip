@@ -475,6 +475,9 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
         wave_lds_sync();
         qi = qn;
       }
+      // the last draw is never used: it must have reached the counter before this workgroup takes its ticket (the
+      // last arriver clears the word)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     // ---- fold the wave: zero-point sums per (head, group) through the wave's strip, entry pairs (c8 = 0 / 1),
     //      codes -> values: 2^24 (acc - sum p' zero point)
