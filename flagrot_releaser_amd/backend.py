@@ -1,0 +1,223 @@
+"""Host side of a decode step, as the serving plugin drives the libraries: split plans per batch bucket, the shared
+split-K workspace, the BF16 sink / window ring bookkeeping, and the write -> attend call sequence of one attention layer.
+
+It mirrors, without vLLM, the decode-row part of the reference's attention backend
+(integrations/vllm_flagrot/vllm_flagrot/attention/backend.py): `plan_bucket` (:638-644), `tile_layout` (:657-662),
+`decode_plan` (:665-676), `decode_workspace` (:699-711), `FlagRotMetadataBuilder.build` (:564-618), `_write`
+(:1234-1248), the decode rows of `_kv_cache_update` (:1266-1299) and `_decode` (:1513-1547).  Everything the builder
+touches per step is a persistent device buffer written in place, so that a captured graph of `DecodeLayer.step` can be
+replayed with new lengths, slots and ring positions.  Kinds: the key-only 2x2 codebooks (konly, konlya, konlya2) and the
+static formats (int4, int4a, int2a); the transform-before-write variants of the reference are out of scope here.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import kernels as K
+
+PAGE = 16
+D = 128
+LOG2E = 1.4426950408889634
+STATIC_KINDS = ("int4", "int4a", "int2a")
+
+
+def is_static(kind: str) -> bool:
+    return kind in STATIC_KINDS
+
+
+def plan_bucket(B: int) -> int:
+    """decode batch size a split plan is made for: 1, 2, 4, then multiples of 8 up to 256, of 16 beyond (the graph
+    capture sizes), so that a padded graph batch and the same batch run eagerly sum in the same order."""
+    if B <= 4:
+        return 1 << (B - 1).bit_length()
+    return -(-B // 8) * 8 if B <= 256 else -(-B // 16) * 16
+
+
+def tile_layout(kind: str, Hkv: int, G: int, Dh: int = D):
+    """(workgroups per (row, split), q heads per partial slot, head dim) of the decode kernel of `kind`."""
+    if is_static(kind) or (kind in K.K2 and (G != 4 or Dh != D)):
+        return K.vheads(Hkv, G, Dh, kind), K.tile_of(K.v2_variant(kind, G, Dh)), Dh
+    return Hkv, 4, D
+
+
+def decode_plan(kind: str, B: int, max_len: int, Hkv: int, G: int = 4, Dh: int = D):
+    """(nsplit, chunk) of a decode batch of B rows: fixed per (batch bucket, longest context), no device sync."""
+    Bp = plan_bucket(B)
+    if is_static(kind):
+        return K.plan_v2(Bp, max_len, Hkv, PAGE, fmt=kind, G=G, Dh=Dh)
+    return K.plan_cb(Bp, max_len, Hkv, PAGE, kind, G=G, Dh=Dh)
+
+
+_WS: dict = {}
+
+
+def decode_workspace(device, layout, rows: int, plan_fn):
+    """one split-K workspace per device and tile layout, sized once for every decode batch size <= rows (graphs bake
+    the pointers in; layers run one after the other and share it)."""
+    HV, GT, Dh = layout
+    key = (str(device), HV, GT, Dh)
+    ws = _WS.get(key)
+    if ws is None or ws.rows < rows:
+        parts = max(plan_bucket(B) * HV * (plan_fn(B)[0] + 1) for B in range(1, rows + 1))
+        ws = _WS[key] = K.Workspace(rows, HV, parts, device, GT, Dh)
+    return ws
+
+
+def ring_slot(p, S: int, W: int):
+    """BF16 slot of position p inside a request's row of S sink slots followed by a W-slot window ring, or -1 when the
+    position keeps no BF16 copy (W = 0 and p >= S).  p: int or integer tensor."""
+    if isinstance(p, torch.Tensor):
+        if W > 0:
+            return torch.where(p < S, p, S + torch.remainder(p - S, W))
+        return torch.where(p < S, p, torch.full_like(p, -1))
+    if p < S:
+        return p
+    return S + (p - S) % W if W > 0 else -1
+
+
+@dataclass
+class DecodeMetadata:
+    seq_lens: torch.Tensor                   # [n] int32 context lengths including the step's token
+    block_table: torch.Tensor                # [n, max_blocks] int32
+    slot_mapping: torch.Tensor               # [n] int64 page slots of the step's tokens (< 0: padding row)
+    num_decodes: int
+    nsplit: int = 1
+    chunk: int = 64
+    dec_cached: torch.Tensor | None = None   # int32 page tokens read: [0, L - W) with [0, S) masked; 0 if L - W <= S
+    dec_tail_len: torch.Tensor | None = None  # int32 BF16 slots read: min(L, S + W)
+    dec_tail_idx: torch.Tensor | None = None  # int32 ring row (request slot; R = the padding row)
+    dec_ring_pos: torch.Tensor | None = None  # int64 flat BF16 slot of the new token (row * (S + W) + slot)
+
+
+class MetadataBuilder:
+    """per-step bookkeeping of the decode rows (every row has one query token)."""
+
+    def __init__(self, kind: str, Hkv: int, G: int, max_len: int, max_rows: int, ring_rows: int, sink: int, window: int,
+                 device, Dh: int = D, plan_fn=None):
+        self.kind, self.Hkv, self.G, self.Dh = kind, Hkv, G, Dh
+        self._plan_fn = plan_fn          # B -> (nsplit, chunk); default: the library's planner (needs the GPU)
+        self.max_len, self.max_rows, self.R, self.S, self.W = max_len, max_rows, ring_rows, sink, window
+        i32 = dict(dtype=torch.int32, device=device)
+        self._cached = torch.zeros(max_rows, **i32)
+        self._tail_len = torch.zeros(max_rows, **i32)
+        self._tail_idx = torch.full((max_rows,), ring_rows, **i32)
+        self._ring_pos = torch.zeros(max_rows, dtype=torch.int64, device=device)
+        self._plans: dict = {}
+
+    def plan(self, B: int):
+        if B not in self._plans:
+            self._plans[B] = (self._plan_fn(B) if self._plan_fn is not None else
+                              decode_plan(self.kind, B, self.max_len, self.Hkv, self.G, self.Dh))
+        return self._plans[B]
+
+    def build(self, seq_lens, block_table, slot_mapping, req_idx=None) -> DecodeMetadata:
+        """seq_lens [n] int32 (device); req_idx: host array of request slots of the first rows (rows beyond it, and
+        dummy runs without it, are padding: they read and write the extra ring row R)."""
+        nd = int(seq_lens.shape[0])
+        md = DecodeMetadata(seq_lens=seq_lens, block_table=block_table, slot_mapping=slot_mapping, num_decodes=nd)
+        if nd == 0:
+            return md
+        md.nsplit, md.chunk = self.plan(nd)
+        L = seq_lens
+        S, W = self.S, self.W
+        if S == 0 and W == 0:
+            md.dec_cached = L
+            return md
+        T = S + W
+        self._tail_idx[:nd].fill_(self.R)
+        if req_idx is not None:
+            k = min(len(req_idx), nd)
+            self._tail_idx[:k].copy_(torch.from_numpy(np.ascontiguousarray(np.asarray(req_idx)[:k], dtype=np.int32)),
+                                     non_blocking=True)
+        # the pages hold every position; the kernel reads [S, L - W) of them and the BF16 slots [0, min(L, T)) =
+        # the sinks [0, min(L, S)) and the window [max(S, L - W), L)
+        torch.where(L - W > S, L - W, torch.zeros_like(L), out=self._cached[:nd])
+        torch.clamp(L, max=T, out=self._tail_len[:nd])
+        p = L.long() - 1                                                     # the new token
+        row = self._tail_idx[:nd].long() * T
+        slot = ring_slot(p, S, W)
+        torch.where(slot >= 0, row + slot, torch.full_like(p, self.R * T), out=self._ring_pos[:nd])
+        md.dec_cached, md.dec_tail_len = self._cached[:nd], self._tail_len[:nd]
+        md.dec_tail_idx, md.dec_ring_pos = self._tail_idx[:nd], self._ring_pos[:nd]
+        return md
+
+
+class DecodeLayer:
+    """cache state and call sequence of one attention layer: pages + BF16 ring, writer then decode."""
+
+    def __init__(self, kind: str, Hkv: int, G: int, pool: torch.Tensor, builder: MetadataBuilder, scale: float = None,
+                 CT=None, co=None, wmask=None, kmu=None):
+        self.kind, self.Hkv, self.G = kind, Hkv, G
+        self.static = is_static(kind)
+        self.pool = pool                                   # uint8 [num_pages, Hkv, chunk bytes]
+        self.b = builder
+        self.S, self.W, self.T, self.R = builder.S, builder.W, builder.S + builder.W, builder.R
+        self.qscale = (scale if scale is not None else 1.0 / math.sqrt(D)) * LOG2E
+        self.CT, self.co, self.wmask, self.kmu = CT, co, wmask, kmu
+        if self.static:
+            if wmask is None:
+                raise ValueError("static formats need the [2 Hkv, 4] rotation mask")
+        elif CT is None or co is None:
+            raise ValueError("codebook kinds need the calibration (CT, co)")
+        dev = pool.device
+        self.layout = tile_layout(kind, Hkv, G)
+        self.kmask = wmask[:Hkv].contiguous() if self.static else None
+        self.vmask = wmask[Hkv:].contiguous() if self.static else None
+        self.ring = torch.zeros(self.R + 1, max(self.T, 1), 2 * Hkv, D, dtype=torch.bfloat16, device=dev) if self.T else None
+        self.ws = decode_workspace(dev, self.layout, builder.max_rows, builder.plan)
+
+    # -- the BF16 slots hold bf16(k - mu) (fp32 subtraction), V rows unchanged
+    def center_rows(self, kv):
+        if self.kmu is None:
+            return kv
+        H = self.Hkv
+        return torch.cat([(kv[:, :H].float() - self.kmu).to(torch.bfloat16), kv[:, H:]], 1)
+
+    def write_pages(self, kv, slots):
+        """kv bf16 [n, 2 Hkv, 128] -> pages at slots (< 0 skipped); the kernels subtract kmu from the K rows"""
+        if self.static:
+            K.v2_write(kv, slots, self.wmask, 32, self.pool, PAGE, fmt=self.kind, kmu=self.kmu)
+        else:
+            K.cb_write(kv, slots, self.CT, self.co, self.kind, self.pool, PAGE, kmu=self.kmu)
+
+    def prefill(self, kv, slots, req: int):
+        """a prompt of n tokens of request slot `req`: every token to its page, sinks and the newest W tokens also to
+        the request's BF16 row"""
+        self.write_pages(kv, slots)
+        if self.T:
+            n = kv.shape[0]
+            pos = torch.arange(n, device=kv.device)
+            keep = (pos < self.S) | (pos >= n - self.W) if self.W > 0 else pos < self.S
+            sl = ring_slot(pos[keep], self.S, self.W)
+            self.ring[req].index_copy_(0, sl, self.center_rows(kv[keep]))
+
+    def update(self, kv, md: DecodeMetadata):
+        """cache update of a decode step: the new tokens to their pages and to their BF16 slots"""
+        self.write_pages(kv, md.slot_mapping)
+        if self.T:
+            self.ring.view(-1, 2 * self.Hkv, D).index_copy_(0, md.dec_ring_pos, self.center_rows(kv))
+
+    def decode(self, q, md: DecodeMetadata, out):
+        nd = q.shape[0]
+        tkw = {}
+        if self.T:
+            r = self.ring
+            tkw = dict(tail=r, tail_len=md.dec_tail_len, tail_idx=md.dec_tail_idx, tail_bs=r.stride(0),
+                       tail_ts=r.stride(1), kv_start=self.S)        # the sinks are in the pages too, read in BF16
+        if q.stride(1) != D or q.stride(2) != 1:
+            q = q.contiguous()
+        if self.static:
+            K.v2_attn(q, self.pool, md.block_table[:nd], md.dec_cached, out, md.nsplit, md.chunk, self.ws, self.qscale,
+                      kmask=self.kmask, vmask=self.vmask, rb=32, fmt=self.kind, **tkw)
+        else:
+            K.cb_attn(q, self.pool, md.block_table[:nd], md.dec_cached, out, md.nsplit, md.chunk, self.ws, self.qscale,
+                      self.kind, **tkw)
+
+    def step(self, q, kv, md: DecodeMetadata, out):
+        """what a captured decode step of this layer contains"""
+        self.update(kv, md)
+        self.decode(q, md, out)

@@ -1,0 +1,55 @@
+"""Host bookkeeping of the decode step (flagrot_releaser_amd.backend) on the CPU: batch buckets, the BF16 ring slot
+formula against a token-by-token simulation, and the metadata builder against a per-row restatement."""
+import numpy as np
+import pytest
+import torch
+
+from flagrot_releaser_amd import backend as BK
+
+
+def test_plan_bucket():
+    assert [BK.plan_bucket(b) for b in (1, 2, 3, 4, 5, 8, 9, 255, 256, 257, 300)] == [1, 2, 4, 4, 8, 8, 16, 256, 256, 272, 304]
+    for b in range(1, 600):
+        assert BK.plan_bucket(b) >= b and BK.plan_bucket(BK.plan_bucket(b)) == BK.plan_bucket(b)
+
+
+@pytest.mark.parametrize("S,W", [(4, 128), (4, 8), (0, 16), (3, 0), (1, 1)])
+def test_ring_slot_keeps_sinks_and_window(S, W):
+    """writing every position p to ring_slot(p) leaves, after L tokens, exactly the sinks [0, min(L, S)) and the window
+    [max(S, L - W), L) in the slots [0, min(L, S + W)) -- what the decode kernel reads as its BF16 rows"""
+    T = S + W
+    row = [-1] * max(T, 1)
+    for L in range(1, 3 * T + 40):
+        p = L - 1
+        s = BK.ring_slot(p, S, W)
+        assert s == int(BK.ring_slot(torch.tensor([p]), S, W)[0])
+        if s >= 0:
+            row[s] = p
+        held = sorted(x for x in row[:min(L, T)] if x >= 0)
+        want = sorted(set(range(min(L, S))) | set(range(max(S, L - W), L)))
+        assert held == want, (L, held, want)
+        assert all(x >= 0 for x in row[:min(L, T)])
+
+
+@pytest.mark.parametrize("S,W", [(0, 0), (4, 128), (4, 0), (0, 16)])
+def test_metadata_builder_rows(S, W):
+    R, rows = 5, 8
+    b = BK.MetadataBuilder("konlya", 8, 4, 4096, rows, R, S, W, "cpu", plan_fn=lambda B: (3, 1408))
+    lens = torch.tensor([1, 3, 4, 5, 131, 132, 133, 1000], dtype=torch.int32)
+    req = np.array([2, 0, 4, 1, 3, 2])                     # two rows more than request slots: padding rows
+    md = b.build(lens, torch.zeros(8, 4, dtype=torch.int32), torch.zeros(8, dtype=torch.int64), req_idx=req)
+    assert (md.nsplit, md.chunk, md.num_decodes) == (3, 1408, 8)
+    if S == 0 and W == 0:
+        assert md.dec_cached is lens and md.dec_tail_len is None
+        return
+    T = S + W
+    for i, L in enumerate(lens.tolist()):
+        row = int(req[i]) if i < len(req) else R
+        assert int(md.dec_tail_idx[i]) == row
+        assert int(md.dec_cached[i]) == (L - W if L - W > S else 0)
+        assert int(md.dec_tail_len[i]) == min(L, T)
+        s = BK.ring_slot(L - 1, S, W)
+        assert int(md.dec_ring_pos[i]) == (row * T + s if s >= 0 else R * T)
+    # the buffers are persistent: a second, shorter build reuses them
+    md2 = b.build(lens[:3] + 1, md.block_table[:3], md.slot_mapping[:3], req_idx=req[:3])
+    assert md2.dec_tail_idx.data_ptr() == md.dec_tail_idx.data_ptr() and md2.dec_ring_pos.shape[0] == 3

@@ -1,0 +1,106 @@
+"""The host-side decode harness on the GPU: prompts prefilled into pages and BF16 rows, then decode steps (cache update
++ attention of one layer) captured once in a HIP graph and replayed with the builder's persistent buffers updated in
+place; every step is checked against fp64 attention over the oracle's parse of the pages and the ring."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attend as A
+from oracle import pages as PG
+from tests.gpu_util import P, bits, make_kv, spd_calib
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("kind,S,W,center", [("konlya2", 4, 16, True), ("konlya", 0, 0, False), ("int4a", 0, 8, False),
+                                              ("konly", 2, 0, True)])
+def test_decode_steps_in_graph(dev, kind, S, W, center):
+    from flagrot_releaser_amd import backend as BK
+    from flagrot_releaser_amd import kernels as K
+    Hkv, G, R, rows, steps = 2, 4, 3, 4, 6
+    g = torch.Generator().manual_seed(41)
+    prompts, req = [37, 70], np.array([2, 0])
+    nreal, nrows = len(prompts), 3                                   # one padding row in the captured batch
+    max_len = max(prompts) + steps
+    nblk = (max_len + P - 1) // P
+    num_pages = nreal * nblk + 3
+    pool = torch.randint(0, 256, (num_pages, Hkv, PG.chunk_bytes(kind, P)), dtype=torch.uint8, generator=g).to(dev)
+    ids = torch.randperm(num_pages, generator=g)[:nreal * nblk].int().view(nreal, nblk)
+    bt = torch.zeros(nrows, nblk, dtype=torch.int32)
+    bt[:nreal] = ids
+    static = BK.is_static(kind)
+    kw = {}
+    if static:
+        kw["wmask"] = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8).to(dev)
+    else:
+        Cq, co = spd_calib(Hkv, g)
+        kw.update(CT=Cq.transpose(1, 2).contiguous().to(dev), co=co.to(dev))
+    if center:
+        kw["kmu"] = (1.5 * torch.randn(Hkv, 128, generator=g)).to(dev)
+    builder = BK.MetadataBuilder(kind, Hkv, G, max_len, rows, R, S, W, dev)
+    layer = BK.DecodeLayer(kind, Hkv, G, pool, builder, **kw)
+
+    def slot_of(b, p):
+        return int(bt[b, p // P]) * P + p % P
+
+    for b, n in enumerate(prompts):
+        kv = make_kv(n, Hkv, g, edge=False).to(dev)
+        layer.prefill(kv, torch.tensor([slot_of(b, p) for p in range(n)], dtype=torch.int64, device=dev), int(req[b]))
+    # persistent step inputs
+    seq = torch.zeros(nrows, dtype=torch.int32, device=dev)
+    slots = torch.full((nrows,), -1, dtype=torch.int64, device=dev)
+    dbt = bt.to(dev)
+    q = torch.zeros(nrows, G * Hkv, 128, dtype=torch.bfloat16, device=dev)
+    kvn = torch.zeros(nrows, 2 * Hkv, 128, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros(nrows, G * Hkv * 128, dtype=torch.bfloat16, device=dev)
+    lens = list(prompts)
+    graph = None
+    T = S + W
+    for step in range(steps):
+        lens = [n + 1 for n in lens]
+        seq.copy_(torch.tensor(lens + [0], dtype=torch.int32))
+        slots.copy_(torch.tensor([slot_of(b, lens[b] - 1) for b in range(nreal)] + [-1], dtype=torch.int64))
+        q.copy_((torch.randn(q.shape, generator=g) * 0.8).bfloat16())
+        kvn.copy_(make_kv(nrows, Hkv, g, edge=False))
+        md = builder.build(seq, dbt, slots, req_idx=req)
+        if graph is None:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            ring0 = None if layer.ring is None else layer.ring.clone()
+            pool0 = pool.clone()
+            with torch.cuda.stream(side):
+                layer.step(q, kvn, md, out)                          # warm-up; the same step is replayed below
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            pool.copy_(pool0)
+            if ring0 is not None:
+                layer.ring.copy_(ring0)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                layer.step(q, kvn, md, out)
+            pool.copy_(pool0)
+            if ring0 is not None:
+                layer.ring.copy_(ring0)
+        graph.replay()
+        torch.cuda.synchronize()
+        # the new tokens sit in their BF16 slots (key rows centred)
+        if T:
+            want = layer.center_rows(kvn[:nreal])
+            for b in range(nreal):
+                s = BK.ring_slot(lens[b] - 1, S, W)
+                if s >= 0:
+                    assert torch.equal(layer.ring[int(req[b]), s], want[b]), (step, b)
+        cached = md.dec_cached[:nreal].cpu().tolist() if T else lens
+        ref = A.decode_reference(bits(q[:nreal]), pool.cpu().numpy(), kind, P, bt[:nreal].numpy(), cached, 1 / math.sqrt(128),
+                                 kmask=kw["wmask"][:Hkv].cpu().numpy() if static else None,
+                                 vmask=kw["wmask"][Hkv:].cpu().numpy() if static else None,
+                                 tail=None if not T else bits(layer.ring),
+                                 tail_len=None if not T else md.dec_tail_len[:nreal].cpu().numpy(),
+                                 tail_idx=None if not T else md.dec_tail_idx[:nreal].cpu().numpy(), kv_start=S)
+        got = out[:nreal].view(nreal, G * Hkv, 128).float().cpu().numpy().astype(np.float64)
+        assert not np.isnan(got).any()
+        lim = 2e-3 + 1e-2 * np.abs(ref) + 1e-5 * np.abs(ref).max(axis=(1, 2), keepdims=True)
+        assert (np.abs(got - ref) <= lim).all(), (kind, step, float(np.abs(got - ref).max()))
+    assert int(layer.ws.counter.abs().sum()) == 0
