@@ -3,11 +3,13 @@ split-K workspace, the BF16 sink / window ring bookkeeping, and the write -> att
 
 It mirrors, without vLLM, the decode-row part of the reference's attention backend
 (integrations/vllm_flagrot/vllm_flagrot/attention/backend.py): `plan_bucket` (:638-644), `tile_layout` (:657-662),
-`decode_plan` (:665-676), `decode_workspace` (:699-711), `FlagRotMetadataBuilder.build` (:564-618), `_write`
-(:1234-1248), the decode rows of `_kv_cache_update` (:1266-1299) and `_decode` (:1513-1547).  Everything the builder
+`decode_plan` (:665-676), `decode_workspace` / `kivi_workspace` (:684-711), `FlagRotMetadataBuilder.build` and
+`_kivi_decode_groups` (:564-636), `_write` (:1234-1248), the decode rows of `_kv_cache_update` / `_kivi_update`
+(:1266-1325) and `_decode` (:1513-1547).  Everything the builder
 touches per step is a persistent device buffer written in place, so that a captured graph of `DecodeLayer.step` can be
 replayed with new lengths, slots and ring positions.  Kinds: the key-only 2x2 codebooks (konly, konlya, konlya2) and the
-static formats (int4, int4a, int2a); the transform-before-write variants of the reference are out of scope here.
+static formats (int4, int4a, int2a) through `DecodeLayer`, the KIVI-style pages ("kivi2") through `KiviDecodeLayer`;
+the transform-before-write variants of the reference are out of scope here.
 """
 from __future__ import annotations
 
@@ -18,6 +20,7 @@ import numpy as np
 import torch
 
 from . import kernels as K
+from . import kivi as KIVI
 
 PAGE = 16
 D = 128
@@ -47,6 +50,8 @@ def tile_layout(kind: str, Hkv: int, G: int, Dh: int = D):
 def decode_plan(kind: str, B: int, max_len: int, Hkv: int, G: int = 4, Dh: int = D):
     """(nsplit, chunk) of a decode batch of B rows: fixed per (batch bucket, longest context), no device sync."""
     Bp = plan_bucket(B)
+    if kind == "kivi2":
+        return KIVI.plan(Bp, max_len, Hkv)
     if is_static(kind):
         return K.plan_v2(Bp, max_len, Hkv, PAGE, fmt=kind, G=G, Dh=Dh)
     return K.plan_cb(Bp, max_len, Hkv, PAGE, kind, G=G, Dh=Dh)
@@ -64,6 +69,19 @@ def decode_workspace(device, layout, rows: int, plan_fn):
     if ws is None or ws.rows < rows:
         parts = max(plan_bucket(B) * HV * (plan_fn(B)[0] + 1) for B in range(1, rows + 1))
         ws = _WS[key] = K.Workspace(rows, HV, parts, device, GT, Dh)
+    return ws
+
+
+_KWS: dict = {}
+
+
+def kivi_workspace(device, rows: int, Hkv: int, G: int, Dh: int, plan_fn):
+    """KIVI split-K workspace, sized once for every decode batch size <= rows"""
+    key = (str(device), Hkv, G, Dh)
+    parts = max(plan_bucket(B) * Hkv * (plan_fn(B)[0] + 1) for B in range(1, rows + 1))
+    ws = _KWS.get(key)
+    if ws is None or ws.parts < parts:
+        ws = _KWS[key] = KIVI.Workspace(parts, G, Dh, device)
     return ws
 
 
@@ -91,6 +109,8 @@ class DecodeMetadata:
     dec_tail_len: torch.Tensor | None = None  # int32 BF16 slots read: min(L, S + W)
     dec_tail_idx: torch.Tensor | None = None  # int32 ring row (request slot; R = the padding row)
     dec_ring_pos: torch.Tensor | None = None  # int64 flat BF16 slot of the new token (row * (S + W) + slot)
+    kivi_sidx: torch.Tensor | None = None    # kivi2: [nd, 32] int64 ring rows of the key group the step completes
+    kivi_dslot: torch.Tensor | None = None   # (-1: sinks) and its page slots ([:, 0] < 0: no group completes)
 
 
 class MetadataBuilder:
@@ -107,6 +127,10 @@ class MetadataBuilder:
         self._tail_idx = torch.full((max_rows,), ring_rows, **i32)
         self._ring_pos = torch.zeros(max_rows, dtype=torch.int64, device=device)
         self._plans: dict = {}
+        if kind == "kivi2":
+            self._ksidx = torch.full((max_rows, 32), -1, dtype=torch.int64, device=device)
+            self._kdslot = torch.full((max_rows, 32), -1, dtype=torch.int64, device=device)
+            self._k32 = torch.arange(32, dtype=torch.int64, device=device)
 
     def plan(self, B: int):
         if B not in self._plans:
@@ -143,7 +167,24 @@ class MetadataBuilder:
         torch.where(slot >= 0, row + slot, torch.full_like(p, self.R * T), out=self._ring_pos[:nd])
         md.dec_cached, md.dec_tail_len = self._cached[:nd], self._tail_len[:nd]
         md.dec_tail_idx, md.dec_ring_pos = self._tail_idx[:nd], self._ring_pos[:nd]
+        if self.kind == "kivi2":
+            self._kivi_decode_groups(md, L, block_table[:nd], nd)
         return md
+
+    def _kivi_decode_groups(self, md, L, bt, nd):
+        """kivi2: the key group [32 g, 32 g + 32) a decode step completes (new token p = L - 1 = 32 g + 31) is encoded
+        from the BF16 ring in the same step (device operations on persistent buffers)"""
+        S, W, T = self.S, self.W, self.S + self.W
+        Ll = L.long()
+        act = (Ll % 32 == 0) & (Ll >= 32) & (self._tail_idx[:nd] < self.R)
+        pos = ((Ll - 1) // 32 * 32)[:, None] + self._k32[None]                          # [nd, 32]
+        row = self._tail_idx[:nd].long()[:, None] * T
+        slot = ring_slot(pos, S, W)
+        torch.where((pos < S) | ~act[:, None], torch.full_like(pos, -1), row + slot, out=self._ksidx[:nd])
+        pg = torch.clamp(pos // PAGE, min=0, max=bt.shape[1] - 1)
+        ds = bt.gather(1, pg).long() * PAGE + pos % PAGE
+        torch.where(act[:, None], ds, torch.full_like(ds, -1), out=self._kdslot[:nd])
+        md.kivi_sidx, md.kivi_dslot = self._ksidx[:nd], self._kdslot[:nd]
 
 
 class DecodeLayer:
@@ -219,5 +260,52 @@ class DecodeLayer:
 
     def step(self, q, kv, md: DecodeMetadata, out):
         """what a captured decode step of this layer contains"""
+        self.update(kv, md)
+        self.decode(q, md, out)
+
+
+class KiviDecodeLayer:
+    """KIVI-style pages: values written per token, key groups of 32 tokens encoded when they complete (from the prompt
+    rows at prefill, from the BF16 ring at decode: the window must hold a whole group, W >= 32)."""
+
+    def __init__(self, Hkv: int, G: int, pool: torch.Tensor, builder: MetadataBuilder, qs, lz, co, scale: float = None):
+        assert builder.kind == "kivi2" and builder.W >= 32, "kivi2 needs a BF16 window of at least one key group"
+        self.Hkv, self.G, self.pool, self.b = Hkv, G, pool, builder
+        self.S, self.W, self.T, self.R = builder.S, builder.W, builder.S + builder.W, builder.R
+        self.scale = scale if scale is not None else 1.0 / math.sqrt(D)
+        self.qs, self.lz, self.co = qs, lz, co             # calibration queries, their log normalisers, value weights
+        dev = pool.device
+        self.ring = torch.zeros((self.R + 1) * self.T, 2 * Hkv, D, dtype=torch.bfloat16, device=dev)
+        self.ws = kivi_workspace(dev, builder.max_rows, Hkv, G, D, builder.plan)
+
+    def prefill(self, kv, slots, req: int):
+        """a fresh prompt of n tokens: values of every token, the whole key groups, sinks and newest W rows in BF16"""
+        n = kv.shape[0]
+        dev = kv.device
+        KIVI.v_write(kv, slots, self.co, None, self.pool, self.Hkv, D)
+        pos = torch.arange(n, device=dev)
+        keep = (pos < self.S) | (pos >= n - self.W)
+        self.ring.view(self.R + 1, self.T, 2 * self.Hkv, D)[req].index_copy_(0, ring_slot(pos[keep], self.S, self.W), kv[keep])
+        ng = n // 32
+        if ng:
+            gp = pos[:32 * ng].view(ng, 32)
+            sidx = torch.where(gp < self.S, torch.full_like(gp, -1), gp).contiguous()
+            KIVI.k_encode(kv, sidx, slots[:32 * ng].view(ng, 32).contiguous(), self.qs, self.lz, self.scale, self.pool,
+                          self.Hkv, D)
+
+    def update(self, kv, md: DecodeMetadata):
+        KIVI.v_write(kv, md.slot_mapping, self.co, None, self.pool, self.Hkv, D)
+        self.ring.index_copy_(0, md.dec_ring_pos, kv)
+        KIVI.k_encode(self.ring, md.kivi_sidx, md.kivi_dslot, self.qs, self.lz, self.scale, self.pool, self.Hkv, D)
+
+    def decode(self, q, md: DecodeMetadata, out):
+        nd = q.shape[0]
+        if q.stride(1) != D or q.stride(2) != 1:
+            q = q.contiguous()
+        KIVI.attn(q, self.pool, md.block_table[:nd], md.dec_cached, out, md.nsplit, md.chunk, self.ws,
+                  self.scale * LOG2E, self.S, self.G, ring=self.ring, tail_len=md.dec_tail_len,
+                  tail_idx=md.dec_tail_idx, T=self.T)
+
+    def step(self, q, kv, md: DecodeMetadata, out):
         self.update(kv, md)
         self.decode(q, md, out)

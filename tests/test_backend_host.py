@@ -53,3 +53,23 @@ def test_metadata_builder_rows(S, W):
     # the buffers are persistent: a second, shorter build reuses them
     md2 = b.build(lens[:3] + 1, md.block_table[:3], md.slot_mapping[:3], req_idx=req[:3])
     assert md2.dec_tail_idx.data_ptr() == md.dec_tail_idx.data_ptr() and md2.dec_ring_pos.shape[0] == 3
+
+
+def test_kivi_decode_groups():
+    """the key group a decode step completes: ring rows of its 32 positions (sinks excluded) and their page slots"""
+    S, W, R = 4, 64, 3
+    T = S + W
+    b = BK.MetadataBuilder("kivi2", 2, 4, 4096, 6, R, S, W, "cpu", plan_fn=lambda B: (2, 512))
+    lens = torch.tensor([32, 33, 64, 31, 96, 128], dtype=torch.int32)
+    bt = torch.arange(6 * 16, dtype=torch.int32).view(6, 16) * 3 % 97
+    req = np.array([1, 0, 2, 1])                                           # rows 4, 5: padding (ring row R)
+    md = b.build(lens, bt, torch.zeros(6, dtype=torch.int64), req_idx=req)
+    for i, L in enumerate(lens.tolist()):
+        act = L % 32 == 0 and L >= 32 and i < len(req)
+        if not act:
+            assert int(md.kivi_dslot[i, 0]) < 0 and (md.kivi_sidx[i] == -1).all()
+            continue
+        for j in range(32):
+            p = L - 32 + j
+            assert int(md.kivi_dslot[i, j]) == int(bt[i, p // 16]) * 16 + p % 16
+            assert int(md.kivi_sidx[i, j]) == (-1 if p < S else int(req[i]) * T + BK.ring_slot(p, S, W))

@@ -104,3 +104,80 @@ def test_decode_steps_in_graph(dev, kind, S, W, center):
         lim = 2e-3 + 1e-2 * np.abs(ref) + 1e-5 * np.abs(ref).max(axis=(1, 2), keepdims=True)
         assert (np.abs(got - ref) <= lim).all(), (kind, step, float(np.abs(got - ref).max()))
     assert int(layer.ws.counter.abs().sum()) == 0
+
+
+def test_kivi_decode_steps_in_graph(dev):
+    """KIVI-style pages: prompts prefilled (values per token, whole key groups), then decode steps replayed from one
+    captured graph; steps that complete a 32-token key group encode it from the BF16 ring inside the graph."""
+    from flagrot_releaser_amd import backend as BK
+    from flagrot_releaser_amd import kivi as KV
+    from oracle import kivi as OK
+    from oracle import quant as Q
+    from tests.test_gpu_kivi import _calib, _kv, _ref_attn
+    Hkv, G, R, rows, steps, S, W = 2, 4, 3, 4, 7, 4, 32
+    T = S + W
+    g = torch.Generator().manual_seed(43)
+    prompts, req = [61, 90], np.array([1, 2])                          # groups complete at lengths 64 and 96
+    nreal, nrows = len(prompts), 3
+    max_len = max(prompts) + steps
+    nblk = 2 * (-(-max_len // 32))
+    num_pages = nreal * nblk + 2
+    pool = torch.zeros(num_pages, Hkv, KV.chunk_bytes(128), dtype=torch.uint8, device=dev)
+    bt = torch.zeros(nrows, nblk, dtype=torch.int32)
+    bt[:nreal] = torch.randperm(num_pages, generator=g)[:nreal * nblk].int().view(nreal, nblk)
+    qs, lz, co = _calib(Hkv, 24, g)
+    builder = BK.MetadataBuilder("kivi2", Hkv, G, max_len, rows, R, S, W, dev)
+    layer = BK.KiviDecodeLayer(Hkv, G, pool, builder, qs.to(dev), lz.to(dev), co.to(dev))
+
+    def slot_of(b, p):
+        return int(bt[b, p // P]) * P + p % P
+
+    for b, n in enumerate(prompts):
+        layer.prefill(_kv(n, Hkv, g).to(dev), torch.tensor([slot_of(b, p) for p in range(n)], dtype=torch.int64, device=dev),
+                      int(req[b]))
+    seq = torch.zeros(nrows, dtype=torch.int32, device=dev)
+    slots = torch.full((nrows,), -1, dtype=torch.int64, device=dev)
+    dbt = bt.to(dev)
+    q = torch.zeros(nrows, G * Hkv, 128, dtype=torch.bfloat16, device=dev)
+    kvn = torch.zeros(nrows, 2 * Hkv, 128, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros(nrows, G * Hkv * 128, dtype=torch.bfloat16, device=dev)
+    lens = list(prompts)
+    graph = None
+    encoded = 0
+    for step in range(steps):
+        lens = [n + 1 for n in lens]
+        seq.copy_(torch.tensor(lens + [0], dtype=torch.int32))
+        slots.copy_(torch.tensor([slot_of(b, lens[b] - 1) for b in range(nreal)] + [-1], dtype=torch.int64))
+        q.copy_((torch.randn(q.shape, generator=g) * 1.2).bfloat16())
+        kvn.copy_(_kv(nrows, Hkv, g))
+        md = builder.build(seq, dbt, slots, req_idx=req)
+        encoded += int((md.kivi_dslot[:, 0] >= 0).sum())
+        if graph is None:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            ring0, pool0 = layer.ring.clone(), pool.clone()
+            with torch.cuda.stream(side):
+                layer.step(q, kvn, md, out)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            pool.copy_(pool0); layer.ring.copy_(ring0)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                layer.step(q, kvn, md, out)
+            pool.copy_(pool0); layer.ring.copy_(ring0)
+        graph.replay()
+        torch.cuda.synchronize()
+        pnp = pool.cpu().numpy()
+        ringf = Q.bf16_to_f32(bits(layer.ring)).astype(np.float64).reshape(R + 1, T, 2 * Hkv, 128)
+        qf = Q.bf16_to_f32(bits(q)).astype(np.float64)
+        got = Q.bf16_to_f32(bits(out)).astype(np.float64).reshape(nrows, G * Hkv, 128)
+        for b in range(nreal):
+            L = lens[b]
+            cached, tl = int(md.dec_cached[b]), int(md.dec_tail_len[b])
+            assert cached == (L - W if L - W > S else 0) and tl == min(L, T) and cached <= 32 * (L // 32)
+            Kp, Vp = OK.dequant_groups(pnp[bt[b, :2 * (-(-max(cached, 1) // 32))].numpy()], 128)
+            tb = ringf[int(req[b]), :tl]
+            ref = _ref_attn(qf[b], Kp, Vp, min(S, cached), cached, tb[:, :Hkv], tb[:, Hkv:], G, 1 / math.sqrt(128))
+            tol = 1e-2 * np.abs(ref).max() + 1e-6
+            assert np.abs(got[b] - ref).max() <= tol, (step, b, float(np.abs(got[b] - ref).max()), tol)
+    assert encoded == 2                                               # lengths 64 and 96 were reached
