@@ -265,8 +265,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path is measured on ONE GPU (every (sequence, KV head) is independent; see DESIGN.md "
-              "for how it shards); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this path is measured on ONE GPU (every (sequence, KV head) is independent: tensor-parallel "
+              "ranks own KV heads and exchange nothing here); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
     from flagrot_releaser_amd import kernels as K
