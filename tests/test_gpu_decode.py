@@ -144,6 +144,13 @@ def test_large_workgroup_shape(dev, mode, fmt):
     run_case(dev, mode, [2200], fmt, seed=22, Hkv=1, G=8, nsplit=1)
 
 
+def test_block_table_beyond_the_lds_cache(dev):
+    """more than 1024 pages per sequence: the block-table entries past the workgroup's LDS cache are read from memory
+    (shared-range workgroups and, with one split of 17 k tokens, the large workgroup)"""
+    run_case(dev, "codebook", [17000, 40], "konlya", seed=23, Hkv=1)
+    run_case(dev, "codebook", [16500], "konlya2", seed=24, Hkv=1, nsplit=3)
+
+
 @pytest.mark.parametrize("shared", ["copy", "stride0"])
 def test_shared_block_table_row(dev, shared):
     run_case(dev, "codebook", [100, 37, 64], "konlya", bt_shared=shared, seed=9, Hkv=2)
