@@ -198,7 +198,9 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float sc0, fl
 #pragma unroll
     for (int tg = 0; tg < 4; ++tg) {
       uint32_t x[4];
-      if constexpr (QM == QM_ASYM2) UnpackD<QM>::run((j & 1) ? (r.kc[tg][j >> 1] >> 4) : r.kc[tg][j >> 1], x);
+      if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher, 2^4 folded into its scale
+        if (j & 1) UnpackD<QM>::run_hi(r.kc[tg][j >> 1], x); else UnpackD<QM>::run(r.kc[tg][j >> 1], x);
+      }
       else UnpackD<QM>::run(r.kc[tg][j], x);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
@@ -214,7 +216,7 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float sc0, fl
     }
     // a = 2^-24 sum code q: score += scale (2^24 a - zero point * sum q)
     const float sj = f16_value(kw[j] & 0x7FFFu) * qscale;
-    const float sj24 = sj * 16777216.f;
+    const float sj24 = sj * ((QM == QM_ASYM2 && (j & 1)) ? 1048576.f : 16777216.f);
     if constexpr (ZM != 0) {
       const float4 qs = *reinterpret_cast<const float4*>(&S.qsum[var][j][0]);
       const float sz = -sj * static_cast<float>(kw[j] & ZM);
@@ -299,7 +301,9 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
       for (int s2 = 0; s2 < 2; ++s2) {
         const int sub = 2 * half + s2;
         uint32_t x[4];
-        if constexpr (QM == QM_ASYM2) UnpackD<QM>::run((sub & 1) ? (r.vc[k][sub >> 1] >> 4) : r.vc[k][sub >> 1], x);
+        if constexpr (QM == QM_ASYM2) {   // two sub-vectors per word: the odd one's sums carry 2^4 until the fold
+          if (sub & 1) UnpackD<QM>::run_hi(r.vc[k][sub >> 1], x); else UnpackD<QM>::run(r.vc[k][sub >> 1], x);
+        }
         else UnpackD<QM>::run(r.vc[k][sub], x);
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
@@ -493,6 +497,7 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
     const float unfold = (lane & 1) ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;   // lane & 1 = token parity
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
+      if constexpr (QM == QM_ASYM2) { st.acc[h][1] *= 0.0625f; st.acc[h][3] *= 0.0625f; }   // fields unpacked 4 bits up
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
       if constexpr (QM != QM_SYM4) {

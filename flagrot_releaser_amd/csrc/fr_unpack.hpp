@@ -63,11 +63,18 @@ template <> struct UnpackD<QM_ASYM4> {
     x[0] = w & 0x000F000Fu; x[1] = w & 0x00F000F0u; x[2] = t & 0x000F000Fu; x[3] = t & 0x00F000F0u;
   }
 };
-template <> struct UnpackD<QM_ASYM2> {   // fields at bits 0, 2, 8, 10 (+16) of the (pre-shifted) word
+template <> struct UnpackD<QM_ASYM2> {   // fields at bits 0, 2, 8, 10 (+16) of the word
   static constexpr int SH = 2;
+  static constexpr int HI = 4;             // run_hi: the fields 4 bits higher (the other group / sub-vector of the word)
   static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
     const uint32_t t = w >> 8;
     x[0] = w & 0x00030003u; x[1] = w & 0x000C000Cu; x[2] = t & 0x00030003u; x[3] = t & 0x000C000Cu;
+  }
+  // still inside the 10 mantissa bits: every pair carries the extra factor 2^HI, which the caller folds into the
+  // scale of the sum instead of shifting the word first
+  static DEVI void run_hi(uint32_t w, uint32_t (&x)[4]) {
+    const uint32_t t = w >> 8;
+    x[0] = w & 0x00300030u; x[1] = w & 0x00C000C0u; x[2] = t & 0x00300030u; x[3] = t & 0x00C000C0u;
   }
 };
 template <> struct UnpackD<QM_SYM4> {    // sign-magnitude bytes s0000mmm -> signed denormals (no extra factor)
