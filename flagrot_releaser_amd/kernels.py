@@ -182,8 +182,9 @@ BIG_CHUNK = 2048          # tokens per split from which the library launches one
 def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, ncu: int = None):
     """(nsplit, chunk) for B sequences x HV (KV head, q tile) pairs: chunk a multiple of 64 tokens, <= 8192,
     nsplit = ceil(Lmax / chunk).  Mirrors the two launch shapes of the library: when the pairs alone nearly fill the
-    CUs with chunks of >= 2048 tokens, one large workgroup per CU (nsplit = CUs // pairs); otherwise workgroups of 4
-    wavefronts that share a pair's page range, `slots` (= CUs x resident workgroups) of them in one round."""
+    CUs allow chunks of >= 2048 tokens, large workgroups, one per CU at most (nsplit = min(CUs // pairs, Lmax // 2048));
+    otherwise workgroups of 4 wavefronts that share a pair's page range, at most `slots` (= CUs x resident workgroups)
+    of them and about sqrt(quads of pages) per pair."""
     gran = max(64, page)
     Lmax = max(1, int(Lmax))
     ncu = ncu or max(1, slots // 4)
@@ -197,12 +198,13 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
     if nsplit is not None:
         return plan(nsplit)
     pairs = B * HV
-    if pairs <= ncu:
-        ns, chunk = plan(ncu // pairs)
-        if chunk >= BIG_CHUNK and pairs * ns >= 0.85 * ncu and pairs * ns <= ncu:
+    if pairs <= ncu and Lmax >= BIG_CHUNK:          # as many large workgroups as keep >= 2048 tokens each (measured best
+        ns, chunk = plan(min(ncu // pairs, Lmax // BIG_CHUNK))     # even when they fill only part of the CUs)
+        if chunk >= BIG_CHUNK and 24 <= pairs * ns <= ncu:
             return ns, chunk
+    # small workgroups: one round at most; a short job is a trade of pages per wavefront against partials to merge
     quads = math.ceil(Lmax / 64)
-    return plan(min(max(1, slots // pairs), max(1, quads // 8)))     # >= 2 quads per wavefront
+    return plan(min(max(1, slots // pairs), max(1, quads // 4), max(1, round(math.sqrt(quads)))))
 
 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
