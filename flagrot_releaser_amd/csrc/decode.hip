@@ -21,6 +21,7 @@
 //
 // Semantics follow the reference's decode entry points: integrations/vllm_flagrot/csrc/flagrot_capi.cu:19-64,131-149,
 // kernels/csrc/attn_codebook_attn.cuh:2093-2126 (per-(token, group) variant selection), attn_merge.cuh:23-84.
+#include <cstdlib>
 #include "fr_common.hpp"
 #include "fr_launch.hpp"
 #include "fr_unpack.hpp"
@@ -669,7 +670,7 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
 #define FR_BIGW 12
 #endif
 constexpr int BIGW = FR_BIGW;   // wavefronts of the large workgroup: 12 leave 168 registers per lane, 16 leave 128
-constexpr int BIG_CHUNK = 2048;   // tokens per split from which the large workgroup pays: >= 2 quads per wavefront
+constexpr int BIG_CHUNK = 1024;   // tokens per split from which the large workgroup pays (measured: batch 1-16, 2-32 k tokens)
 inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? BIGW : 4; }
 
 template <int QM, bool K2>
@@ -711,7 +712,10 @@ int occupancy_qm(int waves) {
 
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) { return decode_dispatch(fmt, p, st); }
 int decode_waves(int chunk_tokens) { return waves_for(chunk_tokens); }
-int decode_big_chunk() { return BIG_CHUNK; }
+int decode_big_chunk() {      // FLAGROT_BIG_CHUNK overrides (experiments)
+  static const int v = getenv("FLAGROT_BIG_CHUNK") != nullptr ? atoi(getenv("FLAGROT_BIG_CHUNK")) : BIG_CHUNK;
+  return v;
+}
 
 // resident workgroups per CU the host split planner may count on (queried once per format and workgroup size)
 int decode_occupancy(int fmt, int waves) {

@@ -176,13 +176,13 @@ def _slots(key, occ_fn) -> int:
     return _OCC[key] * _NUM_CU
 
 
-BIG_CHUNK = 2048          # tokens per split from which the library launches one large workgroup per CU
+BIG_CHUNK = int(os.environ.get("FLAGROT_BIG_CHUNK", "1024"))   # tokens per split from which the library launches large workgroups
 
 
 def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, ncu: int = None):
     """(nsplit, chunk) for B sequences x HV (KV head, q tile) pairs: chunk a multiple of 64 tokens, <= 8192,
     nsplit = ceil(Lmax / chunk).  Mirrors the two launch shapes of the library: when the pairs alone nearly fill the
-    CUs allow chunks of >= 2048 tokens, large workgroups, one per CU at most (nsplit = min(CUs // pairs, Lmax // 2048));
+    CUs allow chunks of >= 1024 tokens, large workgroups, one per CU at most (nsplit = min(CUs // pairs, Lmax // 1024));
     otherwise workgroups of 4 wavefronts that share a pair's page range, at most `slots` (= CUs x resident workgroups)
     of them and about sqrt(quads of pages) per pair."""
     gran = max(64, page)
@@ -198,7 +198,7 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
     if nsplit is not None:
         return plan(nsplit)
     pairs = B * HV
-    if pairs <= ncu and Lmax >= BIG_CHUNK:          # as many large workgroups as keep >= 2048 tokens each (measured best
+    if pairs <= ncu and Lmax >= BIG_CHUNK:          # as many large workgroups as keep >= 1024 tokens each (measured best
         ns, chunk = plan(min(ncu // pairs, Lmax // BIG_CHUNK))     # even when they fill only part of the CUs)
         if chunk >= BIG_CHUNK and 24 <= pairs * ns <= ncu:
             return ns, chunk

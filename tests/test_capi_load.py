@@ -74,10 +74,10 @@ def test_host_planner_invariants():
     assert K.plan_splits(32, 8192, 8, 16, 1024, ncu=256) == (1, 8192)
     assert K.plan_splits(8, 32768, 8, 16, 1024, ncu=256) == (4, 8192)
     assert K.plan_splits(64, 16256, 8, 16, 1024, ncu=256) == (2, 8128)
-    assert K.plan_splits(2, 4097, 8, 16, 1024, ncu=256) == (2, 2112)
+    assert K.plan_splits(2, 4097, 8, 16, 1024, ncu=256) == (4, 1088)
     assert K.plan_splits(1, 1024, 8, 16, 1024, ncu=256) == (4, 256)
     assert K.plan_splits(1, 2048, 8, 16, 1024, ncu=256) == (6, 384)
-    assert K.plan_splits(1, 32768, 8, 16, 1024, ncu=256) == (16, 2048)
+    assert K.plan_splits(1, 32768, 8, 16, 1024, ncu=256) == (32, 1024)
     assert K.plan_splits(64, 2048, 8, 16, 1024, ncu=256) == (2, 1024)
     assert K.v2_variant("int4a", 4) == 264 and K.tile_of(K.v2_variant("konlya", 8)) == 8
     assert K.vheads(8, 8, 128, "konlya") == 8 and K.vheads(4, 12, 128, "int4") == 12

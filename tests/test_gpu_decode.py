@@ -136,7 +136,7 @@ def test_window_and_kv_start(dev, mode, fmt):
 @pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
                                       ("static", "int4a"), ("static", "int2a")])
 def test_large_workgroup_shape(dev, mode, fmt):
-    """chunks of >= 2048 tokens on few (sequence, head) pairs: one 12-wavefront workgroup per split, quads drawn from
+    """chunks of >= 1024 tokens on few (sequence, head) pairs: one 12-wavefront workgroup per split, quads drawn from
     a counter in LDS (the other tests run the 4-wavefront shapes); with splits, tail rows, kv_start and a q tile pair."""
     ns, ch = run_case(dev, mode, [2300, 2100], fmt, seed=20, Hkv=2, nsplit=1)
     assert (ns, ch) == (1, 2304)
