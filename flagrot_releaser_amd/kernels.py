@@ -267,8 +267,23 @@ def v2_write(kv, slots, mask, rb, pool, page, fmt="int4", kmu=None):
                              mask.data_ptr(), rb, pool.data_ptr(), _stream(), Dh, _kmu(kmu, kv)), "fr_v2_write")
 
 
+def _launcher(fn, args, what, bound):
+    """launch now, or (bound) return a zero-argument callable that launches with these very arguments: the checks and
+    the pointer marshalling are done once, as under graph capture; the tensors must stay alive and in place"""
+    if not bound:
+        _check(fn(*args), what)
+        return None
+
+    def launch():
+        rc = fn(*args)
+        if rc:
+            _check(rc, what)
+    return launch
+
+
 def v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kmask=None, vmask=None, rb=32,
-            tail=None, tail_len=None, tail_idx=None, tail_bs=None, tail_ts=None, page=16, fmt="int4", kv_start=0):
+            tail=None, tail_len=None, tail_idx=None, tail_bs=None, tail_ts=None, page=16, fmt="int4", kv_start=0,
+            bound=False):
     """q bf16 [B, G*Hkv, Dh] -> out bf16 [B, G*Hkv*Dh].  block_table int32 [B, *] (row stride may be 0), seq_lens int32
     [B]; tail: bf16 window rows (strides tail_bs / tail_ts elements) with tail_len int32 [B] (+ tail_idx int32 [B]).
     qscale = softmax scale * log2(e).  kv_start: tokens [0, kv_start) are masked in the paged body."""
@@ -279,13 +294,13 @@ def v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kmas
     v = v2_variant(fmt, G, Dh)
     GT = tile_of(v)
     assert ws.fits(B, vheads(Hkv, G, Dh, fmt), nsplit + (tail is not None), GT, Dh), "split-K workspace too small"
-    _check(lib().fr_v2_attn(V2_FMT[fmt], q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(),
-                            block_table.stride(0), seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale,
-                            _ptr(kmask), _ptr(vmask), rb, int(kmask is not None), int(vmask is not None), v, STAGES,
-                            ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
-                            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
-                            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), G,
-                            int(kv_start)), "fr_v2_attn")
+    args = (V2_FMT[fmt], q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(),
+            block_table.stride(0), seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale,
+            _ptr(kmask), _ptr(vmask), rb, int(kmask is not None), int(vmask is not None), v, STAGES,
+            ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
+            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
+            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), G, int(kv_start))
+    return _launcher(lib().fr_v2_attn, args, "fr_v2_attn", bound)
 
 
 def cb_write(kv, slots, CT, co, kind, pool, page, tg=None, kmu=None):
@@ -374,21 +389,22 @@ def w3_static_write(kv, slots, mask, hfull, pool, page, fmt="int4", path=0, kmu=
 
 
 def cb_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kind, tail=None, tail_len=None,
-            tail_idx=None, tail_bs=None, tail_ts=None, page=16, kv_start=0):
+            tail_idx=None, tail_bs=None, tail_ts=None, page=16, kv_start=0, bound=False):
     B, Hq, Dh = q.shape
     if kind in K2 and (Hq != 4 * pool.shape[1] or Dh != 128):
         return v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, tail=tail, tail_len=tail_len,
-                       tail_idx=tail_idx, tail_bs=tail_bs, tail_ts=tail_ts, page=page, fmt=kind, kv_start=kv_start)
+                       tail_idx=tail_idx, tail_bs=tail_bs, tail_ts=tail_ts, page=page, fmt=kind, kv_start=kv_start,
+                       bound=bound)
     Hkv = Hq // 4
     assert Hq == 4 * pool.shape[1] and Dh == D, f"codebook {kind}: GQA 4, head dim 128 only"
     assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
     assert ws.fits(B, Hkv, nsplit + (tail is not None)), "split-K workspace too small"
-    _check(lib().fr_cb_attn(q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
-                            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, sign_words(), CB_KINDS[kind], 0,
-                            STAGES, ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
-                            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
-                            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), int(kv_start)),
-           "fr_cb_attn")
+    args = (q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, sign_words(), CB_KINDS[kind], 0,
+            STAGES, ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
+            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
+            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), int(kv_start))
+    return _launcher(lib().fr_cb_attn, args, "fr_cb_attn", bound)
 
 
 def head_fwht(x, flags, scale, out=None):
