@@ -183,28 +183,26 @@ DEVI void load_raw(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, in
   }
 }
 
-template <int QM, bool K2, int NT>
-DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
+// K tile entry idx = (token tk = idx >> 2 of the block, quarter tg = idx & 3) from the token's raw words
+template <int QM, bool K2>
+DEVI void convert_k_entry(uint8_t* kt, int idx, const u32x4 kc, const u32x2 sw, uint32_t vf, int kb, int kend, const Consts& cst) {
   using F = Fmt<QM>;
-#pragma unroll
-  for (int it = 0; it < Raw<NT>::NI; ++it) {
-    const int idx = threadIdx.x + it * NT;
+  {
     const int tk = idx >> 2, tg = idx & 3;
     const int j = kb * BN + tk;
     const int row = 32 * (tk >> 5) + krow_of_token(tk & 31);
-    u32x4* dst = reinterpret_cast<u32x4*>(S.kt + row * KROW);
+    u32x4* dst = reinterpret_cast<u32x4*>(kt + row * KROW);
     if (j >= kend) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) dst[4 * g + tg] = u32x4{0u, 0u, 0u, 0u};
-      continue;
+      return;
     }
     uint32_t w[4];
     if constexpr (QM == QM_ASYM2) {
-      w[0] = R.kc[it].x; w[1] = R.kc[it].x >> 4; w[2] = R.kc[it].y; w[3] = R.kc[it].y >> 4;
+      w[0] = kc.x; w[1] = kc.x >> 4; w[2] = kc.y; w[3] = kc.y >> 4;
     } else {
-      w[0] = R.kc[it].x; w[1] = R.kc[it].y; w[2] = R.kc[it].z; w[3] = R.kc[it].w;
+      w[0] = kc.x; w[1] = kc.y; w[2] = kc.z; w[3] = kc.w;
     }
-    const u32x2 sw = R.ks[it];
     const uint32_t s16[4] = {sw.x & 0xFFFFu, sw.x >> 16, sw.y & 0xFFFFu, sw.y >> 16};
     if constexpr (!K2) {
 #pragma unroll
@@ -217,7 +215,7 @@ DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
       }
     } else {
       // key-only pages: the token's flags select identity / H32 per group / whole-head H128 (the quad of a token agrees)
-      const bool ff = (R.vf[it] >> 15) & 1u;
+      const bool ff = (vf >> 15) & 1u;
       const uint32_t sgn1 = (tg & 1) ? 0xBC00BC00u : 0x3C003C00u, sgn2 = (tg & 2) ? 0xBC00BC00u : 0x3C003C00u;
       uint32_t x[4][4], y[4][4];
       bool rot[4];
@@ -260,6 +258,13 @@ DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
       }
     }
   }
+}
+
+template <int QM, bool K2, int NT>
+DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
+#pragma unroll
+  for (int it = 0; it < Raw<NT>::NI; ++it)
+    convert_k_entry<QM, K2>(S.kt, threadIdx.x + it * NT, R.kc[it], R.ks[it], K2 ? R.vf[it] : 0u, kb, kend, cst);
 }
 
 // per (group, run) scale / zero point pairs in the run order; tokens at or beyond kend get scale 0
@@ -317,43 +322,44 @@ DEVI void convert_v(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& c
 }
 
 // ------------------------------------------------------------------------------------------------ one 64-key block
-// scores, mask, online softmax and values of the wavefront's 32 rows against the tiles in LDS
-DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
-                       bool rvalid, int kmin, int l32, int hh) {
-  // S^T = K q^T: two 32-key tiles (two independent accumulator chains), eight 16-element steps; the K operands of four
-  // steps are requested ahead, and the scheduler is told to keep the reads that far in front of the matrix instructions
-  f32x16 sacc[2];
+// scores, mask, online softmax and values of the wavefront's 32 rows against the tiles in LDS, in three parts
+// S^T = K q^T: two 32-key tiles (two independent accumulator chains), eight 16-element steps; the K operands of four
+// steps are requested ahead, and the scheduler is told to keep the reads that far in front of the matrix instructions
+DEVI void qk_block(const uint8_t* kt, const u32x4 (&qf)[8], f32x16 (&sacc)[2], int l32, int hh) {
 #pragma unroll
-  for (int kt = 0; kt < 2; ++kt)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[kt][i] = 0.f;
-  {
-    const uint8_t* k0 = S.kt + l32 * KROW + 16 * hh;
-    const uint8_t* k1 = k0 + 32 * KROW;
-    u32x4 a0[8], a1[8];
+    for (int i = 0; i < 16; ++i) sacc[t][i] = 0.f;
+  const uint8_t* k0 = kt + l32 * KROW + 16 * hh;
+  const uint8_t* k1 = k0 + 32 * KROW;
+  u32x4 a0[8], a1[8];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      a0[s] = *reinterpret_cast<const u32x4*>(k0 + 64 * (s >> 1) + 32 * (s & 1));
-      a1[s] = *reinterpret_cast<const u32x4*>(k1 + 64 * (s >> 1) + 32 * (s & 1));
-    }
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      if (s + 4 < 8) {
-        a0[s + 4] = *reinterpret_cast<const u32x4*>(k0 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
-        a1[s + 4] = *reinterpret_cast<const u32x4*>(k1 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
-      }
-      sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a0[s]), as_h8(qf[s]), sacc[0], 0, 0, 0);
-      sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a1[s]), as_h8(qf[s]), sacc[1], 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // 8 LDS reads
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     // 2 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // 2 LDS reads
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+  for (int s = 0; s < 4; ++s) {
+    a0[s] = *reinterpret_cast<const u32x4*>(k0 + 64 * (s >> 1) + 32 * (s & 1));
+    a1[s] = *reinterpret_cast<const u32x4*>(k1 + 64 * (s >> 1) + 32 * (s & 1));
   }
-  // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys)
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    if (s + 4 < 8) {
+      a0[s + 4] = *reinterpret_cast<const u32x4*>(k0 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+      a1[s + 4] = *reinterpret_cast<const u32x4*>(k1 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+    }
+    sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a0[s]), as_h8(qf[s]), sacc[0], 0, 0, 0);
+    sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a1[s]), as_h8(qf[s]), sacc[1], 0, 0, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // 8 LDS reads
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     // 2 MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // 2 LDS reads
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+}
+
+// mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys); the probabilities leave as the
+// fp16 B operands of the value product, in the V^T token order
+DEVI void softmax_block(f32x16 (&sacc)[2], u32x4 (&pb)[4], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
+                        bool rvalid, int kmin, int hh) {
   const int jb = kb * BN;
   const bool full = __all(rvalid && jb + BN - 1 <= lim) && jb >= kmin;
   if (!full) {
@@ -390,37 +396,47 @@ DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], floa
       for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
   }
   mrow = mnew;
-  // O^T += V^T P^T: four independent accumulator chains (the 32-dim blocks); V^T operands requested two steps ahead
-  {
-    u32x4 pb[4], va[4][4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {      // ks = 2 kt + s
-      const int kt = ks >> 1, s2 = ks & 1;
-      pb[ks] = u32x4{pack_h2_rn(sacc[kt][8 * s2], sacc[kt][8 * s2 + 1]), pack_h2_rn(sacc[kt][8 * s2 + 2], sacc[kt][8 * s2 + 3]),
-                     pack_h2_rn(sacc[kt][8 * s2 + 4], sacc[kt][8 * s2 + 5]), pack_h2_rn(sacc[kt][8 * s2 + 6], sacc[kt][8 * s2 + 7])};
-    }
-    const uint8_t* v0 = S.vt + l32 * VROW + 16 * hh;
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-      for (int db = 0; db < 4; ++db) va[ks][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * ks);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      if (ks + 2 < 4) {
-#pragma unroll
-        for (int db = 0; db < 4; ++db) va[ks + 2][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * (ks + 2));
-      }
-#pragma unroll
-      for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(va[ks][db]), as_h8(pb[ks]), o[db], 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 1);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
+  for (int ks = 0; ks < 4; ++ks) {      // ks = 2 kt + s
+    const int kt = ks >> 1, s2 = ks & 1;
+    pb[ks] = u32x4{pack_h2_rn(sacc[kt][8 * s2], sacc[kt][8 * s2 + 1]), pack_h2_rn(sacc[kt][8 * s2 + 2], sacc[kt][8 * s2 + 3]),
+                   pack_h2_rn(sacc[kt][8 * s2 + 4], sacc[kt][8 * s2 + 5]), pack_h2_rn(sacc[kt][8 * s2 + 6], sacc[kt][8 * s2 + 7])};
   }
+}
+
+// O^T += V^T P^T: four independent accumulator chains (the 32-dim blocks); V^T operands requested two steps ahead
+DEVI void pv_block(const uint8_t* vt, const u32x4 (&pb)[4], f32x16 (&o)[4], int l32, int hh) {
+  u32x4 va[4][4];
+  const uint8_t* v0 = vt + l32 * VROW + 16 * hh;
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int db = 0; db < 4; ++db) va[ks][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * ks);
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    if (ks + 2 < 4) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db) va[ks + 2][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * (ks + 2));
+    }
+#pragma unroll
+    for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(va[ks][db]), as_h8(pb[ks]), o[db], 0, 0, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 1);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
+}
+
+DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
+                       bool rvalid, int kmin, int l32, int hh) {
+  f32x16 sacc[2];
+  u32x4 pb[4];
+  qk_block(S.kt, qf, sacc, l32, hh);
+  softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, kmin, hh);
+  pv_block(S.vt, pb, o, l32, hh);
 }
 
 // ------------------------------------------------------------------------------------------------ main kernel
@@ -504,6 +520,280 @@ __global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
     if (kb + 1 < kb1) block_step(rawB, kb + 1);
   }
   // partials
+  const float l = lrow + __shfl_xor(lrow, 32, 64);
+  if (rvalid) {
+    const long long base = (static_cast<long long>(item) * p.Hkv + h) * ROWS + r;
+    float* op = p.opart + base * D;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<float4*>(op + 32 * db + 8 * q4 + 4 * hh) =
+            make_float4(o[db][4 * q4], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]);
+    if (hh == 0) *reinterpret_cast<float2*>(p.ml + base * 2) = make_float2(mrow, l);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ 256-row kernel
+// Eight wavefronts, 256 rows, two groups of four wavefronts (one of each group per SIMD) that alternate between a
+// matrix slot and a vector slot, half a block apart, so that the matrix instructions of one group run under the vector
+// instructions of the other:
+//   slot 2k      group A: O += P(k-1) V(k-1), S = K(k) q      group B: softmax(k-1), V(k) -> tile
+//   slot 2k + 1  group A: softmax(k), K(k+1) -> tile          group B: O += P(k-1) V(k-1), S = K(k) q
+// One barrier per slot; a wavefront raises its issue priority for its matrix slot (the arbiter otherwise serves the
+// older wavefronts' vector instructions first and the matrix pipe starves).  Group A converts the K tiles, group B the V^T tiles, each into the buffer the other block
+// parity is not reading; a tile is complete one barrier before its first reader.  The raw words of a tile are fetched
+// by the converting group right after the previous conversion (two slots ahead).
+struct Smem8 {
+  alignas(16) uint8_t kt[2][KT_BYTES];
+  alignas(16) uint8_t vt[2][VT_BYTES];
+  int pages[PG_CACHE];
+};
+static_assert(256 * QROW <= 2 * (KT_BYTES + VT_BYTES), "q staging aliases the tiles");
+
+// The thread index as a value the compiler must take as new at every use site: what a converter derives from it (tile
+// addresses, lane offsets) is recomputed per block with a few integer operations instead of being kept in registers
+// across the whole key loop, where the accumulators leave no room for it.
+DEVI int tid_now() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
+// Raw page words of a thread's tile entry, one register set for both groups (a set per group would let the compiler
+// reuse the other group's registers for LDS operands and guard them with waits on outstanding fetches):
+//   group A  w[0] = K code words of (token, tg) (INT2: .x .y), w[1].xy = the token's four K scale words,
+//            w[1].z = the token's group-0 V scale word (whole-head flag of key-only pages)
+//   group B  w[0] = V^T entry (e, c8) of a page, w[1], w[2] = V scale words of the entry's run (eight tokens) in its
+//            two groups: t0 t2 | t4 t6 | t1 t3 | t5 t7
+struct Raw8 {
+  u32x4 w[3];
+};
+
+// A wavefront of the group fetches one page of the block (page = its index in the group): the page base is
+// wave-uniform, the lane adds a 32-bit offset.  Lane = (token pos = lane >> 2, quarter tg) for the K words.
+template <int QM, bool K2>
+DEVI void load_k8(Raw8& R, const Params& p, const int* pg, int h, int kb, int kend, int t256) {
+  using F = Fmt<QM>;
+  const uint32_t lane = t256 & 63, pos = lane >> 2, tg = lane & 3u;
+  const int pgi = __builtin_amdgcn_readfirstlane(t256 >> 6);
+  const int j0 = kb * BN + PAGE * pgi;
+  if (j0 + static_cast<int>(pos) < kend) {
+    const int page = __builtin_amdgcn_readfirstlane(pg[pgi]);
+    const uint8_t* ch = p.pool + static_cast<long long>(page) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 c = gload<u32x2>(ch + (32u * (pos ^ ((pos >> 1) & 2u)) + 8u * tg));
+      R.w[0] = u32x4{c.x, c.y, 0u, 0u};
+    } else {
+      R.w[0] = gload<u32x4>(ch + 16u * lane);
+    }
+    const u32x2 ks = gload<u32x2>(ch + (F::KS_OFF + 8u * pos));
+    R.w[1].x = ks.x; R.w[1].y = ks.y;
+    if constexpr (K2) R.w[1].z = gload<uint16_t>(ch + (F::VS_OFF + (8u * (pos >> 3) + static_cast<uint32_t>(vs_slot8(pos))) * 2u));
+  }
+}
+template <int QM>
+DEVI void load_v8(Raw8& R, const Params& p, const int* pg, int h, int kb, int kend, int t256) {
+  using F = Fmt<QM>;
+  const uint32_t lane = t256 & 63, g = lane >> 5, c8 = lane & 1u;      // entry e = lane >> 1: its dims lie in groups g, g + 2
+  const int pgi = __builtin_amdgcn_readfirstlane(t256 >> 6);
+  const int j0 = kb * BN + PAGE * pgi;
+  if (j0 < kend) {
+    const int page = __builtin_amdgcn_readfirstlane(pg[pgi]);
+    const uint8_t* ch = p.pool + static_cast<long long>(page) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 c = gload<u32x2>(ch + (F::V_OFF + 8u * lane));
+      R.w[0] = u32x4{c.x, c.y, 0u, 0u};
+    } else {
+      R.w[0] = gload<u32x4>(ch + (F::V_OFF + 16u * lane));
+    }
+    R.w[1] = gload<u32x4>(ch + (F::VS_OFF + (g * PAGE + 8u * c8) * 2u));
+    R.w[2] = gload<u32x4>(ch + (F::VS_OFF + ((g + 2u) * PAGE + 8u * c8) * 2u));
+  }
+}
+
+// V^T tile entry: the scale / zero point pairs of the entry's run come from the thread's own scale words, in the run
+// order (t0,t4) (t1,t5) (t2,t6) (t3,t7); tokens at or beyond kend get scale 0
+template <int QM>
+DEVI void convert_v8(uint8_t* vt, const Raw8& R, int kb, int kend, const Consts& cst, int t256) {
+  using F = Fmt<QM>;
+  const int pgi = t256 >> 6, e = (t256 & 63) >> 1, c8 = t256 & 1, run = 2 * pgi + c8;
+  const bool have = kb * BN + PAGE * pgi < kend;
+  const bool ragged = kb * BN + BN > kend;                         // uniform: only the last block of an item
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (have) {
+    if constexpr (QM == QM_ASYM2) {
+      w[0] = R.w[0].x; w[1] = R.w[0].x >> 4; w[2] = R.w[0].y; w[3] = R.w[0].y >> 4;
+    } else {
+      w[0] = R.w[0].x; w[1] = R.w[0].y; w[2] = R.w[0].z; w[3] = R.w[0].w;
+    }
+  }
+  uint32_t sc[2][4], nz[2][4];
+#pragma unroll
+  for (int gg = 0; gg < 2; ++gg) {
+    const u32x4 v = R.w[1 + gg];
+    const uint32_t pr[4] = {__builtin_amdgcn_perm(v.y, v.x, 0x05040100u), __builtin_amdgcn_perm(v.w, v.z, 0x05040100u),
+                            __builtin_amdgcn_perm(v.y, v.x, 0x07060302u), __builtin_amdgcn_perm(v.w, v.z, 0x07060302u)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[gg][i] = have ? pr[i] & 0x7FFF7FFFu : 0u;
+      nz[gg][i] = (pr[i] & (F::ZM * 0x10001u)) | 0xE400E400u;
+    }
+  }
+  if (ragged) {
+    const int t0 = kb * BN + 8 * run;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t m = (t0 + i < kend ? 0xFFFFu : 0u) | (t0 + i + 4 < kend ? 0xFFFF0000u : 0u);
+      sc[0][i] &= m; sc[1][i] &= m;
+    }
+  }
+#pragma unroll
+  for (int sub = 0; sub < 4; ++sub) {
+    const int d = 64 * (sub >> 1) + 16 * (e >> 3) + 8 * (sub & 1) + (e & 7);   // group d >> 5 = 2 (sub >> 1) + (e >> 4)
+    uint32_t x[4];
+    Unpack<QM>::run(w[sub], nz[sub >> 1], cst, x);
+    *reinterpret_cast<u32x4*>(vt + d * VROW + 16 * run) =
+        u32x4{pk_mul(x[0], sc[sub >> 1][0]), pk_mul(x[1], sc[sub >> 1][1]), pk_mul(x[2], sc[sub >> 1][2]), pk_mul(x[3], sc[sub >> 1][3])};
+  }
+}
+
+template <int QM, bool K2>
+__global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
+  constexpr int NT = 512, ROWS = 256;
+  extern __shared__ __align__(16) uint8_t lds[];
+  Smem8& S = *reinterpret_cast<Smem8*>(lds);
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int grp = __builtin_amdgcn_readfirstlane(wv >> 2);
+  const int item = blockIdx.x, h = blockIdx.y;
+  const int* it = p.items + ITEM_INTS * item;
+  const int* tl = p.tiles + TILE_INTS * it[0];
+  const int req = tl[0], crow0 = tl[1], ntok = tl[3], pos0 = tl[4], nk = tl[5], ext = tl[8];
+  const int G = p.G, Hq = p.Hkv * G, TQ = ROWS / G;
+  const int* bt = p.bt + static_cast<long long>(req) * p.bt_stride;
+  const int kend = min(min(nk, it[2] * BN), max(pos0 + ntok - p.shift, ext + 1));
+  const int kb0 = it[1];
+  const int kb1 = kend > kb0 * BN ? (kend + BN - 1) / BN : kb0;
+  const Consts cst = make_consts();
+
+  const int r = 32 * wv + l32, rt = r / G;
+  const bool rvalid = r < TQ * G && rt < ntok;
+  const int lim = rvalid ? min(kend - 1, max(pos0 + rt - p.shift, ext)) : -1;   // last visible key
+
+  int cb = kb0;
+  auto fill_pages = [&]() {
+    for (int i = tid; i < PG_CACHE; i += NT) {
+      const int pgx = 4 * cb + i;
+      S.pages[i] = pgx * PAGE < kend ? bt[pgx] : 0;
+    }
+  };
+  fill_pages();
+
+  u32x4 qf[8];
+  for (int row = tid >> 5; row < ROWS; row += NT / 32) {
+    const int t = row / G, lq = tid & 31;
+    u32x2 raw = {0u, 0u};
+    if (row < TQ * G && t < ntok) raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
+    *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = raw;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const int dA = 32 * (s >> 1) + 4 * (2 * (s & 1) + hh);
+    const u32x2 a = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * dA);
+    const u32x2 b = *reinterpret_cast<const u32x2*>(lds + r * QROW + 2 * (dA + 16));
+    qf[s] = u32x4{(a.x & 0xFFFFu) | (a.y << 16), (b.x & 0xFFFFu) | (b.y << 16),
+                  (a.x >> 16) | (a.y & 0xFFFF0000u), (b.x >> 16) | (b.y & 0xFFFF0000u)};
+  }
+
+  f32x16 o[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float mrow = -INFINITY, lrow = 0.f;
+  // The pipeline starts and drains through harmless work instead of branches: probabilities 0 against zeroed V^T
+  // tiles add nothing, scores of -inf leave the running maximum and sum alone.
+  f32x16 sacc[2];
+  u32x4 pb[4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[t][i] = -INFINITY;
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) pb[ks] = u32x4{0u, 0u, 0u, 0u};
+  Raw8 raw;                                            // fetched in a vector slot, converted in the next matrix slot
+  auto fetched = [&]() {                               // no fetch may be outstanding in a matrix slot: the LDS operand
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // registers there are guarded by waits on ALL outstanding fetches
+  };
+  const int nb = kb1 - kb0;                            // blocks of the item
+  __syncthreads();                                     // the q staging is no longer read
+  for (int i = tid; i < 2 * VT_BYTES / 16; i += NT) reinterpret_cast<u32x4*>(&S.vt[0][0])[i] = u32x4{0u, 0u, 0u, 0u};
+  if (grp == 0) {                                      // K(0) before the first slot, K(1) on its way
+    load_k8<QM, K2>(raw, p, S.pages, h, kb0, kend, tid_now() & 255);
+    convert_k_entry<QM, K2>(S.kt[0], tid_now() & 255, raw.w[0], u32x2{raw.w[1].x, raw.w[1].y}, K2 ? raw.w[1].z : 0u, kb0, kend, cst);
+    load_k8<QM, K2>(raw, p, S.pages + 4, h, kb0 + 1, kend, tid_now() & 255);
+  }
+  fetched();
+  __syncthreads();
+
+  auto slot_barrier = [&]() {                          // nothing of a slot may move into the next one
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto slide = [&](int kb) {
+    if (kb + 2 >= cb + PG_CACHE / 4) {                 // blocks kb (V) and kb + 2 (K) are fetched in this step: slide the window
+      slot_barrier();
+      cb = kb;
+      fill_pages();
+      slot_barrier();
+    }
+  };
+  // one loop per group (the same number of barriers in both): the register allocation of one path does not bind the other
+  if (grp == 0) {
+    for (int k = 0; k < nb; ++k) {
+      const int kb = kb0 + k;
+      slide(kb);
+      __builtin_amdgcn_s_setprio(3);                   // slot 2k: matrix.  V(k - 1), K(k); K(k + 1) is written
+      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);
+      __builtin_amdgcn_sched_barrier(0);
+      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      convert_k_entry<QM, K2>(S.kt[(k & 1) ^ 1], tid_now() & 255, raw.w[0], u32x2{raw.w[1].x, raw.w[1].y}, K2 ? raw.w[1].z : 0u, kb + 1, kend, cst);
+      slot_barrier();
+      load_k8<QM, K2>(raw, p, S.pages + 4 * (kb + 2 - cb), h, kb + 2, kend, tid_now() & 255);   // slot 2k + 1: vector
+      __builtin_amdgcn_sched_barrier(0);
+      softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, p.kmin, hh);
+      fetched();
+      slot_barrier();
+    }
+    if (nb > 0) pv_block(S.vt[(nb - 1) & 1], pb, o, l32, hh);
+  } else {
+    for (int k = 0; k < nb; ++k) {
+      const int kb = kb0 + k;
+      slide(kb);
+      load_v8<QM>(raw, p, S.pages + 4 * (kb - cb), h, kb, kend, tid_now() & 255);   // slot 2k: vector
+      __builtin_amdgcn_sched_barrier(0);
+      softmax_block(sacc, pb, o, mrow, lrow, kb - 1, lim, rvalid, p.kmin, hh);   // block k - 1
+      fetched();
+      slot_barrier();
+      __builtin_amdgcn_s_setprio(3);                   // slot 2k + 1: matrix.  V(k - 1), K(k); V(k) is written
+      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);
+      __builtin_amdgcn_sched_barrier(0);
+      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      convert_v8<QM>(S.vt[k & 1], raw, kb, kend, cst, tid_now() & 255);
+      slot_barrier();
+    }
+    if (nb > 0) {                                      // group B is one slot behind
+      softmax_block(sacc, pb, o, mrow, lrow, kb1 - 1, lim, rvalid, p.kmin, hh);
+      pv_block(S.vt[(nb - 1) & 1], pb, o, l32, hh);
+    }
+  }
+
   const float l = lrow + __shfl_xor(lrow, 32, 64);
   if (rvalid) {
     const long long base = (static_cast<long long>(item) * p.Hkv + h) * ROWS + r;
@@ -691,6 +981,17 @@ template <int QM, bool K2, int NW> int launch_mq(const Params& p, int nitems, hi
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
 
+template <int QM, bool K2> int launch_mq8(const Params& p, int nitems, hipStream_t st) {
+  static bool attr = false;
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_mq8<QM, K2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(sizeof(Smem8))) != hipSuccess) return -1;
+    attr = true;
+  }
+  hipLaunchKernelGGL((k_mq8<QM, K2>), dim3(nitems, p.Hkv), dim3(512), sizeof(Smem8), st, p);
+  return hipPeekAtLastError() == hipSuccess ? 0 : -1;
+}
+
 int done(int rc, const char* what) {
   if (rc == -1) std::snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(hipGetLastError()));
   return rc;
@@ -709,7 +1010,7 @@ extern "C" {
 
 int frmq_abi_version(void) { return 7; }
 const char* frmq_last_error(void) { return g_err; }
-int frmq_smem_bytes(void) { return static_cast<int>(sizeof(Smem)); }
+int frmq_smem_bytes(void) { return static_cast<int>(sizeof(Smem8) > sizeof(Smem) ? sizeof(Smem8) : sizeof(Smem)); }
 
 int frmq_prep_q(const void* q, int q_fp32, long long q_ts, const int* idx, int m, int Hq, int G, const uint8_t* kfull,
                 const uint8_t* kmask, float qscale, void* q16, int Dh, void* stream) {
@@ -725,17 +1026,20 @@ int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const
               const int* tiles, const int* items, int nitems, int Hkv, int G, int shift, int konly, float* opart,
               float* ml, int kernel, int Dh, void* stream, int kmin) {
   if (nitems <= 0) return 0;
-  const int rows = kernel == 1 ? 64 : 128;
+  const int rows = kernel == 1 ? 64 : kernel == 4 ? 256 : 128;
   if (G < 1 || G > rows) return bad(-3, "frmq_attn: G out of range");
   if (Dh != D) return bad(-4, "frmq_attn: head dim 128 only");
-  if (kernel < 1 || kernel > 3) return bad(-2, "frmq_attn: kernel must be 1, 2 or 3");
+  if (kernel < 1 || kernel > 4) return bad(-2, "frmq_attn: kernel must be 1, 2, 3 or 4");
   Params p{};
   p.q = static_cast<const uint16_t*>(q16); p.pool = pool; p.page_stride = page_stride; p.bt = bt; p.bt_stride = bt_stride;
   p.tiles = tiles; p.items = items; p.Hkv = Hkv; p.G = G; p.shift = shift; p.kmin = kmin; p.opart = opart; p.ml = ml;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool k2 = konly & 1, i2 = konly & 2;
   int rc;
-  if (rows == 64) {
+  if (rows == 256) {
+    rc = i2 ? (k2 ? launch_mq8<QM_ASYM2, true>(p, nitems, st) : launch_mq8<QM_ASYM2, false>(p, nitems, st))
+            : (k2 ? launch_mq8<QM_ASYM4, true>(p, nitems, st) : launch_mq8<QM_ASYM4, false>(p, nitems, st));
+  } else if (rows == 64) {
     rc = i2 ? (k2 ? launch_mq<QM_ASYM2, true, 2>(p, nitems, st) : launch_mq<QM_ASYM2, false, 2>(p, nitems, st))
             : (k2 ? launch_mq<QM_ASYM4, true, 2>(p, nitems, st) : launch_mq<QM_ASYM4, false, 2>(p, nitems, st));
   } else {

@@ -10,7 +10,8 @@
  * Plan buffers (host planner, prefill_mq.py:128-210): tiles int32 [nt][9] = (block-table row, compact row0, output
  * row0, tokens, position of the first token, page keys nk, first item, items, ext); items int32 [ni][4] = (tile,
  * first 64-key block, end block, 0).  Row r of a tile = token r / G, q head h G + r % G; rows per tile = 64 for
- * kernel 1, 128 for kernel 2 / 3.  Key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext)
+ * kernel 1, 128 for kernel 2 / 3 (the reference's selectors), 256 for kernel 4 (this library only: eight wavefronts in
+ * two groups that alternate between the matrix and the vector half of a block).  Key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext)
  * and j < nk.
  */
 #ifndef FLAGROT_MQ_H
@@ -36,7 +37,7 @@ int frmq_prep_q(const void* q, int q_fp32, long long q_ts, const int* idx, int m
 /* mq_prefill.cu:1490-1544.  q16 from frmq_prep_q (pre-scaled by softmax scale * log2 e); pool uint8 pages with byte
  * stride page_stride, KV head h at + h * chunk bytes; konly bit 0: key-only 2x2 pages (per-token H32 / H128 flags),
  * bit 1: INT2 pages (80 B per token) instead of INT4 (144 B); opart fp32 [nitems, Hkv, rows, Dh] unnormalised, ml fp32
- * [nitems, Hkv, rows, 2] = (running maximum in log2 units, sum); kernel 1 | 2 | 3 selects rows per tile only. */
+ * [nitems, Hkv, rows, 2] = (running maximum in log2 units, sum); kernel 1 | 2 | 3 | 4 selects rows per tile (64 | 128 | 128 | 256). */
 int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const int* bt, long long bt_stride,
               const int* tiles, const int* items, int nitems, int Hkv, int G, int shift, int konly, float* opart,
               float* ml, int kernel, int Dh, void* stream, int kmin);

@@ -97,13 +97,30 @@ CASES = [  # (requests [(L, nq)], shift, sink, G, fmt, kernel, ext)
     ([(1500, 200), (300, 300)], 0, 0, 8, "konlya2", 1, None),
     ([(1500, 200)], 0, 0, 1, "int4a", 3, None),
     ([(900, 200), (400, 100)], 128, 4, 8, "konlya", 3, {0: 650}),
+    # kernel 4: 256-row tiles, two wavefront groups half a block apart
+    ([(1000, 1000)], 0, 0, 4, "int4a", 4, None),
+    ([(10145, 145)], 0, 0, 4, "konlya", 4, None),
+    ([(16, 5)], 0, 0, 4, "int2a", 4, None),
+    ([(64, 64)], 0, 0, 4, "konlya2", 4, None),
+    ([(3000, 1)], 0, 0, 4, "int4a", 4, None),
+    ([(2000, 145), (1200, 300), (503, 17), (700, 700), (4000, 64)], 0, 0, 4, "konlya", 4, None),
+    ([(2048, 600)], 128, 0, 4, "int4a", 4, None),
+    ([(1191, 300), (600, 600)], 128, 4, 4, "konlya", 4, None),
+    ([(1500, 200), (300, 300)], 0, 0, 5, "konlya", 4, None),
+    ([(1500, 200), (300, 300)], 0, 0, 8, "konlya2", 4, None),
+    ([(1500, 200)], 0, 0, 1, "int4a", 4, None),
+    ([(900, 200), (400, 100)], 128, 4, 8, "konlya", 4, {0: 650}),
+    # items longer than the page-id window of the kernels (256 blocks): the window slides
+    ([(30000, 40)], 0, 0, 4, "int4a", 4, None, 400),
+    ([(30000, 40)], 0, 0, 4, "konlya", 3, None, 400),
 ]
 
 
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_mq_attention_against_fp64(dev, case):
     from flagrot_releaser_amd import prefill_mq as MQ
-    reqs_in, shift, sink, G, fmt, kernel, ext = CASES[case]
+    reqs_in, shift, sink, G, fmt, kernel, ext = CASES[case][:7]
+    min_blocks = CASES[case][7] if len(CASES[case]) > 7 else None
     k2, int2, _ = FMT[fmt]
     g = torch.Generator().manual_seed(200 + case)
     Hkv = 2
@@ -120,8 +137,11 @@ def test_mq_attention_against_fp64(dev, case):
     n = row + 2
     q = (torch.randn(n, Hq, D, generator=g) * 1.5).bfloat16()
     scale = 1 / math.sqrt(D)
-    plan = MQ.build_plan(reqs, G, Hkv, shift, dev, sink=sink, kernel=kernel, ext=ext)
+    plan = MQ.build_plan(reqs, G, Hkv, shift, dev, sink=sink, kernel=kernel, ext=ext, min_blocks=min_blocks)
     assert plan.m == sum(nq for _, nq in reqs_in)
+    if min_blocks:
+        it = plan.items.cpu().numpy().reshape(-1, 4)
+        assert (it[:, 2] - it[:, 1]).max() > 256
     q16 = MQ.prep_q(q.to(dev), scale * LOG2E, G, plan.idx, None if k2 else kfull.to(dev), None if k2 else kmask.to(dev))
     want16 = OM.prep_q(Q.bf16_to_f32(bits(q)), G, scale * LOG2E, plan.idx.cpu().numpy(),
                        None if k2 else kfull.numpy(), None if k2 else kmask.numpy())

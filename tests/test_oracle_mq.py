@@ -120,7 +120,7 @@ def test_merge_items_equals_single_pass():
 def test_plan_arrays_invariants():
     from flagrot_releaser_amd.prefill_mq import BN, KROWS, plan_arrays
     reqs = [(2, 0, 145, 9000, 9000 - 145), (0, 145, 445, 12000, 11700), (1, 445, 462, 5003, 4986), (3, 462, 1162, 700, 0)]
-    for kernel in (1, 3):
+    for kernel in (1, 3, 4):
         for G in (1, 4, 5, 8):
             for shift, ext in ((0, None), (128, None), (128, {0: 11650})):
                 T, I, idx, rows = plan_arrays(reqs, G, 8, shift, ncu=256, kernel=kernel, ext=ext)
@@ -137,6 +137,15 @@ def test_plan_arrays_invariants():
                     assert its[0, 1] == 0 and (its[1:, 1] == its[:-1, 2]).all()          # contiguous, no overlap
                     assert its[-1, 2] == nb or (nb == 0 and its[-1, 2] == 0)
                 assert len(I) * 8 <= 4 * 2 * 4 * 256 + len(T) * 8                         # about `waves` rounds of the GPU
+
+
+def test_pick_kernel_by_rows_per_request():
+    from flagrot_releaser_amd.prefill_mq import pick_kernel
+    assert pick_kernel([(0, 0, 512, 16896, 16384)], 8) == 4          # 4096 rows
+    assert pick_kernel([(0, 0, 16, 4096, 4080)], 8) == 3             # 128 rows: one 128-row tile
+    assert pick_kernel([(0, 0, 16, 4096, 4080), (1, 16, 48, 900, 868)], 8) == 4
+    assert pick_kernel([(0, 0, 100, 900, 800)], 1) == 3
+    assert pick_kernel([], 4) == 3
 
 
 def test_bf_merge_is_attention_over_the_union():
