@@ -722,19 +722,16 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
     for (int i = 0; i < 16; ++i) sacc[t][i] = -INFINITY;
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) pb[ks] = u32x4{0u, 0u, 0u, 0u};
-  Raw8 raw;                                            // fetched in a vector slot, converted in the next matrix slot
-  auto fetched = [&]() {                               // no fetch may be outstanding in a matrix slot: the LDS operand
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // registers there are guarded by waits on ALL outstanding fetches
-  };
+  Raw8 raw;                                            // fetched at the end of a matrix slot, converted in the next vector slot
   const int nb = kb1 - kb0;                            // blocks of the item
   __syncthreads();                                     // the q staging is no longer read
   for (int i = tid; i < 2 * VT_BYTES / 16; i += NT) reinterpret_cast<u32x4*>(&S.vt[0][0])[i] = u32x4{0u, 0u, 0u, 0u};
-  if (grp == 0) {                                      // K(0) before the first slot, K(1) on its way
+  if (grp == 0) {                                      // K(0) before the first slot
     load_k8<QM, K2>(raw, p, S.pages, h, kb0, kend, tid_now() & 255);
     convert_k_entry<QM, K2>(S.kt[0], tid_now() & 255, raw.w[0], u32x2{raw.w[1].x, raw.w[1].y}, K2 ? raw.w[1].z : 0u, kb0, kend, cst);
-    load_k8<QM, K2>(raw, p, S.pages + 4, h, kb0 + 1, kend, tid_now() & 255);
+  } else {
+    load_v8<QM>(raw, p, S.pages, h, kb0, kend, tid_now() & 255);
   }
-  fetched();
   __syncthreads();
 
   auto slot_barrier = [&]() {                          // nothing of a slot may move into the next one
@@ -742,31 +739,38 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The packed probabilities are pure register values: without this the compiler sinks their conversion past the
+  // barrier to their use, between the matrix instructions of the next slot, where a vector instruction stalls them.
+  auto pin = [&]() {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) asm volatile("" : "+v"(pb[ks]));
+  };
   auto slide = [&](int kb) {
-    if (kb + 2 >= cb + PG_CACHE / 4) {                 // blocks kb (V) and kb + 2 (K) are fetched in this step: slide the window
+    if (kb + 1 >= cb + PG_CACHE / 4) {                 // block kb + 1 is fetched in this step: slide the window
       slot_barrier();
-      cb = kb;
+      cb = kb + 1;
       fill_pages();
       slot_barrier();
     }
   };
-  // one loop per group (the same number of barriers in both): the register allocation of one path does not bind the other
+  // One loop per group (the same number of barriers in both): the register allocation of one path does not bind the
+  // other.  A wavefront issues no vector work between its matrix instructions (on this chip a vector instruction behind
+  // a matrix instruction of the same wavefront waits for it); the fetch of the next raw words, mostly latency, follows
+  // the last matrix instruction, and nothing is outstanding when the next matrix slot starts.
   if (grp == 0) {
     for (int k = 0; k < nb; ++k) {
       const int kb = kb0 + k;
       slide(kb);
-      __builtin_amdgcn_s_setprio(3);                   // slot 2k: matrix.  V(k - 1), K(k); K(k + 1) is written
-      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);
+      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);     // slot 2k: matrix.  V(k - 1), K(k)
       __builtin_amdgcn_sched_barrier(0);
       qk_block(S.kt[k & 1], qf, sacc, l32, hh);
-      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_k8<QM, K2>(raw, p, S.pages + 4 * (kb + 1 - cb), h, kb + 1, kend, tid_now() & 255);
+      slot_barrier();
+      softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, p.kmin, hh);   // slot 2k + 1: vector; K(k + 1) is written
+      pin();
       __builtin_amdgcn_sched_barrier(0);
       convert_k_entry<QM, K2>(S.kt[(k & 1) ^ 1], tid_now() & 255, raw.w[0], u32x2{raw.w[1].x, raw.w[1].y}, K2 ? raw.w[1].z : 0u, kb + 1, kend, cst);
-      slot_barrier();
-      load_k8<QM, K2>(raw, p, S.pages + 4 * (kb + 2 - cb), h, kb + 2, kend, tid_now() & 255);   // slot 2k + 1: vector
-      __builtin_amdgcn_sched_barrier(0);
-      softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, p.kmin, hh);
-      fetched();
       slot_barrier();
     }
     if (nb > 0) pv_block(S.vt[(nb - 1) & 1], pb, o, l32, hh);
@@ -774,22 +778,21 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
     for (int k = 0; k < nb; ++k) {
       const int kb = kb0 + k;
       slide(kb);
-      load_v8<QM>(raw, p, S.pages + 4 * (kb - cb), h, kb, kend, tid_now() & 255);   // slot 2k: vector
-      __builtin_amdgcn_sched_barrier(0);
-      softmax_block(sacc, pb, o, mrow, lrow, kb - 1, lim, rvalid, p.kmin, hh);   // block k - 1
-      fetched();
-      slot_barrier();
-      __builtin_amdgcn_s_setprio(3);                   // slot 2k + 1: matrix.  V(k - 1), K(k); V(k) is written
-      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);
-      __builtin_amdgcn_sched_barrier(0);
-      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
-      __builtin_amdgcn_s_setprio(0);
+      softmax_block(sacc, pb, o, mrow, lrow, kb - 1, lim, rvalid, p.kmin, hh);   // slot 2k: vector (block k - 1); V(k) is written
+      pin();
       __builtin_amdgcn_sched_barrier(0);
       convert_v8<QM>(S.vt[k & 1], raw, kb, kend, cst, tid_now() & 255);
+      slot_barrier();
+      pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);     // slot 2k + 1: matrix.  V(k - 1), K(k)
+      __builtin_amdgcn_sched_barrier(0);
+      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
+      __builtin_amdgcn_sched_barrier(0);
+      load_v8<QM>(raw, p, S.pages + 4 * (kb + 1 - cb), h, kb + 1, kend, tid_now() & 255);
       slot_barrier();
     }
     if (nb > 0) {                                      // group B is one slot behind
       softmax_block(sacc, pb, o, mrow, lrow, kb1 - 1, lim, rvalid, p.kmin, hh);
+      pin();
       pv_block(S.vt[(nb - 1) & 1], pb, o, l32, hh);
     }
   }
