@@ -11,6 +11,9 @@
 // O^T = V^T P^T.  Key-only pages (per-token H32 / H128 flags): the conversion applies the token's inverse transform to
 // the fp16 pairs in registers (packed butterflies, the quad of a token exchanging by DPP) before the tile is stored, so
 // the matrix part is the same for every format.
+// Two kernels: k_mq (64 / 128 rows, two or four wavefronts that convert, then attend, with barriers in between; the
+// reference's selectors 1 - 3) and k_mq8 (256 rows, selector 4: eight wavefronts in two groups half a block apart, the
+// matrix instructions of one group under the vector instructions of the other; described at its definition).
 // Causal rule: key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext), j < nk.
 // Partials (unnormalised O, running maximum in log2 units, sum) per (item, KV head, row); k_merge combines the items
 // of a tile.  Semantics follow integrations/vllm_flagrot/csrc/mq_prefill.cu:345-498 (k_mq), :716-772 (merge),
