@@ -359,6 +359,13 @@ DEVI void qk_block(const uint8_t* kt, const u32x4 (&qf)[8], f32x16 (&sacc)[2], i
   __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
 }
 
+// max over lanes l and l + 32, in both: one v_permlane32_swap, no trip through the LDS queue (which the other group's
+// matrix operand reads keep full)
+DEVI float max_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);   // (lo, lo), (hi, hi)
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys); the probabilities leave as the
 // fp16 B operands of the value product, in the V^T token order
 DEVI void softmax_block(f32x16 (&sacc)[2], u32x4 (&pb)[4], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
@@ -379,7 +386,7 @@ DEVI void softmax_block(f32x16 (&sacc)[2], u32x4 (&pb)[4], f32x16 (&o)[4], float
   for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = max_halves(mx);
   const float mnew = fmaxf(mrow, mx);
   const float base = mnew == -INFINITY ? 0.f : mnew;
   const float alpha = fexp2(mrow - base);
