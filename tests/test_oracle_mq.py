@@ -139,6 +139,29 @@ def test_plan_arrays_invariants():
                 assert len(I) * 8 <= 4 * 2 * 4 * 256 + len(T) * 8                         # about `waves` rounds of the GPU
 
 
+def test_split_items_equal_items_and_whole_rounds():
+    from flagrot_releaser_amd.prefill_mq import BN, plan_arrays, split_items
+    # the workload the bench measures: 64 tiles of 257 .. 264 key blocks, 8 KV heads, 256 resident workgroups
+    reqs = [(r, r * 512, (r + 1) * 512, 16896, 16384) for r in range(4)]
+    T, I, _, rows = plan_arrays(reqs, 8, 8, 0, ncu=256, kernel=4)
+    assert rows == 256 and len(T) == 64 and len(I) == 64                     # one item per tile: 512 workgroups = 2 rounds
+    assert (np.diff(I[:, 2] - I[:, 1]) <= 0).all()                          # longest tiles first
+    # one request: 16 tiles x 8 heads = half a round -> two items per tile, of equal length
+    T, I, _, _ = plan_arrays(reqs[:1], 8, 8, 0, ncu=256, kernel=4)
+    assert len(I) == 32
+    ln = (I[:, 2] - I[:, 1]).reshape(16, 2)
+    assert (np.abs(ln[:, 0] - ln[:, 1]) <= 1).all() and ln.min() >= 128
+    # properties on ragged inputs
+    rng = np.random.default_rng(3)
+    for _ in range(50):
+        nb = rng.integers(0, 400, size=int(rng.integers(1, 40)))
+        for waves in (None, 1.0, 2.5):
+            n = split_items(nb, 8, 256, waves, 4)
+            assert n.shape == nb.shape and (n >= 1).all()
+            assert ((nb // n >= 4) | (n == 1)).all()                         # at least min_blocks blocks per item
+    assert split_items(np.zeros(0, np.int64), 8, 256, None, 4).size == 0
+
+
 def test_pick_kernel_by_rows_per_request():
     from flagrot_releaser_amd.prefill_mq import pick_kernel
     assert pick_kernel([(0, 0, 512, 16896, 16384)], 8) == 4          # 4096 rows
