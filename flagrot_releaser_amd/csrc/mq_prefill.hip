@@ -668,6 +668,92 @@ DEVI void convert_v8(uint8_t* vt, const Raw8& R, int kb, int kend, const Consts&
   }
 }
 
+// The 256-row kernel keeps a per-row REFERENCE instead of the running maximum: the score accumulators start at
+// -reference (qk8), so that exp2 applies to them as they are; the reference moves (and O, l are rescaled) only when a
+// score exceeds it by more than 2^8, which keeps p <= 256 in fp16.  Any reference gives the same O / l; the partial's
+// (m, l) carry it to the merge.
+DEVI void qk8(const uint8_t* kt, const u32x4 (&qf)[8], f32x16 (&sacc)[2], float ref, int l32, int hh) {
+  f32x16 init;
+  const float c0 = ref == -INFINITY ? 0.f : -ref;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) init[i] = c0;
+  const uint8_t* k0 = kt + l32 * KROW + 16 * hh;
+  const uint8_t* k1 = k0 + 32 * KROW;
+  u32x4 a0[8], a1[8];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    a0[s] = *reinterpret_cast<const u32x4*>(k0 + 64 * (s >> 1) + 32 * (s & 1));
+    a1[s] = *reinterpret_cast<const u32x4*>(k1 + 64 * (s >> 1) + 32 * (s & 1));
+  }
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    if (s + 4 < 8) {
+      a0[s + 4] = *reinterpret_cast<const u32x4*>(k0 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+      a1[s + 4] = *reinterpret_cast<const u32x4*>(k1 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
+    }
+    sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a0[s]), as_h8(qf[s]), s ? sacc[0] : init, 0, 0, 0);
+    sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a1[s]), as_h8(qf[s]), s ? sacc[1] : init, 0, 0, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // 8 LDS reads
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     // 2 MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // 2 LDS reads
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+}
+
+// lane = row, lanes l and l + 32 hold the two halves of its 64 keys; sacc = score - reference.  full: no key of the
+// block is masked for any row of the wavefront.
+DEVI void softmax8(f32x16 (&sacc)[2], u32x4 (&pb)[4], f32x16 (&o)[4], float& ref, float& lrow, bool full, int kb, int lim,
+                   int kmin, int hh) {
+  if (!full) {
+    const int jb = kb * BN;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = jb + 32 * kt + token_of_acc(i, hh);
+        if (!(j <= lim && j >= kmin)) sacc[kt][i] = -INFINITY;
+      }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
+  mx = max_halves(mx);
+  const bool bump = (mx > 8.f || ref == -INFINITY) && mx != -INFINITY;
+  if (__any(bump)) {                                     // rare after the first blocks: move the reference to the row maximum
+    const float delta = bump ? mx : 0.f;
+    const float alpha = ref == -INFINITY ? 0.f : fexp2(-delta);   // no reference yet: O and l are still zero
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[kt][i] -= delta;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    lrow *= alpha;
+    if (bump) ref = (ref == -INFINITY ? 0.f : ref) + delta;
+  }
+  typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+  const h2v ones = {static_cast<_Float16>(1.f), static_cast<_Float16>(1.f)};
+  float s4[4] = {0.f, 0.f, 0.f, 0.f};                   // the sum of what the value product uses
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {      // ks = 2 kt + s
+    const int kt = ks >> 1, s2 = ks & 1;
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = pack_h2_rn(fexp2(sacc[kt][8 * s2 + 2 * j]), fexp2(sacc[kt][8 * s2 + 2 * j + 1]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s4[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, w[j]), ones, s4[j], false);
+    pb[ks] = u32x4{w[0], w[1], w[2], w[3]};
+  }
+  lrow += (s4[0] + s4[1]) + (s4[2] + s4[3]);
+}
+
 template <int QM, bool K2>
 __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   constexpr int NT = 512, ROWS = 256;
@@ -721,7 +807,10 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
-  float mrow = -INFINITY, lrow = 0.f;
+  float mrow = -INFINITY, lrow = 0.f;                  // mrow: the row's reference (see qk8)
+  // no key of block kb is masked for any row of the wavefront iff kmin <= 64 kb and 64 kb + 63 <= the smallest limit
+  const int lim_min = -static_cast<int>(wave_max64(-static_cast<float>(rvalid ? lim : -1)));   // exact: key indices < 2^24
+  auto is_full = [&](int kb) { return kb * BN >= p.kmin && kb * BN + BN - 1 <= lim_min; };
   // The pipeline starts and drains through harmless work instead of branches: probabilities 0 against zeroed V^T
   // tiles add nothing, scores of -inf leave the running maximum and sum alone.
   f32x16 sacc[2];
@@ -773,11 +862,11 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
       slide(kb);
       pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);     // slot 2k: matrix.  V(k - 1), K(k)
       __builtin_amdgcn_sched_barrier(0);
-      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
+      qk8(S.kt[k & 1], qf, sacc, mrow, l32, hh);
       __builtin_amdgcn_sched_barrier(0);
       load_k8<QM, K2>(raw, p, S.pages + 4 * (kb + 1 - cb), h, kb + 1, kend, tid_now() & 255);
       slot_barrier();
-      softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, p.kmin, hh);   // slot 2k + 1: vector; K(k + 1) is written
+      softmax8(sacc, pb, o, mrow, lrow, is_full(kb), kb, lim, p.kmin, hh);   // slot 2k + 1: vector; K(k + 1) is written
       pin();
       __builtin_amdgcn_sched_barrier(0);
       convert_k_entry<QM, K2>(S.kt[(k & 1) ^ 1], tid_now() & 255, raw.w[0], u32x2{raw.w[1].x, raw.w[1].y}, K2 ? raw.w[1].z : 0u, kb + 1, kend, cst);
@@ -788,20 +877,20 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
     for (int k = 0; k < nb; ++k) {
       const int kb = kb0 + k;
       slide(kb);
-      softmax_block(sacc, pb, o, mrow, lrow, kb - 1, lim, rvalid, p.kmin, hh);   // slot 2k: vector (block k - 1); V(k) is written
+      softmax8(sacc, pb, o, mrow, lrow, is_full(kb - 1), kb - 1, lim, p.kmin, hh);   // slot 2k: vector (block k - 1); V(k) is written
       pin();
       __builtin_amdgcn_sched_barrier(0);
       convert_v8<QM>(S.vt[k & 1], raw, kb, kend, cst, tid_now() & 255);
       slot_barrier();
       pv_block(S.vt[(k & 1) ^ 1], pb, o, l32, hh);     // slot 2k + 1: matrix.  V(k - 1), K(k)
       __builtin_amdgcn_sched_barrier(0);
-      qk_block(S.kt[k & 1], qf, sacc, l32, hh);
+      qk8(S.kt[k & 1], qf, sacc, mrow, l32, hh);
       __builtin_amdgcn_sched_barrier(0);
       load_v8<QM>(raw, p, S.pages + 4 * (kb + 1 - cb), h, kb + 1, kend, tid_now() & 255);
       slot_barrier();
     }
     if (nb > 0) {                                      // group B is one slot behind
-      softmax_block(sacc, pb, o, mrow, lrow, kb1 - 1, lim, rvalid, p.kmin, hh);
+      softmax8(sacc, pb, o, mrow, lrow, is_full(kb1 - 1), kb1 - 1, lim, p.kmin, hh);
       pin();
       pv_block(S.vt[(nb - 1) & 1], pb, o, l32, hh);
     }
