@@ -116,6 +116,29 @@ CASES = [  # (requests [(L, nq)], shift, sink, G, fmt, kernel, ext)
 ]
 
 
+def _random_cases(n, seed):
+    """seeded shapes for the 256-row kernel: every format, odd group sizes, ragged lengths, shift / sink / ext, the
+    planner's own kernel choice (None) among them"""
+    rng = np.random.default_rng(seed)
+    fmts = ["int4a", "konlya", "int2a", "konlya2"]
+    out = []
+    for i in range(n):
+        G = int(rng.choice([1, 2, 3, 4, 6, 7, 8]))
+        nreq = int(rng.integers(1, 4))
+        reqs = []
+        for _ in range(nreq):
+            nq = int(rng.integers(1, 400))
+            reqs.append((nq + int(rng.integers(0, 1200)), nq))
+        shift = int(rng.choice([0, 0, 64, 128]))
+        sink = int(rng.choice([0, 4])) if shift else 0
+        ext = {0: int(rng.integers(0, reqs[0][0]))} if shift and rng.random() < 0.5 else None
+        out.append((reqs, shift, sink, G, fmts[i % 4], None if i % 5 == 4 else 4, ext))
+    return out
+
+
+CASES += _random_cases(12, 77)
+
+
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_mq_attention_against_fp64(dev, case):
     from flagrot_releaser_amd import prefill_mq as MQ
