@@ -93,7 +93,7 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   // wavefronts, and where the slot's counter word can hold both (one q tile per slot, tickets above the draw bits) the
   // body workgroups of a (sequence, KV head, q tile) share its whole page range and draw quads from the slot's
   // counter: the split plan then only says how many workgroups there are.  FLAGROT_DECODE_STATIC=1 keeps fixed
-  // ranges, FLAGROT_WG_WAVES=4 | 12 forces a workgroup size.
+  // ranges, FLAGROT_WG_WAVES=4 | 16 forces a workgroup size (above 4: the large one).
   const int nparts = nsplit + (tail != nullptr ? 1 : 0);
   static const bool force_static = getenv("FLAGROT_DECODE_STATIC") != nullptr && getenv("FLAGROT_DECODE_STATIC")[0] == '1';
   static const int env_waves = getenv("FLAGROT_WG_WAVES") != nullptr ? atoi(getenv("FLAGROT_WG_WAVES")) : 0;

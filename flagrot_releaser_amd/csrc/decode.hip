@@ -51,6 +51,7 @@ struct Smem {
   alignas(16) uint8_t qv[QV_BYTES];
   // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
   alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
+  alignas(16) uint32_t zero[4 * (4 * PB_RSTRIDE + 1)];   // zeros where the matrix value phase reads the strip rows of foreign groups
   alignas(16) float qsum[3][4][4];                   // [variant][group][head]: sum of the group's (fp16) query elements
   float m[NW][4], l[NW][4];
   int btc[BT_CACHE];
@@ -131,9 +132,13 @@ template <int QM> struct KRegs {
   uint2 ks;                 // the token's 4 K scale words
   uint32_t vs[4];           // the token's 4 V scale words (one per group)
 };
+// The value product P' V runs on the matrix pipe: sixteen v_mfma_f32_16x16x32_f16 per quad of pages, rows = 16 V^T
+// entries, columns = (group, head), 32 tokens deep.  An entry word masked in place (eight tokens as fp16 denormal
+// pairs; the matrix pipe keeps denormal inputs) is the A operand of its lane, one 16-byte strip row (p' of a run's eight
+// tokens for a (group, head)) the B operand.  The scores stay on the vector pipe (v_dot2_f32_f16).
 template <int QM> struct VRegs {
   static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;
-  uint32_t vc[4][NW];       // [page][entry word]
+  uint32_t vc[4][NW];       // [2 (page pair s) + entry half][entry word] of lane (entry m = lane & 15, run kc = lane >> 4)
 };
 
 template <int QM, int P>
@@ -163,25 +168,34 @@ DEVI void load_k(KRegs<QM>& r, const uint8_t* chunk, int pos) {
 template <int QM, int P>
 DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
   using L = Lay<QM, P>;
+  // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of pages 2 s, 2 s + 1)
+  const int m = lane & 15, kc = lane >> 4;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    if constexpr (QM == QM_ASYM2) {
-      const u32x2 v = gload<u32x2>(chunk[k] + L::V_OFF + 8 * lane);
-      r.vc[k][0] = v.x; r.vc[k][1] = v.y;
-    } else {
-      const u32x4 v = gload<u32x4>(chunk[k] + L::V_OFF + 16 * lane);
-      r.vc[k][0] = v.x; r.vc[k][1] = v.y; r.vc[k][2] = v.z; r.vc[k][3] = v.w;
+  for (int s2 = 0; s2 < 2; ++s2) {
+    const uint8_t* ch = (kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2];
+#pragma unroll
+    for (int eh = 0; eh < 2; ++eh) {
+      if constexpr (QM == QM_ASYM2) {
+        const u32x2 v = gload<u32x2>(ch + L::V_OFF + 8 * (2 * (16 * eh + m) + (kc & 1)));
+        r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y;
+      } else {
+        const u32x4 v = gload<u32x4>(ch + L::V_OFF + 16 * (2 * (16 * eh + m) + (kc & 1)));
+        r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y; r.vc[2 * s2 + eh][2] = v.z; r.vc[2 * s2 + eh][3] = v.w;
+      }
     }
   }
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 struct WaveState {
   float m[4];        // running maximum per head (wave uniform)
   float l[4];        // this lane's share of the running sum per head
-  float acc[4][4];   // [head][entry word] of the lane's V^T entries: 2^-24 sum p' code (zero points not yet removed)
+  // 2^-24 sum p' code (zero points not yet removed), [entry word parity]: column lane & 15 = (group g, head), rows =
+  // entries 16 (g & 1) + 4 (lane >> 4) + r, entry word 2 (g >> 1) + parity
+  f32x4 ot[2];
   float z[2];        // lane = (page, half, group, head pair): its share of sum p' zero point, heads 2 hp and 2 hp + 1
 };
-
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
 template <int QM, bool K2, class SM>
@@ -252,8 +266,10 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
     st.l[h] *= alpha[h];
-#pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= alpha[h];
+  }
+  {   // the lane's accumulator column belongs to head lane & 3
+    const float al = (lane & 2) ? ((lane & 1) ? alpha[3] : alpha[2]) : ((lane & 1) ? alpha[1] : alpha[0]);
+    st.ot[0] *= al; st.ot[1] *= al;
   }
   st.z[0] *= (lane & 1) ? alpha[2] : alpha[0];
   st.z[1] *= (lane & 1) ? alpha[3] : alpha[1];
@@ -288,35 +304,31 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
 
 template <int QM, class SM>
 DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
-  const int c8 = lane & 1, g0 = lane >> 5;
+  // An entry word (entry half eh, word sub) holds channels of group 2 (sub >> 1) + eh only.  The products of all
+  // four groups share one accumulator per word parity: the B operand of a group is the strip row with the columns of
+  // the other groups zero (those lanes read a row of zeros instead), so each column collects its own group's rows.
+  const int n = lane & 15, kc = lane >> 4;
+  const uint4* own = reinterpret_cast<const uint4*>(S.pb(wave)) + kc * PB_RSTRIDE + n;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + (k * 2 + c8) * PB_RSTRIDE;   // + group * 4 + head
+  for (int s2 = 0; s2 < 2; ++s2) {            // 32 tokens: the runs (page 2 s + (kc >> 1), c8 = kc & 1) = strip row group 4 s + kc
+    half8 b[4];
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {      // entry words 0, 1 belong to group g0, words 2, 3 to group 2 + g0
-      const int g = 2 * half + g0;
-      uint4 pq[4];
+    for (int g = 0; g < 4; ++g) {
+      const uint4* src = (n >> 2) == g ? own : reinterpret_cast<const uint4*>(S.zero);
+      b[g] = __builtin_bit_cast(half8, src[4 * s2 * PB_RSTRIDE]);
+    }
 #pragma unroll
-      for (int h = 0; h < 4; ++h) pq[h] = pp[g * 4 + h];
+    for (int eh = 0; eh < 2; ++eh)
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const int sub = 2 * half + s2;
+      for (int sub = 0; sub < 4; ++sub) {
         uint32_t x[4];
         if constexpr (QM == QM_ASYM2) {   // two sub-vectors per word: the odd one's sums carry 2^4 until the fold
-          if (sub & 1) UnpackD<QM>::run_hi(r.vc[k][sub >> 1], x); else UnpackD<QM>::run(r.vc[k][sub >> 1], x);
+          if (sub & 1) UnpackD<QM>::run_hi(r.vc[2 * s2 + eh][sub >> 1], x); else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub >> 1], x);
         }
-        else UnpackD<QM>::run(r.vc[k][sub], x);
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          float a = st.acc[h][sub];
-          a = dot2(x[0], pq[h].x, a);
-          a = dot2(x[1], pq[h].y, a);
-          a = dot2(x[2], pq[h].z, a);
-          a = dot2(x[3], pq[h].w, a);
-          st.acc[h][sub] = a;
-        }
+        else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub], x);
+        const uint4 aq = make_uint4(x[0], x[1], x[2], x[3]);
+        st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aq), b[2 * (sub >> 1) + eh], st.ot[sub & 1], 0, 0, 0);
       }
-    }
   }
   if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (page, page half, group, head pair)
     const int rg = lane >> 3, g = (lane >> 1) & 3, hp = lane & 1;
@@ -373,7 +385,7 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&
 }
 
 template <int QM, bool K2, int P, int NW>
-__global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW == 16 ? 4 : 3) : (K2 ? 4 : 1)) k_decode(const DecodeParams p, int ntile, int nparts) {
+__global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4 : 1)) k_decode(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
   __shared__ Smem<NW> S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -396,12 +408,9 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
     const int hi = dyn ? len : min(len, (split + 1) * p.chunk);
     WaveState st;
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      st.m[h] = -INFINITY; st.l[h] = 0.f;
-#pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] = 0.f;
-    }
+    for (int h = 0; h < 4; ++h) { st.m[h] = -INFINITY; st.l[h] = 0.f; }
     st.z[0] = st.z[1] = 0.f;
+    st.ot[0] = st.ot[1] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (lo < hi) {   // uniform over the workgroup
       const int pg0 = lo / P, pg1 = (hi + P - 1) / P;
       const int* bt = p.block_table + static_cast<long long>(b) * p.bt_stride;
@@ -417,6 +426,7 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
       if (dyn) take = draw();        // the first round trip to the device-scope counter hides behind the prologue
       for (int i = threadIdx.x; i < min(pg1 - pg0, BT_CACHE); i += 64 * NW) S.btc[i] = bt[pg0 + i];
       if (threadIdx.x == 0) S.next = NW;
+      for (int i = threadIdx.x; i < 4 * (4 * PB_RSTRIDE + 1); i += 64 * NW) S.zero[i] = 0u;
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
       const int nquad = (pg1 - pg0 + 3) >> 2;
@@ -484,8 +494,8 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
       // last arriver clears the word)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    // ---- fold the wave: zero-point sums per (head, group) through the wave's strip, entry pairs (c8 = 0 / 1),
-    //      codes -> values: 2^24 (acc - sum p' zero point)
+    // ---- fold the wave: zero-point sums per (head, group) through the wave's strip, codes -> values:
+    //      2^24 (acc - sum p' zero point)
     if constexpr (QM != QM_SYM4) {
       float z0 = st.z[0], z1 = st.z[1];
       z0 += swz_xor<8>(z0); z1 += swz_xor<8>(z1);
@@ -496,38 +506,35 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
       wave_lds_sync();
     }
     const float unfold = (lane & 1) ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;   // lane & 1 = token parity
+    const int hl = lane & 3, gl = (lane >> 2) & 3;      // the lane's accumulator column: head hl, group gl
+    {
+      float zg = 0.f;
+      if constexpr (QM != QM_SYM4) zg = reinterpret_cast<const float*>(S.pb(wave))[hl * 4 + gl];
+      if constexpr (QM == QM_ASYM2) st.ot[1] *= 0.0625f;            // fields unpacked 4 bits up
+#pragma unroll
+      for (int y = 0; y < 2; ++y)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) st.ot[y][r4] = (st.ot[y][r4] - zg) * 16777216.f;
+    }
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      if constexpr (QM == QM_ASYM2) { st.acc[h][1] *= 0.0625f; st.acc[h][3] *= 0.0625f; }   // fields unpacked 4 bits up
-#pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] += dpp_xor1(st.acc[h][s4]);
-      if constexpr (QM != QM_SYM4) {
-        const float* zs = reinterpret_cast<const float*>(S.pb(wave)) + h * 4 + (lane >> 5);
-        const float z01 = zs[0], z23 = zs[2];
-        st.acc[h][0] -= z01; st.acc[h][1] -= z01; st.acc[h][2] -= z23; st.acc[h][3] -= z23;
-      }
-#pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) st.acc[h][s4] *= 16777216.f;
       const float lsum = wave_sum64(st.l[h] * unfold);
       if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = lsum; }
     }
     __syncthreads();     // every wave is done with its strip: the partial outputs may overwrite them
     {
-      const int wq = lane >> 4, gid = (lane >> 1) & 7;
+      const int kc = lane >> 4;      // the lane's four entry rows: 4 kc + r
+      float M = S.m[0][hl];
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        float M = S.m[0][h];
+      for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][hl]);
+      const float mh = (hl & 2) ? ((hl & 1) ? st.m[3] : st.m[2]) : ((hl & 1) ? st.m[1] : st.m[0]);
+      const float f = mh == -INFINITY ? 0.f : fexp2(mh - M);
+      float* o = S.o(wave, hl);
 #pragma unroll
-        for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][h]);
-        const float f = st.m[h] == -INFINITY ? 0.f : fexp2(st.m[h] - M);
-        if ((lane & 1) == 0) {
-          float* o = S.o(wave, h);
-#pragma unroll
-          for (int sub = 0; sub < 4; ++sub) {
-            const int d = 64 * (sub >> 1) + 16 * wq + gid + 8 * (sub & 1);
-            o[d] = f * st.acc[h][sub];
-          }
-        }
+      for (int y = 0; y < 2; ++y) {
+        // entry e = 16 (gl & 1) + 4 kc + r, word sub = 2 (gl >> 1) + y: dim 64 (sub >> 1) + 16 (e >> 3) + 8 (sub & 1) + (e & 7)
+        const int d = 32 * gl + 16 * (kc >> 1) + 8 * y + 4 * (kc & 1);
+        *reinterpret_cast<float4*>(o + d) = make_float4(f * st.ot[y][0], f * st.ot[y][1], f * st.ot[y][2], f * st.ot[y][3]);
       }
     }
     __syncthreads();
@@ -664,14 +671,11 @@ __global__ void __launch_bounds__(64 * NW, NW > 4 ? 16 / (NW / 4) / 1 * 0 + (NW 
   }
 }
 
-// Wavefronts per workgroup: 16 (one workgroup fills a CU: 4 wavefronts per SIMD at 128 registers) when every wavefront
-// has at least two quads of pages to draw, else 4.
-#ifndef FR_BIGW
-#define FR_BIGW 12
-#endif
-constexpr int BIGW = FR_BIGW;   // wavefronts of the large workgroup: 12 leave 168 registers per lane, 16 leave 128
+// Wavefronts per workgroup: 4, or from 1024 tokens per split one large workgroup that fills a CU.  The codebook
+// kernels fit 128 registers per lane: 16 wavefronts (4 per SIMD); the static-mask kernels need more: 12 (168 registers).
+template <bool K2> constexpr int BIGW = K2 ? 16 : 12;
 constexpr int BIG_CHUNK = 1024;   // tokens per split from which the large workgroup pays (measured: batch 1-16, 2-32 k tokens)
-inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? BIGW : 4; }
+inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? 16 : 4; }   // > 4 selects the large workgroup
 
 template <int QM, bool K2>
 int launch_qm(const DecodeParams& p, hipStream_t st) {
@@ -680,7 +684,7 @@ int launch_qm(const DecodeParams& p, hipStream_t st) {
   const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
-  if (p.wg_waves == BIGW) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW>), grid, dim3(64 * BIGW), 0, st, p, ntile, nparts);
+  if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
   else hipLaunchKernelGGL((k_decode<QM, K2, 16, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
@@ -700,8 +704,8 @@ int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
 template <int QM, bool K2>
 int occupancy_qm(int waves) {
   int n = 0;
-  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * waves, 0) != hipSuccess || n < 1) {
+  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW<K2>>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * (waves > 4 ? BIGW<K2> : 4), 0) != hipSuccess || n < 1) {
     (void)hipGetLastError();
     return waves > 4 ? 1 : 2;
   }
@@ -722,7 +726,6 @@ int decode_occupancy(int fmt, int waves) {
   static int cache[16][2] = {{0}};
   if (fmt < 0 || fmt >= 16) return 0;
   const int wi = waves > 4 ? 1 : 0;
-  waves = wi ? BIGW : 4;
   if (cache[fmt][wi] == 0) {
     switch (fmt) {
       case FMT_INT4: cache[fmt][wi] = occupancy_qm<QM_SYM4, false>(waves); break;

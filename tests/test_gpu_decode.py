@@ -2,11 +2,12 @@
 
 Bar (floating point, the tolerance of the build's north star: max-abs 2e-3 / rel 1e-2):
   * rows of ordinary data: |out - ref| <= 2e-3 + 1e-2 * |ref| element-wise;
-  * row 0, which carries the reference tests' adversarial groups (values x300, x1e-5, constants, one-hots: log2
-    scores of +-1000, outputs of several hundred, so that a 1e-5 relative change of one score moves a weight by
-    percents): |out - ref| <= 2e-3 + 1e-2 * max |ref[0]| (the reference's own tests measure every row against the
-    global max |ref| with a 4e-3 floor, test_kernels.py:173).  The rotated query variants are held in fp16 (11-bit
-    mantissa); the identity variant of a bf16 query is exact.
+  * row 0 (and every row when the sequences share one block-table row), which carries the reference tests'
+    adversarial groups (values x300, x1e-5, constants, one-hots: log2 scores of +-1000, outputs of several hundred, so
+    that a 1e-5 relative change of one score moves a weight by percents): |out - ref| <= 2e-3 + 1e-2 * max |ref[row]|
+    (the reference's own tests measure every row against the global max |ref| with a 4e-3 floor,
+    test_kernels.py:173).  The rotated query variants are held in fp16 (11-bit mantissa); the identity variant of a
+    bf16 query is exact.
 ref = fp64 softmax attention over the pages parsed by the oracle's independent layout parser (the cache bytes are
 written by the HIP writers, whose bit-exactness tests/test_gpu_writers.py establishes)."""
 import math
@@ -97,6 +98,8 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
         # whose rounding scales with the largest value-group scale of the row (1e-5 of a quantisation step)
         lim = ATOL + RTOL * np.abs(ref) + 1e-5 * np.abs(ref).max(axis=(1, 2), keepdims=True)
         lim[0] = ATOL + RTOL * np.abs(ref[0]).max()                          # row 0: adversarial groups
+        if bt_shared:                                                        # every sequence reads row 0's pages
+            lim = ATOL + RTOL * np.abs(ref).max(axis=(1, 2), keepdims=True) + 0 * lim
         err = np.where(valid[:, None, None], np.abs(got - ref), 0.0)
         worst = np.unravel_index(np.argmax(err / lim), err.shape)
         assert (err <= lim).all(), (f"{fmt} {lens} ns={ns} ch={ch} worst(b,head,d)={tuple(int(i) for i in worst)} "
@@ -136,7 +139,7 @@ def test_window_and_kv_start(dev, mode, fmt):
 @pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
                                       ("static", "int4a"), ("static", "int2a")])
 def test_large_workgroup_shape(dev, mode, fmt):
-    """chunks of >= 1024 tokens on few (sequence, head) pairs: one 12-wavefront workgroup per split, quads drawn from
+    """chunks of >= 1024 tokens on few (sequence, head) pairs: one large (16- or 12-wavefront) workgroup per split, quads drawn from
     a counter in LDS (the other tests run the 4-wavefront shapes); with splits, tail rows, kv_start and a q tile pair."""
     ns, ch = run_case(dev, mode, [2300, 2100], fmt, seed=20, Hkv=2, nsplit=1)
     assert (ns, ch) == (1, 2304)
