@@ -1,6 +1,7 @@
-// Paged split-K GQA decode attention over FlagRot INT4 / INT2 pages for gfx950 (wave64, no matrix cores).
+// Paged split-K GQA decode attention over FlagRot INT4 / INT2 pages for gfx950 (wave64; scores on the vector
+// pipe, the value product on the matrix pipe).
 //
-// One workgroup (16 wavefronts = a whole CU's register file, or 4 for short chunks) per (KV head x q tile of 4 heads,
+// One workgroup (16 or 12 wavefronts = a whole CU's register file, or 4 for short chunks) per (KV head x q tile of 4 heads,
 // split, sequence).  Its wavefronts draw quads of 4 pages from a counter in LDS, so they finish together whatever
 // share of the issue slots each one got.  A wavefront streams whole pages (16 tokens x one KV head = one contiguous
 // 2304 / 1280 byte chunk) with 128-bit loads:
@@ -11,10 +12,11 @@
 //                the variant its token / group flags ask for, so selection costs no arithmetic.  The exponent offsets
 //                and the zero points are removed with per-(variant, head, group) query sums.
 //   softmax      exp2-domain online softmax per wavefront; p * V-scale is written to LDS as fp16 in V^T token order.
-//   value phase  lane = one 16-byte V^T entry (4 dims x 8 tokens): a code field masked in place is an fp16 denormal
-//                (value code * 2^(position - 24), exact), contracted with p * scale over the tokens by v_dot2; the
-//                powers of two ride on the p * scale operand and one final multiply, the zero points leave through
-//                sum p * scale * zero point, contracted once per (page half, group, head) from the same LDS strips.
+//   value phase  lane = one 16-byte V^T entry (4 dims x 8 tokens) of a run of 8 tokens: its words masked in place (fp16
+//                denormals, value code * 2^(position - 24), exact) are the A operands of v_mfma_f32_16x16x32_f16, the
+//                p * scale strip rows the B operands (columns = (group, head)); the powers of two ride on the
+//                p * scale operand and one final multiply, the zero points leave through sum p * scale * zero point,
+//                contracted by v_dot2 once per (page half, group, head) from the same LDS strips.
 // The wavefronts are merged through LDS; splits through the caller's workspace with a ticket counter (the last
 // arriving workgroup of a (sequence, KV head) merges, normalises, optionally rotates back, and stores bf16).
 // The BF16 sink / window rows are one more split handled by an extra workgroup of the same grid.
