@@ -45,24 +45,33 @@ template <class T> DEVI T gload(const uint8_t* p) {
   return *(gp)(p);
 }
 constexpr int CHUNK = 1552, KM_OFF = 512, VC_OFF = 768, VM_OFF = 1280, VF_OFF = 1536;
-constexpr int NPAIR = 18;                       // token pairs per (group, sub-vector): 32 tokens + two odd-class pads
+constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
+constexpr int QROW = 68;                        // words per row of the query strips: 64 + 4 pad (conflict-free 128-bit rows)
+constexpr int OROW = 132;                       // floats per row of the merged accumulators: 128 + 4 pad
 
-template <int G> struct Scr {                   // per wavefront; G = heads of the tile (<= 4)
-  uint32_t qs[G][64];                           // fp16 pairs of q' * scale * 2^-shift, per (head, channel pair)
-  alignas(16) uint32_t pp[4][NPAIR][4];         // (p * scale) of the pair's two tokens, per (sub-vector, pair, head)
-  alignas(16) uint32_t pm[4][NPAIR][4];         // (p * min)
-  alignas(8) uint8_t vord[4][2 * NPAIR][8];     // the 8 code bytes of (sub-vector, slot)
-  int cnt[4][2];                                // tokens of class 0 / 1 per sub-vector
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct Scr {                                    // per wavefront, rewritten for every 32-token group
+  alignas(16) uint32_t qs[GT][QROW];            // fp16 pairs of q' * scale * 2^-shift per (head, channel pair)
+  alignas(16) uint32_t qm[GT][QROW];            // fp16 pairs of q' * min
+  alignas(16) _Float16 pst[GT][32];             // p per (head, token)
+  alignas(16) uint16_t vsm[3][4][32];           // value scale (fp16 bits) per (class, sub-vector, token), 0 off its class
+  alignas(16) uint16_t vmm[3][4][32];           // value min likewise
+  alignas(16) uint8_t vt[4][8][32];             // value code bytes per (sub-vector, byte, token)
 };
-template <int G> struct Smem {
-  float qv[3][G][128];                          // query rotations (fp32)
-  Scr<G> w[4];
-  float ob[3][G][128];                          // merged accumulators per class
-  float mw[4][G], lw[4][G];
+struct Smem {
+  float qv[3][GT][128];                         // query rotations (fp32)
+  union {
+    Scr w[4];
+    float ob[3][GT][OROW];                      // merged accumulators per class (after the page loop)
+  };
+  float mw[4][GT], lw[4][GT];
 };
 
 struct GroupRegs {
-  u32x4 kc;      // lane (token, half): the token's 4 code words of its 64 channels
+  u32x2 ka, kb;  // lane (token m = lane & 15 of page A / B, quarter kc = lane >> 4): code words 2 kc, 2 kc + 1 of the token
   u32x2 km;      // lane = channel pair: (scale | min << 16) of channels 2 l, 2 l + 1
   u32x4 vc;      // lane (token, half): the token's code bytes of sub-vectors 2 half, 2 half + 1
   u32x2 vm;      // lane (token, half): (scale | min << 16) of sub-vectors 2 half, 2 half + 1
@@ -72,7 +81,8 @@ struct GroupRegs {
 DEVI void load_group(GroupRegs& r, const uint8_t* chA, const uint8_t* chB, int lane) {
   const int t = lane & 31, hh = lane >> 5;
   const uint8_t* cht = t < 16 ? chA : chB;
-  r.kc = gload<u32x4>(cht + (t & 15) * 32 + 16 * hh);
+  r.ka = gload<u32x2>(chA + (lane & 15) * 32 + 8 * (lane >> 4));
+  r.kb = gload<u32x2>(chB + (lane & 15) * 32 + 8 * (lane >> 4));
   r.km = gload<u32x2>((lane < 32 ? chA : chB) + KM_OFF + (lane & 31) * 8);
   r.vc = gload<u32x4>(cht + VC_OFF + (t & 15) * 32 + 16 * hh);
   r.vm = gload<u32x2>(cht + VM_OFF + (t & 15) * 16 + 8 * hh);
@@ -82,7 +92,7 @@ DEVI void load_group(GroupRegs& r, const uint8_t* chA, const uint8_t* chB, int l
 // The BF16 ring rows of one sequence (split index NS): rows [0, tail_len) of ring block tail_idx, K row h, V row Hkv + h,
 // original basis.  A wavefront takes every fourth row, lanes own 2 dims; same partial format as the page splits.
 template <int G>
-DEVI void tail_split(Smem<G>& S, const uint16_t* __restrict__ q, long long q_rs, const uint16_t* __restrict__ ring,
+DEVI void tail_split(Smem& S, const uint16_t* __restrict__ q, long long q_rs, const uint16_t* __restrict__ ring,
                      const int* __restrict__ tail_len, const int* __restrict__ tail_idx, int T, int Hkv, int Gq, int b, int h,
                      int g0, float qscale, float* __restrict__ op, float* __restrict__ mlp) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
@@ -148,37 +158,36 @@ DEVI void tail_split(Smem<G>& S, const uint16_t* __restrict__ q, long long q_rs,
   }
 }
 
-template <int G>
 __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restrict__ q, long long q_rs,
                                                     const uint8_t* __restrict__ pool, const int* __restrict__ bt,
                                                     long long bt_rs, const int* __restrict__ cached, int kv_start, int Hkv,
                                                     int NS, int chunk, float qscale, float* __restrict__ opart,
-                                                    float* __restrict__ ml, int Gq, int ntile,
+                                                    float* __restrict__ ml, int Gq,
                                                     const uint16_t* __restrict__ ring, const int* __restrict__ tail_len,
                                                     const int* __restrict__ tail_idx, int T) {
-  constexpr int GP = 4;
+  constexpr int G = GT;
   extern __shared__ __align__(16) uint8_t lds[];
-  Smem<G>& S = *reinterpret_cast<Smem<G>*>(lds);
-  const int b = blockIdx.x, h = blockIdx.y / ntile, g0 = (blockIdx.y % ntile) * G, sp = blockIdx.z;   // heads g0 .. g0 + G - 1
+  Smem& S = *reinterpret_cast<Smem*>(lds);
+  const int b = blockIdx.x, h = blockIdx.y, g0 = 0, sp = blockIdx.z;
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
   const long long pidx = (static_cast<long long>(b) * Hkv + h) * (NS + 1) + sp;
-  float* op = opart + (pidx * Gq + g0) * 128;
-  float* mlp = ml + (pidx * Gq + g0) * 2;
+  float* op = opart + pidx * Gq * 128;
+  float* mlp = ml + pidx * Gq * 2;
   if (sp == NS) {
     tail_split<G>(S, q, q_rs, ring, tail_len, tail_idx, T, Hkv, Gq, b, h, g0, qscale, op, mlp);
     return;
   }
   const int t0 = max(sp * chunk, kv_start), t1 = min((sp + 1) * chunk, cached[b]);
   if (t1 <= t0) {
-    if (tid < G && g0 + tid < Gq) { mlp[2 * tid] = -INFINITY; mlp[2 * tid + 1] = 0.f; }
+    if (tid < Gq) { mlp[2 * tid] = -INFINITY; mlp[2 * tid + 1] = 0.f; }
     return;
   }
-  // query rotations: half wave per (variant, head)
+  // query rotations: half wave per (variant, head); heads past the group are zero
   for (int r = tid >> 5; r < 3 * G; r += 8) {
     const int var = r / G, g = r % G, lq = tid & 31;
     float x[4] = {0.f, 0.f, 0.f, 0.f};
-    if (g0 + g < Gq) {
-      const uint2 raw = *reinterpret_cast<const uint2*>(q + static_cast<long long>(b) * q_rs + (static_cast<long long>(h) * Gq + g0 + g) * 128 + 4 * lq);
+    if (g < Gq) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(q + static_cast<long long>(b) * q_rs + (static_cast<long long>(h) * Gq + g) * 128 + 4 * lq);
       x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
     }
     if (var == 1) fwht<32>(x, lq);
@@ -187,14 +196,19 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   }
   __syncthreads();
 
-  Scr<G>& W = S.w[wv];
-  float m_run[G], l_run[G];
-  float accI[G][4], accH[G][4], accF[G][4], mI[G], mH[G], mF[G];
+  Scr& W = S.w[wv];
+  // Score layout: lane = (head sn = lane & 15 (heads 8..15 repeat 0..7 and are ignored), token quarter kc = lane >> 4);
+  // value layout: lane = (column vn = lane & 31 = (class vn >> 3, head vn & 7; columns 24..31 ignored), token half lane >> 5).
+  const int sn = lane & 15, kc = lane >> 4, sh = sn & 7;
+  const int vcl = min(l32 >> 3, 2), vh = l32 & 7;
+  float m_run = -INFINITY, l_run = 0.f;          // of head sh, over this lane's tokens
+  f32x16 accv[4];                                // [sub-vector]: rows = the 32 channels, this lane's column; codes * 2^-24 * 2^(2 field)
+  float am[4];                                   // [sub-vector]: sum p * min of this lane's (class, head) over its tokens
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m_run[g] = -INFINITY; l_run[g] = 0.f; mI[g] = mH[g] = mF[g] = 0.f;
+  for (int j = 0; j < 4; ++j) {
+    am[j] = 0.f;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) accI[g][k] = accH[g][k] = accF[g][k] = 0.f;
+    for (int i = 0; i < 16; ++i) accv[j][i] = 0.f;
   }
   const int* btb = bt + static_cast<long long>(b) * bt_rs;
   const int g_first = t0 / 32, g_end = (t1 + 31) / 32;
@@ -202,7 +216,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   // fields 0..4 are masked in place (code * 2^(2k - 24)), fields 5..7 after a shift by 10 (code * 2^(2(k-5) - 24))
   const int kq = lane & 7;
   const float qfold = __uint_as_float((127u - 2u * static_cast<uint32_t>(kq < 5 ? kq : kq - 5)) << 23);
-  const int jv = l32 >> 3;                                  // sub-vector of this lane's 4 value channels
+  const uint32_t vmask = 0x00030003u << (2 * (l32 & 3));      // value layout row = channel l32: field l32 & 3 of byte l32 >> 2
+  const half8 tiny = __builtin_bit_cast(half8, u32x4{0x00010001u, 0x00010001u, 0x00010001u, 0x00010001u});   // 2^-24 in every slot
 
   GroupRegs cur;
   int gi = g_first + wv;
@@ -212,189 +227,179 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     GroupRegs nxt;
     if (gi + 4 < g_end) load_group(nxt, pool + (static_cast<long long>(btb[2 * (gi + 4)]) * Hkv + h) * CHUNK,
                                    pool + (static_cast<long long>(btb[2 * (gi + 4) + 1]) * Hkv + h) * CHUNK, lane);
-    // ---- group flags, q' * scale, bias
-    const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = __builtin_amdgcn_readlane(cur.km.y, 0),
-                   s2 = __builtin_amdgcn_readlane(cur.km.x, 1), s3 = __builtin_amdgcn_readlane(cur.km.y, 1),
-                   s4 = __builtin_amdgcn_readlane(cur.km.x, 2);
-    const bool useF = (s4 >> 15) & 1u;
-    const uint32_t lmask = ((s0 >> 15) & 1u) | (((s1 >> 15) & 1u) << 1) | (((s2 >> 15) & 1u) << 2) | (((s3 >> 15) & 1u) << 3);
-    const int which = useF ? 2 : static_cast<int>((lmask >> (lane >> 4)) & 1u);
-    const float sa = f16_value(cur.km.x & 0x7FFFu), ma = f16_value(cur.km.x >> 16);
-    const float sb = f16_value(cur.km.y & 0x7FFFu), mb = f16_value(cur.km.y >> 16);
-    float bias[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float2 qq = *reinterpret_cast<const float2*>(&S.qv[which][g][2 * lane]);
-      W.qs[g][lane] = pack_rn(qq.x * sa * qfold, qq.y * sb * qfold);
-      bias[g] = wave_sum64(qq.x * ma + qq.y * mb);
-    }
-    // reset of the ordered strips (the pad slots of odd classes must weigh nothing)
-    for (int i = lane; i < 2 * 4 * NPAIR * GP / 4; i += 64) reinterpret_cast<u32x4*>(&W.pp[0][0][0])[i] = u32x4{0u, 0u, 0u, 0u};
-    wave_lds_sync();
-    // ---- scores: lane = (token l32, channel half hh)
-    float a[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) a[g] = 0.f;
-#pragma unroll
-    for (int wi = 0; wi < 4; ++wi) {
-      const uint32_t w = cur.kc[wi], w10 = w >> 10;
-      const uint32_t x[8] = {w & 0x00030003u, w & 0x000C000Cu, w & 0x00300030u, w & 0x00C000C0u, w & 0x03000300u,
-                             w10 & 0x00030003u, w10 & 0x000C000Cu, w10 & 0x00300030u};
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const u32x4 qa = *reinterpret_cast<const u32x4*>(&W.qs[g][8 * (4 * hh + wi)]);
-        const u32x4 qb = *reinterpret_cast<const u32x4*>(&W.qs[g][8 * (4 * hh + wi) + 4]);
-        float v = a[g];
-        v = dot2(x[0], qa.x, v); v = dot2(x[1], qa.y, v); v = dot2(x[2], qa.z, v); v = dot2(x[3], qa.w, v);
-        v = dot2(x[4], qb.x, v); v = dot2(x[5], qb.y, v); v = dot2(x[6], qb.z, v); v = dot2(x[7], qb.w, v);
-        a[g] = v;
-      }
-    }
-    const int pos = gi * 32 + l32;
-    const bool valid = pos >= t0 && pos < t1;
-    float sc[G];
-    bool beat = false;
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float tot = (a[g] + __shfl_xor(a[g], 32, 64)) * 16777216.f + bias[g];
-      sc[g] = valid ? tot * qscale : -INFINITY;
-      beat |= sc[g] > m_run[g];
-    }
-    if (__any(beat)) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const float mn = fmaxf(m_run[g], wave_max64(sc[g]));
-        const float alpha = m_run[g] == -INFINITY ? 0.f : fexp2(m_run[g] - mn);
-        m_run[g] = mn;
-        l_run[g] *= alpha;
-        mI[g] *= alpha; mH[g] *= alpha; mF[g] *= alpha;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) { accI[g][k] *= alpha; accH[g][k] *= alpha; accF[g][k] *= alpha; }
-      }
-    }
-    // ---- p, class order, ordered strips: lane (token, half) serves sub-vectors 2 hh, 2 hh + 1
-    uint32_t ph[GP / 2];                                    // p as fp16 pairs of heads
+    // ---- group flags; q' * scale and q' * min strips: lane = channel pair
     {
-      float p[GP];
-#pragma unroll
-      for (int g = 0; g < GP; ++g) p[g] = 0.f;
+      const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = __builtin_amdgcn_readlane(cur.km.y, 0),
+                     s2 = __builtin_amdgcn_readlane(cur.km.x, 1), s3 = __builtin_amdgcn_readlane(cur.km.y, 1),
+                     s4 = __builtin_amdgcn_readlane(cur.km.x, 2);
+      const bool useF = (s4 >> 15) & 1u;
+      const uint32_t lmask = ((s0 >> 15) & 1u) | (((s1 >> 15) & 1u) << 1) | (((s2 >> 15) & 1u) << 2) | (((s3 >> 15) & 1u) << 3);
+      const int which = useF ? 2 : static_cast<int>((lmask >> (lane >> 4)) & 1u);
+      const float sa = f16_value(cur.km.x & 0x7FFFu) * qfold, ma = f16_value(cur.km.x >> 16);
+      const float sb = f16_value(cur.km.y & 0x7FFFu) * qfold, mb = f16_value(cur.km.y >> 16);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        p[g] = valid ? fexp2(sc[g] - m_run[g]) : 0.f;
-        if (hh == 0) l_run[g] += p[g];
-      }
-#pragma unroll
-      for (int g2 = 0; g2 < GP / 2; ++g2) ph[g2] = pack_rn(p[2 * g2], p[2 * g2 + 1]);
-    }
-    const bool vF = cur.vf != 0;
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-      const uint32_t w = jj ? cur.vm.y : cur.vm.x;
-      const int j = 2 * hh + jj;
-      const int cls = vF ? 2 : static_cast<int>((w >> 15) & 1u);
-      const unsigned long long b0 = __ballot(cls == 0), b1 = __ballot(cls == 1), b2 = __ballot(cls == 2);
-      const uint32_t m0 = static_cast<uint32_t>(hh ? (b0 >> 32) : b0), m1 = static_cast<uint32_t>(hh ? (b1 >> 32) : b1),
-                     m2 = static_cast<uint32_t>(hh ? (b2 >> 32) : b2);
-      const uint32_t below = (1u << l32) - 1u;
-      const int n0 = __popc(m0), n1 = __popc(m1);
-      const int base1 = (n0 + 1) & ~1, base2 = base1 + ((n1 + 1) & ~1);
-      const int slot = cls == 0 ? __popc(m0 & below) : cls == 1 ? base1 + __popc(m1 & below) : base2 + __popc(m2 & below);
-      *reinterpret_cast<u32x2*>(&W.vord[j][slot][0]) = jj ? u32x2{cur.vc.z, cur.vc.w} : u32x2{cur.vc.x, cur.vc.y};
-      if (l32 == 0) { W.cnt[j][0] = n0; W.cnt[j][1] = n1; }
-      const uint32_t s2x = (w & 0x7FFFu) * 0x10001u, m2x = (w >> 16) * 0x10001u;
-      _Float16* dp = reinterpret_cast<_Float16*>(&W.pp[j][slot >> 1][0]) + (slot & 1);
-      _Float16* dm = reinterpret_cast<_Float16*>(&W.pm[j][slot >> 1][0]) + (slot & 1);
-#pragma unroll
-      for (int g2 = 0; g2 < GP / 2; ++g2) {
-        const half2_t ps = __builtin_bit_cast(half2_t, pk_mul(ph[g2], s2x));
-        const half2_t pn = __builtin_bit_cast(half2_t, pk_mul(ph[g2], m2x));
-        dp[4 * g2] = ps.x; dp[4 * g2 + 2] = ps.y;
-        dm[4 * g2] = pn.x; dm[4 * g2 + 2] = pn.y;
+        const float2 qq = *reinterpret_cast<const float2*>(&S.qv[which][g][2 * lane]);
+        W.qs[g][lane] = pack_rn(qq.x * sa, qq.y * sb);
+        W.qm[g][lane] = pack_rn(qq.x * ma, qq.y * mb);
       }
     }
-    wave_lds_sync();
-    // ---- values: lane = (4 channels of byte l32, pair parity hh)
+    // ---- value strips: lane = (token l32, half hh) serves sub-vectors 2 hh, 2 hh + 1.  Scale and min go to the strip of
+    //      the token's class (0 in the other two; tokens outside the range have no class), the code bytes to byte rows.
     {
-      const int n0 = W.cnt[jv][0], n1 = W.cnt[jv][1];
-      const int e0 = (n0 + 1) >> 1, e1 = e0 + ((n1 + 1) >> 1), e2 = e1 + ((32 - n0 - n1 + 1) >> 1);
-      // every lane walks its own pair range in lockstep; lanes past their range contribute zero operands (no
-      // divergent control flow: the accumulators stay in place)
-      auto run = [&](int kb, int ke, float (&acc)[G][4], float (&am)[G]) {
-        int kp = kb + ((kb ^ hh) & 1);
-        int nit = max(0, (ke - kp + 1) >> 1);
-        nit = max(nit, __builtin_amdgcn_ds_swizzle(nit, (8 << 10) | 0x1F));      // other sub-vectors
-        nit = max(nit, __builtin_amdgcn_ds_swizzle(nit, (16 << 10) | 0x1F));
-        nit = max(nit, __shfl_xor(nit, 32, 64));                                   // other pair parity
-        nit = __builtin_amdgcn_readfirstlane(nit);
-        for (int it = 0; it < nit; ++it, kp += 2) {
-          const bool live = kp < ke;
-          const int kr = live ? kp : 0;
-          uint32_t comb = static_cast<uint32_t>(W.vord[jv][2 * kr][l32 & 7]) |
-                          (static_cast<uint32_t>(W.vord[jv][2 * kr + 1][l32 & 7]) << 16);
-          comb = live ? comb : 0u;
-          const uint32_t ones = live ? 0x3C003C00u : 0u;
-          const uint32_t x0 = comb & 0x00030003u, x1 = comb & 0x000C000Cu, x2 = comb & 0x00300030u, x3 = comb & 0x00C000C0u;
-          const u32x4 pq = *reinterpret_cast<const u32x4*>(&W.pp[jv][kr][0]);
-          const u32x4 mq = *reinterpret_cast<const u32x4*>(&W.pm[jv][kr][0]);
+      const int pos = gi * 32 + l32;
+      const bool valid = pos >= t0 && pos < t1;
+      const bool vF = cur.vf != 0;
 #pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const uint32_t pv = pq[g];
-            acc[g][0] = dot2(x0, pv, acc[g][0]);
-            acc[g][1] = dot2(x1, pv, acc[g][1]);
-            acc[g][2] = dot2(x2, pv, acc[g][2]);
-            acc[g][3] = dot2(x3, pv, acc[g][3]);
-            am[g] = dot2(ones, mq[g], am[g]);
-          }
+      for (int jj = 0; jj < 2; ++jj) {
+        const uint32_t w = jj ? cur.vm.y : cur.vm.x;
+        const int j = 2 * hh + jj;
+        const int cls = !valid ? 3 : vF ? 2 : static_cast<int>((w >> 15) & 1u);
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+          W.vsm[c][j][l32] = cls == c ? static_cast<uint16_t>(w & 0x7FFFu) : static_cast<uint16_t>(0);
+          W.vmm[c][j][l32] = cls == c ? static_cast<uint16_t>(w >> 16) : static_cast<uint16_t>(0);
         }
-      };
-      run(0, e0, accI, mI);
-      run(e0, e1, accH, mH);
-      run(e1, e2, accF, mF);
+        const uint32_t c0 = jj ? cur.vc.z : cur.vc.x, c1 = jj ? cur.vc.w : cur.vc.y;
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+          W.vt[j][bb][l32] = static_cast<uint8_t>(c0 >> (8 * bb));
+          W.vt[j][4 + bb][l32] = static_cast<uint8_t>(c1 >> (8 * bb));
+        }
+      }
+    }
+    wave_lds_sync();
+    // ---- scores on the matrix pipe: rows = the 16 tokens of a page, columns = heads, 128 channels in four steps of 32.
+    //      A code field masked in place is an fp16 denormal (code * 2^(shift - 24)); the bias sum q' * min enters as
+    //      2^-24 * (q' * min) through the same accumulators.
+    f32x4 sa0, sa1;
+    {
+      f32x4 bias = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 bm = *reinterpret_cast<const u32x4*>(&W.qm[sh][16 * kc + 4 * s]);
+        bias = __builtin_amdgcn_mfma_f32_16x16x32_f16(tiny, __builtin_bit_cast(half8, bm), bias, 0, 0, 0);
+      }
+      sa0 = bias; sa1 = bias;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 bq = *reinterpret_cast<const u32x4*>(&W.qs[sh][16 * kc + 4 * s]);
+        const uint32_t wa = (s >> 1) ? cur.ka.y : cur.ka.x, wb = (s >> 1) ? cur.kb.y : cur.kb.x;
+        u32x4 xa, xb;
+        if (s & 1) {
+          const uint32_t wa10 = wa >> 10, wb10 = wb >> 10;
+          xa = u32x4{wa & 0x03000300u, wa10 & 0x00030003u, wa10 & 0x000C000Cu, wa10 & 0x00300030u};
+          xb = u32x4{wb & 0x03000300u, wb10 & 0x00030003u, wb10 & 0x000C000Cu, wb10 & 0x00300030u};
+        } else {
+          xa = u32x4{wa & 0x00030003u, wa & 0x000C000Cu, wa & 0x00300030u, wa & 0x00C000C0u};
+          xb = u32x4{wb & 0x00030003u, wb & 0x000C000Cu, wb & 0x00300030u, wb & 0x00C000C0u};
+        }
+        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, bq), sa0, 0, 0, 0);
+        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, bq), sa1, 0, 0, 0);
+      }
+    }
+    // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
+    {
+      float sc[8];
+      bool beat = false;
+      const float up = 16777216.f * qscale;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int pos = gi * 32 + 16 * (i >> 2) + 4 * kc + (i & 3);
+        const float v = (i < 4 ? sa0[i & 3] : sa1[i & 3]) * up;
+        sc[i] = (pos >= t0 && pos < t1) ? v : -INFINITY;
+        beat |= sc[i] > m_run;
+      }
+      if (__any(beat)) {
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m_run, mx);
+        const float alpha = m_run == -INFINITY ? 0.f : fexp2(m_run - mn);
+        m_run = mn;
+        l_run *= alpha;
+        const float av = __shfl(alpha, vh, 64);          // the factor of this lane's value column (head vh)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          am[j] *= av;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) accv[j][i] *= av;
+        }
+      }
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        p[i] = sc[i] == -INFINITY ? 0.f : fexp2(sc[i] - m_run);
+        l_run += p[i];
+      }
+      if (sn < 8) {
+        *reinterpret_cast<u32x2*>(&W.pst[sh][4 * kc]) = u32x2{pack_rn(p[0], p[1]), pack_rn(p[2], p[3])};
+        *reinterpret_cast<u32x2*>(&W.pst[sh][16 + 4 * kc]) = u32x2{pack_rn(p[4], p[5]), pack_rn(p[6], p[7])};
+      }
+    }
+    wave_lds_sync();
+    // ---- values on the matrix pipe: rows = the 32 channels of a sub-vector, columns = (class, head), 32 tokens in two
+    //      steps of 16; B = p * scale of the column's class (0 for tokens of another class), A = the tokens' code fields
+    //      masked in place.  sum p * min per (class, head, sub-vector) by v_dot2.
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int tk = 16 * s + 8 * hh;
+      const u32x4 pr = *reinterpret_cast<const u32x4*>(&W.pst[vh][tk]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u32x4 sv = *reinterpret_cast<const u32x4*>(&W.vsm[vcl][j][tk]);
+        const u32x4 mv = *reinterpret_cast<const u32x4*>(&W.vmm[vcl][j][tk]);
+        const u32x2 by = *reinterpret_cast<const u32x2*>(&W.vt[j][l32 >> 2][tk]);
+        const u32x4 bo = u32x4{pk_mul(pr.x, sv.x), pk_mul(pr.y, sv.y), pk_mul(pr.z, sv.z), pk_mul(pr.w, sv.w)};
+        float a = am[j];
+        a = dot2(pr.x, mv.x, a); a = dot2(pr.y, mv.y, a); a = dot2(pr.z, mv.z, a); a = dot2(pr.w, mv.w, a);
+        am[j] = a;
+        // token pairs (0,1) (2,3) of by.x and (4,5) (6,7) of by.y: byte 2 i to bits 0..7, byte 2 i + 1 to bits 16..23
+        const u32x4 ao = u32x4{__builtin_amdgcn_perm(0u, by.x, 0x0C010C00u) & vmask, __builtin_amdgcn_perm(0u, by.x, 0x0C030C02u) & vmask,
+                               __builtin_amdgcn_perm(0u, by.y, 0x0C010C00u) & vmask, __builtin_amdgcn_perm(0u, by.y, 0x0C030C02u) & vmask};
+        accv[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, ao), __builtin_bit_cast(half8, bo), accv[j], 0, 0, 0);
+      }
     }
     wave_lds_sync();
     cur = nxt;
   }
 
   // ---- merge of the wavefronts: maxima, sums, accumulators per class (in wavefront order), inverse transforms
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float lt = wave_sum64(l_run[g]);
-    if (lane == 0) { S.mw[wv][g] = m_run[g]; S.lw[wv][g] = lt; }
+  {
+    float lt = l_run + __shfl_xor(l_run, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (lane < G) { S.mw[wv][lane] = m_run; S.lw[wv][lane] = lt; }
   }
-  __syncthreads();
-  float fac[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float M = fmaxf(fmaxf(S.mw[0][g], S.mw[1][g]), fmaxf(S.mw[2][g], S.mw[3][g]));
-    fac[g] = m_run[g] == -INFINITY ? 0.f : fexp2(m_run[g] - M);
+  __syncthreads();          // every wavefront is done with its strips: the merged accumulators take their place
+  float fac;
+  {
+    const float M = fmaxf(fmaxf(S.mw[0][vh], S.mw[1][vh]), fmaxf(S.mw[2][vh], S.mw[3][vh]));
+    const float mine = S.mw[wv][vh];
+    fac = mine == -INFINITY ? 0.f : fexp2(mine - M);
   }
   for (int r = 0; r < 4; ++r) {
-    if (wv == r) {
+    if (wv == r && l32 < 24) {
+      float* orow = &S.ob[l32 >> 3][vh][0];
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float vi[4], vh[4], vf[4];
+      for (int j = 0; j < 4; ++j) {
+        const float mj = am[j] + __shfl_xor(am[j], 32, 64);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float up = __uint_as_float((127u + 24u - 2u * k) << 23);          // 2^(24 - 2k)
-          vi[k] = accI[g][k] * up + mI[g]; vh[k] = accH[g][k] * up + mH[g]; vf[k] = accF[g][k] * up + mF[g];
-          vi[k] += __shfl_xor(vi[k], 32, 64); vh[k] += __shfl_xor(vh[k], 32, 64); vf[k] += __shfl_xor(vf[k], 32, 64);
-          vi[k] *= fac[g]; vh[k] *= fac[g]; vf[k] *= fac[g];
-        }
-        if (hh == 0) {
-          float4* pI = reinterpret_cast<float4*>(&S.ob[0][g][4 * l32]);
-          float4* pH = reinterpret_cast<float4*>(&S.ob[1][g][4 * l32]);
-          float4* pF = reinterpret_cast<float4*>(&S.ob[2][g][4 * l32]);
-          float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f), b4 = a4, c4 = a4;
-          if (r) { a4 = *pI; b4 = *pH; c4 = *pF; }
-          *pI = make_float4(a4.x + vi[0], a4.y + vi[1], a4.z + vi[2], a4.w + vi[3]);
-          *pH = make_float4(b4.x + vh[0], b4.y + vh[1], b4.z + vh[2], b4.w + vh[3]);
-          *pF = make_float4(c4.x + vf[0], c4.y + vf[1], c4.z + vf[2], c4.w + vf[3]);
+        for (int i4 = 0; i4 < 4; ++i4) {
+          float4* dst = reinterpret_cast<float4*>(orow + 32 * j + 8 * i4 + 4 * hh);      // row = 8 (i >> 2) + 4 hh + (i & 3)
+          float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (r) acc = *dst;
+          // field f = i & 3 of its byte: code * 2^(2 f - 24) was accumulated
+          acc.x += fac * (accv[j][4 * i4 + 0] * 16777216.f + mj);
+          acc.y += fac * (accv[j][4 * i4 + 1] * 4194304.f + mj);
+          acc.z += fac * (accv[j][4 * i4 + 2] * 1048576.f + mj);
+          acc.w += fac * (accv[j][4 * i4 + 3] * 262144.f + mj);
+          *dst = acc;
         }
       }
     }
     __syncthreads();
   }
-  for (int g = tid >> 5; g < G && g0 + g < Gq; g += 8) {
+  for (int g = tid >> 5; g < Gq; g += 8) {
     const int lq = tid & 31;
     const float4 a4 = *reinterpret_cast<const float4*>(&S.ob[0][g][4 * lq]);
     const float4 b4 = *reinterpret_cast<const float4*>(&S.ob[1][g][4 * lq]);
@@ -412,20 +417,18 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   }
 }
 
-template <int G>
 int launch_pages(int Gq, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
                  int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring, const void* tail_len,
                  const void* tail_idx, int T, void* opart, void* ml, hipStream_t st) {
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages<G>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(sizeof(Smem<G>))) != hipSuccess) return 1;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(sizeof(Smem))) != hipSuccess) return 1;
     attr = true;
   }
-  const int ntile = (Gq + G - 1) / G;
-  hipLaunchKernelGGL(k_attn_pages<G>, dim3(B, Hkv * ntile, NS + 1), dim3(256), sizeof(Smem<G>), st, static_cast<const uint16_t*>(q), q_rs,
+  hipLaunchKernelGGL(k_attn_pages, dim3(B, Hkv, NS + 1), dim3(256), sizeof(Smem), st, static_cast<const uint16_t*>(q), q_rs,
                      static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), bt_rs, static_cast<const int*>(cached),
-                     kv_start, Hkv, NS, chunk, qscale, static_cast<float*>(opart), static_cast<float*>(ml), Gq, ntile,
+                     kv_start, Hkv, NS, chunk, qscale, static_cast<float*>(opart), static_cast<float*>(ml), Gq,
                      static_cast<const uint16_t*>(ring), static_cast<const int*>(tail_len), static_cast<const int*>(tail_idx), T);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
@@ -435,14 +438,8 @@ int launch_pages(int Gq, const void* q, long long q_rs, const void* pool, const 
 int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
                        const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
                        const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, hipStream_t st) {
-  // heads per tile: a GQA group of up to 4 in one tile, of 5 .. 8 in two
-  const int gt = G <= 4 ? G : (G + 1) / 2;
-#define FRKV_P(GG) case GG: return launch_pages<GG>(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len, tail_idx, T, opart, ml, st);
-  switch (gt) {
-    FRKV_P(1) FRKV_P(2) FRKV_P(3) FRKV_P(4)
-    default: return 2;
-  }
-#undef FRKV_P
+  if (G < 1 || G > GT) return 2;
+  return launch_pages(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len, tail_idx, T, opart, ml, st);
 }
 
 }  // namespace frkv
