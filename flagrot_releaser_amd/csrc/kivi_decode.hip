@@ -59,14 +59,15 @@ struct Scr {                                    // per wavefront, rewritten for 
   alignas(16) _Float16 pst[GT][32];             // p per (head, token)
   alignas(16) uint16_t vsm[3][4][32];           // value scale (fp16 bits) per (class, sub-vector, token), 0 off its class
   alignas(16) uint16_t vmm[3][4][32];           // value min likewise
-  alignas(16) uint8_t vt[4][8][32];             // value code bytes per (sub-vector, byte, token)
+  alignas(16) uint16_t vt[4][8][32];            // value code bytes (zero-extended) per (sub-vector, byte, token)
 };
 struct Smem {
-  float qv[3][GT][128];                         // query rotations (fp32)
+  uint32_t qh[3][GT][64];                       // query rotations as fp16 pairs per (variant, head, channel pair)
   union {
     Scr w[4];
     float ob[3][GT][OROW];                      // merged accumulators per class (after the page loop)
   };
+  float ams[4][GT][12];                         // per wavefront: sum p * min per (head, class, sub-vector)
   float mw[4][GT], lw[4][GT];
 };
 
@@ -169,7 +170,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   extern __shared__ __align__(16) uint8_t lds[];
   Smem& S = *reinterpret_cast<Smem*>(lds);
   const int b = blockIdx.x, h = blockIdx.y, g0 = 0, sp = blockIdx.z;
-  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
   const long long pidx = (static_cast<long long>(b) * Hkv + h) * (NS + 1) + sp;
   float* op = opart + pidx * Gq * 128;
   float* mlp = ml + pidx * Gq * 2;
@@ -192,7 +193,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     }
     if (var == 1) fwht<32>(x, lq);
     if (var == 2) fwht<128>(x, lq);
-    *reinterpret_cast<float4*>(&S.qv[var][g][4 * lq]) = make_float4(x[0], x[1], x[2], x[3]);
+    *reinterpret_cast<u32x2*>(&S.qh[var][g][2 * lq]) = u32x2{pack_rn(x[0], x[1]), pack_rn(x[2], x[3])};
   }
   __syncthreads();
 
@@ -203,10 +204,9 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   const int vcl = min(l32 >> 3, 2), vh = l32 & 7;
   float m_run = -INFINITY, l_run = 0.f;          // of head sh, over this lane's tokens
   f32x16 accv[4];                                // [sub-vector]: rows = the 32 channels, this lane's column; codes * 2^-24 * 2^(2 field)
-  float am[4];                                   // [sub-vector]: sum p * min of this lane's (class, head) over its tokens
+  f32x4 amd = {0.f, 0.f, 0.f, 0.f};              // score layout: sum p * min, rows = heads 4 kc + r, column sn = (class sn >> 2, sub-vector sn & 3)
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    am[j] = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) accv[j][i] = 0.f;
   }
@@ -224,6 +224,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   if (gi < g_end) load_group(cur, pool + (static_cast<long long>(btb[2 * gi]) * Hkv + h) * CHUNK,
                              pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNK, lane);
   for (; gi < g_end; gi += 4) {
+    const bool full = gi * 32 >= t0 && gi * 32 + 32 <= t1;     // every token of the group is inside the range (wave uniform)
     GroupRegs nxt;
     if (gi + 4 < g_end) load_group(nxt, pool + (static_cast<long long>(btb[2 * (gi + 4)]) * Hkv + h) * CHUNK,
                                    pool + (static_cast<long long>(btb[2 * (gi + 4) + 1]) * Hkv + h) * CHUNK, lane);
@@ -235,26 +236,27 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       const bool useF = (s4 >> 15) & 1u;
       const uint32_t lmask = ((s0 >> 15) & 1u) | (((s1 >> 15) & 1u) << 1) | (((s2 >> 15) & 1u) << 2) | (((s3 >> 15) & 1u) << 3);
       const int which = useF ? 2 : static_cast<int>((lmask >> (lane >> 4)) & 1u);
-      const float sa = f16_value(cur.km.x & 0x7FFFu) * qfold, ma = f16_value(cur.km.x >> 16);
-      const float sb = f16_value(cur.km.y & 0x7FFFu) * qfold, mb = f16_value(cur.km.y >> 16);
+      // fp16 products of the fp16 query pair with (scale * 2^-shift) and with min
+      const uint32_t spair = pack_rn(f16_value(cur.km.x & 0x7FFFu) * qfold, f16_value(cur.km.y & 0x7FFFu) * qfold);
+      const uint32_t mpair = (cur.km.x >> 16) | (cur.km.y & 0xFFFF0000u);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const float2 qq = *reinterpret_cast<const float2*>(&S.qv[which][g][2 * lane]);
-        W.qs[g][lane] = pack_rn(qq.x * sa, qq.y * sb);
-        W.qm[g][lane] = pack_rn(qq.x * ma, qq.y * mb);
+        const uint32_t qq = S.qh[which][g][lane];
+        W.qs[g][lane] = pk_mul(qq, spair);
+        W.qm[g][lane] = pk_mul(qq, mpair);
       }
     }
     // ---- value strips: lane = (token l32, half hh) serves sub-vectors 2 hh, 2 hh + 1.  Scale and min go to the strip of
     //      the token's class (0 in the other two; tokens outside the range have no class), the code bytes to byte rows.
     {
       const int pos = gi * 32 + l32;
-      const bool valid = pos >= t0 && pos < t1;
       const bool vF = cur.vf != 0;
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
         const uint32_t w = jj ? cur.vm.y : cur.vm.x;
         const int j = 2 * hh + jj;
-        const int cls = !valid ? 3 : vF ? 2 : static_cast<int>((w >> 15) & 1u);
+        int cls = vF ? 2 : static_cast<int>((w >> 15) & 1u);
+        if (!full) cls = (pos >= t0 && pos < t1) ? cls : 3;
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
           W.vsm[c][j][l32] = cls == c ? static_cast<uint16_t>(w & 0x7FFFu) : static_cast<uint16_t>(0);
@@ -263,8 +265,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
         const uint32_t c0 = jj ? cur.vc.z : cur.vc.x, c1 = jj ? cur.vc.w : cur.vc.y;
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
-          W.vt[j][bb][l32] = static_cast<uint8_t>(c0 >> (8 * bb));
-          W.vt[j][4 + bb][l32] = static_cast<uint8_t>(c1 >> (8 * bb));
+          W.vt[j][bb][l32] = static_cast<uint16_t>((c0 >> (8 * bb)) & 0xFFu);
+          W.vt[j][4 + bb][l32] = static_cast<uint16_t>((c1 >> (8 * bb)) & 0xFFu);
         }
       }
     }
@@ -301,17 +303,18 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
     {
       float sc[8];
-      bool beat = false;
       const float up = 16777216.f * qscale;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int pos = gi * 32 + 16 * (i >> 2) + 4 * kc + (i & 3);
-        const float v = (i < 4 ? sa0[i & 3] : sa1[i & 3]) * up;
-        sc[i] = (pos >= t0 && pos < t1) ? v : -INFINITY;
-        beat |= sc[i] > m_run;
+      for (int i = 0; i < 8; ++i) sc[i] = (i < 4 ? sa0[i & 3] : sa1[i & 3]) * up;
+      if (!full) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int pos = gi * 32 + 16 * (i >> 2) + 4 * kc + (i & 3);
+          sc[i] = (pos >= t0 && pos < t1) ? sc[i] : -INFINITY;
+        }
       }
-      if (__any(beat)) {
-        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      if (__any(mx > m_run)) {
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m_run, mx);
@@ -321,15 +324,17 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
         const float av = __shfl(alpha, vh, 64);          // the factor of this lane's value column (head vh)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          am[j] *= av;
 #pragma unroll
           for (int i = 0; i < 16; ++i) accv[j][i] *= av;
         }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) amd[r] *= __shfl(alpha, 4 * kc + r, 64);      // rows = heads 4 kc + r (8..15 repeat 0..7)
       }
+      // a wavefront's group always holds a token of the range: the maximum is finite from its first group on
       float p[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        p[i] = sc[i] == -INFINITY ? 0.f : fexp2(sc[i] - m_run);
+        p[i] = fexp2(sc[i] - m_run);
         l_run += p[i];
       }
       if (sn < 8) {
@@ -341,6 +346,11 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     // ---- values on the matrix pipe: rows = the 32 channels of a sub-vector, columns = (class, head), 32 tokens in two
     //      steps of 16; B = p * scale of the column's class (0 for tokens of another class), A = the tokens' code fields
     //      masked in place.  sum p * min per (class, head, sub-vector) by v_dot2.
+    {   // sum p * min: rows = heads, columns = (class, sub-vector), the 32 tokens in one step
+      const u32x4 pa = *reinterpret_cast<const u32x4*>(&W.pst[sh][8 * kc]);
+      const u32x4 mb = *reinterpret_cast<const u32x4*>(&W.vmm[min(sn >> 2, 2)][sn & 3][8 * kc]);
+      amd = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, pa), __builtin_bit_cast(half8, mb), amd, 0, 0, 0);
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       const int tk = 16 * s + 8 * hh;
@@ -348,15 +358,9 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const u32x4 sv = *reinterpret_cast<const u32x4*>(&W.vsm[vcl][j][tk]);
-        const u32x4 mv = *reinterpret_cast<const u32x4*>(&W.vmm[vcl][j][tk]);
-        const u32x2 by = *reinterpret_cast<const u32x2*>(&W.vt[j][l32 >> 2][tk]);
+        const u32x4 by = *reinterpret_cast<const u32x4*>(&W.vt[j][l32 >> 2][tk]);     // (token 2 i | token 2 i + 1 << 16) per word
         const u32x4 bo = u32x4{pk_mul(pr.x, sv.x), pk_mul(pr.y, sv.y), pk_mul(pr.z, sv.z), pk_mul(pr.w, sv.w)};
-        float a = am[j];
-        a = dot2(pr.x, mv.x, a); a = dot2(pr.y, mv.y, a); a = dot2(pr.z, mv.z, a); a = dot2(pr.w, mv.w, a);
-        am[j] = a;
-        // token pairs (0,1) (2,3) of by.x and (4,5) (6,7) of by.y: byte 2 i to bits 0..7, byte 2 i + 1 to bits 16..23
-        const u32x4 ao = u32x4{__builtin_amdgcn_perm(0u, by.x, 0x0C010C00u) & vmask, __builtin_amdgcn_perm(0u, by.x, 0x0C030C02u) & vmask,
-                               __builtin_amdgcn_perm(0u, by.y, 0x0C010C00u) & vmask, __builtin_amdgcn_perm(0u, by.y, 0x0C030C02u) & vmask};
+        const u32x4 ao = u32x4{by.x & vmask, by.y & vmask, by.z & vmask, by.w & vmask};
         accv[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, ao), __builtin_bit_cast(half8, bo), accv[j], 0, 0, 0);
       }
     }
@@ -369,6 +373,10 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     float lt = l_run + __shfl_xor(l_run, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (lane < G) { S.mw[wv][lane] = m_run; S.lw[wv][lane] = lt; }
+    if (sn < 12 && kc < 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) S.ams[wv][4 * kc + r][sn] = amd[r];
+    }
   }
   __syncthreads();          // every wavefront is done with its strips: the merged accumulators take their place
   float fac;
@@ -382,7 +390,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       float* orow = &S.ob[l32 >> 3][vh][0];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float mj = am[j] + __shfl_xor(am[j], 32, 64);
+        const float mj = S.ams[wv][vh][4 * (l32 >> 3) + j];
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
           float4* dst = reinterpret_cast<float4*>(orow + 32 * j + 8 * i4 + 4 * hh);      // row = 8 (i >> 2) + 4 hh + (i & 3)
