@@ -47,6 +47,7 @@ template <class T> DEVI T gload(const uint8_t* p) {
 constexpr int CHUNK = 1552, KM_OFF = 512, VC_OFF = 768, VM_OFF = 1280, VF_OFF = 1536;
 constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
 constexpr int QROW = 68;                        // words per row of the query strips: 64 + 4 pad (conflict-free 128-bit rows)
+constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad
 constexpr int OROW = 132;                       // floats per row of the merged accumulators: 128 + 4 pad
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -56,10 +57,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 struct Scr {                                    // per wavefront, rewritten for every 32-token group
   alignas(16) uint32_t qs[GT][QROW];            // fp16 pairs of q' * scale * 2^-shift per (head, channel pair)
   alignas(16) uint32_t qm[GT][QROW];            // fp16 pairs of q' * min
-  alignas(16) _Float16 pst[GT][32];             // p per (head, token)
-  alignas(16) uint16_t vsm[3][4][32];           // value scale (fp16 bits) per (class, sub-vector, token), 0 off its class
-  alignas(16) uint16_t vmm[3][4][32];           // value min likewise
-  alignas(16) uint16_t vt[4][8][32];            // value code bytes (zero-extended) per (sub-vector, byte, token)
+  // rows and blocks padded so that the 128-bit rows one instruction reads fall into different banks
+  alignas(16) _Float16 pst[GT][PROW];           // p per (head, token)
+  alignas(16) uint16_t vsm[3][4 * 32 + 8];      // value scale (fp16 bits) per (class, sub-vector * 32 + token), 0 off its class
+  alignas(16) uint16_t vmm[3][4 * 32 + 8];      // value min likewise
+  alignas(16) uint16_t vt[4][8 * PROW + 16];    // value code bytes (zero-extended) per (sub-vector, byte * PROW + token)
 };
 struct Smem {
   uint32_t qh[3][GT][64];                       // query rotations as fp16 pairs per (variant, head, channel pair)
@@ -259,15 +261,18 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
         if (!full) cls = (pos >= t0 && pos < t1) ? cls : 3;
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
-          W.vsm[c][j][l32] = cls == c ? static_cast<uint16_t>(w & 0x7FFFu) : static_cast<uint16_t>(0);
-          W.vmm[c][j][l32] = cls == c ? static_cast<uint16_t>(w >> 16) : static_cast<uint16_t>(0);
+          W.vsm[c][32 * j + l32] = cls == c ? static_cast<uint16_t>(w & 0x7FFFu) : static_cast<uint16_t>(0);
+          W.vmm[c][32 * j + l32] = cls == c ? static_cast<uint16_t>(w >> 16) : static_cast<uint16_t>(0);
         }
         const uint32_t c0 = jj ? cur.vc.z : cur.vc.x, c1 = jj ? cur.vc.w : cur.vc.y;
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-          W.vt[j][bb][l32] = static_cast<uint16_t>((c0 >> (8 * bb)) & 0xFFu);
-          W.vt[j][4 + bb][l32] = static_cast<uint16_t>((c1 >> (8 * bb)) & 0xFFu);
-        }
+        // bytes 0, 1 and 2, 3 of a word side by side in the two halves of one register: one permute per pair
+        const uint32_t c01 = __builtin_amdgcn_perm(0u, c0, 0x0C010C00u), c23 = __builtin_amdgcn_perm(0u, c0, 0x0C030C02u);
+        const uint32_t c45 = __builtin_amdgcn_perm(0u, c1, 0x0C010C00u), c67 = __builtin_amdgcn_perm(0u, c1, 0x0C030C02u);
+        uint16_t* vt = &W.vt[j][l32];
+        vt[0 * PROW] = static_cast<uint16_t>(c01); vt[1 * PROW] = static_cast<uint16_t>(c01 >> 16);
+        vt[2 * PROW] = static_cast<uint16_t>(c23); vt[3 * PROW] = static_cast<uint16_t>(c23 >> 16);
+        vt[4 * PROW] = static_cast<uint16_t>(c45); vt[5 * PROW] = static_cast<uint16_t>(c45 >> 16);
+        vt[6 * PROW] = static_cast<uint16_t>(c67); vt[7 * PROW] = static_cast<uint16_t>(c67 >> 16);
       }
     }
     wave_lds_sync();
@@ -302,10 +307,10 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     }
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
     {
-      float sc[8];
+      float sc[8];                       // raw accumulators: score = sc * 2^24 * qscale (a positive factor)
       const float up = 16777216.f * qscale;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sc[i] = (i < 4 ? sa0[i & 3] : sa1[i & 3]) * up;
+      for (int i = 0; i < 8; ++i) sc[i] = i < 4 ? sa0[i & 3] : sa1[i & 3];
       if (!full) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -313,7 +318,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
           sc[i] = (pos >= t0 && pos < t1) ? sc[i] : -INFINITY;
         }
       }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))) * up;
       if (__any(mx > m_run)) {
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -334,7 +339,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       float p[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        p[i] = fexp2(sc[i] - m_run);
+        p[i] = fexp2(__builtin_fmaf(sc[i], up, -m_run));
         l_run += p[i];
       }
       if (sn < 8) {
@@ -348,7 +353,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     //      masked in place.  sum p * min per (class, head, sub-vector) by v_dot2.
     {   // sum p * min: rows = heads, columns = (class, sub-vector), the 32 tokens in one step
       const u32x4 pa = *reinterpret_cast<const u32x4*>(&W.pst[sh][8 * kc]);
-      const u32x4 mb = *reinterpret_cast<const u32x4*>(&W.vmm[min(sn >> 2, 2)][sn & 3][8 * kc]);
+      const u32x4 mb = *reinterpret_cast<const u32x4*>(&W.vmm[min(sn >> 2, 2)][32 * (sn & 3) + 8 * kc]);
       amd = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, pa), __builtin_bit_cast(half8, mb), amd, 0, 0, 0);
     }
 #pragma unroll
@@ -357,8 +362,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       const u32x4 pr = *reinterpret_cast<const u32x4*>(&W.pst[vh][tk]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const u32x4 sv = *reinterpret_cast<const u32x4*>(&W.vsm[vcl][j][tk]);
-        const u32x4 by = *reinterpret_cast<const u32x4*>(&W.vt[j][l32 >> 2][tk]);     // (token 2 i | token 2 i + 1 << 16) per word
+        const u32x4 sv = *reinterpret_cast<const u32x4*>(&W.vsm[vcl][32 * j + tk]);
+        const u32x4 by = *reinterpret_cast<const u32x4*>(&W.vt[j][(l32 >> 2) * PROW + tk]);     // (token 2 i | token 2 i + 1 << 16) per word
         const u32x4 bo = u32x4{pk_mul(pr.x, sv.x), pk_mul(pr.y, sv.y), pk_mul(pr.z, sv.z), pk_mul(pr.w, sv.w)};
         const u32x4 ao = u32x4{by.x & vmask, by.y & vmask, by.z & vmask, by.w & vmask};
         accv[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, ao), __builtin_bit_cast(half8, bo), accv[j], 0, 0, 0);
