@@ -1,22 +1,23 @@
-// Paged split-K decode attention over KIVI-style FlagRot INT2 pages for gfx950 (wave64, no matrix cores): the page
-// splits and the BF16 ring rows (one more split).  (The split merge and the C ABI live in kivi_attn.hip.)
+// Paged split-K decode attention over KIVI-style FlagRot INT2 pages for gfx950 (wave64, matrix pipe for both products):
+// the page splits and the BF16 ring rows (one more split).  (The split merge and the C ABI live in kivi_attn.hip.)
 //
-// Workgroup = 4 wavefronts per (sequence, KV head x tile of up to 4 query heads, split); a wavefront owns whole
-// 32-token groups (two pages) and keeps its own running maximum, sum and accumulators; the wavefronts are merged
-// through LDS at the end.  (Tiles of 4 heads keep the three accumulator classes in registers at 3 waves per SIMD; a
-// GQA group of 8 reads its pages twice, which the path can afford: it is instruction bound, not bandwidth bound.)
-// Per group:
-//   q' * scale   lane = channel pair: the group's channel scales are folded into the query rotation the group's flags
-//                select (identity / H32 per sub-vector / H128; the three rotations are made once per workgroup), stored
-//                as fp16 pairs; q' . min becomes a per-head bias.
-//   scores       lane = (token, 64-channel half): a 2-bit code field masked in place is an fp16 DENORMAL whose value is
-//                code * 2^(shift - 24); the power of two is folded into the fp16 query operand, so a pair of codes costs
-//                one v_and and feeds v_dot2_f32_f16 directly (exact products, fp32 accumulation).
-//   softmax      exp2-domain, the running maximum is re-reduced only when some token beats it.
-//   values       tokens of a (group, sub-vector) are ordered by class (stored as is / H32 / H128) with ballots; p * scale,
-//                p * min (fp16) and the token's 8 code bytes are written in that order, so that lane = 4 channels walks
-//                PAIRS of tokens of one class: the two code bytes are merged and masked into four denormal pairs,
-//                contracted with v_dot2 into the accumulators of that class.  o = accI + H32(accH) + H128(accF) once per workgroup.
+// Workgroup = 4 wavefronts per (sequence, KV head with its whole GQA group of up to 8 query heads, split); a wavefront
+// owns whole 32-token groups (two pages) and keeps its own running maxima, sums and accumulators; the wavefronts are
+// merged through LDS at the end.  Per group:
+//   q' * scale   lane = channel pair: the group's channel scales (and mins) times the query rotation the group's flags
+//                select (identity / H32 per sub-vector / H128; the three rotations are made once per workgroup and
+//                kept as fp16 pairs), packed fp16 products written to LDS strips.
+//   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads, 128 channels in four steps:
+//                a 2-bit code field masked in place is an fp16 DENORMAL whose value is code * 2^(shift - 24) (the
+//                matrix pipe keeps denormal inputs); the power of two is folded into the query operand.  The bias
+//                sum q' * min enters through the same accumulators (A = 2^-24 in every slot, B = q' * min).
+//   softmax      exp2-domain, lane = (head, 8 tokens); the running maximum is re-reduced only when some token beats it.
+//   values       v_mfma_f32_32x32x16_f16, rows = the 32 channels of a sub-vector, columns = (class, head) with class =
+//                stored as is / H32 / H128, 32 tokens in two steps.  B = p * scale of the token if it belongs to the
+//                column's class, else 0 (class-masked scale strips written by the token lanes); A = the tokens' code
+//                bytes (transposed through LDS as zero-extended 16-bit values, so a 128-bit read is four token pairs)
+//                masked in place to the row's 2-bit field.  sum p * min per (head, class, sub-vector): one more
+//                16x16x32 product.  o = accI + H32(accH) + H128(accF) once per workgroup.
 // Semantics follow integrations/vllm_flagrot/csrc/kivi.cu:729-980 (k_attn).
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
