@@ -9,6 +9,8 @@
 // Mapping: one half wave (32 lanes) owns one 128-d row, 4 consecutive dims per lane.  The selecting writer keeps the
 // head's 64 KB C_q^T in LDS for the whole workgroup and walks its tokens eight rows at a time; the error vectors of
 // the candidates live in a small per-half-wave LDS strip so that the fixed-order matvec reads them as broadcasts.
+#include <cstdlib>
+
 #include "fr_common.hpp"
 #include "fr_launch.hpp"
 
@@ -269,6 +271,159 @@ __global__ void __launch_bounds__(256) k_k2_write(const K2WriteParams p, int tok
   }
 }
 
+
+// Low-latency form of k_k2_write for a handful of tokens (a decode step): four half waves per (token, head) instead of
+// one, two tokens per workgroup.  Every half wave repeats the cheap part (quantised candidates, transforms); the
+// weighted error sums are shared out without touching the order of any sum: in the local pass half wave r carries the
+// chains of output 4 l + r, in the whole-head pass half wave b carries the block sums of block b, and the block sums are
+// added in block order as in k_k2_write.  Results are bit-identical to k_k2_write.
+constexpr int K2LL_LDS = K2_LDS_C + 2 * (2 * 128 + 4 * 2 * 32 + 4 * 8 * 32) * 4;
+template <int QM, int P>
+__global__ void __launch_bounds__(256) k_k2_write_ll(const K2WriteParams p) {
+  using L = Lay<QM, P>;
+  extern __shared__ __align__(16) uint8_t lds[];
+  float* Cs = reinterpret_cast<float*>(lds);                   // [k][i] = C_q[i][k]
+  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31, role = hw & 3, ts = hw >> 2;
+  float* es = reinterpret_cast<float*>(lds + K2_LDS_C) + ts * (2 * 128 + 4 * 2 * 32 + 4 * 8 * 32);  // [2][128]
+  float* xs = es + 2 * 128;                                    // [role][candidate][lane]: local sums of output 4 l + role
+  float* ys = xs + 4 * 2 * 32;                                 // [block][8][lane]: block sums ub[4], uf[4]
+  const int h = blockIdx.x;
+  const int t = blockIdx.y * 2 + ts;
+  const bool do_k = p.passes & 1, do_v = p.passes & 2;
+  if (do_k) {
+    const float4* src = reinterpret_cast<const float4*>(p.CT + static_cast<size_t>(h) * 128 * 128);
+    float4* dst = reinterpret_cast<float4*>(Cs);
+    for (int i = threadIdx.x; i < 128 * 128 / 4; i += 256) dst[i] = src[i];
+  }
+  __syncthreads();
+  const int g = l32 >> 3;
+  long long slot = -1;
+  if (t < p.T) slot = p.slots[static_cast<long long>(t) * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
+  const bool live = slot >= 0;                                 // the barriers below are passed by every thread
+  uint8_t* chunk = p.pool + ((live ? slot / P : 0) * p.Hkv + h) * L::CHUNK;
+  const int pos = live ? static_cast<int>(slot % P) : 0;
+  bool key_full = false;
+  if (do_k) {
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+      load_row(p.kv, static_cast<long long>(t) * p.kv_ts + h * 128 + 4 * l32, x);
+      if (p.kmu != nullptr) {
+        const float4 m = *reinterpret_cast<const float4*>(p.kmu + h * 128 + 4 * l32);
+        x[0] = x[0] - m.x; x[1] = x[1] - m.y; x[2] = x[2] - m.z; x[3] = x[3] - m.w;
+      }
+    }
+    // ---- local candidates: identity and H32 of every 32-group
+    float qi[4], ei[4], qh[4], eh[4], y[4];
+    const uint32_t wi = quant_group<QM, true>(x, qi, ei);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { ei[i] = ei[i] - x[i]; y[i] = x[i]; }
+    fwht<32>(y, l32);
+    const uint32_t wh = quant_group<QM, true>(y, qh, eh);
+    fwht<32>(eh, l32);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) eh[i] = eh[i] - x[i];
+    if (role == 0) {
+      *reinterpret_cast<float4*>(es + 4 * l32) = make_float4(ei[0], ei[1], ei[2], ei[3]);
+      *reinterpret_cast<float4*>(es + 128 + 4 * l32) = make_float4(eh[0], eh[1], eh[2], eh[3]);
+    }
+    __syncthreads();
+    {
+      float ui = 0.f, uh = 0.f;
+      const float* crow = Cs + (32 * g) * 128 + 4 * l32 + role;   // C[4 l + role][32 g + k] at crow[k * 128]
+      const float* e0 = es + 32 * g;
+#pragma unroll 8
+      for (int k = 0; k < 32; ++k) {
+        const float c = crow[k * 128];
+        const float pa = c * e0[k], pb = c * e0[128 + k];
+        ui = k == 0 ? pa : ui + pa;
+        uh = k == 0 ? pb : uh + pb;
+      }
+      xs[(role * 2 + 0) * 32 + l32] = ui;
+      xs[(role * 2 + 1) * 32 + l32] = uh;
+    }
+    __syncthreads();
+    float pi[4], ph[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { pi[i] = ei[i] * xs[(i * 2 + 0) * 32 + l32]; ph[i] = eh[i] * xs[(i * 2 + 1) * 32 + l32]; }
+    const bool use_h = tree32(ph) < tree32(pi);   // strict: ties keep the identity
+    float qb[4], eb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { qb[i] = use_h ? qh[i] : qi[i]; eb[i] = use_h ? eh[i] : ei[i]; }
+    const uint32_t wb = use_h ? wh : wi;
+    // ---- whole-head candidate
+    float qf[4], ef[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) y[i] = x[i];
+    fwht<128>(y, l32);
+    const uint32_t wf = quant_group<QM, true>(y, qf, ef);
+    fwht<128>(ef, l32);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ef[i] = ef[i] - x[i];
+    if (role == 0) {      // every half wave has read the local strips (second barrier above)
+      *reinterpret_cast<float4*>(es + 4 * l32) = make_float4(eb[0], eb[1], eb[2], eb[3]);
+      *reinterpret_cast<float4*>(es + 128 + 4 * l32) = make_float4(ef[0], ef[1], ef[2], ef[3]);
+    }
+    __syncthreads();
+    {
+      float ub[4], uf[4];
+      const int b = role;
+      const float* crow = Cs + (32 * b) * 128 + 4 * l32;
+      const float* e0 = es + 32 * b;
+#pragma unroll 4
+      for (int k = 0; k < 32; ++k) {
+        const float4 cv = *reinterpret_cast<const float4*>(crow + k * 128);
+        const float a = e0[k], f = e0[128 + k];
+        const float c[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pa = c[i] * a, pf = c[i] * f;
+          ub[i] = k == 0 ? pa : ub[i] + pa;
+          uf[i] = k == 0 ? pf : uf[i] + pf;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { ys[(b * 8 + i) * 32 + l32] = ub[i]; ys[(b * 8 + 4 + i) * 32 + l32] = uf[i]; }
+    }
+    __syncthreads();
+    float tb[4], tf[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float ub = ys[(b * 8 + i) * 32 + l32], uf = ys[(b * 8 + 4 + i) * 32 + l32];
+        tb[i] = b == 0 ? ub : tb[i] + ub;
+        tf[i] = b == 0 ? uf : tf[i] + uf;
+      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { tb[i] = eb[i] * tb[i]; tf[i] = ef[i] * tf[i]; }
+    key_full = tree128(tf) < tree128(tb);
+    if (live && role == 0) {
+      uint32_t code[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) code[i] = code_bits(key_full ? qf[i] : qb[i], QM == QM_SYM4);
+      uint32_t word = key_full ? wf : wb;
+      if (!key_full && use_h) word |= 0x8000u;
+      store_row<QM, P>(chunk, pos, false, code, word, l32, false);
+      if (!do_v && l32 == 0) {  // key-only pass: own bit 15 of the token's group-0 V scale word
+        const int off = L::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2;
+        uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + (off & ~3));
+        const uint32_t bit = 0x8000u << ((off & 2) * 8);
+        if (key_full) atomicOr(wp, bit); else atomicAnd(wp, ~bit);
+      }
+    }
+  }
+  if (do_v && live && role == 1) {
+    float x[4], q[4], deq[4];
+    load_row(p.kv, static_cast<long long>(t) * p.kv_ts + (p.Hkv + h) * 128 + 4 * l32, x);
+    uint32_t word = quant_group<QM, false>(x, q, deq);
+    if (do_k && g == 0 && key_full) word |= 0x8000u;
+    uint32_t code[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) code[i] = code_bits(q[i], QM == QM_SYM4);
+    store_row<QM, P>(chunk, pos, true, code, word, l32, !do_k);
+  }
+}
+
 template <int QM>
 int static_write_qm(const StaticWriteParams& p, hipStream_t st) {
   const long long rows = static_cast<long long>(p.T) * 2 * p.Hkv;
@@ -283,13 +438,21 @@ int static_write_qm(const StaticWriteParams& p, hipStream_t st) {
 template <int QM, int P>
 int k2_write_p(const K2WriteParams& p, hipStream_t st) {
   auto k = k_k2_write<QM, P>;
+  auto kll = k_k2_write_ll<QM, P>;
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, K2_LDS) != hipSuccess) {
-      set_error("selecting writer: cannot reserve 72 KB of LDS");
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, K2_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kll), hipFuncAttributeMaxDynamicSharedMemorySize, K2LL_LDS) != hipSuccess) {
+      set_error("selecting writer: cannot reserve 76 KB of LDS");
       return -2;
     }
     attr = true;
+  }
+  // a decode step's worth of tokens: four half waves per (token, head), at most two workgroups per CU in one round
+  static const bool no_ll = getenv("FLAGROT_WRITER_LL") != nullptr && getenv("FLAGROT_WRITER_LL")[0] == '0';
+  if (!no_ll && static_cast<long long>(p.T) * p.Hkv <= 1024) {
+    hipLaunchKernelGGL(kll, dim3(p.Hkv, (p.T + 1) / 2), dim3(256), K2LL_LDS, st, p);
+    return hipPeekAtLastError() == hipSuccess ? 0 : -1;
   }
   // tokens per workgroup: enough workgroups to fill 256 CUs twice, at least one round of 8 rows each
   int tpw = K2_ROWS;
