@@ -62,8 +62,9 @@ def test_static_writer_bytes(dev, fmt, T):
 
 
 @pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
-@pytest.mark.parametrize("T", [1, 5, 64, 333])
+@pytest.mark.parametrize("T", [1, 5, 64, 333, 700])
 def test_selecting_writer_bytes(dev, kind, T):
+    """T * Hkv <= 1024 runs the low-latency kernel (four half waves per token and head), T = 700 the one-half-wave kernel"""
     from flagrot_releaser_amd import kernels as K
     g = torch.Generator().manual_seed(2000 + T)
     Hkv = 2
