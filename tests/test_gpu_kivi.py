@@ -253,6 +253,12 @@ CASES = [
     ([700], 1, 5, 0, (3, 256), [0]),
     ([2048, 1500], 8, 4, 32, None, [40, 128]),
     ([40, 40], 2, 2, 64, (1, 256), [3, 0]),       # nothing left in the pages: tail only (and one empty sequence)
+    # ragged ends inside a 32-token group, kv_start inside a group, group sizes that leave matrix columns idle
+    ([333, 97, 1], 2, 3, 37, (2, 256), [2, 0, 9]),
+    ([1500, 31], 1, 6, 5, (5, 320), [0, 128]),
+    ([777], 4, 7, 255, (3, 288), [64]),
+    ([2049, 2047], 2, 8, 1, None, [1, 127]),
+    ([65, 64, 63], 3, 1, 33, (1, 256), [0, 0, 0]),
 ]
 
 
