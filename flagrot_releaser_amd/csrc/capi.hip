@@ -146,6 +146,7 @@ int fr_cb_write3(const void* kv, long long kv_ts, const long long* slots, int sl
   p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.slot_ph = slot_ph; p.T = T; p.Hkv = Hkv; p.page = page;
   p.CT = CT; p.kmu = kmu; p.pool = pool;
   p.passes = (nchunk >= 0 ? 1 : 0) | (nchunk_v >= 0 ? 2 : 0);
+  p.screen = 1;
   if (p.passes == 0) return 0;
   return launched(k2_write_launch(kind, p, static_cast<hipStream_t>(stream)), "fr_cb_write3");
 }

@@ -197,6 +197,77 @@ DEVI void place4(uint32_t c, bool isB, int i, uint32_t& mask, uint32_t& bits) {
   }
 }
 
+// V^T fields of one token by 32-bit atomics (tokens of a page may arrive from different waves): the lane's 4 codes
+template <int QM, int P>
+DEVI void store_v_codes(uint8_t* chunk, int pos, const uint32_t (&code)[4], int l32) {
+  using L = Lay<QM, P>;
+  const int c8 = pos >> 3, ii = (pos & 7) >> 1;
+  const bool isB = pos & 1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int dd = 4 * l32 + i;
+    const int e = ((dd & 63) >> 4) * 8 + (dd & 7);
+    if constexpr (QM == QM_ASYM2) {
+      uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 8 + 4 * (dd >> 6));
+      const int sh = 8 * ii + 4 * ((dd & 15) >> 3) + 2 * (isB ? 1 : 0);
+      atomicAnd(wp, ~(3u << sh));
+      atomicOr(wp, code[i] << sh);
+    } else {
+      const int sub = 2 * (dd >> 6) + ((dd & 15) >> 3);
+      uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 16 + 4 * sub);
+      uint32_t m, b;
+      place4<QM>(code[i], isB, ii, m, b);
+      atomicAnd(wp, ~m);
+      atomicOr(wp, b);
+    }
+  }
+}
+// the V scale word of the lane's group (lanes 0, 8, 16, 24 of the half wave store)
+template <int QM, int P>
+DEVI void store_v_word(uint8_t* chunk, int pos, uint32_t word, int l32, bool keep_flag) {
+  using L = Lay<QM, P>;
+  const int g = l32 >> 3, c8 = pos >> 3;
+  if ((l32 & 7) == 0) {
+    const int off = L::VS_OFF + (g * P + 8 * c8 + vs_slot8(pos)) * 2;
+    if (keep_flag && g == 0) {  // the low 15 bits only; bit 15 belongs to the key pass
+      uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + (off & ~3));
+      const int sh = (off & 2) * 8;
+      atomicAnd(wp, ~(0x7FFFu << sh));
+      atomicOr(wp, (word & 0x7FFFu) << sh);
+    } else {
+      *reinterpret_cast<uint16_t*>(chunk + off) = static_cast<uint16_t>(word);
+    }
+  }
+}
+// One V^T word of an aligned run of 8 tokens (slots 8 c8 .. 8 c8 + 7 of one page), whole: word j of the run is
+// (entry e = j >> 2, sub = j & 3) for the 4-bit formats, (entry e = j >> 1, half m = j & 1) for the 2-bit format;
+// codes[token of the run][dim].
+template <int QM, int P>
+DEVI void store_v_run_word(uint8_t* chunk, int c8, int j, const uint8_t (*codes)[128]) {
+  using L = Lay<QM, P>;
+  if constexpr (QM == QM_ASYM2) {
+    const int e = j >> 1, m = j & 1;
+    uint32_t wd = 0;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int dd = 64 * m + 16 * (e >> 3) + 8 * r + (e & 7);
+#pragma unroll
+      for (int tk = 0; tk < 8; ++tk) wd |= static_cast<uint32_t>(codes[tk][dd]) << (8 * (tk >> 1) + 4 * r + 2 * (tk & 1));
+    }
+    *reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 8 + 4 * m) = wd;
+  } else {
+    const int e = j >> 2, sub = j & 3;
+    const int dd = 64 * (sub >> 1) + 16 * (e >> 3) + 8 * (sub & 1) + (e & 7);
+    uint32_t wd = 0;
+#pragma unroll
+    for (int tk = 0; tk < 8; ++tk) {
+      uint32_t m, b;
+      place4<QM>(codes[tk][dd], (tk & 1) != 0, tk >> 1, m, b);
+      wd |= b;
+    }
+    *reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 16 + 4 * sub) = wd;
+  }
+}
 // Writes one row (K or V) of one token: the lane's 4 codes (d = 4 * l32 + i) and its group's scale word.
 // K rows are stored as whole words; V^T fields with 32-bit atomics (tokens of a page arrive from different waves).
 // VW: 0 plain 16-bit store of the V scale word, 1 keep bit 15 of V word 0 (a concurrent key pass owns it).
@@ -230,37 +301,8 @@ DEVI void store_row(uint8_t* chunk, int pos, bool isv, const uint32_t (&code)[4]
     }
     if ((l32 & 7) == 0) *reinterpret_cast<uint16_t*>(chunk + L::KS_OFF + 8 * pos + 2 * g) = static_cast<uint16_t>(word);
   } else {
-    const int c8 = pos >> 3, ii = (pos & 7) >> 1;
-    const bool isB = pos & 1;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int dd = 4 * l32 + i;
-      const int e = ((dd & 63) >> 4) * 8 + (dd & 7);
-      if constexpr (QM == QM_ASYM2) {
-        uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 8 + 4 * (dd >> 6));
-        const int sh = 8 * ii + 4 * ((dd & 15) >> 3) + 2 * (isB ? 1 : 0);
-        atomicAnd(wp, ~(3u << sh));
-        atomicOr(wp, code[i] << sh);
-      } else {
-        const int sub = 2 * (dd >> 6) + ((dd & 15) >> 3);
-        uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + L::V_OFF + (e * (P / 8) + c8) * 16 + 4 * sub);
-        uint32_t m, b;
-        place4<QM>(code[i], isB, ii, m, b);
-        atomicAnd(wp, ~m);
-        atomicOr(wp, b);
-      }
-    }
-    if ((l32 & 7) == 0) {
-      const int off = L::VS_OFF + (g * P + 8 * c8 + vs_slot8(pos)) * 2;
-      if (keep_flag && g == 0) {  // the low 15 bits only; bit 15 belongs to the key pass
-        uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + (off & ~3));
-        const int sh = (off & 2) * 8;
-        atomicAnd(wp, ~(0x7FFFu << sh));
-        atomicOr(wp, (word & 0x7FFFu) << sh);
-      } else {
-        *reinterpret_cast<uint16_t*>(chunk + off) = static_cast<uint16_t>(word);
-      }
-    }
+    store_v_codes<QM, P>(chunk, pos, code, l32);
+    store_v_word<QM, P>(chunk, pos, word, l32, keep_flag);
   }
 }
 

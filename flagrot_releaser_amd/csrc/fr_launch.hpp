@@ -27,6 +27,7 @@ struct K2WriteParams {
   const float* kmu;
   uint8_t* pool;
   int passes;              // bit 0: key rows, bit 1: value rows
+  int screen;              // 1: large key passes may run the screened kernel (same bytes; fr_cb_write3)
 };
 int k2_write_launch(int kind, const K2WriteParams& p, hipStream_t st);
 int k2_write_lds_bytes();

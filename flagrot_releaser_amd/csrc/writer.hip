@@ -153,13 +153,17 @@ __global__ void __launch_bounds__(256) k_k2_write(const K2WriteParams p, int tok
   }
   __syncthreads();
   const int g = l32 >> 3;
-  for (int t = t_lo + hw; t < t_hi; t += K2_ROWS) {
-    const long long slot = p.slots[static_cast<long long>(t) * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
-    if (slot < 0) continue;
-    uint8_t* chunk = p.pool + ((slot / P) * p.Hkv + h) * L::CHUNK;
-    const int pos = static_cast<int>(slot % P);
+  __shared__ long long vslot[K2_ROWS];
+  __shared__ __align__(16) uint8_t vcodes[K2_ROWS][128];
+  for (int tb = t_lo; tb < t_hi; tb += K2_ROWS) {      // one token per half wave; the trip count is the workgroup's
+    const int t = tb + hw;
+    long long slot = -1;
+    if (t < t_hi) slot = p.slots[static_cast<long long>(t) * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
+    const bool live = slot >= 0;
+    uint8_t* chunk = p.pool + ((live ? slot / P : 0) * p.Hkv + h) * L::CHUNK;
+    const int pos = live ? static_cast<int>(slot % P) : 0;
     bool key_full = false;
-    if (do_k) {
+    if (do_k && live) {
       float x[4];
       load_row(p.kv, static_cast<long long>(t) * p.kv_ts + h * 128 + 4 * l32, x);
       if (p.kmu != nullptr) {
@@ -259,14 +263,33 @@ __global__ void __launch_bounds__(256) k_k2_write(const K2WriteParams p, int tok
       }
     }
     if (do_v) {
-      float x[4], q[4], deq[4];
-      load_row(p.kv, static_cast<long long>(t) * p.kv_ts + (p.Hkv + h) * 128 + 4 * l32, x);
-      uint32_t word = quant_group<QM, false>(x, q, deq);
-      if (do_k && g == 0 && key_full) word |= 0x8000u;
-      uint32_t code[4];
+      // Value rows.  The eight tokens of the step usually fill one aligned run of 8 slots of a page: their V^T words
+      // are then assembled in LDS and stored whole; otherwise field by field with atomics.
+      uint32_t code[4] = {0u, 0u, 0u, 0u};
+      if (live) {
+        float x[4], q[4], deq[4];
+        load_row(p.kv, static_cast<long long>(t) * p.kv_ts + (p.Hkv + h) * 128 + 4 * l32, x);
+        uint32_t word = quant_group<QM, false>(x, q, deq);
+        if (do_k && g == 0 && key_full) word |= 0x8000u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) code[i] = code_bits(q[i], QM == QM_SYM4);
-      store_row<QM, P>(chunk, pos, true, code, word, l32, !do_k);
+        for (int i = 0; i < 4; ++i) code[i] = code_bits(q[i], QM == QM_SYM4);
+        store_v_word<QM, P>(chunk, pos, word, l32, !do_k);
+      }
+      if (l32 == 0) vslot[hw] = slot;
+      *reinterpret_cast<uint32_t*>(&vcodes[hw][4 * l32]) = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+      __syncthreads();
+      const long long s0 = vslot[0];
+      bool run = s0 >= 0 && (s0 & 7) == 0;
+#pragma unroll
+      for (int i = 1; i < K2_ROWS; ++i) run = run && vslot[i] == s0 + i;
+      if (run) {
+        constexpr int NWORD = QM == QM_ASYM2 ? 64 : 128;
+        uint8_t* c0 = p.pool + ((s0 / P) * p.Hkv + h) * L::CHUNK;
+        if (threadIdx.x < NWORD) store_v_run_word<QM, P>(c0, static_cast<int>(s0 % P) >> 3, threadIdx.x, vcodes);
+      } else if (live) {
+        store_v_codes<QM, P>(chunk, pos, code, l32);
+      }
+      __syncthreads();
     }
   }
 }
@@ -424,6 +447,437 @@ __global__ void __launch_bounds__(256) k_k2_write_ll(const K2WriteParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------ screened selecting writer
+// Same bytes as k_k2_write at a fraction of its vector instructions: the quadratic forms d^T C d of the candidates'
+// error vectors are ESTIMATED on the matrix pipe (v_mfma_f32_32x32x2f32, fp32 operands) and a choice is taken from the
+// estimates only where it cannot differ from the choice of the exactly ordered fp32 evaluation; every other token is
+// evaluated exactly, in the reference's order, at the end of the workgroup.
+//   Bound: with S = |d|^T |C| |d|, the reference's value (sums of <= 35 terms, one product, a tree of depth 7) lies
+//   within 44 u S of the true form (u = 2^-24), the estimate (at most 128 products and sums inside the matrix pipe,
+//   each taken as accurate to 2 u whatever its order and rounding mode, a 16-term dot, 6 more sums) within 300 u S;
+//   S <= rho |d|^2 with rho = max(largest row sum, largest column sum of |C|), computed by the workgroup itself.  The
+//   screen uses b = 2^-15 rho |d|^2 (1.5 x the sum of the two) + 2^-100: candidate a beats candidate b for certain when
+//   e~_a + b_a < e~_b - b_b.
+// Workgroup = (KV head, tile of tokens), four wavefronts; wavefront w keeps rows 32 w .. 32 w + 31 of C in registers as
+// matrix A operands (the whole row for the whole-head forms, its diagonal 32-block for the local forms).  A step takes
+// 16 tokens, two per half wave: candidates in registers exactly as in k_k2_write, error vectors as the 32 columns of a
+// matrix in LDS, forms by MFMA, choices back through LDS.
+constexpr int W3_TOK = 16;                   // tokens per step
+constexpr int W3_DROW = 132;                 // floats per column of the error matrix in LDS: 128 + 4 pad
+constexpr int W3_MAXTILE = 128;              // tokens per workgroup at most (fallback list)
+constexpr float W3_KAPPA = 3.0517578125e-05f;   // 2^-15
+
+struct W3Smem {
+  float dm[2 * W3_TOK][W3_DROW];             // column 2 t + c: error vector of candidate c of token t of the step
+  float part[2][4][2 * W3_TOK];              // [form | squared norm][row tile = wavefront][column]
+  float colsum[128];
+  float rinf[4];                             // largest row sum of |C| per row tile
+  float es[8][256];                          // strips of the exact evaluation (per half wave)
+  int fb[W3_MAXTILE];                        // tokens left to the exact evaluation
+  int nfb;
+  uint8_t choice[W3_TOK][4];                 // per (token, 32-group): 0 identity, 1 H32, 2 undecided
+  long long vslot[W3_TOK];
+  alignas(16) uint8_t vcodes[W3_TOK][128];   // value codes of the step's tokens
+};
+
+// the exact choice of one token, half wave: k_k2_write's evaluation with C^T read through `C` (LDS or memory)
+template <int QM>
+DEVI void k2_exact_choice(const float (&x)[4], const float* C, float* es, int l32, float (&qsel)[4], uint32_t& word, bool& key_full) {
+  const int g = l32 >> 3;
+  float qi[4], ei[4], qh[4], eh[4], y[4];
+  const uint32_t wi = quant_group<QM, true>(x, qi, ei);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { ei[i] = ei[i] - x[i]; y[i] = x[i]; }
+  fwht<32>(y, l32);
+  const uint32_t wh = quant_group<QM, true>(y, qh, eh);
+  fwht<32>(eh, l32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) eh[i] = eh[i] - x[i];
+  wave_lds_sync();
+  *reinterpret_cast<float4*>(es + 4 * l32) = make_float4(ei[0], ei[1], ei[2], ei[3]);
+  *reinterpret_cast<float4*>(es + 128 + 4 * l32) = make_float4(eh[0], eh[1], eh[2], eh[3]);
+  wave_lds_sync();
+  float ui[4], uh[4];
+  {
+    const float* crow = C + (32 * g) * 128 + 4 * l32;
+    const float* e0 = es + 32 * g;
+#pragma unroll 4
+    for (int k = 0; k < 32; ++k) {
+      const float4 cv = *reinterpret_cast<const float4*>(crow + k * 128);
+      const float a = e0[k], b = e0[128 + k];
+      const float c[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pa = c[i] * a, pb = c[i] * b;
+        ui[i] = k == 0 ? pa : ui[i] + pa;
+        uh[i] = k == 0 ? pb : uh[i] + pb;
+      }
+    }
+  }
+  float pi[4], ph[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { pi[i] = ei[i] * ui[i]; ph[i] = eh[i] * uh[i]; }
+  const bool use_h = tree32(ph) < tree32(pi);
+  float qb[4], eb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { qb[i] = use_h ? qh[i] : qi[i]; eb[i] = use_h ? eh[i] : ei[i]; }
+  const uint32_t wb = use_h ? wh : wi;
+  float qf[4], ef[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) y[i] = x[i];
+  fwht<128>(y, l32);
+  const uint32_t wf = quant_group<QM, true>(y, qf, ef);
+  fwht<128>(ef, l32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ef[i] = ef[i] - x[i];
+  wave_lds_sync();
+  *reinterpret_cast<float4*>(es + 4 * l32) = make_float4(eb[0], eb[1], eb[2], eb[3]);
+  *reinterpret_cast<float4*>(es + 128 + 4 * l32) = make_float4(ef[0], ef[1], ef[2], ef[3]);
+  wave_lds_sync();
+  float tb[4], tf[4];
+#pragma unroll 1
+  for (int b = 0; b < 4; ++b) {
+    float ub[4], uf[4];
+    const float* crow = C + (32 * b) * 128 + 4 * l32;
+    const float* e0 = es + 32 * b;
+#pragma unroll 4
+    for (int k = 0; k < 32; ++k) {
+      const float4 cv = *reinterpret_cast<const float4*>(crow + k * 128);
+      const float a = e0[k], f = e0[128 + k];
+      const float c[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pa = c[i] * a, pf = c[i] * f;
+        ub[i] = k == 0 ? pa : ub[i] + pa;
+        uf[i] = k == 0 ? pf : uf[i] + pf;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      tb[i] = b == 0 ? ub[i] : tb[i] + ub[i];
+      tf[i] = b == 0 ? uf[i] : tf[i] + uf[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { tb[i] = eb[i] * tb[i]; tf[i] = ef[i] * tf[i]; }
+  key_full = tree128(tf) < tree128(tb);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) qsel[i] = key_full ? qf[i] : qb[i];
+  word = key_full ? wf : wb;
+  if (!key_full && use_h) word |= 0x8000u;
+}
+
+// the key row of one token with its choice; in a key-only pass also the flag bit it owns in the value scale word
+template <int QM, int P>
+DEVI void k2_store_key(const K2WriteParams& p, int h, long long slot, bool flag_bit, const float (&qsel)[4], uint32_t word,
+                       bool key_full, int l32) {
+  using L = Lay<QM, P>;
+  uint8_t* chunk = p.pool + ((slot / P) * p.Hkv + h) * L::CHUNK;
+  const int pos = static_cast<int>(slot % P);
+  uint32_t code[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) code[i] = code_bits(qsel[i], QM == QM_SYM4);
+  store_row<QM, P>(chunk, pos, false, code, word, l32, false);
+  if (flag_bit && l32 == 0) {
+    const int off = L::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2;
+    uint32_t* wp = reinterpret_cast<uint32_t*>(chunk + (off & ~3));
+    const uint32_t bit = 0x8000u << ((off & 2) * 8);
+    if (key_full) atomicOr(wp, bit); else atomicAnd(wp, ~bit);
+  }
+}
+// the value scale words of one token (its codes are in the page already), with the key's whole-head flag
+template <int QM, int P>
+DEVI void k2_store_value_words(const K2WriteParams& p, int t, int h, long long slot, bool key_full, int l32) {
+  using L = Lay<QM, P>;
+  float x[4], q[4], deq[4];
+  load_row(p.kv, static_cast<long long>(t) * p.kv_ts + (p.Hkv + h) * 128 + 4 * l32, x);
+  uint32_t vword = quant_group<QM, false>(x, q, deq);
+  if ((l32 >> 3) == 0 && key_full) vword |= 0x8000u;
+  store_v_word<QM, P>(p.pool + ((slot / P) * p.Hkv + h) * L::CHUNK, static_cast<int>(slot % P), vword, l32, false);
+}
+
+DEVI float max32(float v) {   // over the 32 lanes of a half wave
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, hx(v, o));
+  return v;
+}
+DEVI float sum32(float v) {
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) v = v + hx(v, o);
+  return v;
+}
+
+typedef float w3_f32x16 __attribute__((ext_vector_type(16)));
+
+template <int QM, int P>
+__global__ void __launch_bounds__(256) k_k2_screen(const K2WriteParams p, int tile, float kappa) {
+  __shared__ W3Smem S;
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, hw = tid >> 5, l32 = tid & 31, kq = lane >> 5;
+  const int h = blockIdx.x;
+  const int t_lo = blockIdx.y * tile, t_hi = min(p.T, t_lo + tile);
+  const bool do_v = p.passes & 2;
+  const float* CT = p.CT + static_cast<size_t>(h) * 128 * 128;       // CT[k * 128 + i] = C[i][k]
+  // ---- A operands: lane (row m = l32 of tile wv, half kq): C[32 wv + m][64 kq + s] and C[32 wv + m][32 wv + 16 kq + s]
+  // (read from memory at every use: C^T stays in L2, and the registers it would take cost three quarters of the occupancy)
+  const float* ahp = CT + (64 * kq) * 128 + 32 * wv + l32;                 // + s * 128
+  const float* alp = CT + (32 * wv + 16 * kq) * 128 + 32 * wv + l32;       // + s * 128
+  if (tid < 128) S.colsum[tid] = 0.f;
+  if (tid == 0) S.nfb = 0;
+  __syncthreads();
+  float rho_loc, rho_full;
+  {
+    float rs = 0.f, rl = 0.f, cl = 0.f;
+#pragma unroll 8
+    for (int s2 = 0; s2 < 64; ++s2) {
+      const float a = fabsf(ahp[s2 * 128]);
+      rs += a;
+      const float cs = sum32(a);                                 // column 64 kq + s2 over the rows of this tile
+      if (l32 == 0) atomicAdd(&S.colsum[64 * kq + s2], cs);
+    }
+#pragma unroll 8
+    for (int s2 = 0; s2 < 16; ++s2) {
+      const float a = fabsf(alp[s2 * 128]);
+      rl += a;
+      cl = fmaxf(cl, sum32(a));
+    }
+    rs += __shfl_xor(rs, 32, 64); rl += __shfl_xor(rl, 32, 64);
+    cl = fmaxf(cl, __shfl_xor(cl, 32, 64));
+    rho_loc = fmaxf(max32(rl), cl);
+    const float ri = max32(rs);
+    if (lane == 0) S.rinf[wv] = ri;
+    __syncthreads();
+    float c1 = fmaxf(S.colsum[lane], S.colsum[64 + lane]);
+    c1 = max32(c1); c1 = fmaxf(c1, __shfl_xor(c1, 32, 64));
+    rho_full = fmaxf(fmaxf(fmaxf(S.rinf[0], S.rinf[1]), fmaxf(S.rinf[2], S.rinf[3])), c1);
+  }
+  const float beta_loc = kappa * rho_loc, beta_full = kappa * rho_full;
+  const int g = l32 >> 3;
+
+  for (int tb0 = t_lo; tb0 < t_hi; tb0 += W3_TOK) {
+    // ---- P1: candidates of the half wave's two tokens (exactly as in k_k2_write); error vectors to the matrix
+    uint32_t cq[2][3], cw[2][3];        // per token: packed codes (one byte per element) and scale words of I, H, F
+    float ef[2][4];
+    long long slot[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int tk = 2 * hw + u, t = tb0 + tk;
+      slot[u] = -1;
+      if (t < t_hi) slot[u] = p.slots[static_cast<long long>(t) * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
+      float x[4] = {0.f, 0.f, 0.f, 0.f};
+      if (slot[u] >= 0) {
+        load_row(p.kv, static_cast<long long>(t) * p.kv_ts + h * 128 + 4 * l32, x);
+        if (p.kmu != nullptr) {
+          const float4 m = *reinterpret_cast<const float4*>(p.kmu + h * 128 + 4 * l32);
+          x[0] = x[0] - m.x; x[1] = x[1] - m.y; x[2] = x[2] - m.z; x[3] = x[3] - m.w;
+        }
+      }
+      float qi[4], ei[4], qh[4], eh[4], qf[4], y[4];
+      cw[u][0] = quant_group<QM, true>(x, qi, ei);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { ei[i] = ei[i] - x[i]; y[i] = x[i]; }
+      fwht<32>(y, l32);
+      cw[u][1] = quant_group<QM, true>(y, qh, eh);
+      fwht<32>(eh, l32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { eh[i] = eh[i] - x[i]; y[i] = x[i]; }
+      fwht<128>(y, l32);
+      cw[u][2] = quant_group<QM, true>(y, qf, ef[u]);
+      fwht<128>(ef[u], l32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ef[u][i] = ef[u][i] - x[i];
+      cq[u][0] = cq[u][1] = cq[u][2] = 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        cq[u][0] |= code_bits(qi[i], QM == QM_SYM4) << (8 * i);
+        cq[u][1] |= code_bits(qh[i], QM == QM_SYM4) << (8 * i);
+        cq[u][2] |= code_bits(qf[i], QM == QM_SYM4) << (8 * i);
+      }
+      *reinterpret_cast<float4*>(&S.dm[2 * tk][4 * l32]) = make_float4(ei[0], ei[1], ei[2], ei[3]);
+      *reinterpret_cast<float4*>(&S.dm[2 * tk + 1][4 * l32]) = make_float4(eh[0], eh[1], eh[2], eh[3]);
+    }
+    __syncthreads();
+    // ---- P2: local forms of block wv for the 32 columns; lane = (column l32, half kq)
+    {
+      w3_f32x16 acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+      const float* dcol = &S.dm[l32][32 * wv];
+      const float* alq = alp;
+      asm volatile("" : "+v"(alq));             // keeps these loads inside the step (not hoisted into 80 registers)
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const float4 d4 = *reinterpret_cast<const float4*>(dcol + 16 * kq + 4 * s4);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(alq[(4 * s4 + 0) * 128], d4.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(alq[(4 * s4 + 1) * 128], d4.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(alq[(4 * s4 + 2) * 128], d4.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(alq[(4 * s4 + 3) * 128], d4.w, acc, 0, 0, 0);
+      }
+      float f = 0.f, n2 = 0.f;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {          // rows 8 q4 + 4 kq + r of the block
+        const float4 d4 = *reinterpret_cast<const float4*>(dcol + 8 * q4 + 4 * kq);
+        f = __builtin_fmaf(d4.x, acc[4 * q4 + 0], f); f = __builtin_fmaf(d4.y, acc[4 * q4 + 1], f);
+        f = __builtin_fmaf(d4.z, acc[4 * q4 + 2], f); f = __builtin_fmaf(d4.w, acc[4 * q4 + 3], f);
+        n2 = __builtin_fmaf(d4.x, d4.x, n2); n2 = __builtin_fmaf(d4.y, d4.y, n2);
+        n2 = __builtin_fmaf(d4.z, d4.z, n2); n2 = __builtin_fmaf(d4.w, d4.w, n2);
+      }
+      f += __shfl_xor(f, 32, 64); n2 += __shfl_xor(n2, 32, 64);
+      const float bnd = beta_loc * n2 + 7.888609052210118e-31f;
+      // columns 2 t (identity) and 2 t + 1 (H32): the reference takes H32 iff its value is strictly smaller
+      const float fo = hx(f, 1), bo = hx(bnd, 1);
+      if ((l32 & 1) == 0 && kq == 0) {
+        const float eI = f, bI = bnd, eH = fo, bH = bo;
+        S.choice[l32 >> 1][wv] = (eH + bH < eI - bI) ? 1 : (eH - bH > eI + bI) ? 0 : 2;
+      }
+    }
+    __syncthreads();
+    // ---- P3: the half wave's tokens: base candidate from the local choices, or the exact list
+    bool pend[2], kfull[2] = {false, false};
+    uint32_t useh[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int tk = 2 * hw + u;
+      const uint32_t ch = *reinterpret_cast<const uint32_t*>(&S.choice[tk][0]);
+      const bool und = (ch & 0x02020202u) != 0;      // some group undecided
+      pend[u] = slot[u] >= 0 && !und;
+      if (slot[u] >= 0 && und && l32 == 0) S.fb[atomicAdd(&S.nfb, 1)] = tb0 + tk;
+      useh[u] = (ch >> (8 * g)) & 1u;
+      const float4 eI = *reinterpret_cast<const float4*>(&S.dm[2 * tk][4 * l32]);
+      const float4 eH = *reinterpret_cast<const float4*>(&S.dm[2 * tk + 1][4 * l32]);
+      const float4 eb = useh[u] ? eH : eI;
+      wave_lds_sync();
+      *reinterpret_cast<float4*>(&S.dm[2 * tk][4 * l32]) = eb;
+      *reinterpret_cast<float4*>(&S.dm[2 * tk + 1][4 * l32]) = make_float4(ef[u][0], ef[u][1], ef[u][2], ef[u][3]);
+    }
+    __syncthreads();
+    // ---- P4: whole-head forms: rows of tile wv, all 128 columns of C
+    {
+      w3_f32x16 acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+      const float* dcol = &S.dm[l32][0];
+      const float* ahq = ahp;
+      asm volatile("" : "+v"(ahq));
+#pragma unroll 4
+      for (int s4 = 0; s4 < 16; ++s4) {
+        const float4 d4 = *reinterpret_cast<const float4*>(dcol + 64 * kq + 4 * s4);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ahq[(4 * s4 + 0) * 128], d4.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ahq[(4 * s4 + 1) * 128], d4.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ahq[(4 * s4 + 2) * 128], d4.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ahq[(4 * s4 + 3) * 128], d4.w, acc, 0, 0, 0);
+      }
+      float f = 0.f, n2 = 0.f;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const float4 d4 = *reinterpret_cast<const float4*>(dcol + 32 * wv + 8 * q4 + 4 * kq);
+        f = __builtin_fmaf(d4.x, acc[4 * q4 + 0], f); f = __builtin_fmaf(d4.y, acc[4 * q4 + 1], f);
+        f = __builtin_fmaf(d4.z, acc[4 * q4 + 2], f); f = __builtin_fmaf(d4.w, acc[4 * q4 + 3], f);
+        n2 = __builtin_fmaf(d4.x, d4.x, n2); n2 = __builtin_fmaf(d4.y, d4.y, n2);
+        n2 = __builtin_fmaf(d4.z, d4.z, n2); n2 = __builtin_fmaf(d4.w, d4.w, n2);
+      }
+      f += __shfl_xor(f, 32, 64); n2 += __shfl_xor(n2, 32, 64);
+      if (kq == 0) { S.part[0][wv][l32] = f; S.part[1][wv][l32] = n2; }
+    }
+    __syncthreads();
+    // ---- P5: base against whole head; rows of the decided tokens into their pages
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int tk = 2 * hw + u;
+      float e[2], b[2];
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        e[c] = (S.part[0][0][2 * tk + c] + S.part[0][1][2 * tk + c]) + (S.part[0][2][2 * tk + c] + S.part[0][3][2 * tk + c]);
+        const float n2 = (S.part[1][0][2 * tk + c] + S.part[1][1][2 * tk + c]) + (S.part[1][2][2 * tk + c] + S.part[1][3][2 * tk + c]);
+        b[c] = beta_full * n2 + 7.888609052210118e-31f;
+      }
+      const int dec = (e[1] + b[1] < e[0] - b[0]) ? 1 : (e[1] - b[1] > e[0] + b[0]) ? 0 : 2;
+      if (pend[u] && dec == 2) {
+        if (l32 == 0) S.fb[atomicAdd(&S.nfb, 1)] = tb0 + tk;
+        pend[u] = false;
+      } else if (pend[u]) {
+        const bool key_full = dec == 1;
+        kfull[u] = key_full;
+        const uint32_t cpk = key_full ? cq[u][2] : (useh[u] ? cq[u][1] : cq[u][0]);
+        uint32_t word = key_full ? cw[u][2] : (useh[u] ? cw[u][1] : cw[u][0]);
+        if (!key_full && useh[u]) word |= 0x8000u;
+        float qsel[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t cb = (cpk >> (8 * i)) & 0xFFu;
+          qsel[i] = QM == QM_SYM4 ? ((cb & 8u) ? -static_cast<float>(cb & 7u) : static_cast<float>(cb)) : static_cast<float>(cb);
+        }
+        k2_store_key<QM, P>(p, h, slot[u], !do_v, qsel, word, key_full, l32);
+      }
+    }
+    // ---- value rows of the step: codes of all live tokens (whole words for aligned runs of 8 slots, else atomics),
+    //      scale words of the decided tokens (the others' carry the key's flag and follow the exact evaluation)
+    if (do_v) {
+      uint32_t vcode[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int tk = 2 * hw + u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vcode[u][i] = 0u;
+        if (slot[u] >= 0) {
+          float x[4], q[4], deq[4];
+          load_row(p.kv, static_cast<long long>(tb0 + tk) * p.kv_ts + (p.Hkv + h) * 128 + 4 * l32, x);
+          uint32_t vword = quant_group<QM, false>(x, q, deq);
+          if (g == 0 && kfull[u]) vword |= 0x8000u;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vcode[u][i] = code_bits(q[i], QM == QM_SYM4);
+          if (pend[u]) {
+            using L = Lay<QM, P>;
+            store_v_word<QM, P>(p.pool + ((slot[u] / P) * p.Hkv + h) * L::CHUNK, static_cast<int>(slot[u] % P), vword, l32, false);
+          }
+        }
+        if (l32 == 0) S.vslot[tk] = slot[u];
+        *reinterpret_cast<uint32_t*>(&S.vcodes[tk][4 * l32]) = vcode[u][0] | (vcode[u][1] << 8) | (vcode[u][2] << 16) | (vcode[u][3] << 24);
+      }
+      __syncthreads();
+      using L = Lay<QM, P>;
+      constexpr int NWORD = QM == QM_ASYM2 ? 64 : 128;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const long long s0 = S.vslot[8 * r];
+        bool run = s0 >= 0 && (s0 & 7) == 0;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) run = run && S.vslot[8 * r + i] == s0 + i;
+        if (run) {
+          const int j = tid - r * 128;
+          if (j >= 0 && j < NWORD)
+            store_v_run_word<QM, P>(p.pool + ((s0 / P) * p.Hkv + h) * L::CHUNK, static_cast<int>(s0 % P) >> 3, j, &S.vcodes[8 * r]);
+        } else if ((hw >> 2) == r) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            if (slot[u] >= 0)
+              store_v_codes<QM, P>(p.pool + ((slot[u] / P) * p.Hkv + h) * L::CHUNK, static_cast<int>(slot[u] % P), vcode[u], l32);
+        }
+      }
+    }
+    // (the next step's P1 writes the matrix after every wavefront has passed the barrier behind P4; the value strips are
+    //  rewritten after three more barriers)
+  }
+  // ---- the tokens the screen could not decide: exact evaluation, C^T from memory
+  __syncthreads();
+  const int nfb = S.nfb;
+  for (int i = hw; i < nfb; i += 8) {
+    const int t = S.fb[i];
+    const long long slot = p.slots[static_cast<long long>(t) * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
+    float x[4];
+    load_row(p.kv, static_cast<long long>(t) * p.kv_ts + h * 128 + 4 * l32, x);
+    if (p.kmu != nullptr) {
+      const float4 m = *reinterpret_cast<const float4*>(p.kmu + h * 128 + 4 * l32);
+      x[0] = x[0] - m.x; x[1] = x[1] - m.y; x[2] = x[2] - m.z; x[3] = x[3] - m.w;
+    }
+    float qsel[4];
+    uint32_t word;
+    bool key_full;
+    k2_exact_choice<QM>(x, CT, &S.es[hw][0], l32, qsel, word, key_full);
+    k2_store_key<QM, P>(p, h, slot, !do_v, qsel, word, key_full, l32);
+    if (do_v) k2_store_value_words<QM, P>(p, t, h, slot, key_full, l32);
+  }
+}
+
 template <int QM>
 int static_write_qm(const StaticWriteParams& p, hipStream_t st) {
   const long long rows = static_cast<long long>(p.T) * 2 * p.Hkv;
@@ -447,6 +901,16 @@ int k2_write_p(const K2WriteParams& p, hipStream_t st) {
       return -2;
     }
     attr = true;
+  }
+  // prefill-sized key passes: the screened kernel (same bytes)
+  static const int w3mode = getenv("FLAGROT_W3") != nullptr ? atoi(getenv("FLAGROT_W3")) : 1;     // 0 off, 2 every token exact
+  static const float w3kappa = getenv("FLAGROT_W3_KAPPA") != nullptr ? static_cast<float>(atof(getenv("FLAGROT_W3_KAPPA"))) : W3_KAPPA;
+  if (w3mode != 0 && p.screen && (p.passes & 1) && static_cast<long long>(p.T) * p.Hkv > 1024) {
+    int tile = W3_TOK;
+    while (tile < W3_MAXTILE && static_cast<long long>(p.Hkv) * ((p.T + tile - 1) / tile) > 512) tile *= 2;
+    hipLaunchKernelGGL((k_k2_screen<QM, P>), dim3(p.Hkv, (p.T + tile - 1) / tile), dim3(256), 0, st, p, tile,
+                       w3mode == 2 ? 1e30f : w3kappa);
+    return hipPeekAtLastError() == hipSuccess ? 0 : -1;
   }
   // a decode step's worth of tokens: four half waves per (token, head), at most two workgroups per CU in one round
   static const bool no_ll = getenv("FLAGROT_WRITER_LL") != nullptr && getenv("FLAGROT_WRITER_LL")[0] == '0';

@@ -87,6 +87,38 @@ def test_selecting_writer_bytes(dev, kind, T):
 
 
 @pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
+@pytest.mark.parametrize("T,base", [(700, 0), (700, 5), (90, 8), (333, 16)])
+def test_selecting_writer_consecutive_slots(dev, kind, T, base):
+    """prefill-like slots (consecutive positions): aligned runs of 8 slots take the whole-word V^T store, the ragged
+    ends, a hole and a token written twice the atomic one; whole-pool bytes against the oracle's packer"""
+    from flagrot_releaser_amd import kernels as K
+    g = torch.Generator().manual_seed(4000 + T + base)
+    Hkv = 2
+    npg = (T + base) // P + 3
+    pool = _pool(kind, npg, Hkv, g)
+    kv = make_kv(T, Hkv, g)
+    Cq, co = spd_calib(Hkv, g)
+    slots = base + torch.arange(T).long()
+    slots[T // 2] = -1
+    if T > 300:
+        slots[200:216] = slots[200:216].flip(0)            # a run of 16 slots in reverse order
+    dpool = pool.to(dev)
+    CT = Cq.transpose(1, 2).contiguous().to(dev)
+    K.cb_write(kv.to(dev), slots.to(dev), CT, co.to(dev), kind, dpool, P)
+    torch.cuda.synchronize()
+    want = pool.numpy().copy()
+    codes, words, info = Q.k2_encode(bits(kv), Cq.numpy(), kind, None)
+    PG.pack_tokens(want, slots.numpy(), codes, words, kind, P)
+    _same(dpool.cpu().numpy(), want, kind)
+    # the two-pass form (key-only and value-only launches) on the same slots
+    C1, beta = K.w3_calib(Cq.to(dev))
+    d2 = pool.to(dev)
+    K.cb_write3(kv.to(dev), slots.to(dev), CT, co.to(dev), C1, beta, kind, d2, P, split=True)
+    torch.cuda.synchronize()
+    assert torch.equal(d2, dpool)
+
+
+@pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
 def test_two_pass_writer_equals_one_pass(dev, kind):
     """fr_cb_write3: one launch, and key pass / value pass on two streams, write the same bytes as fr_cb_write."""
     from flagrot_releaser_amd import kernels as K
@@ -106,6 +138,40 @@ def test_two_pass_writer_equals_one_pass(dev, kind):
     K.cb_write3(kv, slots, CT, co, C1, beta, kind, c, P, split=True, kmu=kmu)
     torch.cuda.synchronize()
     assert torch.equal(a, b) and torch.equal(a, c)
+
+
+@pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
+@pytest.mark.parametrize("order", ["scattered", "consecutive"])
+def test_screened_writer_equals_exact_writer(dev, kind, order):
+    """fr_cb_write3 at prefill sizes runs the screened kernel (matrix-pipe estimates of the weighted errors, exact
+    evaluation where the estimate cannot decide): whole-pool byte equality with fr_cb_write on ordinary rows, on the
+    adversarial groups of the reference's tests, on rows that tie exactly (zeros, constants, repeated tokens) and on
+    holes; key-only and value-only passes included."""
+    from flagrot_releaser_amd import kernels as K
+    g = torch.Generator().manual_seed(77)
+    Hkv, T = 4, 3000
+    npg = T // P + 9
+    pool = _pool(kind, npg, Hkv, g).to(dev)
+    kv = make_kv(T, Hkv, g, edge=True)
+    kv[100:140] = 0                                        # every candidate reproduces the row: exact ties
+    kv[140:180] = kv[140:141]                              # one token repeated
+    kv[180:200] = 0.37                                     # constants
+    kv[200:260, :, 32:64] = 0                              # ties in one 32-group only
+    kv[260:300] = (kv[260:300].float() * 1e-4).bfloat16()  # tiny rows
+    kv = kv.to(dev)
+    Cq, co = spd_calib(Hkv, g)
+    CT, co = Cq.transpose(1, 2).contiguous().to(dev), co.to(dev)
+    slots = _slots(T, npg, g) if order == "scattered" else 11 + torch.arange(T).long()
+    slots[500:523] = -1
+    slots = slots.to(dev)
+    C1, beta = K.w3_calib(Cq.to(dev))
+    for kmu in (None, torch.randn(Hkv, 128, generator=g).to(dev)):
+        a, b, c = pool.clone(), pool.clone(), pool.clone()
+        K.cb_write(kv, slots, CT, co, kind, a, P, kmu=kmu)
+        K.cb_write3(kv, slots, CT, co, C1, beta, kind, b, P, split=False, kmu=kmu)
+        K.cb_write3(kv, slots, CT, co, C1, beta, kind, c, P, split=True, kmu=kmu)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b) and torch.equal(a, c)
 
 
 @pytest.mark.parametrize("fmt", ["int4", "int4a", "int2a"])
