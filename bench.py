@@ -81,7 +81,7 @@ def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192):
             kv = synth_kv(n, g, dev, torch, mu=kmu)
             pos = torch.arange(s, s + n, device=dev)
             slots = bt[b].long()[pos // P] * P + pos % P
-            K.cb_write(kv, slots, CT, co, kind, pool, P, kmu=kmu)
+            K.cb_write3(kv, slots, CT, co, None, None, kind, pool, P, split=False, kmu=kmu)    # = cb_write bytes
     torch.cuda.synchronize()
     return pool, bt, CT, co, time.perf_counter() - t0
 

@@ -223,7 +223,11 @@ class DecodeLayer:
         if self.static:
             K.v2_write(kv, slots, self.wmask, 32, self.pool, PAGE, fmt=self.kind, kmu=self.kmu)
         else:
-            K.cb_write(kv, slots, self.CT, self.co, self.kind, self.pool, PAGE, kmu=self.kmu)
+            # same bytes either way; fr_cb_write3 runs the screened kernel on prompt-sized launches
+            if kv.shape[0] * self.Hkv > 1024:
+                K.cb_write3(kv, slots, self.CT, self.co, None, None, self.kind, self.pool, PAGE, split=False, kmu=self.kmu)
+            else:
+                K.cb_write(kv, slots, self.CT, self.co, self.kind, self.pool, PAGE, kmu=self.kmu)
 
     def prefill(self, kv, slots, req: int):
         """a prompt of n tokens of request slot `req`: every token to its page, sinks and the newest W tokens also to

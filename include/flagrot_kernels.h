@@ -59,7 +59,10 @@ int fr_cb_write(const void* kv, long long kv_ts, const long long* slots, int slo
 
 /* flagrot_capi.cu:104-115.  Same bytes as fr_cb_write.  nchunk < 0 skips the key pass, nchunk_v < 0 the value
  * pass; the two passes own disjoint bits of the token's group-0 V scale word, so they may run on two streams.
- * C1 / beta (screening constants of the reference's tensor-core writer) are accepted and ignored. */
+ * Key passes of more than 1024 (token, head) rows run the screened kernel: the weighted errors are estimated on the
+ * matrix pipe and a token is decided from the estimates only where the exactly ordered evaluation cannot decide
+ * otherwise; the rest is evaluated exactly.  The error bound is computed from CT by the kernel itself: C1 / beta (the
+ * screening constants of the reference's tensor-core writer) are accepted and ignored (may be null). */
 int fr_cb_write3(const void* kv, long long kv_ts, const long long* slots, int slot_ph, int T, int Hkv, int page,
                  const float* CT, const float* co, const void* C1, const float* beta, const unsigned* sg, int kind,
                  uint8_t* pool, int nchunk, int nchunk_v, void* stream, const float* kmu);
