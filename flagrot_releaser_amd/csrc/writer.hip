@@ -32,20 +32,24 @@ DEVI void load_row(const void* kv, long long off, float (&x)[4]) {
 template <int QM, int P>
 __global__ void __launch_bounds__(256) k_static_write(const StaticWriteParams p) {
   using L = Lay<QM, P>;
-  const int l32 = threadIdx.x & 31;
-  const long long row = static_cast<long long>(blockIdx.x) * 8 + (threadIdx.x >> 5);
+  // workgroup = eight consecutive tokens of one head row (K or V), one per half wave
+  __shared__ long long vslot[8];
+  __shared__ __align__(16) uint8_t vcodes[8][128];
+  const int l32 = threadIdx.x & 31, hw = threadIdx.x >> 5;
   const int H2 = 2 * p.Hkv;
-  if (row >= static_cast<long long>(p.T) * H2) return;
-  const int t = static_cast<int>(row / H2), hr = static_cast<int>(row % H2);
-  const long long slot = p.slots[t];
-  if (slot < 0) return;
+  const int hr = static_cast<int>(blockIdx.x % H2);
+  const int t = static_cast<int>(blockIdx.x / H2) * 8 + hw;
+  long long slot = -1;
+  if (t < p.T) slot = p.slots[t];
+  const bool live = slot >= 0;
   const bool isv = hr >= p.Hkv;
   const int head = isv ? hr - p.Hkv : hr;
-  uint8_t* chunk = p.pool + ((slot / P) * p.Hkv + head) * L::CHUNK;
-  const int pos = static_cast<int>(slot % P);
+  if (!isv && !live) return;             // key rows need no hand-over between the half waves
+  uint8_t* chunk = p.pool + ((live ? slot / P : 0) * p.Hkv + head) * L::CHUNK;
+  const int pos = live ? static_cast<int>(slot % P) : 0;
 
-  float x[4];
-  load_row(p.kv, static_cast<long long>(t) * p.kv_ts + hr * 128 + 4 * l32, x);
+  float x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (live) load_row(p.kv, static_cast<long long>(t) * p.kv_ts + hr * 128 + 4 * l32, x);
   if (p.hfull != nullptr && p.hfull[hr]) {  // whole-head +-1 Hadamard / 16, rounded to bf16 (the stored basis)
     butterflies<128>(x, l32);
 #pragma unroll
@@ -67,7 +71,26 @@ __global__ void __launch_bounds__(256) k_static_write(const StaticWriteParams p)
   uint32_t code[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) code[i] = code_bits(q[i], QM == QM_SYM4);
-  store_row<QM, P>(chunk, pos, isv, code, word, l32, false);
+  if (!isv) {
+    store_row<QM, P>(chunk, pos, false, code, word, l32, false);
+    return;
+  }
+  // value rows: an aligned run of 8 slots of one page gets its V^T words assembled in LDS and stored whole
+  if (live) store_v_word<QM, P>(chunk, pos, word, l32, false);
+  if (l32 == 0) vslot[hw] = slot;
+  *reinterpret_cast<uint32_t*>(&vcodes[hw][4 * l32]) = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+  __syncthreads();
+  const long long s0 = vslot[0];
+  bool run = s0 >= 0 && (s0 & 7) == 0;
+#pragma unroll
+  for (int i = 1; i < 8; ++i) run = run && vslot[i] == s0 + i;
+  if (run) {
+    constexpr int NWORD = QM == QM_ASYM2 ? 64 : 128;
+    if (threadIdx.x < NWORD)
+      store_v_run_word<QM, P>(p.pool + ((s0 / P) * p.Hkv + head) * L::CHUNK, static_cast<int>(s0 % P) >> 3, threadIdx.x, vcodes);
+  } else if (live) {
+    store_v_codes<QM, P>(chunk, pos, code, l32);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ head Hadamard
@@ -880,8 +903,7 @@ __global__ void __launch_bounds__(256) k_k2_screen(const K2WriteParams p, int ti
 
 template <int QM>
 int static_write_qm(const StaticWriteParams& p, hipStream_t st) {
-  const long long rows = static_cast<long long>(p.T) * 2 * p.Hkv;
-  const unsigned grid = static_cast<unsigned>((rows + 7) / 8);
+  const unsigned grid = static_cast<unsigned>(static_cast<long long>((p.T + 7) / 8) * 2 * p.Hkv);
   if (grid == 0) return 0;
   if (p.page == 16) hipLaunchKernelGGL((k_static_write<QM, 16>), dim3(grid), dim3(256), 0, st, p);
   else if (p.page == 32) hipLaunchKernelGGL((k_static_write<QM, 32>), dim3(grid), dim3(256), 0, st, p);

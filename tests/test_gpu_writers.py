@@ -39,9 +39,12 @@ def _slots(T, npg, g, holes=True):
 
 
 @pytest.mark.parametrize("fmt", ["int4", "int4a", "int2a"])
-@pytest.mark.parametrize("T", [1, 5, 64, 1000])
+@pytest.mark.parametrize("T", [1, 5, 64, 1000, -333, -90])
 def test_static_writer_bytes(dev, fmt, T):
+    """T < 0: |T| tokens at consecutive slots (aligned runs of 8 take the whole-word V^T store; ragged ends, a hole and a
+    reversed stretch the atomic one)"""
     from flagrot_releaser_amd import kernels as K
+    consecutive, T = T < 0, abs(T)
     g = torch.Generator().manual_seed(1000 + T)
     Hkv = 4
     npg = T // P + 5
@@ -50,6 +53,10 @@ def test_static_writer_bytes(dev, fmt, T):
     base[:, :2 * Hkv] = make_kv(T, Hkv, g)
     kv = base.to(dev)[:, :2 * Hkv]                                   # token stride (2 Hkv + 1) * 128
     slots = _slots(T, npg, g)
+    if consecutive:
+        slots = 13 + torch.arange(T).long()
+        slots[T // 2] = -1
+        slots[40:56] = slots[40:56].flip(0)
     mask = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8)
     kmu = torch.randn(Hkv, 128, generator=g) if T != 5 else None
     dpool = pool.to(dev)
