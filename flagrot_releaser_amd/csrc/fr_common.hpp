@@ -38,8 +38,20 @@ DEVI float f16_value(uint32_t bits) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
 }
 
-// exchange inside a 32-lane half wave
-DEVI float hx(float v, int m) { return __shfl_xor(v, m, 32); }
+// exchange inside a 32-lane half wave: lane ^ m.  For the distances the butterflies and trees use (1, 2, 4, 8, 16, known
+// after unrolling) this is a DPP move (1, 2: quad permute; 8: rotation of the 16-lane row by 8) or a ds_swizzle (4, 16);
+// any other distance goes through ds_bpermute.
+DEVI float hx(float v, int m) {
+  const int i = __float_as_int(v);
+  if (__builtin_constant_p(m)) {
+    if (m == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0xB1, 0xF, 0xF, true));
+    if (m == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x4E, 0xF, 0xF, true));
+    if (m == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x128, 0xF, 0xF, true));   // row_ror:8
+    if (m == 4) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, (4 << 10) | 0x1F));
+    if (m == 16) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, (16 << 10) | 0x1F));
+  }
+  return __shfl_xor(v, m, 32);
+}
 DEVI uint32_t hdown(uint32_t v, int n) { return __shfl_down(v, n, 32); }
 
 // ---------------------------------------------------------------------------------------------- butterflies
