@@ -125,6 +125,34 @@ def test_selecting_writer_consecutive_slots(dev, kind, T, base):
     assert torch.equal(d2, dpool)
 
 
+@pytest.mark.parametrize("fmt", ["int4a", "int2a", "konlya", "konlya2", "konly"])
+@pytest.mark.parametrize("order", ["scattered", "consecutive"])
+def test_writers_page_32(dev, fmt, order):
+    """32-token pages (four runs of 8 slots per page): whole-pool bytes against the oracle's packer for both writers"""
+    from flagrot_releaser_amd import kernels as K
+    P32 = 32
+    g = torch.Generator().manual_seed(5200 + len(fmt))
+    Hkv, T = 2, 300
+    npg = T // P32 + 4
+    pool = torch.randint(0, 256, (npg, Hkv, PG.chunk_bytes(fmt, P32)), dtype=torch.uint8, generator=g)
+    kv = make_kv(T, Hkv, g)
+    slots = torch.randperm(npg * P32, generator=g)[:T].long() if order == "scattered" else 19 + torch.arange(T).long()
+    slots[77] = -1
+    dpool = pool.to(dev)
+    want = pool.numpy().copy()
+    if fmt in ("int4a", "int2a"):
+        mask = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8)
+        K.v2_write(kv.to(dev), slots.to(dev), mask.to(dev), 32, dpool, P32, fmt=fmt)
+        codes, words = Q.static_encode(bits(kv), mask.numpy(), fmt, None)
+    else:
+        Cq, co = spd_calib(Hkv, g)
+        K.cb_write(kv.to(dev), slots.to(dev), Cq.transpose(1, 2).contiguous().to(dev), co.to(dev), fmt, dpool, P32)
+        codes, words, _ = Q.k2_encode(bits(kv), Cq.numpy(), fmt, None)
+    torch.cuda.synchronize()
+    PG.pack_tokens(want, slots.numpy(), codes, words, fmt, P32)
+    assert np.array_equal(dpool.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
 def test_two_pass_writer_equals_one_pass(dev, kind):
     """fr_cb_write3: one launch, and key pass / value pass on two streams, write the same bytes as fr_cb_write."""
