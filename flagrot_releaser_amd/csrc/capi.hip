@@ -69,12 +69,12 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   if ((variant & ~(GEN | GT8 | HD256)) != 264 && (variant & ~(GEN | GT8 | HD256)) != 0)
     return fail(-3, "fr_v2_attn: unsupported variant");
   if (stages < 1 || stages > 8) return fail(-3, "fr_v2_attn: unsupported stages");
-  if (page != 16) return fail(-5, "fr_v2_attn: page size 16 only");
+  if (page != 16 && page != 32) return fail(-5, "fr_v2_attn: page size 16 or 32");
   if (gqa <= 0) gqa = 4;
   if (gqa > 64) return fail(-7, "fr_v2_attn: gqa out of range");
   if (gqa != 4 && !(variant & GEN)) return fail(-7, "fr_v2_attn: gqa != 4 needs the generalised variant");
   if (rb != 32 && (qrot || vrot)) return fail(-3, "fr_v2_attn: rotation block 32 only");
-  if (nsplit < 1 || chunk <= 0 || chunk % 16) return fail(-3, "fr_v2_attn: bad split plan");
+  if (nsplit < 1 || chunk <= 0 || chunk % page) return fail(-3, "fr_v2_attn: bad split plan");
   const bool k2 = fmt == FMT_KONLY || fmt == FMT_KONLYA || fmt == FMT_KONLYA2;
   DecodeParams p{};
   p.q = q; p.q_bs = q_bs; p.pool = pool; p.block_table = block_table; p.bt_stride = bt_stride; p.seq_lens = seq_lens;
@@ -118,7 +118,7 @@ int fr_v2_write(int fmt, const void* kv, long long kv_ts, const long long* slots
 
 int fr_v2_occupancy(int fmt, int variant, int stages, int page) {
   (void)variant; (void)stages;
-  if (page != 16 || fmt < FMT_INT4 || fmt > FMT_KONLYA2) return 0;
+  if ((page != 16 && page != 32) || fmt < FMT_INT4 || fmt > FMT_KONLYA2) return 0;
   return decode_occupancy(fmt, 4);
 }
 int fr_v2_chunk_bytes(int fmt, int page) { return page * (fmt_int2(fmt) ? 80 : 144); }
@@ -181,7 +181,7 @@ int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* bl
 
 int fr_cb_occupancy(int kind, int variant, int stages, int page) {
   (void)variant; (void)stages;
-  if (page != 16 || fmt_of_kind(kind) < 0) return 0;
+  if ((page != 16 && page != 32) || fmt_of_kind(kind) < 0) return 0;
   return decode_occupancy(fmt_of_kind(kind), 4);
 }
 int fr_cb_chunk_bytes(int kind, int page) { return page * (kind == KIND_KONLYA2 ? 80 : 144); }

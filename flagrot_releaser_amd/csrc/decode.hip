@@ -170,18 +170,21 @@ DEVI void load_k(KRegs<QM>& r, const uint8_t* chunk, int pos) {
 template <int QM, int P>
 DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
   using L = Lay<QM, P>;
-  // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of pages 2 s, 2 s + 1)
+  // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of half s of the quad:
+  // 16-token pages 2 s, 2 s + 1 with two runs each, or the 32-token page s with four)
+  constexpr int R = P / 8;                       // runs of 8 tokens (entries per dim group) per page
   const int m = lane & 15, kc = lane >> 4;
 #pragma unroll
   for (int s2 = 0; s2 < 2; ++s2) {
-    const uint8_t* ch = (kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2];
+    const uint8_t* ch = P == 16 ? ((kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2]) : chunk[s2];
+    const int c8 = P == 16 ? (kc & 1) : kc;
 #pragma unroll
     for (int eh = 0; eh < 2; ++eh) {
       if constexpr (QM == QM_ASYM2) {
-        const u32x2 v = gload<u32x2>(ch + L::V_OFF + 8 * (2 * (16 * eh + m) + (kc & 1)));
+        const u32x2 v = gload<u32x2>(ch + L::V_OFF + 8 * (R * (16 * eh + m) + c8));
         r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y;
       } else {
-        const u32x4 v = gload<u32x4>(ch + L::V_OFF + 16 * (2 * (16 * eh + m) + (kc & 1)));
+        const u32x4 v = gload<u32x4>(ch + L::V_OFF + 16 * (R * (16 * eh + m) + c8));
         r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y; r.vc[2 * s2 + eh][2] = v.z; r.vc[2 * s2 + eh][3] = v.w;
       }
     }
@@ -275,7 +278,6 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
   }
   st.z[0] *= (lane & 1) ? alpha[2] : alpha[0];
   st.z[1] *= (lane & 1) ? alpha[3] : alpha[1];
-  const int pi = lane >> 4, pos = lane & 15;
   float p[4];
 #pragma unroll
   for (int h = 0; h < 4; ++h) {
@@ -285,13 +287,13 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
   // p' = p * V scale per group as fp16 (packed fp16 products of head pairs) and the zero points, in V^T token order
   // of the token's page.  Odd tokens are unpacked with the factor 2^SH (UnpackD): their scores were lowered by SH
   // (p carries 2^-SH), their zero point is raised by 2^SH; zero points are fp16 denormals like the codes.
-  const int rg = pi * 2 + (pos >> 3), sl = vslot(pos & 7);
+  const int rg = lane >> 3, sl = vslot(lane & 7);         // run of 8 tokens (page, page eighth) and the slot inside it
   uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
   uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + rg * ZB_RSTRIDE * 8 + sl;     // + group * 8
   const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[0], p[1]));
   const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[2], p[3]));
   const uint32_t keep = valid ? 0x7FFF7FFFu : 0u;        // unwritten slots may hold any pattern
-  const int zsh = (pos & 1) ? UnpackD<QM>::SH : 0;
+  const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const uint32_t sv2 = (r.vs[g] * 0x10001u) & keep;
@@ -431,15 +433,16 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       for (int i = threadIdx.x; i < 4 * (4 * PB_RSTRIDE + 1); i += 64 * NW) S.zero[i] = 0u;
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
-      const int nquad = (pg1 - pg0 + 3) >> 2;
-      const int pi = lane >> 4, pos = lane & 15;
+      constexpr int PPQ = 64 / P;                 // pages per quad of 64 tokens (the name stays: 4 pages of 16, 2 of 32)
+      const int nquad = (pg1 - pg0 + PPQ - 1) / PPQ;
+      const int pi = lane / P, pos = lane % P;
       // odd tokens: the B fields of a V^T word come out of the unpacking with the factor 2^SH, so their scores are
       // lowered by SH (log2 domain) and their share of the softmax sum is raised again at the end
       const float sc0 = (pos & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
       typedef const __attribute__((address_space(1))) uint8_t* gptr;
       const gptr pool = (gptr)p.pool;
       auto chunk_of = [&](int quad) {   // pages past the range read the last page of the range; their tokens are masked
-        const int i = min(4 * quad + pi, pg1 - pg0 - 1);
+        const int i = min(PPQ * quad + pi, pg1 - pg0 - 1);
         const int page = i < BT_CACHE ? S.btc[i] : bt[pg0 + i];
         return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
       };
@@ -467,14 +470,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
           const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
           const uint8_t* ch[4];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const uint32_t lo32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp), 16 * k);
-            const uint32_t hi32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp >> 32), 16 * k);
+          for (int k = 0; k < 4; ++k) {             // (32-token pages: entries 2, 3 repeat page 1 and are not read)
+            const uint32_t lo32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp), (P * k) & 63);
+            const uint32_t hi32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp >> 32), (P * k) & 63);
             ch[k] = reinterpret_cast<const uint8_t*>((static_cast<unsigned long long>(hi32) << 32) | lo32);
           }
           load_v<QM, P>(vr, ch, lane);
         }
-        const int tok = (pg0 + 4 * qi + pi) * P + pos;
+        const int tok = (pg0 + PPQ * qi + pi) * P + pos;
         const bool valid = tok >= lo && tok < hi;
         float sc[4];
         key_phase<QM, K2>(S, cur, p.qscale, sc0, sc);
@@ -681,12 +684,15 @@ inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? 16 :
 
 template <int QM, bool K2>
 int launch_qm(const DecodeParams& p, hipStream_t st) {
-  if (p.page != 16) return -5;
+  if (p.page != 16 && p.page != 32) return -5;
   const int ntile = (p.gqa + 3) / 4;
   const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
-  if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
+  if (p.page == 32) {
+    if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 32, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
+    else hipLaunchKernelGGL((k_decode<QM, K2, 32, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
+  } else if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
   else hipLaunchKernelGGL((k_decode<QM, K2, 16, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }

@@ -5,7 +5,7 @@
  * integrations/vllm_flagrot/csrc/flagrot_capi.cu).  All pointers are raw device addresses, `stream` is a
  * hipStream_t, every call is asynchronous on that stream, allocates nothing and may be captured in a HIP graph.
  * Return codes: 0 ok; -1 launch error; -2 LDS request refused; -3 unsupported variant / stages; -4 unknown fmt /
- * kind; -5 page not in {16, 32} (decode: 16 only); -7 gqa out of range; -8 head dim not supported.
+ * kind; -5 page not in {16, 32}; -7 gqa out of range; -8 head dim not supported.
  *
  * fmt  (static / generalised decode): 4 int4, 5 int4a, 6 konly, 7 konlya, 8 int2a, 9 konlya2
  * kind (key-only 2x2 codebooks):      6 konly, 10 konlya, 11 konlya2

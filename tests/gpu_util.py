@@ -44,7 +44,7 @@ def spd_calib(Hkv, g, nq=256):
     return Cq, co
 
 
-def alloc_tables(lens, num_pages, g):
+def alloc_tables(lens, num_pages, g, P=P):
     need = [(n + P - 1) // P for n in lens]
     ids = torch.randperm(num_pages, generator=g)[:sum(need)]
     bt = torch.zeros(len(lens), max(max(need), 1), dtype=torch.int32)
@@ -55,6 +55,6 @@ def alloc_tables(lens, num_pages, g):
     return bt
 
 
-def slots_of(bt, b, n):
+def slots_of(bt, b, n, P=P):
     pos = torch.arange(n)
     return bt[b].long()[pos // P] * P + pos % P

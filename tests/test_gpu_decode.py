@@ -18,21 +18,21 @@ import torch
 
 from oracle import attend as A
 from oracle import pages as PG
-from tests.gpu_util import P, alloc_tables, bits, make_kv, slots_of, spd_calib
+from tests.gpu_util import P as P16, alloc_tables, bits, make_kv, slots_of, spd_calib
 
 pytestmark = pytest.mark.gpu
 LOG2E = 1.4426950408889634
 ATOL, RTOL = 2e-3, 1e-2
 
 
-def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None):
+def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None, P=P16):
     from flagrot_releaser_amd import kernels as K
     g = torch.Generator().manual_seed(seed)
     B = len(lens)
     HQ = G * Hkv
     num_pages = sum((n + P - 1) // P for n in lens) + 7
     pool = torch.randint(0, 256, (num_pages, Hkv, PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g).to(dev)
-    bt = alloc_tables(lens, num_pages, g)
+    bt = alloc_tables(lens, num_pages, g, P)
     if bt_shared:
         bt = bt[:1].expand(B, -1)
         if bt_shared != "stride0":
@@ -46,7 +46,7 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
         if n == 0:
             continue
         kv = make_kv(n, Hkv, g, edge=(b == 0)).to(dev)
-        sl = slots_of(bt, b, n).to(dev)
+        sl = slots_of(bt, b, n, P).to(dev)
         if mode == "static":
             K.v2_write(kv, sl, mask.to(dev), 32, pool, P, fmt=fmt)
         else:
@@ -87,9 +87,9 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
         out.fill_(float("nan"))
         if mode == "static":
             K.v2_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, kmask=mask[:Hkv].to(dev),
-                      vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, **tkw)
+                      vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, page=P, **tkw)
         else:
-            K.cb_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start, **tkw)
+            K.cb_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start, page=P, **tkw)
         torch.cuda.synchronize()
         got = out.view(B, HQ, 128).float().cpu().numpy().astype(np.float64)
         valid = np.array([min(kv_start, lens[b]) < lens[b] or (tail is not None and int(tail_len[b]) > 0) for b in range(B)])
@@ -168,6 +168,16 @@ def test_gqa_groups(dev, G, Hkv):
     run_case(dev, "codebook", [130, 31], "konlya2", seed=13, G=G, Hkv=Hkv)
 
 
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
+                                      ("static", "int4a"), ("static", "int2a")])
+def test_pages_of_32_tokens(dev, mode, fmt):
+    """32-token pages: a quad is two pages of four 8-token runs each; ragged lengths, splits, the large workgroup,
+    tail rows and kv_start"""
+    run_case(dev, mode, [1, 31, 32, 33, 65, 200, 1000, 511], fmt, seed=40, P=32)
+    run_case(dev, mode, [700, 120], fmt, seed=41, Hkv=2, nsplit=3, win=(40, 5), kv_start=37, P=32)
+    run_case(dev, mode, [2300, 2100], fmt, seed=42, Hkv=2, nsplit=1, P=32)
+
+
 def test_decode_error_codes(dev):
     from flagrot_releaser_amd import kernels as K
     L = K.lib()
@@ -176,7 +186,7 @@ def test_decode_error_codes(dev):
     base = [zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, None, None, 32, 0, 0, 264, 4, zp, zp, zp, zp, 512, None, None,
             None, 0, 0, None]
     assert L.fr_v2_attn(99, *base, 4, 0) == -4
-    bad_page = list(base); bad_page[8] = 32
+    bad_page = list(base); bad_page[8] = 64
     assert L.fr_v2_attn(5, *bad_page, 4, 0) == -5
     assert L.fr_v2_attn(5, *base, 8, 0) == -7            # gqa 8 without the generalised variant bits
     hd = list(base); hd[17] = 264 | 1024 | 4096
