@@ -132,7 +132,8 @@ template <int QM> struct KRegs {
   static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;   // code words per 16-byte / 8-byte quarter row
   uint32_t kc[4][NW];       // [quarter tg][word]
   uint2 ks;                 // the token's 4 K scale words
-  uint32_t vs[4];           // the token's 4 V scale words (one per group)
+  uint16_t vs[4];           // the token's 4 V scale words (one per group); 16 bits wide so that their widening belongs to the use
+                            // (a widening at the load would be scheduled right behind it and wait for the keys in flight)
 };
 // The value product P' V runs on the matrix pipe: sixteen v_mfma_f32_16x16x32_f16 per quad of pages, rows = 16 V^T
 // entries, columns = (group, head), 32 tokens deep.  An entry word masked in place (eight tokens as fp16 denormal
@@ -443,7 +444,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       const gptr pool = (gptr)p.pool;
       auto chunk_of = [&](int quad) {   // pages past the range read the last page of the range; their tokens are masked
         const int i = min(PPQ * quad + pi, pg1 - pg0 - 1);
-        const int page = i < BT_CACHE ? S.btc[i] : bt[pg0 + i];
+        // The entry comes from LDS.  Past the cached window it is read from memory inside a branch and consumed there:
+        // a select between the two addresses would be one generic load, which waits for every page load in flight.
+        int page = S.btc[min(i, BT_CACHE - 1)];
+        if (__builtin_expect(i >= BT_CACHE, 0)) {
+          const int far = gload<int>(reinterpret_cast<const uint8_t*>(bt + pg0 + i));
+          asm volatile("v_mov_b32 %0, %1" : "=v"(page) : "v"(far));
+        }
         return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
       };
       __builtin_amdgcn_s_setprio(1);
@@ -482,9 +489,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         float sc[4];
         key_phase<QM, K2>(S, cur, p.qscale, sc0, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
-        if (qn < nquad) {            // the key registers are free: the next quad's keys fly during the value phase
-          mine = chunk_of(qn);
-          load_k<QM, P>(cur, mine, pos);
+        // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
+        // path (past the range chunk_of names the range's last page again, a cache hit nobody uses): were they inside
+        // the branch, the wait counts after the join would be those of the path without them, and the value phase
+        // would wait for these loads as well.
+        mine = chunk_of(qn);
+        load_k<QM, P>(cur, mine, pos);
+        if (qn < nquad) {
           // once the counter has run dry, the wavefronts that still hold a quad go first: they all end together
           if (qn + NW >= nquad) __builtin_amdgcn_s_setprio(3);
         } else {
