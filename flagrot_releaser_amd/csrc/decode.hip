@@ -205,12 +205,10 @@ struct WaveState {
 
 // scores of the lane's token against the 4 q heads (log2 domain, unmasked)
 template <int QM, bool K2, class SM>
-DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float sc0, float (&sc)[4]) {
+DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
   const bool full = K2 && (r.vs[0] & 0x8000u);
-#pragma unroll
-  for (int h = 0; h < 4; ++h) sc[h] = sc0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
@@ -424,7 +422,11 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       auto draw = [&]() {
         int t = 0;
         if (lane == 0)
-          t = dyn ? (__hip_atomic_fetch_add(ctr, DRAW_BATCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & DRAW_MASK) : atomicAdd(&S.next, 1);
+          // (shared counter: one increment = DRAW_BATCH quads.  An increment and not an addition: the compiler rewrites
+          // additions into a wave-wide reduction whose broadcast waits for the counter's round trip on the spot)
+          // what comes back is unpacked where it is used (undraw): any arithmetic on it here would wait for it here
+          t = dyn ? static_cast<int>(__builtin_amdgcn_atomic_inc32(reinterpret_cast<unsigned*>(ctr), 0xFFFFFFFFu, __ATOMIC_RELAXED, "agent"))
+                  : atomicAdd(&S.next, 1);
         return t;
       };
       int take = 0;
@@ -468,26 +470,34 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         int qn;
         if (more > 0) { qn = nextq++; --more; }
         else {
-          qn = __builtin_amdgcn_readfirstlane(take) + nworker;
+          // (the draw made an iteration ago is read here and not before: without the opaque copy its broadcast is
+          // moved up to the draw itself, which then waits for the counter's round trip on the spot)
+          int drawn = take;
+          asm volatile("" : "+v"(drawn));
+          drawn = __builtin_amdgcn_readfirstlane(drawn);
+          qn = (dyn ? (drawn & DRAW_MASK) * DRAW_BATCH : drawn) + nworker;
           take = draw();
           if (dyn) { nextq = qn + 1; more = DRAW_BATCH - 1; }
         }
         VRegs<QM> vr;                // this quad's V^T entries: in flight during the key phase
+        const uint8_t* ch[4];
         {
           const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
-          const uint8_t* ch[4];
 #pragma unroll
           for (int k = 0; k < 4; ++k) {             // (32-token pages: entries 2, 3 repeat page 1 and are not read)
             const uint32_t lo32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp), (P * k) & 63);
             const uint32_t hi32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp >> 32), (P * k) & 63);
             ch[k] = reinterpret_cast<const uint8_t*>((static_cast<unsigned long long>(hi32) << 32) | lo32);
           }
-          load_v<QM, P>(vr, ch, lane);
         }
         const int tok = (pg0 + PPQ * qi + pi) * P + pos;
         const bool valid = tok >= lo && tok < hi;
-        float sc[4];
-        key_phase<QM, K2>(S, cur, p.qscale, sc0, sc);
+        // (The scheduler moves the requests for the value entries below the key phase, where the code words' registers
+        // are free.  Pinning them, or half of them, above or inside it costs registers the loop does not have at four
+        // wavefronts per SIMD, and gains nothing at three: measured.)
+        float sc[4] = {sc0, sc0, sc0, sc0};
+        load_v<QM, P>(vr, ch, lane);
+        key_phase<QM, K2>(S, cur, p.qscale, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
         // path (past the range chunk_of names the range's last page again, a cache hit nobody uses): were they inside
