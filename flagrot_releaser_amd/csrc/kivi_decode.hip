@@ -228,9 +228,15 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
                              pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNK, lane);
   for (; gi < g_end; gi += 4) {
     const bool full = gi * 32 >= t0 && gi * 32 + 32 <= t1;     // every token of the group is inside the range (wave uniform)
+    // The next group is requested on every path (past the range: the range's last group again, a cache hit nobody
+    // uses).  Were the requests inside a branch, the wait counts after the join would be those of the path without
+    // them, and this group's first use would wait for the next group's data as well.
     GroupRegs nxt;
-    if (gi + 4 < g_end) load_group(nxt, pool + (static_cast<long long>(btb[2 * (gi + 4)]) * Hkv + h) * CHUNK,
-                                   pool + (static_cast<long long>(btb[2 * (gi + 4) + 1]) * Hkv + h) * CHUNK, lane);
+    {
+      const int gn = min(gi + 4, g_end - 1);
+      load_group(nxt, pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNK,
+                 pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNK, lane);
+    }
     // ---- group flags; q' * scale and q' * min strips: lane = channel pair
     {
       const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = __builtin_amdgcn_readlane(cur.km.y, 0),
