@@ -84,6 +84,9 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   p.opart = opart; p.mlpart = mlpart; p.counter = counter;
   const int gt = ((variant & GEN) && (variant & GT8)) ? 8 : 4;
   const int ntile = (gqa + 3) / 4, nct = (gqa + gt - 1) / gt;
+  // a counter slot must hold a whole number of 4-head tiles: with tiles of 8 and 9..12 heads (3 tiles, 2 slots) the
+  // kernel would index three counter words where the caller sized two
+  if (ntile % nct != 0) return fail(-7, "fr_v2_attn: the 8-head tile variant needs gqa <= 8 (or a multiple of 8)");
   p.counter_div = ntile / nct;
   p.out = out; p.o_bs = o_bs;
   p.tail = tail; p.tail_len = tail_len; p.tail_idx = tail_idx; p.tail_bs = tail_bs; p.tail_ts = tail_ts;

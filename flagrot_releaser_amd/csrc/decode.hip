@@ -622,8 +622,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   if (nparts > 1) {
     // Partials cross workgroups (and XCDs, each with its own L2) through device-scope relaxed atomic stores / loads,
     // which are write-through / read-through; a device-scope fence here would write back and invalidate the whole
-    // L2 once per workgroup.  Order: stores acknowledged (workgroup release = wait for the store counter), barrier,
-    // ticket; the last arriver reads after its ticket returned.
+    // L2 once per workgroup.  Order: every storing wavefront waits until its stores are acknowledged (an explicit
+    // wait on the vector memory counter, which counts stores on this target: a workgroup-scope fence emits no such
+    // wait), barrier, ticket; the last arriver reads (device-scope loads) after its ticket has returned.
     if (act) {
       float* op = p.opart + part_id * 512 + oh * 128 + 2 * lane;
       __hip_atomic_store(op, po[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -633,6 +634,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         __hip_atomic_store(p.mlpart + part_id * 8 + 2 * oh + 1, pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wavefront's partial stores have been acknowledged
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) {    // every draw of this workgroup precedes its ticket: the last arriver may clear the slot
