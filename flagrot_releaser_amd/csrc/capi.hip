@@ -3,6 +3,7 @@
 #include <cstdlib>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/flagrot_kernels.h"
 #include "fr_common.hpp"
@@ -180,6 +181,87 @@ int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* bl
   return fr_v2_attn(fmt, q, q_bs, pool, block_table, bt_stride, seq_lens, B, Hkv, page, nsplit, chunk, qscale, nullptr,
                     nullptr, 32, 0, 0, 264, stages, opart, mlpart, counter, out, o_bs, tail, tail_len, tail_idx,
                     tail_bs, tail_ts, stream, 4, kv_start);
+}
+
+// ---- the entry point that allocates nothing --------------------------------------------------------------------
+// Split partials, their (max, sum) pairs and the ticket / draw counters of fr_cb_attn_noalloc live in this array
+// instead of a caller-owned workspace.  Every GPU the library runs on holds its own copy, at its own address, until
+// the process ends.  Host code must never use the array's name as a device address: the address is asked for once
+// per device (scratch_of) and only that pointer is handed to kernels.
+}  // extern "C"
+namespace {
+constexpr int NA_MAX_PARTS = FR_NOALLOC_MAX_PARTS;            // partials of 4 heads x 128 floats
+constexpr size_t NA_OPART = size_t(NA_MAX_PARTS) * 512 * 4;   // bytes
+constexpr size_t NA_MLPART = size_t(NA_MAX_PARTS) * 8 * 4;
+constexpr size_t NA_COUNTER = size_t(NA_MAX_PARTS) * 4;
+static __device__ __align__(256) unsigned char scratch[NA_OPART + NA_MLPART + NA_COUNTER];
+
+constexpr int NA_MAX_DEV = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[NA_MAX_DEV] = {nullptr};
+
+// device address of `scratch` on the current device (asked for once per device), or null with the error text set
+unsigned char* scratch_of() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NA_MAX_DEV) {
+    (void)hipGetLastError();
+    set_error("fr_cb_attn_noalloc: no current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      char buf[200];
+      std::snprintf(buf, sizeof(buf), "fr_cb_attn_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      (void)hipGetLastError();
+      set_error(buf);
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+  }
+  return g_scratch_ptr[dev];
+}
+
+// a fill kernel and not hipMemsetAsync: memset nodes recorded into a HIP graph are not reliable on replays
+__global__ void k_clear_words(int* w, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) w[i] = 0;
+}
+}  // namespace
+extern "C" {
+
+int fr_cb_attn_noalloc(const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
+                       const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale, int kind,
+                       void* out, long long o_bs, const void* tail, const int* tail_len, const int* tail_idx,
+                       long long tail_bs, long long tail_ts, void* stream, int gqa, int kv_start) {
+  if (B <= 0) return 0;
+  const int fmt = fmt_of_kind(kind);
+  if (fmt < 0) return fail(-4, "fr_cb_attn_noalloc: kind must be 6 (konly), 10 (konlya) or 11 (konlya2)");
+  if (gqa <= 0) gqa = 4;
+  if (gqa > 64 || Hkv <= 0 || nsplit < 1) return fail(-7, "fr_cb_attn_noalloc: bad gqa / Hkv / nsplit");
+  const long long ntile = (gqa + 3) / 4;
+  const long long parts = static_cast<long long>(B) * Hkv * ntile * (nsplit + 1);
+  if (parts > NA_MAX_PARTS) {
+    char buf[200];
+    std::snprintf(buf, sizeof(buf), "fr_cb_attn_noalloc: B*Hkv*ceil(gqa/4)*(nsplit+1) = %lld partials exceed the built-in "
+                  "workspace of %d", parts, NA_MAX_PARTS);
+    return fail(-2, buf);
+  }
+  unsigned char* base = scratch_of();
+  if (base == nullptr) return -1;
+  float* opart = reinterpret_cast<float*>(base);
+  float* mlpart = reinterpret_cast<float*>(base + NA_OPART);
+  int* counter = reinterpret_cast<int*>(base + NA_OPART + NA_MLPART);
+  // The counters are left at zero by every completed call; they are cleared all the same, so that a call that was cut
+  // short (a failed launch, a device reset of another context) cannot poison the next one.
+  const int nctr = static_cast<int>(static_cast<long long>(B) * Hkv * ntile);
+  hipLaunchKernelGGL(k_clear_words, dim3((nctr + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), counter, nctr);
+  if (hipPeekAtLastError() != hipSuccess) return launched(-1, "fr_cb_attn_noalloc (clear)");
+  return fr_v2_attn(fmt, q, q_bs, pool, block_table, bt_stride, seq_lens, B, Hkv, page, nsplit, chunk, qscale, nullptr,
+                    nullptr, 32, 0, 0, 264 | GEN, 4, opart, mlpart, counter, out, o_bs, tail, tail_len, tail_idx,
+                    tail_bs, tail_ts, stream, gqa, kv_start);
 }
 
 int fr_cb_occupancy(int kind, int variant, int stages, int page) {

@@ -89,6 +89,7 @@ def lib():
         "fr_cb_chunk_bytes": [I, I],
         "fr_cb_write_smem": [I, I, I],
         "fr_head_fwht": [P, LL, P, LL, I, I, P, F, P, I],
+        "fr_cb_attn_noalloc": [P, LL, P, P, I, P, I, I, I, I, I, F, I, P, LL, P, P, P, LL, LL, P, I, I],
     }
     for name, args in sig.items():
         fn = getattr(L, name)
@@ -100,7 +101,8 @@ def lib():
 
 EXPORTS = ("fr_abi_version", "fr_v2_attn", "fr_v2_write", "fr_v2_occupancy", "fr_v2_chunk_bytes", "fr_cb_nsg",
            "fr_cb_write", "fr_cb_write3", "fr_w3_static_write", "fr_cb_attn", "fr_cb_occupancy", "fr_cb_chunk_bytes",
-           "fr_cb_write_smem", "fr_last_error", "fr_head_fwht")
+           "fr_cb_write_smem", "fr_last_error", "fr_head_fwht", "fr_cb_attn_noalloc")
+NOALLOC_MAX_PARTS = 8192     # FR_NOALLOC_MAX_PARTS of include/flagrot_kernels.h
 
 
 def _check(rc: int, what: str):
@@ -405,6 +407,23 @@ def cb_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kind
             out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
             0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), int(kv_start))
     return _launcher(lib().fr_cb_attn, args, "fr_cb_attn", bound)
+
+
+def cb_attn_noalloc(q, pool, block_table, seq_lens, out, nsplit, chunk, qscale, kind, tail=None, tail_len=None,
+                    tail_idx=None, tail_bs=None, tail_ts=None, page=16, kv_start=0, bound=False):
+    """cb_attn for callers that cannot allocate: no workspace argument, the split partials live in an array built
+    into the library (shared by all calls on the GPU: do not overlap calls).  Raises when
+    B * Hkv * ceil(G / 4) * (nsplit + 1) exceeds NOALLOC_MAX_PARTS.  No counterpart in the reference front end."""
+    B, Hq, Dh = q.shape
+    Hkv = pool.shape[1]
+    G = Hq // Hkv
+    assert kind in K2 and Hq == G * Hkv and Dh == D, f"{kind}: key-only 2x2 kinds, head dim 128 only"
+    assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
+    args = (q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, CB_KINDS[kind], out.data_ptr(), out.stride(0),
+            _ptr(tail), _ptr(tail_len), _ptr(tail_idx), 0 if tail is None else tail_bs,
+            0 if tail is None else tail_ts, _stream(), G, int(kv_start))
+    return _launcher(lib().fr_cb_attn_noalloc, args, "fr_cb_attn_noalloc", bound)
 
 
 def head_fwht(x, flags, scale, out=None):

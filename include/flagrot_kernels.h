@@ -80,6 +80,19 @@ int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* bl
                const void* tail, const int* tail_len, const int* tail_idx, long long tail_bs, long long tail_ts,
                void* stream, int kv_start);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): fr_cb_attn for any gqa (<= 64) without the workspace
+ * arguments.  Partials, (max, sum) pairs and counters live in an array built into the library (about 16.3 MiB per GPU,
+ * held until the process ends); the call allocates nothing and clears its counters itself.  Limit:
+ * B*Hkv*ceil(gqa/4)*(nsplit+1) <= FR_NOALLOC_MAX_PARTS, else -2 with a message in fr_last_error().  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are safe.
+ * The first call on a device looks the array's address up (no stream work, no allocation). */
+#define FR_NOALLOC_MAX_PARTS 8192
+int fr_cb_attn_noalloc(const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
+                       const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale, int kind,
+                       void* out, long long o_bs, const void* tail, const int* tail_len, const int* tail_idx,
+                       long long tail_bs, long long tail_ts, void* stream, int gqa, int kv_start);
+
 /* flagrot_capi.cu:151-153 */
 int fr_cb_occupancy(int kind, int variant, int stages, int page);
 int fr_cb_chunk_bytes(int kind, int page);
