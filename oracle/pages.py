@@ -24,7 +24,10 @@ INT2 chunk (80 P bytes):
                 bit 4 r + 2 b = token 8 c8 + 2 i + b
   [64P, 72P)    K scale words, [72P, 80P) V scale words, as INT4.
 
-Parity status: pinned (hand-derived byte positions, pack/parse round trips, whole-pool garbage preservation).
+Parity status: PINNED by vectors the reference's own parsers wrote (vllm_flagrot/kernels.py parse_pages /
+dequant_v2_pages / dequant_cb_pages on pools of random bytes with packed tokens, six formats x pages of 16 and 32
+tokens: tests/golden/pages_*.npz, tests/test_oracle_golden.py), plus hand-derived byte positions, pack/parse round
+trips and whole-pool garbage preservation (tests/test_oracle_pages.py).
 """
 from __future__ import annotations
 
