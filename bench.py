@@ -1,10 +1,15 @@
 """Headline benchmark: paged FlagRot decode attention on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2|kivi|mq]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload int4|int2|kivi|mq] [--only]
 
 A step is one decode layer-step: one launch of the paged decode attention (through the C ABI of
 libflagrot_kernels.so) over the whole batch, on a synthetic cache that is already resident in HBM.  Successive steps
 cycle through several distinct copies of the cache so that no page is served from the last-level cache.
+
+Timing (the reference's method, scripts/bench_attn_int2.py:42-64 of the reference): after W warm-up steps and a
+clock-settling run, the K steps are captured into ONE HIP graph, the graph is replayed 7 times with an event on either
+side on the launch stream, and the figures come from the MEDIAN replay (K steps).  The same K steps launched eagerly
+(arguments bound once) are timed beside it (`eager_us`): they carry the host's launch gap.
 
 Workloads (BASELINE.json configs):
   int4  configs[1]: INT4 FlagRot (key-only 2x2 codebook, kind konlya), Llama-3.1-8B GQA shape 32q/8kv, d=128,
@@ -16,9 +21,12 @@ Workloads (BASELINE.json configs):
   mq    configs[4]: prefix-cached multi-query prefill over INT4 pages (libflagrot_mq.so, the MFMA path): 4 requests x
         512 new tokens over a 16384-token cached prefix, Qwen-32B shape 64q/8kv, d=128; --mq-fmt konlya | int4a.
         value = TFLOP/s of the attention (4 x 128 flops per visible (row, key) pair), roofline bound "mfma".
-Prints ONE JSON line: value = achieved GB/s of page bytes (the reference's convention: B * L * Hkv * bytes per token),
-with `roofline` (HBM, measured with events on the launch stream) and `cpu_baseline` (the numpy oracle's
-dequantise-then-attend path, timed on the host on configs[0]'s shape).
+Prints ONE JSON line for the chosen workload: value = achieved GB/s of page bytes (the reference's convention:
+B * L * Hkv * bytes per token), `roofline`, `cpu_baseline` (the numpy oracle's writer and dequantise-then-attend legs
+timed on the host on configs[0]'s shape, one thread) and `checked` (sampled sequences of the timed launch's output
+compared with the oracle, outside the timed region).  Without --workload (the default run) the other three workloads
+are run as short legs as well and reported under `workloads`, and configs[1] is also run with the split plan the
+reference's own host planner makes from this library's occupancy answer (`reference_planner`).
 """
 from __future__ import annotations
 
@@ -35,7 +43,11 @@ if ROOT not in sys.path:
 
 LOG2E = 1.4426950408889634
 PEAK_HBM_GBPS = 8000.0
+PEAK_F16_TFLOPS = 2500.0
 P, HKV, G, DH = 16, 8, 4, 128
+ATOL, RTOL = 2e-3, 1e-2          # the bar of the attention outputs: |out - ref| <= ATOL + RTOL |ref|
+REPLAYS = 7
+TRAFFIC_FILE = "profiles/decode_traffic.json"
 
 
 def synth_kv(T, g, dev, torch, outliers=4, gain=8.0, mu=None):
@@ -64,6 +76,54 @@ def settle(torch, launch, busy_ms=40.0, batch=16):
         done += e0.elapsed_time(e1)
 
 
+def timed(torch, launch, steps, warmup, eager=None):
+    """launch(i): step i on torch's current stream.  W warm-up steps, clock settling, then (a) the K steps eagerly
+    (through `eager(i)` when given: the same step with pre-bound arguments) and (b) the K steps as one HIP graph
+    replayed REPLAYS times.  Returns per-step microseconds: graph median / min replay, eager average."""
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    run = eager or launch
+    settle(torch, run)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        run(i)
+    e1.record()
+    torch.cuda.synchronize()
+    eager_us = e0.elapsed_time(e1) / steps * 1e3
+    cur = torch.cuda.current_stream()
+    side = torch.cuda.Stream()
+    side.wait_stream(cur)
+    with torch.cuda.stream(side):
+        launch(0)                               # the capture stream's first use of every library, outside the capture
+    cur.wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(steps):
+            launch(i)
+    graph.replay()
+    torch.cuda.synchronize()
+    settle(torch, run)
+    reps = []
+    for _ in range(REPLAYS):
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        reps.append(e0.elapsed_time(e1) / steps * 1e3)
+    reps.sort()
+    del graph
+    return {"graph_us": reps[len(reps) // 2], "graph_min_us": reps[0], "graph_max_us": reps[-1], "eager_us": eager_us}
+
+
+def within(got, ref):
+    """worst |got - ref| / (ATOL + RTOL |ref|) over all elements (<= 1: inside the bar)"""
+    import numpy as np
+    return float((np.abs(got - ref) / (ATOL + RTOL * np.abs(ref))).max())
+
+
 def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192):
     """fills one pool with B sequences of L tokens through the selecting writer; returns pool, block table, calib."""
     g = torch.Generator(device=dev).manual_seed(seed)
@@ -86,50 +146,188 @@ def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192):
     return pool, bt, CT, co, time.perf_counter() - t0
 
 
+def host_threads():
+    try:
+        from threadpoolctl import threadpool_limits
+        return threadpool_limits(limits=1)
+    except Exception:      # no threadpoolctl: numpy runs with whatever its BLAS was built with
+        import contextlib
+        return contextlib.nullcontext()
+
+
 def cpu_baseline(torch, K, dev):
-    """the oracle's decode path (page parse + dequantise + inverse transforms + fp64 softmax attention) on
-    configs[0]'s shape: batch 1, context 2048, 32q/8kv; the cache bytes come from the HIP writer."""
+    """the oracle's two legs on configs[0]'s shape (batch 1, context 2048, 32q/8kv, INT4 groups of 32, uniform
+    calibration weights), one host thread: (i) the selecting writer for the 2048 tokens x 8 KV heads (K and V),
+    (ii) one decode step = page parse + dequantise + inverse transforms + fp64 softmax attention."""
     import numpy as np
     from oracle import attend as A
+    from oracle import quant as Q
     kind, L = "konly", 2048
-    pool, bt, CT, co, _ = build_cache(torch, K, dev, kind, 1, L, seed=0)
-    g = torch.Generator().manual_seed(0)
-    q = torch.randn(1, G * HKV, DH, generator=g).bfloat16()
-    qb = q.view(torch.int16).numpy().view(np.uint16)
-    hp, hbt = pool.cpu().numpy(), bt.cpu().numpy()
-    ts = []
-    for _ in range(4):
+    g = torch.Generator(device=dev).manual_seed(0)
+    kv = synth_kv(L, g, dev, torch).cpu()
+    kvb = kv.view(torch.int16).numpy().view(np.uint16)
+    C = np.stack([np.eye(DH, dtype=np.float32)] * HKV)
+    with host_threads():
         t0 = time.perf_counter()
-        A.decode_reference(qb, hp, kind, P, hbt, [L], 1 / math.sqrt(DH))
-        ts.append(time.perf_counter() - t0)
+        Q.k2_encode(kvb, C, kind)
+        t_write = time.perf_counter() - t0
+        pool, bt, CT, co, _ = build_cache(torch, K, dev, kind, 1, L, seed=0)
+        gq = torch.Generator().manual_seed(0)
+        q = torch.randn(1, G * HKV, DH, generator=gq).bfloat16()
+        qb = q.view(torch.int16).numpy().view(np.uint16)
+        hp, hbt = pool.cpu().numpy(), bt.cpu().numpy()
+        ts = []
+        for _ in range(4):
+            t0 = time.perf_counter()
+            A.decode_reference(qb, hp, kind, P, hbt, [L], 1 / math.sqrt(DH))
+            ts.append(time.perf_counter() - t0)
     t = sorted(ts[1:])[len(ts[1:]) // 2]
     nbytes = L * HKV * 144
-    try:
-        from threadpoolctl import threadpool_info
-        cores = max([i.get("num_threads", 1) for i in threadpool_info()] + [1])
-    except Exception:
-        cores = 1
-    return {"value": round(nbytes / t / 1e9, 6), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"numpy oracle decode_reference, B=1 L={L} 32q/8kv INT4 (konly) pages = {nbytes} page bytes, "
-                      f"median of 3 after 1 warm-up: {t * 1e6:.0f} us per layer-step; host has {os.cpu_count()} cpus"}
+    return {"value": round(nbytes / t / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"numpy oracle on configs[0] (B=1 L={L} 32q/8kv INT4 konly, page 16), one thread of the host's "
+                      f"{os.cpu_count()} cpus: decode step (decode_reference, {nbytes} page bytes) median of 3 after 1 "
+                      f"warm-up = {t * 1e6:.0f} us per layer-step; writer (k2_encode, {L} tokens x {HKV} KV heads, K and V) "
+                      f"one run = {t_write:.2f} s = {t_write / L * 1e6:.0f} us per token",
+            "decode_us_per_layer_step": round(t * 1e6, 0), "writer_us_per_token": round(t_write / L * 1e6, 1)}
 
 
-def main_kivi(args, torch, dev):
+def reference_plan(B, Lmax, Hkv, slots):
+    """the split plan a caller written against the reference makes for a key-only kind: smallest modelled cost
+    ceil(B Hkv ns / slots) (chunk + 1024) + 4 ns [ns > 1] over chunks of whole 64-token blocks of at most 8192 tokens,
+    slots = (what fr_cb_occupancy returns) x (multi_processor_count); integrations/vllm_flagrot/vllm_flagrot/
+    kernels.py:247-265 of the reference."""
+    best = None
+    for ns in range(max(1, math.ceil(Lmax / 8192)), min(512, math.ceil(Lmax / 64)) + 1):
+        chunk = math.ceil(Lmax / ns / 64) * 64
+        if chunk > 8192:
+            continue
+        nse = math.ceil(Lmax / chunk)
+        if best is not None and nse == best[1]:
+            continue
+        cost = math.ceil(B * Hkv * nse / slots) * (chunk + 1024) + (4 * nse if nse > 1 else 0)
+        if best is None or cost < best[0] - 1e-9:
+            best = (cost, nse, chunk)
+    return best[1], best[2]
+
+
+# ------------------------------------------------------------------------------------------------ FlagRot decode
+def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
+    """configs[1] / configs[2] through libflagrot_kernels.so.  Returns {plan: result dict}."""
+    import numpy as np
+    from flagrot_releaser_amd import kernels as K
+    from oracle import attend as A
+    K.lib()
+    if workload == "int4":
+        kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144
+        name = "configs[1]: INT4 FlagRot konlya paged decode, Llama-3.1-8B GQA 32q/8kv d=128, B=32 L=8192 page=16"
+    else:
+        kind, B, L, S, W, cell = "konlya2", 64, 16384, 4, 128, 80
+        name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
+                "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
+    g = torch.Generator(device=dev).manual_seed(1)
+    kmu = None
+    if workload == "int2":
+        kmu = (2.0 * torch.randn(HKV, DH, generator=g, device=dev)).contiguous()
+    pool, bt, CT, co, fill_s = build_cache(torch, K, dev, kind, B, L, seed=1, kmu=kmu)
+    ncopy = max(1, min(8, int(6e9 // pool.numel())))
+    pools = [pool] + [pool.clone() for _ in range(ncopy - 1)]
+    q = torch.randn(B, G * HKV, DH, generator=g, device=dev).bfloat16()
+    out = torch.zeros(B, G * HKV * DH, dtype=torch.bfloat16, device=dev)
+    T = S + W
+    tkw = {}
+    Lpages = L - W if T else L                      # the newest W tokens live in the BF16 ring, not in pages
+    seq = torch.full((B,), Lpages, dtype=torch.int32, device=dev)
+    ring = None
+    if T:
+        ring = torch.randn(B + 1, T, 2 * HKV, DH, generator=g, device=dev).bfloat16()
+        tkw = dict(tail=ring, tail_len=torch.full((B,), T, dtype=torch.int32, device=dev),
+                   tail_idx=torch.arange(B, dtype=torch.int32, device=dev), tail_bs=ring.stride(0),
+                   tail_ts=ring.stride(1), kv_start=S)
+    scale = LOG2E / math.sqrt(DH)
+    page_bytes = B * (Lpages - S) * HKV * cell
+    tail_bytes = B * T * 2 * HKV * DH * 2
+    alg_bytes = page_bytes + tail_bytes
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    results = {}
+    for plan in plans:
+        if plan == "own":
+            ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None)
+        else:      # "reference": the reference front end's cost model fed with this library's occupancy answer
+            occ = K.lib().fr_cb_occupancy(K.CB_KINDS[kind], 0, K.STAGES, P)
+            ns, ch = reference_plan(B, Lpages, HKV, max(1, occ) * cus)
+        ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
+
+        def step(i):
+            K.cb_attn(q, pools[i % ncopy], bt, seq, out, ns, ch, ws, scale, kind, **tkw)
+
+        # eager leg: arguments bound once (checks and pointer marshalling done once, as under graph capture)
+        bound = [K.cb_attn(q, pools[j], bt, seq, out, ns, ch, ws, scale, kind, bound=True, **tkw) for j in range(ncopy)]
+        t = timed(torch, step, steps, warmup, eager=lambda i: bound[i % ncopy]())
+        us = t["graph_us"]
+        gbps = alg_bytes / (us * 1e-6) / 1e9
+        # outside the timed region: sampled sequences of the output of one more launch against the oracle
+        out.zero_()
+        step(0)
+        torch.cuda.synchronize()
+        rows = sorted({0, B // 2 + 1, B - 1})
+        idx = bt[rows].long().reshape(-1)
+        mp = pools[0].index_select(0, idx).cpu().numpy()
+        mbt = np.arange(idx.numel(), dtype=np.int32).reshape(len(rows), -1)
+        qb = q[rows].cpu().view(torch.int16).numpy().view(np.uint16)
+        tb = None if ring is None else ring[rows].cpu().view(torch.int16).numpy().view(np.uint16)
+        ref = A.decode_reference(qb, mp, kind, P, mbt, [Lpages] * len(rows), 1 / math.sqrt(DH), tail=tb,
+                                 tail_len=None if tb is None else [T] * len(rows), kv_start=S)
+        got = out[rows].view(len(rows), G * HKV, DH).float().cpu().numpy().astype(np.float64)
+        worst = within(got, ref)
+        results[plan] = {
+            "workload": name, "us_per_layer_step": round(us, 2), "GBps": round(gbps, 1),
+            "frac": round(gbps / PEAK_HBM_GBPS, 4), "nsplit": ns, "chunk": ch,
+            "graph_min_us": round(t["graph_min_us"], 2), "graph_max_us": round(t["graph_max_us"], 2),
+            "eager_us": round(t["eager_us"], 2), "algorithmic_bytes_per_launch": alg_bytes,
+            "cache_copies_cycled": ncopy, "steps": steps, "sink": S, "window": W,
+            "checked": bool(worst <= 1.0), "check": f"sequences {rows} x all {G * HKV} heads vs the fp64 oracle: worst "
+                                                    f"|err| / (2e-3 + 1e-2 |ref|) = {worst:.3f}",
+        }
+    # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
+    kv_new = synth_kv(B, g, dev, torch, mu=kmu)
+    slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
+    for _ in range(3):
+        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
+    e1.record()
+    torch.cuda.synchronize()
+    first = results[plans[0]]
+    first["writer"] = {"decode_step_us": round(e0.elapsed_time(e1) / 20 * 1e3, 2), "decode_step_tokens": B,
+                       "prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * L,
+                       "note": "prefill_fill_s includes synthetic input generation"}
+    return results
+
+
+# ------------------------------------------------------------------------------------------------ KIVI decode
+def run_kivi(args, torch, dev, steps, warmup):
     """configs[3] through libflagrot_kivi.so: fill by the value writer + key group encoder, time kv_attn."""
+    import numpy as np
     from flagrot_releaser_amd import kivi as KV
+    from oracle import kivi as OK
+    from oracle import quant as Q
     KV.lib()
+    f8 = bool(args.f8)
     B, L, Gq, W, NQ, outl, gain = 16, 32768, 8, 128, 64, 8, 12.0
-    name = ("configs[3]: KIVI-style FlagRot INT2 paged decode (per-channel keys over 32-token groups, per-token values), "
-            "128-token BF16 residual, Qwen-32B GQA 64q/8kv d=128, B=16 L=32768 page=16")
-    CB = KV.chunk_bytes(DH)
+    name = ("configs[3]: KIVI-style FlagRot INT2 paged decode (per-channel keys over 32-token groups, per-token values"
+            + (", FP8 meta" if f8 else "") + "), 128-token BF16 residual, Qwen-32B GQA 64q/8kv d=128, B=16 L=32768 page=16")
+    CB = KV.chunk_bytes(DH, f8)
     g = torch.Generator(device=dev).manual_seed(3)
     Lp = L - W
     npages = B * (Lp // P)
     pool = torch.zeros(npages + 16, HKV, CB, dtype=torch.uint8, device=dev)
     bt = torch.randperm(npages + 16, generator=g, device=dev)[:npages].int().view(B, -1).contiguous()
-    co = (0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)).contiguous()
-    qs = torch.randn(HKV, NQ, DH, generator=g, device=dev).contiguous()
-    lz = torch.full((HKV, NQ), 6.0, device=dev)
+    co = torch.rand(HKV, DH, generator=g, device=dev).contiguous()
+    qs = (0.3 * torch.randn(HKV, NQ, DH, generator=g, device=dev)).contiguous()
+    lz = torch.full((HKV, NQ), 5.0, device=dev)
     t0 = time.perf_counter()
     for b in range(B):
         for s0 in range(0, Lp, 8192):
@@ -137,9 +335,9 @@ def main_kivi(args, torch, dev):
             kv = synth_kv(n, g, dev, torch, outliers=outl, gain=gain)
             pos = torch.arange(s0, s0 + n, device=dev)
             slots = bt[b].long()[pos // P] * P + pos % P
-            KV.v_write(kv, slots, co, None, pool, HKV, DH)
+            KV.v_write(kv, slots, co, None, pool, HKV, DH, f8=f8)
             KV.k_encode(kv, torch.arange(n, device=dev).view(-1, 32), slots.view(-1, 32).contiguous(), qs, lz,
-                        1 / math.sqrt(DH), pool, HKV, DH)
+                        1 / math.sqrt(DH), pool, HKV, DH, f8=f8)
     torch.cuda.synchronize()
     fill_s = time.perf_counter() - t0
     ncopy = max(1, min(8, int(6e9 // pool.numel())))
@@ -160,53 +358,47 @@ def main_kivi(args, torch, dev):
 
     def step(i):
         KV.attn(q, pools[i % ncopy], bt, cached, out, ns, ch, ws, scale, 0, Gq, ring=ring, tail_len=tail_len,
-                tail_idx=tail_idx, T=W)
+                tail_idx=tail_idx, T=W, f8=f8)
 
-    for i in range(args.warmup):
-        step(i)
-    settle(torch, step)              # clocks out of idle
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    ev[0].record()
-    for i in range(args.steps):
-        step(i)
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
-    ms_per_step = ev[0].elapsed_time(ev[-1]) / args.steps
+    t = timed(torch, step, steps, warmup)
+    us = t["graph_us"]
     alg_bytes = B * Lp * HKV * (CB // P) + B * W * 2 * HKV * DH * 2
-    gbps = alg_bytes / (ms_per_step * 1e-3) / 1e9
-    traffic = None
-    try:
-        with open(os.path.join(ROOT, "profiles", "decode_traffic.json")) as f:
-            traffic = json.load(f).get("kivi", {}).get("traffic_bytes")
-    except OSError:
-        pass
-    res = {
-        "metric": "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)",
-        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 6), "us_per_layer_step": round(ms_per_step * 1e3, 2),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 codes, f32 products and accumulate",
-        "data": "synthetic", "config": {"workload": name, "nsplit": ns, "chunk": ch, "cache_copies_cycled": ncopy,
-                                         "sink": 0, "window": W},
-        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": traffic,
-                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(ms_per_step * 1e3, 2),
-                     "median_launch_us": round(per[len(per) // 2] * 1e3, 2), "min_launch_us": round(per[0] * 1e3, 2),
-                     "note": "one step = kv_attn = the split kernel + the merge kernel"},
-        "writer": {"prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * Lp,
-                   "note": "value writer + key group encoder (64 calibration queries), includes synthetic input generation"},
-    }
-    print(json.dumps(res))
+    gbps = alg_bytes / (us * 1e-6) / 1e9
+    # check: one sequence, all heads, against fp64 attention over the oracle's dequantised pages + ring rows
+    out.zero_()
+    step(0)
+    torch.cuda.synchronize()
+    b = B - 1
+    ch_np = pools[0].index_select(0, bt[b].long()).cpu().numpy()
+    Kd, Vd = OK.dequant_groups(ch_np, DH, f8=f8)
+    rg = Q.bf16_to_f32(ring.view(B + 1, W, 2 * HKV, DH)[b].cpu().view(torch.int16).numpy().view(np.uint16)).astype(np.float64)
+    qf = Q.bf16_to_f32(q[b].cpu().view(torch.int16).numpy().view(np.uint16)).astype(np.float64)
+    ref = OK.attention_reference(qf, Kd, Vd, 0, Lp, rg[:, :HKV], rg[:, HKV:], Gq, 1 / math.sqrt(DH))
+    got = out[b].view(Gq * HKV, DH).float().cpu().numpy().astype(np.float64)
+    worst = within(got, ref)
+    return {"workload": name, "us_per_layer_step": round(us, 2), "GBps": round(gbps, 1),
+            "frac": round(gbps / PEAK_HBM_GBPS, 4), "nsplit": ns, "chunk": ch,
+            "graph_min_us": round(t["graph_min_us"], 2), "graph_max_us": round(t["graph_max_us"], 2),
+            "eager_us": round(t["eager_us"], 2), "algorithmic_bytes_per_launch": alg_bytes,
+            "cache_copies_cycled": ncopy, "steps": steps, "sink": 0, "window": W,
+            "checked": bool(worst <= 1.0), "check": f"sequence {b} x all {Gq * HKV} heads vs fp64 attention over the "
+                                                    f"oracle's dequantised pages: worst |err| / (2e-3 + 1e-2 |ref|) = {worst:.3f}",
+            "note": "one step = kv_attn = the split kernel + the merge kernel",
+            "writer": {"prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * Lp,
+                       "note": f"value writer + key group encoder ({NQ} calibration queries), includes synthetic input generation"}}
 
 
-def main_mq(args, torch, dev):
+# ------------------------------------------------------------------------------------------------ MQ prefill
+def run_mq(args, torch, dev, steps, warmup, fmt):
     """configs[4] through libflagrot_mq.so: one step = frmq_prep_q + frmq_attn + frmq_merge of one layer."""
+    import numpy as np
     from flagrot_releaser_amd import kernels as K
     from flagrot_releaser_amd import prefill_mq as MQ
+    from oracle import attend as A
+    from oracle import mq as OM
     MQ.lib()
     R, NQ, PRE, Gq = 4, 512, 16384, 8
     L = PRE + NQ
-    fmt = args.mq_fmt
     k2 = fmt == "konlya"
     name = (f"configs[4]: multi-query prefill over INT4 FlagRot pages ({fmt}), Qwen-32B GQA 64q/8kv d=128, {R} requests x "
             f"{NQ} new tokens over a {PRE}-token cached prefix (L={L}), page=16, causal inside the chunk")
@@ -234,38 +426,52 @@ def main_mq(args, torch, dev):
     q = (2.0 * torch.randn(R * NQ, Gq * HKV, DH, generator=g, device=dev)).bfloat16()
     out = torch.zeros(R * NQ, Gq * HKV * DH, dtype=torch.bfloat16, device=dev)
     scale = LOG2E / math.sqrt(DH)
+    keep = {}
 
     def step(i):
         q16 = MQ.prep_q(q, scale, Gq, plan.idx, None, None if k2 else kmask)
         opart, ml = MQ.attn(q16, pool, bt, plan, Gq, 0, k2, False)
         MQ.merge(plan, opart, ml, Gq, out=out)
+        keep["q16"] = q16
 
-    for i in range(args.warmup):
-        step(i)
-    settle(torch, step)              # clocks out of idle
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    ev[0].record()
-    for i in range(args.steps):
-        step(i)
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
-    ms_per_step = ev[0].elapsed_time(ev[-1]) / args.steps
-    pairs = R * Gq * HKV * sum(PRE + t + 1 for t in range(NQ))
+    t = timed(torch, step, steps, warmup)
+    us = t["graph_us"]
+    pairs = R * Gq * HKV * sum(PRE + t_ + 1 for t_ in range(NQ))
     flops = 4.0 * DH * pairs
-    tflops = flops / (ms_per_step * 1e-3) / 1e12
-    res = {
-        "metric": "multi-query prefill attention over INT4 pages: achieved TFLOP/s per layer (ms per layer alongside)",
-        "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 operands, f32 accumulate", "data": "synthetic",
-        "config": {"workload": name, "tiles": plan.ntiles, "items": plan.nitems, "rows_per_tile": plan.rows},
-        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": 2500.0, "unit": "TFLOP/s",
-                     "frac": round(tflops / 2500.0, 4), "traffic": None, "algorithmic_flops_per_launch": flops,
-                     "avg_launch_us": round(ms_per_step * 1e3, 1), "median_launch_us": round(per[len(per) // 2] * 1e3, 1),
-                     "note": "one step = frmq_prep_q + frmq_attn + frmq_merge; the attention kernel dominates"},
-    }
-    print(json.dumps(res))
+    tflops = flops / (us * 1e-6) / 1e12
+    # check: the first and the last 4 rows of request R - 1, two KV heads (16 q heads), against fp64 attention over
+    # the oracle's dequantised pages (static format: keys in the stored basis, q16 was rotated to match)
+    out.zero_()
+    step(0)
+    torch.cuda.synchronize()
+    r, nh = R - 1, 2
+    mp = pool.index_select(0, bt[r].long())[:, :nh].contiguous().cpu().numpy()
+    Kp, Vp = A.dequant_pages(mp, fmt, P)
+    Kd, Vd = Kp.reshape(-1, nh, DH)[:L], Vp.reshape(-1, nh, DH)[:L]
+    q16 = keep["q16"].view(R * NQ, Gq * HKV, DH)
+    worst = 0.0
+    for t0_ in (0, NQ - 4):
+        rows = slice(r * NQ + t0_, r * NQ + t0_ + 4)
+        qb = q16[rows, :nh * Gq].cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+        ref, _ = OM.attention(qb, {0: Kd}, {0: Vd}, [(0, 0, 4, L, PRE + t0_)], Gq, 0)
+        got = out[rows].view(4, Gq * HKV, DH)[:, :nh * Gq].float().cpu().numpy().astype(np.float64)
+        worst = max(worst, within(got, ref))
+    return {"workload": name, "ms_per_layer": round(us * 1e-3, 4), "TFLOPs": round(tflops, 1),
+            "frac": round(tflops / PEAK_F16_TFLOPS, 4), "bound": "mfma", "peak_TFLOPs": PEAK_F16_TFLOPS,
+            "graph_min_us": round(t["graph_min_us"], 1), "graph_max_us": round(t["graph_max_us"], 1),
+            "eager_us": round(t["eager_us"], 1), "algorithmic_flops_per_launch": flops, "steps": steps,
+            "tiles": plan.ntiles, "items": plan.nitems, "rows_per_tile": plan.rows,
+            "checked": bool(worst <= 1.0), "check": f"request {r}, rows 0-3 and {NQ - 4}-{NQ - 1}, {nh * Gq} q heads vs fp64 "
+                                                    f"attention over the oracle's dequantised pages: worst |err| / (2e-3 + 1e-2 |ref|) = {worst:.3f}",
+            "note": "one step = frmq_prep_q + frmq_attn + frmq_merge; the attention kernel dominates"}
+
+
+def traffic_of(workload):
+    try:   # measured with rocprofv3 --pmc in separate runs (FETCH_SIZE / WRITE_SIZE); a process cannot count its own
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            return json.load(f).get(workload, {}).get("traffic_bytes")
+    except OSError:
+        return None
 
 
 def main():
@@ -273,10 +479,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="int4", choices=["int4", "int2", "kivi", "mq"])
+    ap.add_argument("--workload", default=None, choices=["int4", "int2", "kivi", "mq"])
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
+    ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", action="store_true", help="the chosen workload only (no extra legs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every (sequence, KV head) is independent: tensor-parallel "
@@ -288,105 +496,66 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    if args.workload == "kivi":
-        return main_kivi(args, torch, dev)
-    if args.workload == "mq":
-        return main_mq(args, torch, dev)
-    K.lib()
-    if args.workload == "int4":
-        kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144
-        name = "configs[1]: INT4 FlagRot konlya paged decode, Llama-3.1-8B GQA 32q/8kv d=128, B=32 L=8192 page=16"
+    workload = args.workload or "int4"
+    extras = args.workload is None and not args.only
+    metric = "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)"
+    common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "data": "synthetic"}
+    timing = f"HIP graph of {args.steps} steps, median of {REPLAYS} replays (events on the launch stream)"
+    if workload == "mq":
+        r = run_mq(args, torch, dev, args.steps, args.warmup, args.mq_fmt)
+        res = {"metric": "multi-query prefill attention over INT4 pages: achieved TFLOP/s per layer (ms per layer alongside)",
+               "value": r["TFLOPs"], "unit": "TFLOP/s", **common, "ms_per_step": r["ms_per_layer"],
+               "dtype": "f16 operands, f32 accumulate",
+               "config": {"workload": r["workload"], "tiles": r["tiles"], "items": r["items"],
+                          "rows_per_tile": r["rows_per_tile"], "timing": timing},
+               "roofline": {"bound": "mfma", "achieved": r["TFLOPs"], "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": r["frac"], "traffic": None,
+                            "algorithmic_flops_per_launch": r["algorithmic_flops_per_launch"],
+                            "avg_launch_us": r["ms_per_layer"] * 1e3, "eager_us": r["eager_us"]},
+               "checked": r["checked"], "check": r["check"]}
     else:
-        kind, B, L, S, W, cell = "konlya2", 64, 16384, 4, 128, 80
-        name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
-                "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
-    g = torch.Generator(device=dev).manual_seed(1)
-    kmu = None
-    if args.workload == "int2":
-        kmu = (2.0 * torch.randn(HKV, DH, generator=g, device=dev)).contiguous()
-    pool, bt, CT, co, fill_s = build_cache(torch, K, dev, kind, B, L, seed=1, kmu=kmu)
-    pool_bytes = pool.numel()
-    ncopy = max(1, min(8, int(6e9 // pool_bytes)))
-    pools = [pool] + [pool.clone() for _ in range(ncopy - 1)]
-    q = torch.randn(B, G * HKV, DH, generator=g, device=dev).bfloat16()
-    out = torch.zeros(B, G * HKV * DH, dtype=torch.bfloat16, device=dev)
-    T = S + W
-    tkw = {}
-    Lpages = L - W if T else L                      # the newest W tokens live in the BF16 ring, not in pages
-    seq = torch.full((B,), Lpages, dtype=torch.int32, device=dev)
-    if T:
-        ring = torch.randn(B + 1, T, 2 * HKV, DH, generator=g, device=dev).bfloat16()
-        tkw = dict(tail=ring, tail_len=torch.full((B,), T, dtype=torch.int32, device=dev),
-                   tail_idx=torch.arange(B, dtype=torch.int32, device=dev), tail_bs=ring.stride(0),
-                   tail_ts=ring.stride(1), kv_start=S)
-    ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None)
-    ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
-    scale = LOG2E / math.sqrt(DH)
-
-    def step(i):
-        K.cb_attn(q, pools[i % ncopy], bt, seq, out, ns, ch, ws, scale, kind, **tkw)
-
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    # Launches with pre-bound arguments (checks and pointer marshalling done once, as under graph capture).  The
-    # untimed warm-up continues until the GPU has been busy for 40 ms: out of idle the clocks take about that long to
-    # settle (the first 200 launches after an idle period measured 86 us per step, every later 200 launches 74-76).
-    bound = [K.cb_attn(q, pools[j], bt, seq, out, ns, ch, ws, scale, kind, bound=True, **tkw) for j in range(ncopy)]
-    settle(torch, lambda i: bound[i % ncopy]())
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    ev[0].record()
-    for i in range(args.steps):
-        bound[i % ncopy]()
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps))
-    total_ms = ev[0].elapsed_time(ev[-1])
-    ms_per_step = total_ms / args.steps
-    page_bytes = B * (Lpages - S) * HKV * cell
-    tail_bytes = B * T * 2 * HKV * DH * 2
-    alg_bytes = page_bytes + tail_bytes
-    gbps = alg_bytes / (ms_per_step * 1e-3) / 1e9
-
-    # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
-    kv_new = synth_kv(B, g, dev, torch, mu=kmu)
-    slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
-    for _ in range(3):
-        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(20):
-        K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
-    e1.record()
-    torch.cuda.synchronize()
-    writer_us = e0.elapsed_time(e1) / 20 * 1e3
-
-    traffic = None
-    try:   # measured with rocprofv3 --pmc (see profiles/k_decode_*_flagrot.txt); not measurable from inside this process
-        with open(os.path.join(ROOT, "profiles", "decode_traffic.json")) as f:
-            traffic = json.load(f).get(args.workload, {}).get("traffic_bytes")
-    except OSError:
-        pass
-    res = {
-        "metric": "paged decode attention: achieved HBM GB/s of page bytes per layer-step (us per layer-step alongside)",
-        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 6), "us_per_layer_step": round(ms_per_step * 1e3, 2),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 codes, fp16 products, f32 accumulate",
-        "data": "synthetic", "config": {"workload": name, "nsplit": ns, "chunk": ch, "cache_copies_cycled": ncopy,
-                                         "launch": "eager, arguments bound once",
-                                         "sink": S, "window": W},
-        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": traffic,
-                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(ms_per_step * 1e3, 2),
-                     "median_launch_us": round(per[len(per) // 2] * 1e3, 2), "min_launch_us": round(per[0] * 1e3, 2)},
-        "writer": {"decode_step_us": round(writer_us, 2), "decode_step_tokens": B,
-                   "prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * L,
-                   "note": "prefill_fill_s includes synthetic input generation"},
-        "host_wall_s": round(wall, 4),
-    }
+        if workload == "kivi":
+            r = run_kivi(args, torch, dev, args.steps, args.warmup)
+            dtype = "u8 codes, f16 products, f32 accumulate"
+        else:
+            plans = ("own", "reference") if (extras and workload == "int4") else ("own",)
+            rr = run_flagrot(args, torch, dev, workload, args.steps, args.warmup, plans)
+            r = rr["own"]
+            dtype = "u8 codes, f16 products, f32 accumulate"
+        res = {"metric": metric, "value": r["GBps"], "unit": "GB/s", **common,
+               "ms_per_step": round(r["us_per_layer_step"] * 1e-3, 6), "us_per_layer_step": r["us_per_layer_step"],
+               "dtype": dtype,
+               "config": {"workload": r["workload"], "nsplit": r["nsplit"], "chunk": r["chunk"],
+                          "cache_copies_cycled": r["cache_copies_cycled"], "timing": timing, "sink": r["sink"],
+                          "window": r["window"]},
+               "roofline": {"bound": "hbm", "achieved": r["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": r["frac"],
+                            "traffic": traffic_of("kivi" if workload == "kivi" else workload),
+                            "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this launch in "
+                                              "separate runs, scaled by a device copy; not measured in this run)",
+                            "algorithmic_bytes_per_launch": r["algorithmic_bytes_per_launch"],
+                            "avg_launch_us": r["us_per_layer_step"], "graph_min_us": r["graph_min_us"],
+                            "graph_max_us": r["graph_max_us"], "eager_us": r["eager_us"]},
+               "checked": r["checked"], "check": r["check"]}
+        if "writer" in r:
+            res["writer"] = r["writer"]
+        if workload == "int4" and extras:
+            ref = rr["reference"]
+            res["reference_planner"] = {k: ref[k] for k in ("nsplit", "chunk", "us_per_layer_step", "frac", "eager_us", "checked")}
+            res["reference_planner"]["note"] = ("the split plan the reference front end's own cost model makes from "
+                                                "fr_cb_occupancy x multi_processor_count, run through the same library")
+    if extras:
+        short = max(10, args.steps // 5)
+        wl = {}
+        torch.cuda.empty_cache()
+        wl["int2"] = run_flagrot(args, torch, dev, "int2", short, 5)["own"]
+        torch.cuda.empty_cache()
+        wl["kivi"] = run_kivi(args, torch, dev, short, 5)
+        torch.cuda.empty_cache()
+        wl["mq_" + args.mq_fmt] = run_mq(args, torch, dev, max(5, args.steps // 20), 3, args.mq_fmt)
+        torch.cuda.empty_cache()
+        res["workloads"] = wl
+        res["checked_all"] = bool(res["checked"] and all(v["checked"] for v in wl.values()))
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, K, dev)
     print(json.dumps(res))

@@ -120,10 +120,17 @@ int fr_v2_write(int fmt, const void* kv, long long kv_ts, const long long* slots
   return launched(static_write_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_write");
 }
 
+// What the host split planner multiplies by the CU count to get the number of workgroups that run at once.  The answer
+// is 1: the fastest launch shape is ONE large workgroup per CU (decode_launch takes it whenever the plan's workgroups
+// fit the CUs once with >= 1024 tokens each), and a planner that fills "1 x CUs" slots with the longest chunks that
+// fit (the reference front end's cost model, vllm_flagrot/kernels.py:247-265) lands on exactly that shape: 256
+// (sequence, KV head) pairs of 8192 tokens -> nsplit 1, chunk 8192; 8 pairs of 32768 tokens -> 32 splits of 1024.
+// When more workgroups than CUs are asked for, the library runs 4-wavefront workgroups, of which up to 4 are
+// resident per CU; it then treats nsplit only as the number of workgroups per (sequence, KV head, q tile).
 int fr_v2_occupancy(int fmt, int variant, int stages, int page) {
   (void)variant; (void)stages;
   if ((page != 16 && page != 32) || fmt < FMT_INT4 || fmt > FMT_KONLYA2) return 0;
-  return decode_occupancy(fmt, 4);
+  return 1;
 }
 int fr_v2_chunk_bytes(int fmt, int page) { return page * (fmt_int2(fmt) ? 80 : 144); }
 
@@ -267,7 +274,7 @@ int fr_cb_attn_noalloc(const void* q, long long q_bs, const uint8_t* pool, const
 int fr_cb_occupancy(int kind, int variant, int stages, int page) {
   (void)variant; (void)stages;
   if ((page != 16 && page != 32) || fmt_of_kind(kind) < 0) return 0;
-  return decode_occupancy(fmt_of_kind(kind), 4);
+  return 1;      // as fr_v2_occupancy: one large workgroup per CU is the shape a planner should aim at
 }
 int fr_cb_chunk_bytes(int kind, int page) { return page * (kind == KIND_KONLYA2 ? 80 : 144); }
 int fr_cb_write_smem(int kind, int tg, int hd) {

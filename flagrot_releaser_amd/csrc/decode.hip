@@ -1,17 +1,23 @@
-// Paged split-K GQA decode attention over FlagRot INT4 / INT2 pages for gfx950 (wave64; scores on the vector
-// pipe, the value product on the matrix pipe).
+// Paged split-K GQA decode attention over FlagRot INT4 / INT2 pages for gfx950 (wave64).  The kernel is priced
+// against HBM only: every page byte is read once; both contractions use the matrix pipe as a wide dot product on
+// operands that already sit in the right shape (nothing is reshaped into a GEMM).
 //
 // One workgroup (16 or 12 wavefronts = a whole CU's register file, or 4 for short chunks) per (KV head x q tile of 4 heads,
 // split, sequence).  Its wavefronts draw quads of 4 pages from a counter in LDS, so they finish together whatever
 // share of the issue slots each one got.  A wavefront streams whole pages (16 tokens x one KV head = one contiguous
 // 2304 / 1280 byte chunk) with 128-bit loads:
-//   key phase    lane = token: its code row, 8 elements of each 32-group per 16-byte quarter.  A code field masked in
-//                place is an fp16 denormal (value code * 2^(position - 24), exact) and is contracted with the query by
-//                v_dot2_f32_f16; the powers of two ride on the query operand and the scale.  The query is rotated three ways once per workgroup
-//                (identity, H32 per group, H128) and kept in LDS in the code words' element order; every lane fetches
-//                the variant its token / group flags ask for, so selection costs no arithmetic.  The exponent offsets
-//                and the zero points are removed with per-(variant, head, group) query sums.
-//   softmax      exp2-domain online softmax per wavefront; p * V-scale is written to LDS as fp16 in V^T token order.
+//   key phase    lane = (token t of a page, quarter x of its code row): one 16-byte load is the four code words (one
+//                per 32-group) of that quarter.  A code field masked in place is an fp16 denormal (value
+//                code * 2^(position - 24), exact); the eight fields of a word are the lane's share of the B operand of
+//                v_mfma_f32_16x16x32_f16 (columns = the page's 16 tokens, 32 deep = the group's 32 dims).  The A
+//                operand rows are (head, query variant): the query tile is rotated three ways once per workgroup
+//                (identity, H32 per group, H128), split into an fp16 pair (value + remainder: two products) and kept
+//                in LDS in the code words' element order.  The zero point leaves through one more small product
+//                (zero point x sum of the group's query elements).  A lane then holds, for its (token, head), the
+//                score parts of all variants: the one its (token, group) flag bits ask for is picked and scaled by the
+//                group's scale word.
+//   softmax      exp2-domain online softmax, lane = (token, head); p * V-scale is written to LDS as fp16 in V^T token
+//                order (the four lanes of a token exchange their V scale words).
 //   value phase  lane = one 16-byte V^T entry (4 dims x 8 tokens) of a run of 8 tokens: its words masked in place (fp16
 //                denormals, value code * 2^(position - 24), exact) are the A operands of v_mfma_f32_16x16x32_f16, the
 //                p * scale strip rows the B operands (columns = (group, head)); the powers of two ride on the
@@ -35,10 +41,8 @@ DEVI float dot2(uint32_t a, uint32_t b, float c) { return __builtin_amdgcn_fdot2
 DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 
-// LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per variant /
-// per row group) start in different banks.
-constexpr int QV_VSTRIDE = 65;                     // uint4 per variant: 64 + 1 pad
-constexpr int QV_BYTES = 3 * QV_VSTRIDE * 16;      // [variant][head][tg][j][8 fp16]
+// LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per
+// row group) start in different banks.
 constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (page, c8): 16 + 1 pad
 constexpr int PB_BYTES = 8 * PB_RSTRIDE * 16;      // per wave: [page][c8][group][head][8 fp16]
 constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
@@ -47,14 +51,17 @@ constexpr int STRIP_BYTES = PB_BYTES + ZB_BYTES;   // per wave
 constexpr int DRAW_BATCH = 2;                      // quads per draw from the shared (device-scope) counter
 constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
 constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
+constexpr float QPRE = 16.f;                       // the query operands carry 2^4 (fp16 range: |q| up to 127 in any rotation)
 
 template <int NW>
 struct Smem {
-  alignas(16) uint8_t qv[QV_BYTES];
+  // A operands of the score products: [group j][lane of the matrix instruction = row (head, variant) + 16 x k block]
+  alignas(16) uint4 qhi[4][64];                      // fp16(q * 2^4 / element factor)
+  alignas(16) uint4 qlo[4][64];                      // fp16 of what that rounding left
+  alignas(16) uint4 qz[4][64];                       // -(sum of the group's query elements), fp16 pair in k blocks 0 / 1 (first word)
   // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
   alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
   alignas(16) uint32_t zero[4 * (4 * PB_RSTRIDE + 1)];   // zeros where the matrix value phase reads the strip rows of foreign groups
-  alignas(16) float qsum[3][4][4];                   // [variant][group][head]: sum of the group's (fp16) query elements
   float m[NW][4], l[NW][4];
   int btc[BT_CACHE];
   int next;                                          // next quad of 4 pages nobody has taken yet
@@ -70,10 +77,15 @@ struct Smem {
 DEVI int kslot(int isB, int i) { return 2 * (2 * (i & 1) + isB) + (i >> 1); }
 DEVI int vslot(int r8) { return 2 * (r8 & 3) + (r8 >> 2); }
 
-// Rotates the q tile three ways and stores it as fp16 in code-word order (the identity variant of a bf16 query is
-// exact in fp16; qscale is applied to the fp32 score), with the sums per 32-group that remove the key zero points.
+// Rotates the q tile three ways and stores it as the A operands of the score products: rows = (head, variant), per
+// 32-group j and k block (= quarter tg of a code row) the eight elements in the order the masked code words give
+// them.  An element is held as an fp16 pair (value + what its rounding left), both times 2^4 and divided by the
+// factor its code field comes out of the unpacking with (2^SH for the B elements of a word, 2^4 more for the odd
+// groups of the 2-bit words).  The third operand removes the zero points: -(sum of the group's elements as held).
+// Wavefronts 0..3: one head each; half 0 writes the rows of variants 0 (identity, or the static kmask rotation) and
+// 1 (H32), half 1 those of variant 2 (H128) and the idle row 3; rows of variants a format does not use are zero.
 template <int QM, bool K2, class SM>
-DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {   // wavefronts 0..3: one head each
+DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
   const int w = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
   const int hq = tile * 4 + w;                       // head inside the GQA group
   float x[4] = {0.f, 0.f, 0.f, 0.f};
@@ -83,37 +95,57 @@ DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {  
     const uint2 raw = *reinterpret_cast<const uint2*>(qr);
     x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
   }
-  const int g = l32 >> 3;
-  // half 0: variants 0 (identity, or the static kmask rotation) and 1 (H32); half 1: variant 2 (H128)
-  const int nvar = K2 ? (half == 0 ? 2 : 1) : (half == 0 ? 1 : 0);
+  const int g = l32 >> 3, isB = (l32 >> 2) & 1, tg = l32 & 3;   // the lane's dims 4 l32 + i: group, word half, quarter
   float y[4] = {x[0], x[1], x[2], x[3]};
   if (half == 0) fwht<32>(y, l32); else fwht<128>(y, l32);
-  for (int vi = 0; vi < nvar; ++vi) {
-    int var;
+  // factor of the lane's code fields after the unpacking (the operand is divided by it)
+  const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
+  const float fold = QPRE / beta;
+#pragma unroll
+  for (int vi = 0; vi < 2; ++vi) {
+    const int var = 2 * half + vi;
     float v[4];
+    bool live;
     if (K2) {
-      var = half == 0 ? vi : 2;
+      live = var < 3;
       const bool rot = var != 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
     } else {
-      var = 0;
+      live = var == 0;
       const bool rot = p.kmask != nullptr && p.kmask[kvh * 4 + g] != 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
     }
-    // the B elements of a code word are unpacked with the factor 2^SH (UnpackD): their query slots carry 2^-SH
-    const float fold = ((l32 >> 2) & 1) ? 1.f / static_cast<float>(1 << UnpackD<QM>::SH) : 1.f;
+    uint32_t hb[4], lb[4];
     float qs = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int d = 4 * l32 + i, r = d & 31;
-      const int isB = r >> 4, tg = (r & 15) >> 2, ii = r & 3;
-      qs += static_cast<float>(static_cast<_Float16>(v[i]));
-      reinterpret_cast<_Float16*>(S.qv)[(var * QV_VSTRIDE + (w * 4 + tg) * 4 + g) * 8 + kslot(isB, ii)] = static_cast<_Float16>(v[i] * fold);
+      const float a = live ? v[i] * fold : 0.f;
+      const _Float16 hi = static_cast<_Float16>(a);
+      const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
+      hb[i] = __builtin_bit_cast(uint16_t, hi);
+      lb[i] = __builtin_bit_cast(uint16_t, lo);
+      qs += (static_cast<float>(hi) + static_cast<float>(lo)) * beta;
     }
-    qs += hx(qs, 1); qs += hx(qs, 2); qs += hx(qs, 4);
-    if ((l32 & 7) == 0) S.qsum[var][g][w] = qs;
+    // elements i = 0, 2 are halves 2 isB, 2 isB + 1 of the operand (word isB), i = 1, 3 halves 4 + 2 isB, 5 + 2 isB
+    const int m = 4 * w + var, ln = m + 16 * tg;
+    uint32_t* dh = reinterpret_cast<uint32_t*>(&S.qhi[g][ln]);
+    uint32_t* dl = reinterpret_cast<uint32_t*>(&S.qlo[g][ln]);
+    dh[isB] = hb[0] | (hb[2] << 16); dh[2 + isB] = hb[1] | (hb[3] << 16);
+    dl[isB] = lb[0] | (lb[2] << 16); dl[2 + isB] = lb[1] | (lb[3] << 16);
+    if constexpr (QM != QM_SYM4) {
+      qs += hx(qs, 1); qs += hx(qs, 2); qs += hx(qs, 4);
+      if ((l32 & 7) == 0) {   // k blocks 0 / 1 carry the pair, in the half the zero point of group g is masked into
+        const _Float16 zh = static_cast<_Float16>(-qs);
+        const _Float16 zl = static_cast<_Float16>(-qs - static_cast<float>(zh));
+        const int sh = 16 * (g & 1);
+        S.qz[g][m] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zh)) << sh, 0u, 0u, 0u);
+        S.qz[g][m + 16] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zl)) << sh, 0u, 0u, 0u);
+        S.qz[g][m + 32] = make_uint4(0u, 0u, 0u, 0u);
+        S.qz[g][m + 48] = make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
   }
 }
 
@@ -126,13 +158,14 @@ template <class T> DEVI T gload(const uint8_t* p) {
   return *(gp)(p);
 }
 
-// One wave iteration covers 4 consecutive pages = 64 tokens.  Key phase: lane = token (page lane >> 4, position
-// lane & 15).  Value phase: lane = V^T entry `lane` of each of the 4 pages in turn.
+// One wave iteration covers a quad = 64 consecutive tokens (four 16-token pages or two 32-token pages), as four
+// blocks of 16 tokens.  Key phase: lane = (token t = lane & 15 of a block, quarter x = lane >> 4 of its code row).
+// Value phase: lane = V^T entry `lane` of each of the 4 blocks in turn.
 template <int QM> struct KRegs {
   static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;   // code words per 16-byte / 8-byte quarter row
-  uint32_t kc[4][NW];       // [quarter tg][word]
-  uint2 ks;                 // the token's 4 K scale words
-  uint16_t vs[4];           // the token's 4 V scale words (one per group); 16 bits wide so that their widening belongs to the use
+  uint32_t kc[4][NW];       // [block][word]: quarter x of token t's code row (word j = group j; 2-bit: groups 2 j, 2 j + 1)
+  uint2 ks[4];              // [block]: the token's 4 K scale words
+  uint16_t vs[4];           // [block]: the token's V scale word of group x; 16 bits wide so that the widening belongs to the use
                             // (a widening at the load would be scheduled right behind it and wait for the keys in flight)
 };
 // The value product P' V runs on the matrix pipe: sixteen v_mfma_f32_16x16x32_f16 per quad of pages, rows = 16 V^T
@@ -144,28 +177,35 @@ template <int QM> struct VRegs {
   uint32_t vc[4][NW];       // [2 (page pair s) + entry half][entry word] of lane (entry m = lane & 15, run kc = lane >> 4)
 };
 
+// lane offsets of the key-side loads inside a chunk (block 0 of a page; a 32-token page's second block adds constants)
+template <int QM, int P> struct KOffs { int k, ks, vs; };
 template <int QM, int P>
-DEVI void load_k(KRegs<QM>& r, const uint8_t* chunk, int pos) {
+DEVI KOffs<QM, P> key_offsets(int lane) {
   using L = Lay<QM, P>;
-  if constexpr (QM == QM_ASYM2) {
-    const uint8_t* row = chunk + L::K_OFF + 32 * (pos ^ ((pos >> 1) & 2));
+  const int t = lane & 15, x = lane >> 4;
+  KOffs<QM, P> o;
+  o.k = QM == QM_ASYM2 ? L::K_OFF + 32 * (t ^ ((t >> 1) & 2)) + 8 * x : L::K_OFF + 64 * t + 16 * x;
+  o.ks = L::KS_OFF + 8 * t;
+  o.vs = L::VS_OFF + (x * P + 8 * (t >> 3) + vs_slot8(t)) * 2;
+  return o;
+}
+// chunk[b]: the chunk of block b's page (wave uniform); 32-token pages: blocks 2 s, 2 s + 1 are the halves of page s
+template <int QM, int P>
+DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[4], const KOffs<QM, P>& o) {
 #pragma unroll
-    for (int tg = 0; tg < 4; ++tg) {
-      const u32x2 k = gload<u32x2>(row + 8 * tg);
-      r.kc[tg][0] = k.x; r.kc[tg][1] = k.y;
+  for (int b = 0; b < 4; ++b) {
+    const int hp = P == 32 ? (b & 1) : 0;            // second half of a 32-token page: 16 tokens further
+    const uint8_t* ch = chunk[b];
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 k = gload<u32x2>(ch + o.k + hp * 16 * 32);
+      r.kc[b][0] = k.x; r.kc[b][1] = k.y;
+    } else {
+      const u32x4 k = gload<u32x4>(ch + o.k + hp * 16 * 64);
+      r.kc[b][0] = k.x; r.kc[b][1] = k.y; r.kc[b][2] = k.z; r.kc[b][3] = k.w;
     }
-  } else {
-    const uint8_t* row = chunk + L::K_OFF + 64 * pos;
-#pragma unroll
-    for (int tg = 0; tg < 4; ++tg) {
-      const u32x4 k = gload<u32x4>(row + 16 * tg);
-      r.kc[tg][0] = k.x; r.kc[tg][1] = k.y; r.kc[tg][2] = k.z; r.kc[tg][3] = k.w;
-    }
+    { const u32x2 t2 = gload<u32x2>(ch + o.ks + hp * 16 * 8); r.ks[b] = make_uint2(t2.x, t2.y); }
+    r.vs[b] = gload<uint16_t>(ch + o.vs + hp * 16 * 2);
   }
-  { const u32x2 t2 = gload<u32x2>(chunk + L::KS_OFF + 8 * pos); r.ks = make_uint2(t2.x, t2.y); }
-  const uint8_t* vo = chunk + L::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2;
-#pragma unroll
-  for (int g = 0; g < 4; ++g) r.vs[g] = gload<uint16_t>(vo + g * P * 2);
 }
 
 template <int QM, int P>
@@ -177,7 +217,7 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
   const int m = lane & 15, kc = lane >> 4;
 #pragma unroll
   for (int s2 = 0; s2 < 2; ++s2) {
-    const uint8_t* ch = P == 16 ? ((kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2]) : chunk[s2];
+    const uint8_t* ch = P == 16 ? ((kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2]) : chunk[2 * s2];
     const int c8 = P == 16 ? (kc & 1) : kc;
 #pragma unroll
     for (int eh = 0; eh < 2; ++eh) {
@@ -194,114 +234,161 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 struct WaveState {
-  float m[4];        // running maximum per head (wave uniform)
-  float l[4];        // this lane's share of the running sum per head
+  float m;           // running maximum of head x = lane >> 4 (log2 domain; uniform over the head's 16 lanes)
+  float l;           // this lane's share of the running sum of head x
   // 2^-24 sum p' code (zero points not yet removed), [entry word parity]: column lane & 15 = (group g, head), rows =
   // entries 16 (g & 1) + 4 (lane >> 4) + r, entry word 2 (g >> 1) + parity
   f32x4 ot[2];
   float z[2];        // lane = (page, half, group, head pair): its share of sum p' zero point, heads 2 hp and 2 hp + 1
 };
 
-// scores of the lane's token against the 4 q heads (log2 domain, unmasked)
+// exchange with the lane 16 / 32 further (xor): the four lanes of a token
+DEVI uint32_t lane_xor16(uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_ds_swizzle(static_cast<int>(v), (16 << 10) | 0x1F)); }
+DEVI uint32_t lane_xor32(uint32_t v, int lane) {
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // r[0] = lower half twice, r[1] = upper half twice
+  return lane < 32 ? r[1] : r[0];
+}
+// all-reduce over the 16 lanes of a row (DPP: quad permutes, then the mirrors of 8 and of 16 lanes)
+DEVI float row_max16(float v) {
+  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true)));   // row_half_mirror
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true))); // row_mirror
+}
+DEVI float row_sum16(float v) {
+  v += dpp_xor1(v); v += dpp_xor2(v);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+// the 16-bit scale word `j` of a packed pair as fp32, sign bit (flag) dropped.  Plain code on purpose: instructions
+// written as inline assembly are invisible to the compiler's hazard handling, and a register that a matrix
+// instruction is still writing (an unused row of its result) may be handed to them as their output.
+DEVI float word_scale(uint32_t pair, int j) {
+  const uint16_t w = static_cast<uint16_t>((j & 1) ? (pair >> 16) : pair);
+  return static_cast<float>(__builtin_fabsf16(__builtin_bit_cast(_Float16, w)));
+}
+
+// Scores of the lane's (token, head) for the four blocks of the quad: raw sums 2^-20 sum_j scale_j sum (c - z) q'
+// (the factor and qscale are applied with the softmax).
 template <int QM, bool K2, class SM>
-DEVI void key_phase(const SM& S, const KRegs<QM>& r, float qscale, float (&sc)[4]) {
+DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
-  const uint32_t kw[4] = {r.ks.x & 0xFFFFu, r.ks.x >> 16, r.ks.y & 0xFFFFu, r.ks.y >> 16};
-  const bool full = K2 && (r.vs[0] & 0x8000u);
+  // the zero point of group j, masked in place (an fp16 denormal z 2^-24 in the low half of the pair word for even j,
+  // in the high half for odd j): lanes of k blocks 0 and 1 feed it (first element pair of their eight) against the pair
+  // -(sum q) of the third operand
+  const uint32_t zlane = (lane < 32) ? static_cast<uint32_t>(ZM) : 0u;
+  bool full[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    // the whole-head flag is bit 15 of the token's group-0 V scale word (lane x = 0 of the token's four lanes holds it);
+    // the words of the other value groups never carry that bit (scale words are non-negative fp16 patterns), so the
+    // union over the four lanes names it
+    full[b] = false;
+    if constexpr (K2) {
+      uint32_t f = r.vs[b] & 0x8000u;
+      f |= lane_xor16(f);
+      f |= lane_xor32(f, lane);
+      full[b] = f != 0u;
+    }
+    sc[b] = 0.f;
+  }
+  // group by group (one set of A operands live at a time), the four blocks of a group back to back
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int var = K2 ? (full ? 2 : static_cast<int>(kw[j] >> 15)) : 0;
-    const uint4* qp = reinterpret_cast<const uint4*>(S.qv) + var * QV_VSTRIDE + j;   // + head * 16 + tg * 4
-    float a[4];
+    const half8 qh = __builtin_bit_cast(half8, S.qhi[j][lane]), ql = __builtin_bit_cast(half8, S.qlo[j][lane]);
+    half8 qz;
+    if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[j][lane]);
+    f32x4 acc[4];
 #pragma unroll
-    for (int tg = 0; tg < 4; ++tg) {
+    for (int b = 0; b < 4; ++b) {
       uint32_t x[4];
-      if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher, 2^4 folded into its scale
-        if (j & 1) UnpackD<QM>::run_hi(r.kc[tg][j >> 1], x); else UnpackD<QM>::run(r.kc[tg][j >> 1], x);
+      if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher (2^4 is in its query operand)
+        if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
       }
-      else UnpackD<QM>::run(r.kc[tg][j], x);
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const uint4 qq = qp[h * 16 + tg * 4];
-        float v;
-        if (tg == 0) asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(v) : "v"(x[0]), "v"(qq.x));   // no register clear
-        else v = dot2(x[0], qq.x, a[h]);
-        v = dot2(x[1], qq.y, v);
-        v = dot2(x[2], qq.z, v);
-        v = dot2(x[3], qq.w, v);
-        a[h] = v;
+      else UnpackD<QM>::run(r.kc[b][j], x);
+      const half8 kb = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+      f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh, kb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      a = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql, kb, a, 0, 0, 0);
+      if constexpr (ZM != 0) {
+        const uint32_t kwz = (j & 2) ? r.ks[b].y : r.ks[b].x;
+        const uint32_t zz = kwz & (zlane << (16 * (j & 1)));
+        // (the same instruction as the two products before it: a chain of one kind on one accumulator)
+        a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qz, __builtin_bit_cast(half8, make_uint4(zz, 0u, 0u, 0u)), a, 0, 0, 0);
       }
-    }
-    // a = 2^-24 sum code q: score += scale (2^24 a - zero point * sum q)
-    const float sj = f16_value(kw[j] & 0x7FFFu) * qscale;
-    const float sj24 = sj * ((QM == QM_ASYM2 && (j & 1)) ? 1048576.f : 16777216.f);
-    if constexpr (ZM != 0) {
-      const float4 qs = *reinterpret_cast<const float4*>(&S.qsum[var][j][0]);
-      const float sz = -sj * static_cast<float>(kw[j] & ZM);
-      sc[0] += sz * qs.x; sc[1] += sz * qs.y; sc[2] += sz * qs.z; sc[3] += sz * qs.w;
+      acc[b] = a;
     }
 #pragma unroll
-    for (int h = 0; h < 4; ++h) sc[h] += sj24 * a[h];
+    for (int b = 0; b < 4; ++b) {     // rows 4 x + variant of the product: the lane's head, every variant
+      const uint32_t kw = (j & 2) ? r.ks[b].y : r.ks[b].x;
+      float pick = acc[b][0];
+      if constexpr (K2) {
+        const bool h32 = (kw >> (16 * (j & 1) + 15)) & 1u;
+        pick = full[b] ? acc[b][2] : (h32 ? acc[b][1] : acc[b][0]);
+      }
+      sc[b] += pick * word_scale(kw, j);
+    }
   }
 }
 
-// online softmax step for 64 tokens: the running maximum is only re-reduced over the wave when some lane beats it
+// online softmax step for the quad, lane = (token, head x): the running maximum is only re-reduced when some lane
+// beats it; then p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order.
+// qs20 = qscale * 2^20 (the factor the raw score sums lack); sc0 lowers the scores of odd tokens by SH (below).
 template <int QM, class SM>
-DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], bool valid, int lane, int wave) {
+DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], const bool (&valid)[4],
+                        float qs20, float sc0, int lane, int wave) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   bool beat = false;
+  float mx = -INFINITY;
 #pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    sc[h] = valid ? sc[h] : -INFINITY;
-    beat |= sc[h] > st.m[h];
+  for (int b = 0; b < 4; ++b) {
+    sc[b] = valid[b] ? sc[b] * qs20 + sc0 : -INFINITY;
+    mx = fmaxf(mx, sc[b]);
   }
+  beat = mx > st.m;
   // The state is multiplied every time (by 1 unless the maxima moved): modifying it only inside the rare branch makes
   // the compiler keep two copies of all its registers and move them on the common path.
-  float alpha[4] = {1.f, 1.f, 1.f, 1.f};
+  float al = 1.f, az0 = 1.f, az1 = 1.f, am = 1.f;
   if (__builtin_expect(__any(beat), 0)) {   // rare after the first quads
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const float mn = fmaxf(st.m[h], wave_max64(sc[h]));
-      alpha[h] = mn == -INFINITY ? 1.f : fexp2(st.m[h] - mn);
-      st.m[h] = mn;
-    }
+    const float mn = fmaxf(st.m, row_max16(mx));
+    am = mn == -INFINITY ? 1.f : fexp2(st.m - mn);
+    st.m = mn;
+    // the factors of the four heads (rows of 16 lanes) for the lanes whose accumulator columns belong to them
+    const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 0));
+    const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 16));
+    const float a2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 32));
+    const float a3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 48));
+    al = (lane & 2) ? ((lane & 1) ? a3 : a2) : ((lane & 1) ? a1 : a0);     // accumulator column: head lane & 3
+    az0 = (lane & 1) ? a2 : a0;
+    az1 = (lane & 1) ? a3 : a1;
   }
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    st.l[h] *= alpha[h];
-  }
-  {   // the lane's accumulator column belongs to head lane & 3
-    const float al = (lane & 2) ? ((lane & 1) ? alpha[3] : alpha[2]) : ((lane & 1) ? alpha[1] : alpha[0]);
-    st.ot[0] *= al; st.ot[1] *= al;
-  }
-  st.z[0] *= (lane & 1) ? alpha[2] : alpha[0];
-  st.z[1] *= (lane & 1) ? alpha[3] : alpha[1];
-  float p[4];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    p[h] = fexp2(sc[h] - st.m[h]);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
-    st.l[h] += p[h];
-  }
-  // p' = p * V scale per group as fp16 (packed fp16 products of head pairs) and the zero points, in V^T token order
-  // of the token's page.  Odd tokens are unpacked with the factor 2^SH (UnpackD): their scores were lowered by SH
-  // (p carries 2^-SH), their zero point is raised by 2^SH; zero points are fp16 denormals like the codes.
-  const int rg = lane >> 3, sl = vslot(lane & 7);         // run of 8 tokens (page, page eighth) and the slot inside it
-  uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + rg * PB_RSTRIDE * 8 + sl;     // + (group * 4 + head) * 8
-  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + rg * ZB_RSTRIDE * 8 + sl;     // + group * 8
-  const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[0], p[1]));
-  const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(p[2], p[3]));
-  const uint32_t keep = valid ? 0x7FFF7FFFu : 0u;        // unwritten slots may hold any pattern
+  st.l *= am;
+  st.ot[0] *= al; st.ot[1] *= al;
+  st.z[0] *= az0; st.z[1] *= az1;
+  // Odd tokens are unpacked from the V^T words with the factor 2^SH (UnpackD): their scores were lowered by SH (p
+  // carries 2^-SH), their zero point is raised by 2^SH; zero points are fp16 denormals like the codes.
+  const int t = lane & 15, x = lane >> 4;
+  const int sl = vslot(t & 7);
+  uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + (t >> 3) * PB_RSTRIDE * 8 + sl;   // + block * 2 rows; + (group * 4 + head) * 8
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (t >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
+  const int c0 = ((x) * 4 + x) * 8, c1 = ((x ^ 1) * 4 + x) * 8, c2 = ((x ^ 2) * 4 + x) * 8, c3 = ((x ^ 3) * 4 + x) * 8;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const uint32_t sv2 = (r.vs[g] * 0x10001u) & keep;
-    const uint32_t x01 = pk_mul(p01, sv2), x23 = pk_mul(p23, sv2);
-    pb[(g * 4 + 0) * 8] = static_cast<uint16_t>(x01);
-    pb[(g * 4 + 1) * 8] = static_cast<uint16_t>(x01 >> 16);
-    pb[(g * 4 + 2) * 8] = static_cast<uint16_t>(x23);
-    pb[(g * 4 + 3) * 8] = static_cast<uint16_t>(x23 >> 16);
-    if constexpr (QM != QM_SYM4) zb[g * 8] = static_cast<uint16_t>((r.vs[g] & ZM) << zsh);
+  for (int b = 0; b < 4; ++b) {
+    const float pe = fexp2(sc[b] - st.m);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
+    st.l += pe;
+    const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe, pe));
+    // the token's four V scale words, sign bits stripped: own group x, then the lanes 16, 32, 48 further (groups
+    // x ^ 1, x ^ 2, x ^ 3); unwritten slots may hold any pattern: masked
+    const uint32_t v0 = valid[b] ? (r.vs[b] & 0x7FFFu) : 0u;
+    const uint32_t v1 = lane_xor16(v0), v2 = lane_xor32(v0, lane), v3 = lane_xor32(v1, lane);
+    const uint32_t xa = pk_mul(pp, (v1 << 16) | v0), xb = pk_mul(pp, (v3 << 16) | v2);
+    uint16_t* row = pb + b * 2 * PB_RSTRIDE * 8;
+    row[c0] = static_cast<uint16_t>(xa);
+    row[c1] = static_cast<uint16_t>(xa >> 16);
+    row[c2] = static_cast<uint16_t>(xb);
+    row[c3] = static_cast<uint16_t>(xb >> 16);
+    if constexpr (QM != QM_SYM4) zb[b * 2 * ZB_RSTRIDE * 8] = static_cast<uint16_t>((r.vs[b] & ZM) << zsh);
   }
 }
 
@@ -410,15 +497,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
     const int lo = dyn ? min(p.kv_start, len) : max(split * p.chunk, min(p.kv_start, len));
     const int hi = dyn ? len : min(len, (split + 1) * p.chunk);
     WaveState st;
-#pragma unroll
-    for (int h = 0; h < 4; ++h) { st.m[h] = -INFINITY; st.l[h] = 0.f; }
+    st.m = -INFINITY; st.l = 0.f;
     st.z[0] = st.z[1] = 0.f;
     st.ot[0] = st.ot[1] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (lo < hi) {   // uniform over the workgroup
       const int pg0 = lo / P, pg1 = (hi + P - 1) / P;
       const int* bt = p.block_table + static_cast<long long>(b) * p.bt_stride;
       // quads beyond a wave's first one are drawn: from S.next (the workgroup owns a range) or from the slot's draw
-      // counter (all body wavefronts of the slot share the range); a draw is made a whole iteration before its use
+      // counter (all body wavefronts of the slot share the range)
       auto draw = [&]() {
         int t = 0;
         if (lane == 0)
@@ -437,74 +523,81 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
       constexpr int PPQ = 64 / P;                 // pages per quad of 64 tokens (the name stays: 4 pages of 16, 2 of 32)
-      const int nquad = (pg1 - pg0 + PPQ - 1) / PPQ;
-      const int pi = lane / P, pos = lane % P;
+      const int npg = pg1 - pg0;
+      const int nquad = (npg + PPQ - 1) / PPQ;
       // odd tokens: the B fields of a V^T word come out of the unpacking with the factor 2^SH, so their scores are
       // lowered by SH (log2 domain) and their share of the softmax sum is raised again at the end
-      const float sc0 = (pos & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
+      const float sc0 = (lane & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
+      const float qs20 = p.qscale * (16777216.f / QPRE);         // raw score sums carry 2^-24 from the codes and QPRE from the query
       typedef const __attribute__((address_space(1))) uint8_t* gptr;
       const gptr pool = (gptr)p.pool;
-      auto chunk_of = [&](int quad) {   // pages past the range read the last page of the range; their tokens are masked
-        const int i = min(PPQ * quad + pi, pg1 - pg0 - 1);
-        // The entry comes from LDS.  Past the cached window it is read from memory inside a branch and consumed there:
-        // a select between the two addresses would be one generic load, which waits for every page load in flight.
-        int page = S.btc[min(i, BT_CACHE - 1)];
-        if (__builtin_expect(i >= BT_CACHE, 0)) {
-          const int far = gload<int>(reinterpret_cast<const uint8_t*>(bt + pg0 + i));
-          asm volatile("v_mov_b32 %0, %1" : "=v"(page) : "v"(far));
+      // chunk addresses of a quad's four blocks (wave uniform).  Pages past the range name the range's last page again
+      // (their tokens are masked).  The entry comes from LDS; past the cached window it is read from memory.
+      auto chunks_of = [&](int quad, const uint8_t* (&ch)[4]) {
+#pragma unroll
+        for (int k = 0; k < PPQ; ++k) {
+          const int i = min(PPQ * quad + k, npg - 1);
+          int page = S.btc[min(i, BT_CACHE - 1)];
+          if (__builtin_expect(i >= BT_CACHE, 0)) page = bt[pg0 + i];
+          page = __builtin_amdgcn_readfirstlane(page);
+          const uint8_t* c = (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
+          if constexpr (P == 16) ch[k] = c;
+          else { ch[2 * k] = c; ch[2 * k + 1] = c; }
         }
-        return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
       };
       __builtin_amdgcn_s_setprio(1);
+      const KOffs<QM, P> koff = key_offsets<QM, P>(lane);
       KRegs<QM> cur;
-      // this wave's current quad of 4 pages: the first one by position
+      // this wave's current quad: the first one by position
       const int nworker = dyn ? p.nsplit * NW : 0;
       int qi = dyn ? split * NW + wave : wave;
-      const uint8_t* mine = chunk_of(qi);
-      if (qi < nquad) load_k<QM, P>(cur, mine, pos);
-      if (!dyn) take = draw();
+      const uint8_t* ch[4];
+      chunks_of(qi, ch);
+      if (qi < nquad) load_k<QM, P>(cur, ch, koff);
       int more = 0, nextq = 0;       // quads left of the batch drawn last (the shared counter hands out DRAW_BATCH at a time)
       while (qi < nquad) {
-        // the next quad: read where the keys of this one are awaited anyway (every older memory operation is then
-        // complete), the following draw goes out ahead of this iteration's loads
-        int qn;
-        if (more > 0) { qn = nextq++; --more; }
-        else {
-          // (the draw made an iteration ago is read here and not before: without the opaque copy its broadcast is
-          // moved up to the draw itself, which then waits for the counter's round trip on the spot)
-          int drawn = take;
-          asm volatile("" : "+v"(drawn));
-          drawn = __builtin_amdgcn_readfirstlane(drawn);
-          qn = (dyn ? (drawn & DRAW_MASK) * DRAW_BATCH : drawn) + nworker;
+        // The next quad.  Shared (device-scope) counter: the draw made an iteration ago is read where the keys of this
+        // quad are awaited anyway, and the following draw goes out ahead of this iteration's loads.  Counter in LDS:
+        // the draw goes out here and is read after the softmax, in this same iteration -- a wavefront that held its
+        // next quad for a whole iteration would start the range's last quad a whole iteration after the others ran dry.
+        int qn = 0;
+        if (dyn) {
+          if (more > 0) { qn = nextq++; --more; }
+          else {
+            // (read here and not before: without the opaque copy its broadcast is moved up to the draw itself, which
+            // then waits for the counter's round trip on the spot)
+            int drawn = take;
+            asm volatile("" : "+v"(drawn));
+            drawn = __builtin_amdgcn_readfirstlane(drawn);
+            qn = (drawn & DRAW_MASK) * DRAW_BATCH + nworker;
+            take = draw();
+            nextq = qn + 1; more = DRAW_BATCH - 1;
+          }
+        } else {
           take = draw();
-          if (dyn) { nextq = qn + 1; more = DRAW_BATCH - 1; }
         }
         VRegs<QM> vr;                // this quad's V^T entries: in flight during the key phase
-        const uint8_t* ch[4];
-        {
-          const unsigned long long mp = reinterpret_cast<unsigned long long>(mine);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {             // (32-token pages: entries 2, 3 repeat page 1 and are not read)
-            const uint32_t lo32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp), (P * k) & 63);
-            const uint32_t hi32 = __builtin_amdgcn_readlane(static_cast<uint32_t>(mp >> 32), (P * k) & 63);
-            ch[k] = reinterpret_cast<const uint8_t*>((static_cast<unsigned long long>(hi32) << 32) | lo32);
-          }
-        }
-        const int tok = (pg0 + PPQ * qi + pi) * P + pos;
-        const bool valid = tok >= lo && tok < hi;
-        // (The scheduler moves the requests for the value entries below the key phase, where the code words' registers
-        // are free.  Pinning them, or half of them, above or inside it costs registers the loop does not have at four
-        // wavefronts per SIMD, and gains nothing at three: measured.)
-        float sc[4] = {sc0, sc0, sc0, sc0};
         load_v<QM, P>(vr, ch, lane);
-        key_phase<QM, K2>(S, cur, p.qscale, sc);
-        softmax_phase<QM>(S, st, cur, sc, valid, lane, wave);
+        bool valid[4];
+        {
+          const int tok0 = (pg0 + PPQ * qi) * P + (lane & 15);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) valid[k] = tok0 + 16 * k >= lo && tok0 + 16 * k < hi;
+        }
+        float sc[4];
+        key_phase<QM, K2>(S, cur, lane, sc);
+        softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
-        // path (past the range chunk_of names the range's last page again, a cache hit nobody uses): were they inside
-        // the branch, the wait counts after the join would be those of the path without them, and the value phase
+        // path (past the range chunks_of names the range's last page again, a cache hit nobody uses): were they inside
+        // a branch, the wait counts after the join would be those of the path without them, and the value phase
         // would wait for these loads as well.
-        mine = chunk_of(qn);
-        load_k<QM, P>(cur, mine, pos);
+        if (!dyn) {
+          int drawn = take;
+          asm volatile("" : "+v"(drawn));
+          qn = __builtin_amdgcn_readfirstlane(drawn);
+        }
+        chunks_of(qn, ch);
+        load_k<QM, P>(cur, ch, koff);
         if (qn < nquad) {
           // once the counter has run dry, the wavefronts that still hold a quad go first: they all end together
           if (qn + NW >= nquad) __builtin_amdgcn_s_setprio(3);
@@ -542,10 +635,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) st.ot[y][r4] = (st.ot[y][r4] - zg) * 16777216.f;
     }
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const float lsum = wave_sum64(st.l[h] * unfold);
-      if (lane == 0) { S.m[wave][h] = st.m[h]; S.l[wave][h] = lsum; }
+    {   // head x = lane >> 4 lives in a row of 16 lanes
+      const float lsum = row_sum16(st.l * unfold);
+      if ((lane & 15) == 0) { S.m[wave][lane >> 4] = st.m; S.l[wave][lane >> 4] = lsum; }
     }
     __syncthreads();     // every wave is done with its strip: the partial outputs may overwrite them
     {
@@ -553,7 +645,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       float M = S.m[0][hl];
 #pragma unroll
       for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][hl]);
-      const float mh = (hl & 2) ? ((hl & 1) ? st.m[3] : st.m[2]) : ((hl & 1) ? st.m[1] : st.m[0]);
+      const float mh = S.m[wave][hl];
       const float f = mh == -INFINITY ? 0.f : fexp2(mh - M);
       float* o = S.o(wave, hl);
 #pragma unroll

@@ -165,17 +165,18 @@ def cb_chunk_bytes(kind: str, page: int, Dh: int = 128) -> int:
 
 # ------------------------------------------------------------------------------------------------ split planner
 _NUM_CU = None
-_OCC: dict = {}
+# 4-wavefront workgroups resident per CU (what the small launch shape's planner fills): the codebook kernels fit 128
+# registers (4 per CU), the static-mask kernels 168 (3 per CU).  The library's own occupancy entry points answer 1 on
+# purpose (one LARGE workgroup per CU: the number a caller written against the reference should plan with).
+SMALL_WG_PER_CU = {"k2": 4, "static": 3}
 
 
-def _slots(key, occ_fn) -> int:
-    """workgroups resident on the GPU at once: occupancy per CU x CU count."""
+def _slots(fmt) -> int:
+    """4-wavefront workgroups resident on the GPU at once."""
     global _NUM_CU
     if _NUM_CU is None:
         _NUM_CU = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-    if key not in _OCC:
-        _OCC[key] = max(1, occ_fn())
-    return _OCC[key] * _NUM_CU
+    return SMALL_WG_PER_CU["k2" if fmt in K2 else "static"] * _NUM_CU
 
 
 BIG_CHUNK = int(os.environ.get("FLAGROT_BIG_CHUNK", "1024"))   # tokens per split from which the library launches large workgroups
@@ -211,14 +212,14 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
     HV = Hkv * -(-G // 4)                                  # workgroups per (row, split): q tiles of 4 heads
-    s = _slots(("v2", fmt, page), lambda: lib().fr_v2_occupancy(V2_FMT[fmt], v2_variant(fmt, G, Dh), STAGES, page))
+    s = _slots(fmt)
     return plan_splits(B, Lmax, HV, page, s, nsplit, ncu=_NUM_CU)
 
 
 def plan_cb(B, Lmax, Hkv, page, kind, nsplit=None, G=4, Dh=128):
     if kind in K2 and (G != 4 or Dh != 128):
         return plan_v2(B, Lmax, Hkv, page, nsplit, fmt=kind, G=G, Dh=Dh)
-    s = _slots(("cb", kind, page), lambda: lib().fr_cb_occupancy(CB_KINDS[kind], 0, STAGES, page))
+    s = _slots(kind)
     return plan_splits(B, Lmax, Hkv, page, s, nsplit, ncu=_NUM_CU)
 
 

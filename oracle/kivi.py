@@ -343,6 +343,24 @@ def dequant_groups(ch, D, dtype=np.float64, basis="orig", f8=False):
     return k, v
 
 
+def attention_reference(q, K, V, kv_start, cached, tailK, tailV, G, scale):
+    """fp64 softmax attention of one sequence (the yardstick of kv_attn; reference test:
+    integrations/vllm_flagrot/tests/test_kivi.py:235-247): q [Hq, D]; K, V [n, Hkv, D] dequantised page rows, of which
+    rows [kv_start, cached) count; tailK, tailV [m, Hkv, D] BF16 ring rows.  Rows without any key give 0."""
+    Hq, D = q.shape
+    out = np.zeros((Hq, D))
+    for hq in range(Hq):
+        h = hq // G
+        k = np.concatenate([K[kv_start:cached, h], tailK[:, h]])
+        v = np.concatenate([V[kv_start:cached, h], tailV[:, h]])
+        if len(k) == 0:
+            continue
+        sc = (k @ q[hq]) * scale
+        p = np.exp(sc - sc.max())
+        out[hq] = (p / p.sum()) @ v
+    return out
+
+
 def lse_merge(oa_bits, la, ob_bits, lb):
     """bf16 LSE merge of two partial attentions: oa, ob uint16 [n, H, D] bf16 patterns, la, lb fp32 [H, n] natural-log
     LSE (+inf treated as -inf).  fp32, every operation rounded on its own; exp in fp32 of the library."""

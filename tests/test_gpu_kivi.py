@@ -229,20 +229,7 @@ def _filled_cache(dev, lens, Hkv, g, tail_T=0):
     return pool, bt, Ks, Vs
 
 
-def _ref_attn(q, K, V, kv_start, cached, tailK, tailV, G, scale):
-    """fp64 softmax attention of one sequence: q [Hq, D]; K, V [n, Hkv, D]; rows [kv_start, cached) + tail rows."""
-    Hq = q.shape[0]
-    out = np.zeros((Hq, D))
-    for hq in range(Hq):
-        h = hq // G
-        k = np.concatenate([K[kv_start:cached, h], tailK[:, h]])
-        v = np.concatenate([V[kv_start:cached, h], tailV[:, h]])
-        if len(k) == 0:
-            continue
-        s = (k @ q[hq]) * scale
-        p = np.exp(s - s.max())
-        out[hq] = (p / p.sum()) @ v
-    return out
+_ref_attn = OK.attention_reference
 
 
 CASES = [
