@@ -113,9 +113,11 @@ DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
       for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
     } else {
       live = var == 0;
-      const bool rot = p.kmask != nullptr && p.kmask[kvh * 4 + g] != 0;
+      // (a bit mask and not `rot ? y[i] : x[i]`: the compiler turns that into a choice between the two arrays'
+      // addresses, which puts both into scratch memory)
+      const uint32_t rot = (p.kmask != nullptr && p.kmask[kvh * 4 + g] != 0) ? 0xFFFFFFFFu : 0u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
+      for (int i = 0; i < 4; ++i) v[i] = __uint_as_float((__float_as_uint(y[i]) & rot) | (__float_as_uint(x[i]) & ~rot));
     }
     uint32_t hb[4], lb[4];
     float qs = 0.f;
@@ -474,6 +476,25 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&
   }
 }
 
+// The workgroup's running maxima per head after every wavefront has put its four into S.m: lane w < NW fetches
+// wavefront w's four at once, one row reduction, one broadcast -- a single LDS round trip (a loop over the
+// wavefronts is NW dependent ones).
+template <int NW, class SM>
+DEVI void workgroup_max(const SM& S, int lane, float (&M)[4]) {
+  float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  if (lane < NW) v = *reinterpret_cast<const float4*>(&S.m[lane][0]);
+  M[0] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.x))));
+  M[1] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.y))));
+  M[2] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.z))));
+  M[3] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.w))));
+}
+// element i of four values held in registers (selects on values: an index into an array of locals would put the
+// array into scratch memory, and a kernel that uses scratch starts its workgroups late)
+DEVI float pick4(float v0, float v1, float v2, float v3, int i) {
+  const float lo = (i & 1) ? v1 : v0, hi = (i & 1) ? v3 : v2;
+  return (i & 2) ? hi : lo;
+}
+
 template <int QM, bool K2, int P, int NW>
 __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4 : 1)) k_decode(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
@@ -485,6 +506,24 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   const int lin = blockIdx.z * gridDim.y + blockIdx.y;
   const int split = lin / p.B, b = lin % p.B;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
+  // The block-table entries of the workgroup's page range are requested before the sequence length is known (the
+  // length load and these loads are then in flight together: one memory latency less before the first page arrives).
+  // If the range is not empty it starts at this token; entries are bounded by the row's length, and whatever lies
+  // past the sequence's last page is never used (page indices are clamped to the range).  Shared rows (stride 0)
+  // have no known length: they are fetched once the length is there.
+  const bool dyn = p.dyn != 0;    // the body workgroups of a (sequence, KV head, q tile) draw quads from one counter
+  const int* const btrow = p.block_table + static_cast<long long>(b) * p.bt_stride;
+  const int pg0s = (dyn ? p.kv_start : max(split * p.chunk, p.kv_start)) / P;
+  constexpr int SPEC = BT_CACHE / (64 * NW);      // entries per thread
+  int spec[SPEC];
+  int nspec = 0;
+  if (!is_tail && p.bt_stride > 0)
+    nspec = min(min(BT_CACHE, p.bt_stride - pg0s), ((dyn ? p.nsplit : 1) * p.chunk + P - 1) / P + 1);
+#pragma unroll
+  for (int k = 0; k < SPEC; ++k) {
+    const int i = threadIdx.x + k * 64 * NW;
+    spec[k] = i < nspec ? btrow[pg0s + i] : 0;
+  }
   const int len = p.seq_lens[b];
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   const bool act = wave < 4;      // the 256 threads that own the workgroup's 4 x 128 outputs
@@ -492,7 +531,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   // the (sequence, KV head, q tile)'s counter slot: merge ticket, and in the dynamic mode the quad draw counter
   const int tpc = p.counter_div;                                 // q tiles that share one counter slot
   int* const ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
-  const bool dyn = p.dyn != 0;    // the body workgroups of a (sequence, KV head, q tile) draw quads from one counter
+  float Mwg[4];                   // the workgroup's maxima per head (uniform)
   if (!is_tail) {
     const int lo = dyn ? min(p.kv_start, len) : max(split * p.chunk, min(p.kv_start, len));
     const int hi = dyn ? len : min(len, (split + 1) * p.chunk);
@@ -517,7 +556,15 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       };
       int take = 0;
       if (dyn) take = draw();        // the first round trip to the device-scope counter hides behind the prologue
-      for (int i = threadIdx.x; i < min(pg1 - pg0, BT_CACHE); i += 64 * NW) S.btc[i] = bt[pg0 + i];
+      if (nspec > 0) {      // (pg0 == pg0s whenever the range is not empty)
+#pragma unroll
+        for (int k = 0; k < SPEC; ++k) {
+          const int i = threadIdx.x + k * 64 * NW;
+          if (i < nspec) S.btc[i] = spec[k];
+        }
+      } else {
+        for (int i = threadIdx.x; i < min(pg1 - pg0, BT_CACHE); i += 64 * NW) S.btc[i] = bt[pg0 + i];
+      }
       if (threadIdx.x == 0) S.next = NW;
       for (int i = threadIdx.x; i < 4 * (4 * PB_RSTRIDE + 1); i += 64 * NW) S.zero[i] = 0u;
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
@@ -635,40 +682,41 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) st.ot[y][r4] = (st.ot[y][r4] - zg) * 16777216.f;
     }
-    {   // head x = lane >> 4 lives in a row of 16 lanes
-      const float lsum = row_sum16(st.l * unfold);
-      if ((lane & 15) == 0) { S.m[wave][lane >> 4] = st.m; S.l[wave][lane >> 4] = lsum; }
-    }
+    // head x = lane >> 4 lives in a row of 16 lanes
+    const float lsum = row_sum16(st.l * unfold);
+    if ((lane & 15) == 0) S.m[wave][lane >> 4] = st.m;
     __syncthreads();     // every wave is done with its strip: the partial outputs may overwrite them
     {
-      const int kc = lane >> 4;      // the lane's four entry rows: 4 kc + r
-      float M = S.m[0][hl];
+      workgroup_max<NW>(S, lane, Mwg);
+      // this wavefront's factors 2^(m - M) per head (uniform): its own maxima sit in lanes 0, 16, 32, 48
+      float f[4];
 #pragma unroll
-      for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][hl]);
-      const float mh = S.m[wave][hl];
-      const float f = mh == -INFINITY ? 0.f : fexp2(mh - M);
+      for (int h = 0; h < 4; ++h) {
+        const float mh = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, st.m), 16 * h));
+        f[h] = mh == -INFINITY ? 0.f : fexp2(mh - Mwg[h]);
+      }
+      if ((lane & 15) == 0) S.l[wave][lane >> 4] = pick4(f[0], f[1], f[2], f[3], lane >> 4) * lsum;
+      const float fl = pick4(f[0], f[1], f[2], f[3], hl);
+      const int kc = lane >> 4;      // the lane's four entry rows: 4 kc + r
       float* o = S.o(wave, hl);
 #pragma unroll
       for (int y = 0; y < 2; ++y) {
         // entry e = 16 (gl & 1) + 4 kc + r, word sub = 2 (gl >> 1) + y: dim 64 (sub >> 1) + 16 (e >> 3) + 8 (sub & 1) + (e & 7)
         const int d = 32 * gl + 16 * (kc >> 1) + 8 * y + 4 * (kc & 1);
-        *reinterpret_cast<float4*>(o + d) = make_float4(f * st.ot[y][0], f * st.ot[y][1], f * st.ot[y][2], f * st.ot[y][3]);
+        *reinterpret_cast<float4*>(o + d) = make_float4(fl * st.ot[y][0], fl * st.ot[y][1], fl * st.ot[y][2], fl * st.ot[y][3]);
       }
     }
     __syncthreads();
   } else {
     float m[4], l[4], o[4][2];
     tail_partial<NW>(p, b, kvh, tile, m, l, o);
-#pragma unroll
-    for (int h = 0; h < 4; ++h)
-      if (lane == 0) { S.m[wave][h] = m[h]; S.l[wave][h] = l[h]; }
+    if (lane < 4) S.m[wave][lane] = pick4(m[0], m[1], m[2], m[3], lane);
     __syncthreads();
+    workgroup_max<NW>(S, lane, Mwg);
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      float M = S.m[0][h];
-#pragma unroll
-      for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][h]);
-      const float f = m[h] == -INFINITY ? 0.f : fexp2(m[h] - M);
+      const float f = m[h] == -INFINITY ? 0.f : fexp2(m[h] - Mwg[h]);
+      if (lane == 0) S.l[wave][h] = f * l[h];
       float* so = S.o(wave, h);
       so[2 * lane] = f * o[h][0];
       so[2 * lane + 1] = f * o[h][1];
@@ -679,13 +727,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   float po[2] = {0.f, 0.f}, pm = -INFINITY, pl = 0.f;
   const int oh = wave & 3;           // head of this thread's two outputs
   if (act) {
-    float M = S.m[0][oh];
-#pragma unroll
-    for (int w = 1; w < NW; ++w) M = fmaxf(M, S.m[w][oh]);
-    float Lsum = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) Lsum += S.m[w][oh] == -INFINITY ? 0.f : fexp2(S.m[w][oh] - M) * S.l[w][oh];
-    pm = M; pl = Lsum;
+    // the sums were scaled by their wavefront's factor when they were stored: lane w fetches wavefront w's
+    const float lw = lane < NW ? S.l[lane][oh] : 0.f;
+    pm = pick4(Mwg[0], Mwg[1], Mwg[2], Mwg[3], oh);
+    pl = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_sum16(lw))));
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
       const float2 v = *reinterpret_cast<const float2*>(S.o(w, oh) + 2 * lane);
