@@ -524,6 +524,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
     const int i = threadIdx.x + k * 64 * NW;
     spec[k] = i < nspec ? btrow[pg0s + i] : 0;
   }
+  // ... and each wavefront asks for the entries of its own first quad itself (lanes 0..3), so that the quad's keys can
+  // be requested as soon as the length has confirmed that the quad lies inside the range: before the query prologue
+  // and its barrier, not after them
+  constexpr int PPQ = 64 / P;                 // pages per quad of 64 tokens (the name stays: 4 pages of 16, 2 of 32)
+  const int qi0 = dyn ? split * NW + wave : wave;
+  int mine4 = 0;
+  if (nspec > 0 && lane < PPQ && PPQ * qi0 + lane < p.bt_stride - pg0s) mine4 = btrow[pg0s + PPQ * qi0 + lane];
   const int len = p.seq_lens[b];
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   const bool act = wave < 4;      // the 256 threads that own the workgroup's 4 x 128 outputs
@@ -556,6 +563,23 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       };
       int take = 0;
       if (dyn) take = draw();        // the first round trip to the device-scope counter hides behind the prologue
+      // this wavefront's first quad, requested now if it lies wholly inside the range (its entries came with mine4)
+      typedef const __attribute__((address_space(1))) uint8_t* gptr;
+      const gptr pool = (gptr)p.pool;
+      const KOffs<QM, P> koff = key_offsets<QM, P>(lane);
+      KRegs<QM> cur;
+      const uint8_t* ch[4];
+      const bool early = nspec > 0 && PPQ * (qi0 + 1) <= pg1 - pg0;      // uniform over the wavefront
+      if (early) {
+#pragma unroll
+        for (int k = 0; k < PPQ; ++k) {
+          const int page = __builtin_amdgcn_readlane(mine4, k);
+          const uint8_t* c = (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
+          if constexpr (P == 16) ch[k] = c;
+          else { ch[2 * k] = c; ch[2 * k + 1] = c; }
+        }
+        load_k<QM, P>(cur, ch, koff);
+      }
       if (nspec > 0) {      // (pg0 == pg0s whenever the range is not empty)
 #pragma unroll
         for (int k = 0; k < SPEC; ++k) {
@@ -569,15 +593,12 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       for (int i = threadIdx.x; i < 4 * (4 * PB_RSTRIDE + 1); i += 64 * NW) S.zero[i] = 0u;
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
-      constexpr int PPQ = 64 / P;                 // pages per quad of 64 tokens (the name stays: 4 pages of 16, 2 of 32)
       const int npg = pg1 - pg0;
       const int nquad = (npg + PPQ - 1) / PPQ;
       // odd tokens: the B fields of a V^T word come out of the unpacking with the factor 2^SH, so their scores are
       // lowered by SH (log2 domain) and their share of the softmax sum is raised again at the end
       const float sc0 = (lane & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
       const float qs20 = p.qscale * (16777216.f / QPRE);         // raw score sums carry 2^-24 from the codes and QPRE from the query
-      typedef const __attribute__((address_space(1))) uint8_t* gptr;
-      const gptr pool = (gptr)p.pool;
       // chunk addresses of a quad's four blocks (wave uniform).  Pages past the range name the range's last page again
       // (their tokens are masked).  The entry comes from LDS; past the cached window it is read from memory.
       auto chunks_of = [&](int quad, const uint8_t* (&ch)[4]) {
@@ -593,14 +614,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         }
       };
       __builtin_amdgcn_s_setprio(1);
-      const KOffs<QM, P> koff = key_offsets<QM, P>(lane);
-      KRegs<QM> cur;
       // this wave's current quad: the first one by position
       const int nworker = dyn ? p.nsplit * NW : 0;
-      int qi = dyn ? split * NW + wave : wave;
-      const uint8_t* ch[4];
-      chunks_of(qi, ch);
-      if (qi < nquad) load_k<QM, P>(cur, ch, koff);
+      int qi = qi0;
+      if (!early) {
+        chunks_of(qi, ch);
+        if (qi < nquad) load_k<QM, P>(cur, ch, koff);
+      }
       int more = 0, nextq = 0;       // quads left of the batch drawn last (the shared counter hands out DRAW_BATCH at a time)
       while (qi < nquad) {
         // The next quad.  Shared (device-scope) counter: the draw made an iteration ago is read where the keys of this
