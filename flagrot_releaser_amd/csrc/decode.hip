@@ -246,11 +246,10 @@ struct WaveState {
   float z[2];        // lane = (page, half, group, head pair): its share of sum p' zero point, heads 2 hp and 2 hp + 1
 };
 
-// exchange with the lane 16 / 32 further (xor): the four lanes of a token
-DEVI uint32_t lane_xor16(uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_ds_swizzle(static_cast<int>(v), (16 << 10) | 0x1F)); }
-DEVI uint32_t lane_xor32(uint32_t v, int lane) {
-  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // r[0] = lower half twice, r[1] = upper half twice
-  return lane < 32 ? r[1] : r[0];
+// exchange among the four lanes of a token (lane ^ 16, ^ 32, ^ 48): one crossbar instruction each, no vector ALU work
+// (a v_permlane32_swap costs two copies, a wait state and a select around it).  byte address of the source lane: 4 x lane
+DEVI uint32_t lane_from(uint32_t v, int src_lane4) {
+  return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(src_lane4, static_cast<int>(v)));
 }
 // all-reduce over the 16 lanes of a row (DPP: quad permutes, then the mirrors of 8 and of 16 lanes)
 DEVI float row_max16(float v) {
@@ -263,12 +262,13 @@ DEVI float row_sum16(float v) {
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
   return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
 }
-// the 16-bit scale word `j` of a packed pair as fp32, sign bit (flag) dropped.  Plain code on purpose: instructions
-// written as inline assembly are invisible to the compiler's hazard handling, and a register that a matrix
-// instruction is still writing (an unused row of its result) may be handed to them as their output.
-DEVI float word_scale(uint32_t pair, int j) {
+// the 16-bit scale word `j` of a packed pair as fp32; its sign bit is a flag, which the caller drops with fabsf (a
+// source modifier of the multiply-add that uses the value).  Plain code on purpose: instructions written as inline
+// assembly are invisible to the compiler's hazard handling, and a register that a matrix instruction is still
+// writing (an unused row of its result) may be handed to them as their output.
+DEVI float word_value(uint32_t pair, int j) {
   const uint16_t w = static_cast<uint16_t>((j & 1) ? (pair >> 16) : pair);
-  return static_cast<float>(__builtin_fabsf16(__builtin_bit_cast(_Float16, w)));
+  return static_cast<float>(__builtin_bit_cast(_Float16, w));
 }
 
 // Scores of the lane's (token, head) for the four blocks of the quad: raw sums 2^-20 sum_j scale_j sum (c - z) q'
@@ -289,8 +289,8 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
     full[b] = false;
     if constexpr (K2) {
       uint32_t f = r.vs[b] & 0x8000u;
-      f |= lane_xor16(f);
-      f |= lane_xor32(f, lane);
+      f |= lane_from(f, 4 * (lane ^ 16));
+      f |= lane_from(f, 4 * (lane ^ 32));
       full[b] = f != 0u;
     }
     sc[b] = 0.f;
@@ -328,7 +328,7 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
         const bool h32 = (kw >> (16 * (j & 1) + 15)) & 1u;
         pick = full[b] ? acc[b][2] : (h32 ? acc[b][1] : acc[b][0]);
       }
-      sc[b] += pick * word_scale(kw, j);
+      sc[b] += pick * fabsf(word_value(kw, j));
     }
   }
 }
@@ -383,7 +383,7 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
     // the token's four V scale words, sign bits stripped: own group x, then the lanes 16, 32, 48 further (groups
     // x ^ 1, x ^ 2, x ^ 3); unwritten slots may hold any pattern: masked
     const uint32_t v0 = valid[b] ? (r.vs[b] & 0x7FFFu) : 0u;
-    const uint32_t v1 = lane_xor16(v0), v2 = lane_xor32(v0, lane), v3 = lane_xor32(v1, lane);
+    const uint32_t v1 = lane_from(v0, 4 * (lane ^ 16)), v2 = lane_from(v0, 4 * (lane ^ 32)), v3 = lane_from(v0, 4 * (lane ^ 48));
     const uint32_t xa = pk_mul(pp, (v1 << 16) | v0), xb = pk_mul(pp, (v3 << 16) | v2);
     uint16_t* row = pb + b * 2 * PB_RSTRIDE * 8;
     row[c0] = static_cast<uint16_t>(xa);
