@@ -43,25 +43,32 @@ DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per
 // row group) start in different banks.
-constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (page, c8): 16 + 1 pad
-constexpr int PB_BYTES = 8 * PB_RSTRIDE * 16;      // per wave: [page][c8][group][head][8 fp16]
+// A wave iteration covers QB blocks of 16 tokens: 4 (64 tokens) for every format.  (Measured for the 2-bit formats:
+// 8 blocks per iteration -- the bytes in flight of a 4-bit iteration -- need 155 registers, i.e. three wavefronts per
+// SIMD instead of four, and are 4 % slower on configs[2]: that loop is bound by instruction issue, not by latency.)
+template <int QM> constexpr int QBLK = 4;
+constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (block, c8): 16 + 1 pad (the pad stays zero: below)
 constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
-constexpr int ZB_BYTES = 8 * ZB_RSTRIDE * 16;      // per wave: [page][c8][group][8 fp16] = zero point (x 2^SH for odd tokens)
-constexpr int STRIP_BYTES = PB_BYTES + ZB_BYTES;   // per wave
+template <int QM> struct Strip {
+  static constexpr int ROWS = 2 * QBLK<QM>;                    // row groups = runs of 8 tokens
+  static constexpr int PB_BYTES = ROWS * PB_RSTRIDE * 16;      // per wave: [block][c8][group][head][8 fp16]
+  static constexpr int ZB_BYTES = ROWS * ZB_RSTRIDE * 16;      // per wave: [block][c8][group][8 fp16] = zero point (x 2^SH for odd tokens)
+  static constexpr int BYTES = PB_BYTES + ZB_BYTES;            // per wave
+};
 constexpr int DRAW_BATCH = 2;                      // quads per draw from the shared (device-scope) counter
 constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
 constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
 constexpr float QPRE = 16.f;                       // the query operands carry 2^4 (fp16 range: |q| up to 127 in any rotation)
 
-template <int NW>
+template <int QM, int NW>
 struct Smem {
+  static constexpr int STRIP_BYTES = Strip<QM>::BYTES, PB_BYTES = Strip<QM>::PB_BYTES;
   // A operands of the score products: [group j][lane of the matrix instruction = row (head, variant) + 16 x k block]
   alignas(16) uint4 qhi[4][64];                      // fp16(q * 2^4 / element factor)
   alignas(16) uint4 qlo[4][64];                      // fp16 of what that rounding left
   alignas(16) uint4 qz[4][64];                       // -(sum of the group's query elements), fp16 pair in k blocks 0 / 1 (first word)
   // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
   alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
-  alignas(16) uint32_t zero[4 * (4 * PB_RSTRIDE + 1)];   // zeros where the matrix value phase reads the strip rows of foreign groups
   float m[NW][4], l[NW][4];
   int btc[BT_CACHE];
   int next;                                          // next quad of 4 pages nobody has taken yet
@@ -165,9 +172,10 @@ template <class T> DEVI T gload(const uint8_t* p) {
 // Value phase: lane = V^T entry `lane` of each of the 4 blocks in turn.
 template <int QM> struct KRegs {
   static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;   // code words per 16-byte / 8-byte quarter row
-  uint32_t kc[4][NW];       // [block][word]: quarter x of token t's code row (word j = group j; 2-bit: groups 2 j, 2 j + 1)
-  uint2 ks[4];              // [block]: the token's 4 K scale words
-  uint16_t vs[4];           // [block]: the token's V scale word of group x; 16 bits wide so that the widening belongs to the use
+  static constexpr int QB = QBLK<QM>;
+  uint32_t kc[QB][NW];      // [block][word]: quarter x of token t's code row (word j = group j; 2-bit: groups 2 j, 2 j + 1)
+  uint2 ks[QB];             // [block]: the token's 4 K scale words
+  uint16_t vs[QB];          // [block]: the token's V scale word of group x; 16 bits wide so that the widening belongs to the use
                             // (a widening at the load would be scheduled right behind it and wait for the keys in flight)
 };
 // The value product P' V runs on the matrix pipe: sixteen v_mfma_f32_16x16x32_f16 per quad of pages, rows = 16 V^T
@@ -176,7 +184,7 @@ template <int QM> struct KRegs {
 // tokens for a (group, head)) the B operand.  The scores stay on the vector pipe (v_dot2_f32_f16).
 template <int QM> struct VRegs {
   static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;
-  uint32_t vc[4][NW];       // [2 (page pair s) + entry half][entry word] of lane (entry m = lane & 15, run kc = lane >> 4)
+  uint32_t vc[QBLK<QM>][NW];   // [2 (block pair s) + entry half][entry word] of lane (entry m = lane & 15, run kc = lane >> 4)
 };
 
 // lane offsets of the key-side loads inside a chunk (block 0 of a page; a 32-token page's second block adds constants)
@@ -193,9 +201,9 @@ DEVI KOffs<QM, P> key_offsets(int lane) {
 }
 // chunk[b]: the chunk of block b's page (wave uniform); 32-token pages: blocks 2 s, 2 s + 1 are the halves of page s
 template <int QM, int P>
-DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[4], const KOffs<QM, P>& o) {
+DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], const KOffs<QM, P>& o) {
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < QBLK<QM>; ++b) {
     const int hp = P == 32 ? (b & 1) : 0;            // second half of a 32-token page: 16 tokens further
     const uint8_t* ch = chunk[b];
     if constexpr (QM == QM_ASYM2) {
@@ -211,14 +219,14 @@ DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[4], const KOffs<QM,
 }
 
 template <int QM, int P>
-DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[4], int lane) {
+DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], int lane) {
   using L = Lay<QM, P>;
   // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of half s of the quad:
   // 16-token pages 2 s, 2 s + 1 with two runs each, or the 32-token page s with four)
   constexpr int R = P / 8;                       // runs of 8 tokens (entries per dim group) per page
   const int m = lane & 15, kc = lane >> 4;
 #pragma unroll
-  for (int s2 = 0; s2 < 2; ++s2) {
+  for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {
     const uint8_t* ch = P == 16 ? ((kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2]) : chunk[2 * s2];
     const int c8 = P == 16 ? (kc & 1) : kc;
 #pragma unroll
@@ -274,15 +282,16 @@ DEVI float word_value(uint32_t pair, int j) {
 // Scores of the lane's (token, head) for the four blocks of the quad: raw sums 2^-20 sum_j scale_j sum (c - z) q'
 // (the factor and qscale are applied with the softmax).
 template <int QM, bool K2, class SM>
-DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
+DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[QBLK<QM>]) {
+  constexpr int QB = QBLK<QM>;
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   // the zero point of group j, masked in place (an fp16 denormal z 2^-24 in the low half of the pair word for even j,
   // in the high half for odd j): lanes of k blocks 0 and 1 feed it (first element pair of their eight) against the pair
   // -(sum q) of the third operand
   const uint32_t zlane = (lane < 32) ? static_cast<uint32_t>(ZM) : 0u;
-  bool full[4];
+  bool full[QB];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < QB; ++b) {
     // the whole-head flag is bit 15 of the token's group-0 V scale word (lane x = 0 of the token's four lanes holds it);
     // the words of the other value groups never carry that bit (scale words are non-negative fp16 patterns), so the
     // union over the four lanes names it
@@ -301,9 +310,12 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
     const half8 qh = __builtin_bit_cast(half8, S.qhi[j][lane]), ql = __builtin_bit_cast(half8, S.qlo[j][lane]);
     half8 qz;
     if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[j][lane]);
+#pragma unroll
+    for (int b0 = 0; b0 < QB; b0 += 4) {
     f32x4 acc[4];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int bb = 0; bb < 4; ++bb) {
+      const int b = b0 + bb;
       uint32_t x[4];
       if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher (2^4 is in its query operand)
         if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
@@ -318,17 +330,19 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
         // (the same instruction as the two products before it: a chain of one kind on one accumulator)
         a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qz, __builtin_bit_cast(half8, make_uint4(zz, 0u, 0u, 0u)), a, 0, 0, 0);
       }
-      acc[b] = a;
+      acc[bb] = a;
     }
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {     // rows 4 x + variant of the product: the lane's head, every variant
+    for (int bb = 0; bb < 4; ++bb) {     // rows 4 x + variant of the product: the lane's head, every variant
+      const int b = b0 + bb;
       const uint32_t kw = (j & 2) ? r.ks[b].y : r.ks[b].x;
-      float pick = acc[b][0];
+      float pick = acc[bb][0];
       if constexpr (K2) {
         const bool h32 = (kw >> (16 * (j & 1) + 15)) & 1u;
-        pick = full[b] ? acc[b][2] : (h32 ? acc[b][1] : acc[b][0]);
+        pick = full[b] ? acc[bb][2] : (h32 ? acc[bb][1] : acc[bb][0]);
       }
       sc[b] += pick * fabsf(word_value(kw, j));
+    }
     }
   }
 }
@@ -337,13 +351,14 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[4]) {
 // beats it; then p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order.
 // qs20 = qscale * 2^20 (the factor the raw score sums lack); sc0 lowers the scores of odd tokens by SH (below).
 template <int QM, class SM>
-DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4], const bool (&valid)[4],
+DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
                         float qs20, float sc0, int lane, int wave) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  constexpr int QB = QBLK<QM>;
   bool beat = false;
   float mx = -INFINITY;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < QB; ++b) {
     sc[b] = valid[b] ? sc[b] * qs20 + sc0 : -INFINITY;
     mx = fmaxf(mx, sc[b]);
   }
@@ -376,7 +391,7 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[4]
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
   const int c0 = ((x) * 4 + x) * 8, c1 = ((x ^ 1) * 4 + x) * 8, c2 = ((x ^ 2) * 4 + x) * 8, c3 = ((x ^ 3) * 4 + x) * 8;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < QB; ++b) {
     const float pe = fexp2(sc[b] - st.m);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
     st.l += pe;
     const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe, pe));
@@ -398,15 +413,16 @@ template <int QM, class SM>
 DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
   // An entry word (entry half eh, word sub) holds channels of group 2 (sub >> 1) + eh only.  The products of all
   // four groups share one accumulator per word parity: the B operand of a group is the strip row with the columns of
-  // the other groups zero (those lanes read a row of zeros instead), so each column collects its own group's rows.
+  // the other groups zero (those lanes read the row group's pad entry, which nobody writes and which is zeroed once),
+  // so each column collects its own group's rows.
   const int n = lane & 15, kc = lane >> 4;
-  const uint4* own = reinterpret_cast<const uint4*>(S.pb(wave)) + kc * PB_RSTRIDE + n;
+  const uint4* rowg = reinterpret_cast<const uint4*>(S.pb(wave)) + kc * PB_RSTRIDE;
 #pragma unroll
-  for (int s2 = 0; s2 < 2; ++s2) {            // 32 tokens: the runs (page 2 s + (kc >> 1), c8 = kc & 1) = strip row group 4 s + kc
+  for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {   // 32 tokens: the runs (block 2 s + (kc >> 1), c8 = kc & 1) = strip row group 4 s + kc
     half8 b[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const uint4* src = (n >> 2) == g ? own : reinterpret_cast<const uint4*>(S.zero);
+      const uint4* src = rowg + ((n >> 2) == g ? n : 16);
       b[g] = __builtin_bit_cast(half8, src[4 * s2 * PB_RSTRIDE]);
     }
 #pragma unroll
@@ -422,8 +438,10 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
         st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aq), b[2 * (sub >> 1) + eh], st.ot[sub & 1], 0, 0, 0);
       }
   }
-  if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (page, page half, group, head pair)
-    const int rg = lane >> 3, g = (lane >> 1) & 3, hp = lane & 1;
+  if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (block, block half, group, head pair), 8 row groups at a time
+#pragma unroll
+    for (int r8 = 0; r8 < Strip<QM>::ROWS; r8 += 8) {
+    const int rg = r8 + (lane >> 3), g = (lane >> 1) & 3, hp = lane & 1;
     const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
     const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
 #pragma unroll
@@ -432,6 +450,7 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
       float a = st.z[e];
       a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
       st.z[e] = a;
+    }
     }
   }
 }
@@ -496,9 +515,9 @@ DEVI float pick4(float v0, float v1, float v2, float v3, int i) {
 }
 
 template <int QM, bool K2, int P, int NW>
-__global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4 : 1)) k_decode(const DecodeParams p, int ntile, int nparts) {
+__global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
-  __shared__ Smem<NW> S;
+  __shared__ Smem<QM, NW> S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile;
   // Workgroups are dispatched in linear order and the CU's arbiter favours the older wavefronts: the splits of one
@@ -527,10 +546,11 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   // ... and each wavefront asks for the entries of its own first quad itself (lanes 0..3), so that the quad's keys can
   // be requested as soon as the length has confirmed that the quad lies inside the range: before the query prologue
   // and its barrier, not after them
-  constexpr int PPQ = 64 / P;                 // pages per quad of 64 tokens (the name stays: 4 pages of 16, 2 of 32)
+  constexpr int QB = QBLK<QM>;                // blocks of 16 tokens per wave iteration ("quad": the name stays)
+  constexpr int PPQ = 16 * QB / P;            // pages per wave iteration
   const int qi0 = dyn ? split * NW + wave : wave;
   int mine4 = 0;
-  if (nspec > 0 && lane < PPQ && PPQ * qi0 + lane < p.bt_stride - pg0s) mine4 = btrow[pg0s + PPQ * qi0 + lane];
+  if (nspec > 0 && lane < PPQ && PPQ * qi0 + lane < p.bt_stride - pg0s) mine4 = btrow[pg0s + PPQ * qi0 + lane];   // (PPQ <= 8)
   const int len = p.seq_lens[b];
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   const bool act = wave < 4;      // the 256 threads that own the workgroup's 4 x 128 outputs
@@ -568,7 +588,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       const gptr pool = (gptr)p.pool;
       const KOffs<QM, P> koff = key_offsets<QM, P>(lane);
       KRegs<QM> cur;
-      const uint8_t* ch[4];
+      const uint8_t* ch[QB];
       const bool early = nspec > 0 && PPQ * (qi0 + 1) <= pg1 - pg0;      // uniform over the wavefront
       if (early) {
 #pragma unroll
@@ -590,7 +610,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         for (int i = threadIdx.x; i < min(pg1 - pg0, BT_CACHE); i += 64 * NW) S.btc[i] = bt[pg0 + i];
       }
       if (threadIdx.x == 0) S.next = NW;
-      for (int i = threadIdx.x; i < 4 * (4 * PB_RSTRIDE + 1); i += 64 * NW) S.zero[i] = 0u;
+      // the pad entry of every strip row group: what the value phase reads for the columns of foreign groups
+      for (int i = threadIdx.x; i < NW * Strip<QM>::ROWS; i += 64 * NW)
+        (reinterpret_cast<uint4*>(S.pb(i / Strip<QM>::ROWS)) + (i % Strip<QM>::ROWS) * PB_RSTRIDE)[16] = make_uint4(0u, 0u, 0u, 0u);
       if (act) q_prologue<QM, K2>(S, p, b, kvh, tile);
       __syncthreads();
       const int npg = pg1 - pg0;
@@ -601,7 +623,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
       const float qs20 = p.qscale * (16777216.f / QPRE);         // raw score sums carry 2^-24 from the codes and QPRE from the query
       // chunk addresses of a quad's four blocks (wave uniform).  Pages past the range name the range's last page again
       // (their tokens are masked).  The entry comes from LDS; past the cached window it is read from memory.
-      auto chunks_of = [&](int quad, const uint8_t* (&ch)[4]) {
+      auto chunks_of = [&](int quad, const uint8_t* (&ch)[QB]) {
 #pragma unroll
         for (int k = 0; k < PPQ; ++k) {
           const int i = min(PPQ * quad + k, npg - 1);
@@ -645,13 +667,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
         }
         VRegs<QM> vr;                // this quad's V^T entries: in flight during the key phase
         load_v<QM, P>(vr, ch, lane);
-        bool valid[4];
+        bool valid[QB];
         {
           const int tok0 = (pg0 + PPQ * qi) * P + (lane & 15);
 #pragma unroll
-          for (int k = 0; k < 4; ++k) valid[k] = tok0 + 16 * k >= lo && tok0 + 16 * k < hi;
+          for (int k = 0; k < QB; ++k) valid[k] = tok0 + 16 * k >= lo && tok0 + 16 * k < hi;
         }
-        float sc[4];
+        float sc[QB];
         key_phase<QM, K2>(S, cur, lane, sc);
         softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
@@ -856,9 +878,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 16 ? 4 : NW == 12 ? 3 : (K2 ? 4
   }
 }
 
-// Wavefronts per workgroup: 4, or from 1024 tokens per split one large workgroup that fills a CU.  The codebook
-// kernels fit 128 registers per lane: 16 wavefronts (4 per SIMD); the static-mask kernels need more: 12 (168 registers).
-template <bool K2> constexpr int BIGW = K2 ? 16 : 12;
+// Wavefronts per workgroup: 4, or from 1024 tokens per split one large workgroup that fills a CU: 16 wavefronts
+// (4 per SIMD; every format's loop fits 128 registers per lane).
+template <int QM> constexpr int BIGW = 16;
 constexpr int BIG_CHUNK = 1024;   // tokens per split from which the large workgroup pays (measured: batch 1-16, 2-32 k tokens)
 inline int waves_for(int chunk_tokens) { return chunk_tokens >= BIG_CHUNK ? 16 : 4; }   // > 4 selects the large workgroup
 
@@ -870,9 +892,9 @@ int launch_qm(const DecodeParams& p, hipStream_t st) {
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
   if (p.page == 32) {
-    if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 32, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
+    if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 32, BIGW<QM>>), grid, dim3(64 * BIGW<QM>), 0, st, p, ntile, nparts);
     else hipLaunchKernelGGL((k_decode<QM, K2, 32, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
-  } else if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW<K2>>), grid, dim3(64 * BIGW<K2>), 0, st, p, ntile, nparts);
+  } else if (p.wg_waves > 4) hipLaunchKernelGGL((k_decode<QM, K2, 16, BIGW<QM>>), grid, dim3(64 * BIGW<QM>), 0, st, p, ntile, nparts);
   else hipLaunchKernelGGL((k_decode<QM, K2, 16, 4>), grid, dim3(256), 0, st, p, ntile, nparts);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
@@ -892,8 +914,8 @@ int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
 template <int QM, bool K2>
 int occupancy_qm(int waves) {
   int n = 0;
-  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW<K2>>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * (waves > 4 ? BIGW<K2> : 4), 0) != hipSuccess || n < 1) {
+  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW<QM>>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * (waves > 4 ? BIGW<QM> : 4), 0) != hipSuccess || n < 1) {
     (void)hipGetLastError();
     return waves > 4 ? 1 : 2;
   }

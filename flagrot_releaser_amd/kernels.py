@@ -165,18 +165,15 @@ def cb_chunk_bytes(kind: str, page: int, Dh: int = 128) -> int:
 
 # ------------------------------------------------------------------------------------------------ split planner
 _NUM_CU = None
-# 4-wavefront workgroups resident per CU (what the small launch shape's planner fills): the codebook kernels fit 128
-# registers (4 per CU), the static-mask kernels 168 (3 per CU).  The library's own occupancy entry points answer 1 on
-# purpose (one LARGE workgroup per CU: the number a caller written against the reference should plan with).
-SMALL_WG_PER_CU = {"k2": 4, "static": 3}
-
-
+# 4-wavefront workgroups resident per CU (what the small launch shape's planner fills): 4 (every format's loop fits
+# 128 registers).  The library's own occupancy entry points answer 1 on purpose (one LARGE workgroup per CU: the number
+# a caller written against the reference should plan with).
 def _slots(fmt) -> int:
     """4-wavefront workgroups resident on the GPU at once."""
     global _NUM_CU
     if _NUM_CU is None:
         _NUM_CU = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-    return SMALL_WG_PER_CU["k2" if fmt in K2 else "static"] * _NUM_CU
+    return 4 * _NUM_CU
 
 
 BIG_CHUNK = int(os.environ.get("FLAGROT_BIG_CHUNK", "1024"))   # tokens per split from which the library launches large workgroups
