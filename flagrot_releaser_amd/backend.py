@@ -272,9 +272,13 @@ class KiviDecodeLayer:
     """KIVI-style pages: values written per token, key groups of 32 tokens encoded when they complete (from the prompt
     rows at prefill, from the BF16 ring at decode: the window must hold a whole group, W >= 32)."""
 
-    def __init__(self, Hkv: int, G: int, pool: torch.Tensor, builder: MetadataBuilder, qs, lz, co, scale: float = None):
+    def __init__(self, Hkv: int, G: int, pool: torch.Tensor, builder: MetadataBuilder, qs, lz, co, scale: float = None,
+                 f8: bool = False):
+        """f8: FP8-meta pages (the reference's `kivi_f8` option, attention/backend.py:365-366): pool chunks of
+        KIVI.chunk_bytes(D, True) bytes."""
         assert builder.kind == "kivi2" and builder.W >= 32, "kivi2 needs a BF16 window of at least one key group"
-        self.Hkv, self.G, self.pool, self.b = Hkv, G, pool, builder
+        assert pool.shape[-1] == KIVI.chunk_bytes(D, f8), "pool chunk size does not match the page format"
+        self.Hkv, self.G, self.pool, self.b, self.f8 = Hkv, G, pool, builder, f8
         self.S, self.W, self.T, self.R = builder.S, builder.W, builder.S + builder.W, builder.R
         self.scale = scale if scale is not None else 1.0 / math.sqrt(D)
         self.qs, self.lz, self.co = qs, lz, co             # calibration queries, their log normalisers, value weights
@@ -286,7 +290,7 @@ class KiviDecodeLayer:
         """a fresh prompt of n tokens: values of every token, the whole key groups, sinks and newest W rows in BF16"""
         n = kv.shape[0]
         dev = kv.device
-        KIVI.v_write(kv, slots, self.co, None, self.pool, self.Hkv, D)
+        KIVI.v_write(kv, slots, self.co, None, self.pool, self.Hkv, D, f8=self.f8)
         pos = torch.arange(n, device=dev)
         keep = (pos < self.S) | (pos >= n - self.W)
         self.ring.view(self.R + 1, self.T, 2 * self.Hkv, D)[req].index_copy_(0, ring_slot(pos[keep], self.S, self.W), kv[keep])
@@ -295,12 +299,13 @@ class KiviDecodeLayer:
             gp = pos[:32 * ng].view(ng, 32)
             sidx = torch.where(gp < self.S, torch.full_like(gp, -1), gp).contiguous()
             KIVI.k_encode(kv, sidx, slots[:32 * ng].view(ng, 32).contiguous(), self.qs, self.lz, self.scale, self.pool,
-                          self.Hkv, D)
+                          self.Hkv, D, f8=self.f8)
 
     def update(self, kv, md: DecodeMetadata):
-        KIVI.v_write(kv, md.slot_mapping, self.co, None, self.pool, self.Hkv, D)
+        KIVI.v_write(kv, md.slot_mapping, self.co, None, self.pool, self.Hkv, D, f8=self.f8)
         self.ring.index_copy_(0, md.dec_ring_pos, kv)
-        KIVI.k_encode(self.ring, md.kivi_sidx, md.kivi_dslot, self.qs, self.lz, self.scale, self.pool, self.Hkv, D)
+        KIVI.k_encode(self.ring, md.kivi_sidx, md.kivi_dslot, self.qs, self.lz, self.scale, self.pool, self.Hkv, D,
+                      f8=self.f8)
 
     def decode(self, q, md: DecodeMetadata, out):
         nd = q.shape[0]
@@ -308,7 +313,7 @@ class KiviDecodeLayer:
             q = q.contiguous()
         KIVI.attn(q, self.pool, md.block_table[:nd], md.dec_cached, out, md.nsplit, md.chunk, self.ws,
                   self.scale * LOG2E, self.S, self.G, ring=self.ring, tail_len=md.dec_tail_len,
-                  tail_idx=md.dec_tail_idx, T=self.T)
+                  tail_idx=md.dec_tail_idx, T=self.T, f8=self.f8)
 
     def step(self, q, kv, md: DecodeMetadata, out):
         self.update(kv, md)

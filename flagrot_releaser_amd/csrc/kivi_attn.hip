@@ -59,10 +59,9 @@ int kv_v_write(const void* kv, long long kv_rs, int n, int Hkv, int D, const voi
                void* pool, int ident, const void* vfix, int f8, void* stream) {
   if (n <= 0) return 0;
   if (D != 128) return bad("kv_v_write: head dim 128 only");
-  if (f8) return bad("kv_v_write: FP8-meta pages are not built");
   if (M != nullptr) return bad("kv_v_write: matrix weighting M is not built (diag co only)");
   return launched(v_write_launch(kv, kv_rs, n, Hkv, static_cast<const long long*>(slots), static_cast<const float*>(co),
-                                 static_cast<uint8_t*>(pool), ident, static_cast<const int*>(vfix),
+                                 static_cast<uint8_t*>(pool), ident, static_cast<const int*>(vfix), f8 & 1,
                                  static_cast<hipStream_t>(stream)), "kv_v_write");
 }
 
@@ -71,11 +70,10 @@ int kv_k_encode(const void* src, long long src_rs, const void* src2, long long s
                 int ident, const void* kfix, int f8, void* stream) {
   if (N <= 0) return 0;
   if (D != 128) return bad("kv_k_encode: head dim 128 only");
-  if (f8) return bad("kv_k_encode: FP8-meta pages are not built");
   return launched(k_encode_launch(src, src_rs, src2, src2_rs, static_cast<const long long*>(sidx),
                                   static_cast<const long long*>(dslot), N, Hkv, static_cast<const float*>(qs),
                                   static_cast<const float*>(lz), NQ, qsc, static_cast<uint8_t*>(pool), ident,
-                                  static_cast<const int*>(kfix), static_cast<hipStream_t>(stream)), "kv_k_encode");
+                                  static_cast<const int*>(kfix), f8 & 1, static_cast<hipStream_t>(stream)), "kv_k_encode");
 }
 
 int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
@@ -85,10 +83,9 @@ int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, lon
   if (B <= 0) return 0;
   if (G > 8 || G < 1 || chunk % 32 || chunk <= 0) { std::snprintf(g_err, sizeof(g_err), "kv_attn: G %d chunk %d", G, chunk); return 2; }
   if (D != 128) return bad("kv_attn: head dim 128 only");
-  if (f8 & 1) return bad("kv_attn: FP8-meta pages are not built");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int rc = attn_splits_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
-                                    tail_idx, T, opart, ml, st);
+                                    tail_idx, T, opart, ml, f8 & 1, st);
   if (rc) return launched(rc, "kv_attn");
   hipLaunchKernelGGL(k_merge, dim3(B, Hkv * G), dim3(128), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
                      Hkv, G, NS, static_cast<uint16_t*>(out), out_rs);
@@ -99,9 +96,8 @@ int kv_dequant(const void* pool, const void* bt, int g0, int g1, int nvalid, int
                int f8, void* stream) {
   if (g1 <= g0) return 0;
   if (D != 128) return bad("kv_dequant: head dim 128 only");
-  if (f8 & 1) return bad("kv_dequant: FP8-meta pages are not built");
   return launched(dequant_launch(static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), g0, g1, nvalid, Hkv, fp32, ok,
-                                 ov, static_cast<hipStream_t>(stream)), "kv_dequant");
+                                 ov, f8 & 1, static_cast<hipStream_t>(stream)), "kv_dequant");
 }
 
 int kv_lse_merge(const void* oa, const void* la, long long la_hs, const void* ob, const void* lb, long long lb_hs,

@@ -18,6 +18,10 @@
 //                bytes (transposed through LDS as zero-extended 16-bit values, so a 128-bit read is four token pairs)
 //                masked in place to the row's 2-bit field.  sum p * min per (head, class, sub-vector): one more
 //                16x16x32 product.  o = accI + H32(accH) + H128(accF) once per workgroup.
+// FP8-meta pages (template flag F8; 1280-byte chunks, kivi.cu:28-35): scale and min are E4M3 bytes.  An E4M3 pattern
+// shifted left by 7 is the fp16 pattern of value / 256 (same mantissa position, exponent bias 15 instead of 7; E4M3
+// subnormals land on fp16 subnormals), so one packed fp16 multiply by 256 -- folded into a factor the f16 path applies
+// anyway where there is one -- gives the exact value, and the rest of the loop is shared with the FP16-meta pages.
 // Semantics follow integrations/vllm_flagrot/csrc/kivi.cu:729-980 (k_attn).
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
@@ -45,7 +49,11 @@ template <class T> DEVI T gload(const uint8_t* p) {
   typedef const __attribute__((address_space(1))) T* gp;
   return *(gp)(p);
 }
-constexpr int CHUNK = 1552, KM_OFF = 512, VC_OFF = 768, VM_OFF = 1280, VF_OFF = 1536;
+constexpr int KM_OFF = 512, VF_OFF = 1536;                                     // VF: FP16-meta pages only
+template <bool F8> constexpr int CHUNK = F8 ? 1280 : 1552;
+template <bool F8> constexpr int VC_OFF = F8 ? 640 : 768;
+template <bool F8> constexpr int VM_OFF = F8 ? 1152 : 1280;
+constexpr uint32_t X256 = 0x5C005C00u;                                         // fp16 pair (256, 256)
 constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
 constexpr int QROW = 68;                        // words per row of the query strips: 64 + 4 pad (conflict-free 128-bit rows)
 constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad
@@ -76,21 +84,29 @@ struct Smem {
 
 struct GroupRegs {
   u32x2 ka, kb;  // lane (token m = lane & 15 of page A / B, quarter kc = lane >> 4): code words 2 kc, 2 kc + 1 of the token
-  u32x2 km;      // lane = channel pair: (scale | min << 16) of channels 2 l, 2 l + 1
+  u32x2 km;      // lane = channel pair: (scale | min << 16) of channels 2 l, 2 l + 1; F8: .x = bytes (s, m, s, m) of the pair
   u32x4 vc;      // lane (token, half): the token's code bytes of sub-vectors 2 half, 2 half + 1
-  u32x2 vm;      // lane (token, half): (scale | min << 16) of sub-vectors 2 half, 2 half + 1
-  uint32_t vf;   // the token's whole-head flag byte
+  u32x2 vm;      // lane (token, half): (scale | min << 16) of sub-vectors 2 half, 2 half + 1; F8: .x = bytes (s, m, s, m)
+  uint32_t vf;   // the token's whole-head flag: non-zero = H128
 };
 
+template <bool F8>
 DEVI void load_group(GroupRegs& r, const uint8_t* chA, const uint8_t* chB, int lane) {
   const int t = lane & 31, hh = lane >> 5;
   const uint8_t* cht = t < 16 ? chA : chB;
   r.ka = gload<u32x2>(chA + (lane & 15) * 32 + 8 * (lane >> 4));
   r.kb = gload<u32x2>(chB + (lane & 15) * 32 + 8 * (lane >> 4));
-  r.km = gload<u32x2>((lane < 32 ? chA : chB) + KM_OFF + (lane & 31) * 8);
-  r.vc = gload<u32x4>(cht + VC_OFF + (t & 15) * 32 + 16 * hh);
-  r.vm = gload<u32x2>(cht + VM_OFF + (t & 15) * 16 + 8 * hh);
-  r.vf = gload<uint8_t>(cht + VF_OFF + (t & 15));
+  r.vc = gload<u32x4>(cht + VC_OFF<F8> + (t & 15) * 32 + 16 * hh);
+  if (F8) {
+    // channels 2 l, 2 l + 1 = slots 2 (l & 1), 2 (l & 1) + 1 of cell l >> 1: four bytes at 4 l
+    r.km = u32x2{gload<uint32_t>((lane < 32 ? chA : chB) + KM_OFF + (lane & 31) * 4), 0u};
+    r.vm = u32x2{gload<uint32_t>(cht + VM_OFF<true> + (t & 15) * 8 + 4 * hh), 0u};
+    r.vf = gload<uint8_t>(cht + KM_OFF + (t & 15) * 8 + 6) & 0x80u;      // bit 7 of the key scale byte in slot 3 of the token's cell
+  } else {
+    r.km = gload<u32x2>((lane < 32 ? chA : chB) + KM_OFF + (lane & 31) * 8);
+    r.vm = gload<u32x2>(cht + VM_OFF<false> + (t & 15) * 16 + 8 * hh);
+    r.vf = gload<uint8_t>(cht + VF_OFF + (t & 15));
+  }
 }
 
 // The BF16 ring rows of one sequence (split index NS): rows [0, tail_len) of ring block tail_idx, K row h, V row Hkv + h,
@@ -162,6 +178,7 @@ DEVI void tail_split(Smem& S, const uint16_t* __restrict__ q, long long q_rs, co
   }
 }
 
+template <bool F8>
 __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restrict__ q, long long q_rs,
                                                     const uint8_t* __restrict__ pool, const int* __restrict__ bt,
                                                     long long bt_rs, const int* __restrict__ cached, int kv_start, int Hkv,
@@ -220,12 +237,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   const int kq = lane & 7;
   const float qfold = __uint_as_float((127u - 2u * static_cast<uint32_t>(kq < 5 ? kq : kq - 5)) << 23);
   const uint32_t vmask = 0x00030003u << (2 * (l32 & 3));      // value layout row = channel l32: field l32 & 3 of byte l32 >> 2
+  const uint32_t qfold8 = pack_rn(256.f * qfold, 256.f * qfold);
   const half8 tiny = __builtin_bit_cast(half8, u32x4{0x00010001u, 0x00010001u, 0x00010001u, 0x00010001u});   // 2^-24 in every slot
 
   GroupRegs cur;
   int gi = g_first + wv;
-  if (gi < g_end) load_group(cur, pool + (static_cast<long long>(btb[2 * gi]) * Hkv + h) * CHUNK,
-                             pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNK, lane);
+  if (gi < g_end) load_group<F8>(cur, pool + (static_cast<long long>(btb[2 * gi]) * Hkv + h) * CHUNK<F8>,
+                                 pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNK<F8>, lane);
   for (; gi < g_end; gi += 4) {
     const bool full = gi * 32 >= t0 && gi * 32 + 32 <= t1;     // every token of the group is inside the range (wave uniform)
     // The next group is requested on every path (past the range: the range's last group again, a cache hit nobody
@@ -234,20 +252,29 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     GroupRegs nxt;
     {
       const int gn = min(gi + 4, g_end - 1);
-      load_group(nxt, pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNK,
-                 pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNK, lane);
+      load_group<F8>(nxt, pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNK<F8>,
+                     pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNK<F8>, lane);
     }
     // ---- group flags; q' * scale and q' * min strips: lane = channel pair
     {
-      const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = __builtin_amdgcn_readlane(cur.km.y, 0),
-                     s2 = __builtin_amdgcn_readlane(cur.km.x, 1), s3 = __builtin_amdgcn_readlane(cur.km.y, 1),
-                     s4 = __builtin_amdgcn_readlane(cur.km.x, 2);
-      const bool useF = (s4 >> 15) & 1u;
-      const uint32_t lmask = ((s0 >> 15) & 1u) | (((s1 >> 15) & 1u) << 1) | (((s2 >> 15) & 1u) << 2) | (((s3 >> 15) & 1u) << 3);
+      // flag channels: 0 .. 3 and 4 (F8: 0, 4, 8, 12 and 16, the first byte of lanes 0, 2, 4, 6 and 8)
+      const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = F8 ? __builtin_amdgcn_readlane(cur.km.x, 2) : __builtin_amdgcn_readlane(cur.km.y, 0),
+                     s2 = __builtin_amdgcn_readlane(cur.km.x, F8 ? 4 : 1), s3 = F8 ? __builtin_amdgcn_readlane(cur.km.x, 6) : __builtin_amdgcn_readlane(cur.km.y, 1),
+                     s4 = __builtin_amdgcn_readlane(cur.km.x, F8 ? 8 : 2);
+      constexpr int FB = F8 ? 7 : 15;
+      const bool useF = (s4 >> FB) & 1u;
+      const uint32_t lmask = ((s0 >> FB) & 1u) | (((s1 >> FB) & 1u) << 1) | (((s2 >> FB) & 1u) << 2) | (((s3 >> FB) & 1u) << 3);
       const int which = useF ? 2 : static_cast<int>((lmask >> (lane >> 4)) & 1u);
       // fp16 products of the fp16 query pair with (scale * 2^-shift) and with min
-      const uint32_t spair = pack_rn(f16_value(cur.km.x & 0x7FFFu) * qfold, f16_value(cur.km.y & 0x7FFFu) * qfold);
-      const uint32_t mpair = (cur.km.x >> 16) | (cur.km.y & 0xFFFF0000u);
+      uint32_t spair, mpair;
+      if (F8) {
+        const uint32_t mb = (cur.km.x >> 8) & 0x00FF00FFu;
+        spair = pk_mul((cur.km.x & 0x007F007Fu) << 7, qfold8);
+        mpair = pk_mul(((mb & 0x007F007Fu) << 7) | ((mb & 0x00800080u) << 8), X256);
+      } else {
+        spair = pack_rn(f16_value(cur.km.x & 0x7FFFu) * qfold, f16_value(cur.km.y & 0x7FFFu) * qfold);
+        mpair = (cur.km.x >> 16) | (cur.km.y & 0xFFFF0000u);
+      }
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const uint32_t qq = S.qh[which][g][lane];
@@ -262,7 +289,11 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       const bool vF = cur.vf != 0;
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
-        const uint32_t w = jj ? cur.vm.y : cur.vm.x;
+        uint32_t w;                                    // fp16 scale (bit 15 = H32) | fp16 min << 16
+        if (F8) {
+          const uint32_t b2 = jj ? cur.vm.x >> 16 : cur.vm.x;                         // s8 | m8 << 8
+          w = pk_mul(((b2 & 0x7Fu) << 7) | ((b2 & 0x7F00u) << 15) | ((b2 & 0x8000u) << 16), X256) | ((b2 & 0x80u) << 8);
+        } else w = jj ? cur.vm.y : cur.vm.x;
         const int j = 2 * hh + jj;
         int cls = vF ? 2 : static_cast<int>((w >> 15) & 1u);
         if (!full) cls = (pos >= t0 && pos < t1) ? cls : 3;
@@ -439,14 +470,17 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
 
 int launch_pages(int Gq, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
                  int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring, const void* tail_len,
-                 const void* tail_idx, int T, void* opart, void* ml, hipStream_t st) {
+                 const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st) {
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages), hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(sizeof(Smem))) != hipSuccess) return 1;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(sizeof(Smem))) != hipSuccess) return 1;
     attr = true;
   }
-  hipLaunchKernelGGL(k_attn_pages, dim3(B, Hkv, NS + 1), dim3(256), sizeof(Smem), st, static_cast<const uint16_t*>(q), q_rs,
+  const auto kern = f8 ? k_attn_pages<true> : k_attn_pages<false>;
+  hipLaunchKernelGGL(kern, dim3(B, Hkv, NS + 1), dim3(256), sizeof(Smem), st, static_cast<const uint16_t*>(q), q_rs,
                      static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), bt_rs, static_cast<const int*>(cached),
                      kv_start, Hkv, NS, chunk, qscale, static_cast<float*>(opart), static_cast<float*>(ml), Gq,
                      static_cast<const uint16_t*>(ring), static_cast<const int*>(tail_len), static_cast<const int*>(tail_idx), T);
@@ -457,9 +491,9 @@ int launch_pages(int Gq, const void* q, long long q_rs, const void* pool, const 
 
 int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
                        const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
-                       const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, hipStream_t st) {
+                       const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st) {
   if (G < 1 || G > GT) return 2;
-  return launch_pages(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len, tail_idx, T, opart, ml, st);
+  return launch_pages(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len, tail_idx, T, opart, ml, f8, st);
 }
 
 }  // namespace frkv

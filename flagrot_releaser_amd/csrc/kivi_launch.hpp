@@ -1,4 +1,4 @@
-// Launcher prototypes shared by the translation units of libflagrot_kivi.so (head dim 128, FP16 scale / min).
+// Launcher prototypes shared by the translation units of libflagrot_kivi.so (head dim 128; f8: FP8-meta pages).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -6,18 +6,18 @@
 namespace frkv {
 
 int v_write_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
-                   int ident, const int* vfix, hipStream_t st);
+                   int ident, const int* vfix, int f8, hipStream_t st);
 int k_encode_launch(const void* src, long long src_rs, const void* src2, long long src2_rs, const long long* sidx,
                     const long long* dslot, int N, int Hkv, const float* qs, const float* lz, int NQ, float qsc,
-                    uint8_t* pool, int ident, const int* kfix, hipStream_t st);
+                    uint8_t* pool, int ident, const int* kfix, int f8, hipStream_t st);
 int dequant_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nvalid, int Hkv, int fp32, void* ok, void* ov,
-                   hipStream_t st);
+                   int f8, hipStream_t st);
 int lse_merge_launch(const void* oa, const float* la, long long la_hs, const void* ob, const float* lb, long long lb_hs,
                      void* out, long long out_rs, int na, int H, int D, hipStream_t st);
 // splits [0, NS) over the pages and split NS over the BF16 ring rows (kivi_decode.hip): partials per (sequence, KV head,
 // split): opart fp32 [.., G, 128] unnormalised, ml fp32 [.., G, 2] = (maximum in log2 units, sum)
 int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
                        const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
-                       const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, hipStream_t st);
+                       const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st);
 
 }  // namespace frkv

@@ -8,6 +8,13 @@
 // (fp16 scale with sign = H32, fp16 min) | VF @1536 [16] u8 (value uses H_128).  Key flags: scale sign of channel
 // j < 4 = sub-vector j is H32; of channel 4 = whole head H_128.
 //
+// FP8-meta pages (F8; kivi.cu:28-35, 84-88, 123-128): scale and min are rounded to E4M3 (nearest even, saturating at
+// +-448) BEFORE the codes are computed, so the codes belong to the stored values.  Chunk of 1280 bytes: KC @0 | KM8 @512
+// [16][4] byte pairs (s8 | flag << 7, m8) | VC @640 | VM8 @1152 [16][4] byte pairs (bit 7 of s8 = H32).  Key flags: bit 7
+// of the scale byte of channel 4 j (slot 0 of cell j) = sub-vector j is H32, of channel 16 (slot 0 of cell 4) = whole
+// head.  Bit 7 of the KEY scale byte in slot 3 of a cell is the whole-head flag of the VALUE row stored in that cell: the
+// value writer sets it with a byte read-modify-write, the key encoder keeps what it finds there.
+//
 // One half wave (32 lanes) owns a 128-d row, 4 channels per lane (the helpers of fr_common.hpp).
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
@@ -17,6 +24,31 @@ using namespace fr;
 namespace {
 
 DEVI float kv_scale(float mn, float mx) { return (mx - mn) * (1.0f / 3.0f); }
+// fp32 -> E4M3 byte (1 sign, 4 exponent bits of bias 7, 3 mantissa bits, no infinities; kivi.cu:113-121): nearest even,
+// saturating at +-448.  Below 2^-6 the grid is m 2^-9 (pattern = m, and m = 8 is the pattern of 2^-6); above, the fp32
+// mantissa is rounded to 3 bits in place (a carry moves into the exponent, never past 448 = 1.75 2^8).
+DEVI uint32_t e4m3_bits(float x) {
+  const float a = fminf(fabsf(x), 448.f);
+  uint32_t code;
+  if (a < 0.015625f) code = static_cast<uint32_t>(rintf(a * 512.f));
+  else {
+    uint32_t b = __float_as_uint(a);
+    b += 0x7FFFFu + ((b >> 20) & 1u);
+    code = (b >> 20) - (120u << 3);
+  }
+  return code | ((__float_as_uint(x) >> 24) & 0x80u);
+}
+DEVI float e4m3_value(uint32_t b) {
+  const uint32_t e = (b >> 3) & 15u, m = b & 7u;
+  const float a = e == 0 ? static_cast<float>(m) * 0.001953125f : __uint_as_float(((e + 120u) << 23) | (m << 20));
+  return (b & 0x80u) ? -a : a;
+}
+template <bool F8> constexpr long long CHUNK = F8 ? 1280 : 1552;
+template <bool F8> constexpr int VC_AT = F8 ? 640 : 768;
+template <bool F8> constexpr int VM_AT = F8 ? 1152 : 1280;
+template <bool F8> DEVI void kv_params(float& mn, float& s) {         // the (min, scale) the codes are computed from
+  if (F8) { mn = e4m3_value(e4m3_bits(mn)); s = e4m3_value(e4m3_bits(s)); }
+}
 DEVI int kv_code(float x, float mn, float s) {
   const float d = s == 0.f ? 1.f : s;
   float q = (x - mn) / d;
@@ -30,6 +62,7 @@ template <int C> DEVI void to_basis(float (&y)[4], int l32) {   // candidate 0 i
 }
 
 // ------------------------------------------------------------------------------------------------ value writer
+template <bool F8>
 __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv, long long kv_rs, int n, int Hkv,
                                                  const long long* __restrict__ slots, const float* __restrict__ co,
                                                  uint8_t* __restrict__ pool, int ident, const int* __restrict__ vfix) {
@@ -52,7 +85,8 @@ __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv
     if (c == 2) fwht<128>(y, l32);
     float mn = fminf(fminf(y[0], y[1]), fminf(y[2], y[3])), mx = fmaxf(fmaxf(y[0], y[1]), fmaxf(y[2], y[3]));
     mn = gmin8(mn); mx = gmax8(mx);
-    const float s = kv_scale(mn, mx);
+    float s = kv_scale(mn, mx);
+    kv_params<F8>(mn, s);
     sc[c] = s; mnv[c] = mn;
 #pragma unroll
     for (int i = 0; i < 4; ++i) { code[c][i] = kv_code(y[i], mn, s); y[i] = kv_rec(code[c][i], mn, s); }
@@ -81,16 +115,26 @@ __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv
   }
   const int cand = useF ? 2 : (useH ? 1 : 0);
   const int* cd = cand == 0 ? code[0] : cand == 1 ? code[1] : code[2];
-  uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * 1552ll;
+  uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * CHUNK<F8>;
   const int off = static_cast<int>(slot % 16);
-  chunk[768 + off * 32 + l32] = static_cast<uint8_t>((cd[0] & 3) | ((cd[1] & 3) << 2) | ((cd[2] & 3) << 4) | ((cd[3] & 3) << 6));
+  chunk[VC_AT<F8> + off * 32 + l32] = static_cast<uint8_t>((cd[0] & 3) | ((cd[1] & 3) << 2) | ((cd[2] & 3) << 4) | ((cd[3] & 3) << 6));
   if ((l32 & 7) == 0) {
     const float s = cand == 0 ? sc[0] : cand == 1 ? sc[1] : sc[2], m0 = cand == 0 ? mnv[0] : cand == 1 ? mnv[1] : mnv[2];
-    uint32_t sb = f16_bits_rn(s) & 0x7FFFu;
-    if (cand == 1) sb |= 0x8000u;
-    *reinterpret_cast<uint32_t*>(chunk + 1280 + off * 16 + 4 * j) = sb | (f16_bits_rn(m0) << 16);
+    if (F8) {
+      const uint32_t sb = e4m3_bits(s) | (cand == 1 ? 0x80u : 0u);
+      *reinterpret_cast<uint16_t*>(chunk + VM_AT<true> + off * 8 + 2 * j) = static_cast<uint16_t>(sb | (e4m3_bits(m0) << 8));
+    } else {
+      uint32_t sb = f16_bits_rn(s) & 0x7FFFu;
+      if (cand == 1) sb |= 0x8000u;
+      *reinterpret_cast<uint32_t*>(chunk + VM_AT<false> + off * 16 + 4 * j) = sb | (f16_bits_rn(m0) << 16);
+    }
   }
-  if (l32 == 0) chunk[1536 + off] = useF ? 1 : 0;
+  if (l32 == 0) {
+    if (F8) {                                            // bit 7 of the key scale byte in slot 3 of this token's cell
+      uint8_t* kb = chunk + 512 + off * 8 + 6;
+      *kb = static_cast<uint8_t>((*kb & 0x7Fu) | (useF ? 0x80u : 0u));
+    } else chunk[1536 + off] = useF ? 1 : 0;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ key group encoder
@@ -108,6 +152,7 @@ struct KEnc {
   float ef;
 };
 
+template <bool F8>
 __global__ void __launch_bounds__(256) k_k_encode(const uint16_t* __restrict__ src, long long src_rs,
                                                   const uint16_t* __restrict__ src2, long long src2_rs,
                                                   const long long* __restrict__ sidx, const long long* __restrict__ dslot,
@@ -149,7 +194,8 @@ __global__ void __launch_bounds__(256) k_k_encode(const uint16_t* __restrict__ s
     float mn = INFINITY, mx = -INFINITY;
     for (int t = 0; t < 32; ++t)
       if (S.valid[t]) { const float v = S.es[c][t][ch]; mn = fminf(mn, v); mx = fmaxf(mx, v); }
-    const float s = kv_scale(mn, mx);
+    float s = kv_scale(mn, mx);
+    kv_params<F8>(mn, s);
     S.par[c][0][ch] = mn; S.par[c][1][ch] = s;
     for (int t = 0; t < 32; ++t)
       if (S.valid[t]) S.es[c][t][ch] = kv_rec(kv_code(S.es[c][t][ch], mn, s), mn, s);
@@ -263,19 +309,27 @@ __global__ void __launch_bounds__(256) k_k_encode(const uint16_t* __restrict__ s
     word |= __shfl_xor(word, 1, 32);
     word |= __shfl_xor(word, 2, 32);
     const long long slot = ds[t];
-    uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * 1552ll;
+    uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * CHUNK<F8>;
     if ((l32 & 3) == 0) reinterpret_cast<uint32_t*>(chunk + (slot % 16) * 32)[l32 >> 2] = word;
   }
   // meta of all 32 cells: cell i holds channels [4 i, 4 i + 4)
   for (int c = tid; c < 128; c += 256) {
     const int cand = useF ? 2 : S.choice[c >> 5];
-    uint32_t sb = f16_bits_rn(S.par[cand][1][c]) & 0x7FFFu;
-    const bool neg = c < 4 ? (!useF && S.choice[c] != 0) : (c == 4 ? useF : false);
-    if (neg) sb |= 0x8000u;
     const long long slot = ds[c >> 2];
     if (slot < 0) continue;
-    uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * 1552ll;
-    reinterpret_cast<uint32_t*>(chunk + 512 + (slot % 16) * 16)[c & 3] = sb | (f16_bits_rn(S.par[cand][0][c]) << 16);
+    uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * CHUNK<F8>;
+    if (F8) {                                                     // flags at slot 0 of cells 0 .. 4
+      const bool neg = (c & 3) == 0 && (c < 16 ? (!useF && S.choice[c >> 2] != 0) : (c == 16 ? useF : false));
+      uint8_t* at = chunk + 512 + (slot % 16) * 8 + 2 * (c & 3);
+      uint32_t sb = e4m3_bits(S.par[cand][1][c]) | (neg ? 0x80u : 0u);
+      if ((c & 3) == 3) sb |= at[0] & 0x80u;                      // the value row's whole-head flag lives here
+      *reinterpret_cast<uint16_t*>(at) = static_cast<uint16_t>(sb | (e4m3_bits(S.par[cand][0][c]) << 8));
+    } else {
+      uint32_t sb = f16_bits_rn(S.par[cand][1][c]) & 0x7FFFu;
+      const bool neg = c < 4 ? (!useF && S.choice[c] != 0) : (c == 4 ? useF : false);
+      if (neg) sb |= 0x8000u;
+      reinterpret_cast<uint32_t*>(chunk + 512 + (slot % 16) * 16)[c & 3] = sb | (f16_bits_rn(S.par[cand][0][c]) << 16);
+    }
   }
 }
 
@@ -284,22 +338,31 @@ template <typename OT> DEVI OT cvt_out(float v);
 template <> DEVI float cvt_out<float>(float v) { return v; }
 template <> DEVI uint16_t cvt_out<uint16_t>(float v) { return static_cast<uint16_t>(bf16_rn(v)); }
 
-template <typename OT>
+template <typename OT, bool F8>
 __global__ void __launch_bounds__(256) k_dequant(const uint8_t* __restrict__ pool, const int* __restrict__ bt, int g0,
                                                  int Hkv, int nvalid, OT* __restrict__ ok, OT* __restrict__ ov) {
   const int gi = blockIdx.x, h = blockIdx.y, hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
   const int g = g0 + gi;
-  const uint8_t* chA = pool + (static_cast<long long>(bt[2 * g]) * Hkv + h) * 1552ll;
-  const uint8_t* chB = pool + (static_cast<long long>(bt[2 * g + 1]) * Hkv + h) * 1552ll;
-  const uint32_t* m0 = reinterpret_cast<const uint32_t*>(chA + 512);
+  const uint8_t* chA = pool + (static_cast<long long>(bt[2 * g]) * Hkv + h) * CHUNK<F8>;
+  const uint8_t* chB = pool + (static_cast<long long>(bt[2 * g + 1]) * Hkv + h) * CHUNK<F8>;
   uint32_t lm = 0;
-  for (int j = 0; j < 4; ++j) lm |= ((m0[j] >> 15) & 1u) << j;
-  const bool kF = (m0[4] >> 15) & 1u;                           // cell 1, slot 0
-  // this lane's channels [4 l32, 4 l32 + 4) = key cell l32
-  const uint32_t* km = reinterpret_cast<const uint32_t*>((l32 < 16 ? chA : chB) + 512 + (l32 & 15) * 16);
+  bool kF;
   float ks[4], kmn[4];
+  // this lane's channels [4 l32, 4 l32 + 4) = key cell l32
+  if (F8) {
+    for (int j = 0; j < 4; ++j) lm |= static_cast<uint32_t>(chA[512 + 8 * j] >> 7) << j;
+    kF = chA[512 + 8 * 4] >> 7;
+    const uint8_t* km = (l32 < 16 ? chA : chB) + 512 + (l32 & 15) * 8;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { ks[i] = f16_value(km[i] & 0x7FFFu); kmn[i] = f16_value(km[i] >> 16); }
+    for (int i = 0; i < 4; ++i) { ks[i] = e4m3_value(km[2 * i] & 0x7Fu); kmn[i] = e4m3_value(km[2 * i + 1]); }
+  } else {
+    const uint32_t* m0 = reinterpret_cast<const uint32_t*>(chA + 512);
+    for (int j = 0; j < 4; ++j) lm |= ((m0[j] >> 15) & 1u) << j;
+    kF = (m0[4] >> 15) & 1u;                                    // cell 1, slot 0
+    const uint32_t* km = reinterpret_cast<const uint32_t*>((l32 < 16 ? chA : chB) + 512 + (l32 & 15) * 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { ks[i] = f16_value(km[i] & 0x7FFFu); kmn[i] = f16_value(km[i] >> 16); }
+  }
   const int j = l32 >> 3;
   for (int t = hw; t < 32; t += 8) {
     const long long o = static_cast<long long>(gi) * 32 + t;
@@ -326,12 +389,21 @@ __global__ void __launch_bounds__(256) k_dequant(const uint8_t* __restrict__ poo
     }
     // values
     {
-      const uint32_t* vm = reinterpret_cast<const uint32_t*>(ch + 1280 + cell * 16);
       uint32_t l = 0;
-      for (int jj = 0; jj < 4; ++jj) l |= ((vm[jj] >> 15) & 1u) << jj;
-      const bool f = ch[1536 + cell] != 0;
-      const float vs = f16_value(vm[j] & 0x7FFFu), vmn = f16_value(vm[j] >> 16);
-      const uint32_t byte = ch[768 + cell * 32 + l32];
+      bool f;
+      float vs, vmn;
+      if (F8) {
+        const uint8_t* vm = ch + VM_AT<true> + cell * 8;
+        for (int jj = 0; jj < 4; ++jj) l |= static_cast<uint32_t>(vm[2 * jj] >> 7) << jj;
+        f = ch[512 + cell * 8 + 6] >> 7;
+        vs = e4m3_value(vm[2 * j] & 0x7Fu); vmn = e4m3_value(vm[2 * j + 1]);
+      } else {
+        const uint32_t* vm = reinterpret_cast<const uint32_t*>(ch + VM_AT<false> + cell * 16);
+        for (int jj = 0; jj < 4; ++jj) l |= ((vm[jj] >> 15) & 1u) << jj;
+        f = ch[1536 + cell] != 0;
+        vs = f16_value(vm[j] & 0x7FFFu); vmn = f16_value(vm[j] >> 16);
+      }
+      const uint32_t byte = ch[VC_AT<F8> + cell * 32 + l32];
       float x[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = static_cast<float>((byte >> (2 * i)) & 3u) * vs + vmn;
@@ -371,32 +443,41 @@ __global__ void k_lse_merge(const uint16_t* __restrict__ oa, const float* __rest
 }  // namespace
 
 int v_write_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
-                   int ident, const int* vfix, hipStream_t st) {
+                   int ident, const int* vfix, int f8, hipStream_t st) {
   const long long items = static_cast<long long>(n) * Hkv;
-  hipLaunchKernelGGL(k_v_write, dim3(static_cast<unsigned>((items + 7) / 8)), dim3(256), 0, st,
+  const auto kern = f8 ? k_v_write<true> : k_v_write<false>;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((items + 7) / 8)), dim3(256), 0, st,
                      static_cast<const uint16_t*>(kv), kv_rs, n, Hkv, slots, co, pool, ident, vfix);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 
 int k_encode_launch(const void* src, long long src_rs, const void* src2, long long src2_rs, const long long* sidx,
                     const long long* dslot, int N, int Hkv, const float* qs, const float* lz, int NQ, float qsc,
-                    uint8_t* pool, int ident, const int* kfix, hipStream_t st) {
+                    uint8_t* pool, int ident, const int* kfix, int f8, hipStream_t st) {
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_k_encode), hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_k_encode<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(sizeof(KEnc))) != hipSuccess) return 1;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_k_encode<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(sizeof(KEnc))) != hipSuccess) return 1;
     attr = true;
   }
-  hipLaunchKernelGGL(k_k_encode, dim3(N, Hkv), dim3(256), sizeof(KEnc), st, static_cast<const uint16_t*>(src), src_rs,
+  const auto kern = f8 ? k_k_encode<true> : k_k_encode<false>;
+  hipLaunchKernelGGL(kern, dim3(N, Hkv), dim3(256), sizeof(KEnc), st, static_cast<const uint16_t*>(src), src_rs,
                      static_cast<const uint16_t*>(src2), src2_rs, sidx, dslot, Hkv, qs, lz, NQ, qsc, pool, ident, kfix);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 
 int dequant_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nvalid, int Hkv, int fp32, void* ok, void* ov,
-                   hipStream_t st) {
+                   int f8, hipStream_t st) {
   dim3 grid(g1 - g0, Hkv);
-  if (fp32) hipLaunchKernelGGL(k_dequant<float>, grid, dim3(256), 0, st, pool, bt, g0, Hkv, nvalid, static_cast<float*>(ok), static_cast<float*>(ov));
-  else hipLaunchKernelGGL(k_dequant<uint16_t>, grid, dim3(256), 0, st, pool, bt, g0, Hkv, nvalid, static_cast<uint16_t*>(ok), static_cast<uint16_t*>(ov));
+  if (fp32) {
+    const auto kern = f8 ? k_dequant<float, true> : k_dequant<float, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, pool, bt, g0, Hkv, nvalid, static_cast<float*>(ok), static_cast<float*>(ov));
+  } else {
+    const auto kern = f8 ? k_dequant<uint16_t, true> : k_dequant<uint16_t, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, pool, bt, g0, Hkv, nvalid, static_cast<uint16_t*>(ok), static_cast<uint16_t*>(ov));
+  }
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 

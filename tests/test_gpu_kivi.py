@@ -10,6 +10,8 @@ Bars:
              (the reference's bar, tests/test_kivi.py:243);
   dequant    fp32 within 2e-6 max|ref| of the fp64 oracle; bf16 = round of it within one ulp;
   lse_merge  bf16 patterns equal to the oracle's, up to one ulp on at most 0.1 % (library exp).
+Every page test runs on both meta formats: FP16 scale / min (1552-byte chunks) and FP8 E4M3 (1280-byte chunks, codes
+computed from the stored values, value whole-head flag in a key scale byte).
 """
 import math
 
@@ -23,11 +25,16 @@ from tests.gpu_util import bits
 
 pytestmark = pytest.mark.gpu
 D, PAGE = 128, 16
-CB = OK.chunk_bytes(D)
+F8 = pytest.mark.parametrize("f8", [False, True], ids=["f16meta", "f8meta"])
 
 
-def _kv(T, Hkv, g, shift=2.0):
-    """rows with per-channel offsets (what makes rotated bases win or lose per group) and a few outlier channels."""
+def _cb(f8):
+    return OK.chunk_bytes(D, f8)
+
+
+def _kv(T, Hkv, g, shift=2.0, big=200.0):
+    """rows with per-channel offsets (what makes rotated bases win or lose per group), a few outlier channels, a zero
+    row, a constant sub-vector, a tiny row and a row scaled by `big`."""
     mu = torch.randn(2 * Hkv, D, generator=g) * shift
     x = mu[None] + torch.randn(T, 2 * Hkv, D, generator=g) * (0.3 + torch.rand(2 * Hkv, D, generator=g))
     x[:, :, 5] *= 6
@@ -35,7 +42,7 @@ def _kv(T, Hkv, g, shift=2.0):
         x[3] = 0.0
         x[4, :, 32:64] = 1.25
         x[5] *= 1e-4
-        x[6] *= 200
+        x[6] *= big
     return x.bfloat16()
 
 
@@ -46,13 +53,14 @@ def _calib(Hkv, NQ, g):
     return qs, lz, co
 
 
-def _stored_value_flags(pool_np):
-    _, _, _, vm, vf = OK.parse_chunks(pool_np, D)
-    return (vm[..., 0] >> 15).astype(bool), vf.astype(bool)          # [np, H, 16, NV], [np, H, 16]
+def _stored_value_flags(pool_np, f8=False):
+    _, _, _, vm, vf = OK.parse_chunks(pool_np, D, f8)
+    return (vm[..., 0] >> (7 if f8 else 15)).astype(bool), vf.astype(bool)          # [np, H, 16, NV], [np, H, 16]
 
 
+@F8
 @pytest.mark.parametrize("seed,T,Hkv", [(0, 64, 2), (1, 333, 8), (2, 1, 1)])
-def test_v_write_given_flags(dev, seed, T, Hkv):
+def test_v_write_given_flags(dev, seed, T, Hkv, f8):
     from flagrot_releaser_amd import kivi as KV
     g = torch.Generator().manual_seed(seed)
     kv = _kv(T, Hkv, g)
@@ -61,21 +69,21 @@ def test_v_write_given_flags(dev, seed, T, Hkv):
     slots = torch.randperm(npg * 16, generator=g)[:T].long()
     if T > 10:
         slots[7] = -1
-    init = torch.randint(0, 256, (npg, Hkv, CB), generator=g, dtype=torch.uint8)
+    init = torch.randint(0, 256, (npg, Hkv, _cb(f8)), generator=g, dtype=torch.uint8)
     pool = init.to(dev)
-    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, pool, Hkv, D)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, pool, Hkv, D, f8=f8)
     torch.cuda.synchronize()
     got = pool.cpu().numpy()
-    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy())
-    sH, sF = _stored_value_flags(got)
+    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy(), f8=f8)
+    sH, sF = _stored_value_flags(got, f8)
     useH = np.zeros((T, Hkv, 4), bool)
     useF = np.zeros((T, Hkv), bool)
     for t, s in enumerate(slots.tolist()):
         if s >= 0:
             useH[t], useF[t] = sH[s // 16, :, s % 16], sF[s // 16, :, s % 16]
-    codes, meta, vf = OK.v_stored(enc, useH, useF)
+    codes, meta, vf = OK.v_stored(enc, useH, useF, f8=f8)
     want = init.numpy().copy()
-    OK.pack_values(want, slots.numpy(), codes, meta, vf)
+    OK.pack_values(want, slots.numpy(), codes, meta, vf, f8=f8)
     assert np.array_equal(got, want), "value codes / meta differ from the oracle given the stored flags"
     live = (slots.numpy() >= 0)
     badF = (useF != enc["useF"]) & live[:, None]
@@ -87,8 +95,9 @@ def test_v_write_given_flags(dev, seed, T, Hkv):
         assert useH.any() and (~useH).any()
 
 
+@F8
 @pytest.mark.parametrize("mode", ["ident", "fix"])
-def test_v_write_pinned_modes(dev, mode):
+def test_v_write_pinned_modes(dev, mode, f8):
     from flagrot_releaser_amd import kivi as KV
     g = torch.Generator().manual_seed(5)
     T, Hkv = 200, 4
@@ -97,12 +106,13 @@ def test_v_write_pinned_modes(dev, mode):
     npg = 14
     slots = torch.randperm(npg * 16, generator=g)[:T].long()
     fix = torch.tensor([0b0101, 1 << 16, 0b1111, 0], dtype=torch.int32)
-    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
+    pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
     KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, pool, Hkv, D, ident=mode == "ident",
-               fix=fix.to(dev) if mode == "fix" else None)
-    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy(), ident=mode == "ident", fix=fix.numpy() if mode == "fix" else None)
-    want = np.zeros((npg, Hkv, CB), np.uint8)
-    OK.pack_values(want, slots.numpy(), *OK.v_stored(enc))
+               fix=fix.to(dev) if mode == "fix" else None, f8=f8)
+    enc = OK.v_encode(bits(kv)[:, Hkv:], co.numpy(), ident=mode == "ident", fix=fix.numpy() if mode == "fix" else None,
+                      f8=f8)
+    want = np.zeros((npg, Hkv, _cb(f8)), np.uint8)
+    OK.pack_values(want, slots.numpy(), *OK.v_stored(enc, f8=f8), f8=f8)
     assert np.array_equal(pool.cpu().numpy(), want)
 
 
@@ -130,24 +140,27 @@ def _group_rows(rows, rows2, sidx_row, Hkv):
     return xb, (sidx_row.numpy() != -1)
 
 
-def _stored_key_flags(pool_np, dslot_row, h):
+def _stored_key_flags(pool_np, dslot_row, h, f8=False):
     pg0 = int(dslot_row[0]) // 16
     pg1 = int(dslot_row[16]) // 16
-    _, km, *_ = OK.parse_chunks(pool_np[[pg0, pg1]][:, h:h + 1], D)
+    _, km, *_ = OK.parse_chunks(pool_np[[pg0, pg1]][:, h:h + 1], D, f8)
     s = km[:, 0, :, :, 0].reshape(-1)                                 # 128 channel scales, cell-major
-    return (s[:4] >> 15).astype(bool), bool(s[4] >> 15)
+    st, fb = (4, 7) if f8 else (1, 15)                                # flag channels 0, st, 2 st, 3 st and 4 st
+    return (s[0:4 * st:st] >> fb).astype(bool), bool(s[4 * st] >> fb)
 
 
+@F8
 @pytest.mark.parametrize("seed,NG,Hkv,NQ", [(0, 4, 2, 64), (1, 6, 8, 37), (2, 1, 1, 8)])
-def test_k_encode_given_flags(dev, seed, NG, Hkv, NQ):
+def test_k_encode_given_flags(dev, seed, NG, Hkv, NQ, f8):
     from flagrot_releaser_amd import kivi as KV
     g = torch.Generator().manual_seed(seed)
     rows, rows2, sidx, dslot = _groups(NG, Hkv, g)
     qs, lz, _ = _calib(Hkv, NQ, g)
     qsc = 1 / math.sqrt(D)
     npg = 2 * NG + 3
-    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
-    KV.k_encode(rows.to(dev), sidx.to(dev), dslot.to(dev), qs.to(dev), lz.to(dev), qsc, pool, Hkv, D, src2=rows2.to(dev))
+    pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
+    KV.k_encode(rows.to(dev), sidx.to(dev), dslot.to(dev), qs.to(dev), lz.to(dev), qsc, pool, Hkv, D, src2=rows2.to(dev),
+                f8=f8)
     torch.cuda.synchronize()
     got = pool.cpu().numpy()
     want = np.zeros_like(got)
@@ -156,10 +169,10 @@ def test_k_encode_given_flags(dev, seed, NG, Hkv, NQ):
     for n in range(NG):
         xb, valid = _group_rows(rows, rows2, sidx[n], Hkv)
         for h in range(Hkv):
-            enc = OK.k_encode_group(xb[:, h], valid, qs[h].numpy(), lz[h].numpy(), qsc)
-            uH, uF = _stored_key_flags(got, dslot[n].numpy(), h)
-            codes, meta = OK.k_stored(enc, uH, uF)
-            OK.pack_key_group(want, h, dslot[n].numpy(), valid, codes, meta)
+            enc = OK.k_encode_group(xb[:, h], valid, qs[h].numpy(), lz[h].numpy(), qsc, f8=f8)
+            uH, uF = _stored_key_flags(got, dslot[n].numpy(), h, f8)
+            codes, meta = OK.k_stored(enc, uH, uF, f8=f8)
+            OK.pack_key_group(want, h, dslot[n].numpy(), valid, codes, meta, f8=f8)
             if uF != enc["useF"]:
                 assert enc["marginF"] < 1e-3, (n, h, enc["marginF"])
                 nbad += 1
@@ -175,8 +188,9 @@ def test_k_encode_given_flags(dev, seed, NG, Hkv, NQ):
         assert seenH == {True, False}
 
 
+@F8
 @pytest.mark.parametrize("mode", ["ident", "fix"])
-def test_k_encode_pinned_modes_keep_value_fields(dev, mode):
+def test_k_encode_pinned_modes_keep_value_fields(dev, mode, f8):
     from flagrot_releaser_amd import kivi as KV
     g = torch.Generator().manual_seed(9)
     NG, Hkv = 5, 4
@@ -184,21 +198,22 @@ def test_k_encode_pinned_modes_keep_value_fields(dev, mode):
     qs, lz, co = _calib(Hkv, 16, g)
     fix = torch.tensor([0b0011, 1 << 16, 0b1000, 0], dtype=torch.int32)
     npg = 2 * NG + 3
-    init = torch.randint(0, 256, (npg, Hkv, CB), generator=g, dtype=torch.uint8)
+    init = torch.randint(0, 256, (npg, Hkv, _cb(f8)), generator=g, dtype=torch.uint8)
     pool = init.to(dev)
     KV.k_encode(rows.to(dev), sidx.to(dev), dslot.to(dev), qs.to(dev), lz.to(dev), 0.1, pool, Hkv, D, src2=rows2.to(dev),
-                ident=mode == "ident", fix=fix.to(dev) if mode == "fix" else None)
+                ident=mode == "ident", fix=fix.to(dev) if mode == "fix" else None, f8=f8)
     want = init.numpy().copy()
     for n in range(NG):
         xb, valid = _group_rows(rows, rows2, sidx[n], Hkv)
         for h in range(Hkv):
             enc = OK.k_encode_group(xb[:, h], valid, qs[h].numpy(), lz[h].numpy(), 0.1, ident=mode == "ident",
-                                    fix=int(fix[h]) if mode == "fix" else None)
-            OK.pack_key_group(want, h, dslot[n].numpy(), valid, *OK.k_stored(enc))
-    assert np.array_equal(pool.cpu().numpy(), want)       # value fields and unused pages keep their bytes
+                                    fix=int(fix[h]) if mode == "fix" else None, f8=f8)
+            OK.pack_key_group(want, h, dslot[n].numpy(), valid, *OK.k_stored(enc, f8=f8), f8=f8)
+    # value fields and unused pages keep their bytes (f8: also the value rows' whole-head flags inside the key meta)
+    assert np.array_equal(pool.cpu().numpy(), want)
 
 
-def _filled_cache(dev, lens, Hkv, g, tail_T=0):
+def _filled_cache(dev, lens, Hkv, g, tail_T=0, f8=False):
     """pages of B sequences written by the GPU writers (whole groups), block table, and the fp64 K / V the oracle
     reads back from the same bytes."""
     from flagrot_releaser_amd import kivi as KV
@@ -207,7 +222,7 @@ def _filled_cache(dev, lens, Hkv, g, tail_T=0):
     npg = 2 * sum(ngs) + 1
     perm = torch.randperm(npg, generator=g)
     bt = torch.zeros(B, 2 * max(ngs), dtype=torch.int32)
-    pool = torch.zeros(npg, Hkv, CB, dtype=torch.uint8, device=dev)
+    pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
     qs, lz, co = _calib(Hkv, 24, g)
     o = 0
     Ks, Vs = [], []
@@ -217,13 +232,14 @@ def _filled_cache(dev, lens, Hkv, g, tail_T=0):
         o += 2 * ngs[b]
         kv = _kv(n, Hkv, g).to(dev)
         slots = (bt[b].long()[torch.arange(n) // 16] * 16 + torch.arange(n) % 16)
-        KV.v_write(kv, slots.to(dev), co.to(dev), None, pool, Hkv, D)
+        KV.v_write(kv, slots.to(dev), co.to(dev), None, pool, Hkv, D, f8=f8)
         sidx = torch.arange(n).reshape(-1, 32).long()
-        KV.k_encode(kv, sidx.to(dev), slots.reshape(-1, 32).to(dev), qs.to(dev), lz.to(dev), 1 / math.sqrt(D), pool, Hkv, D)
+        KV.k_encode(kv, sidx.to(dev), slots.reshape(-1, 32).to(dev), qs.to(dev), lz.to(dev), 1 / math.sqrt(D), pool, Hkv, D,
+                    f8=f8)
     torch.cuda.synchronize()
     pnp = pool.cpu().numpy()
     for b in range(B):
-        k, v = OK.dequant_groups(pnp[bt[b, :2 * ngs[b]].numpy()], D)
+        k, v = OK.dequant_groups(pnp[bt[b, :2 * ngs[b]].numpy()], D, f8=f8)
         Ks.append(k)
         Vs.append(v)
     return pool, bt, Ks, Vs
@@ -249,13 +265,14 @@ CASES = [
 ]
 
 
+@F8
 @pytest.mark.parametrize("case", range(len(CASES)))
-def test_attn_against_fp64(dev, case):
+def test_attn_against_fp64(dev, case, f8):
     from flagrot_releaser_amd import kivi as KV
     lens, Hkv, G, kv_start, split, tails = CASES[case]
     g = torch.Generator().manual_seed(100 + case)
     B, Hq = len(lens), Hkv * G
-    pool, bt, Ks, Vs = _filled_cache(dev, lens, Hkv, g)
+    pool, bt, Ks, Vs = _filled_cache(dev, lens, Hkv, g, f8=f8)
     T = 128
     R = B + 1
     ring = (torch.randn((R + 1) * T, 2 * Hkv, D, generator=g) * 1.5).bfloat16()
@@ -270,7 +287,7 @@ def test_attn_against_fp64(dev, case):
     out = outbuf[:, :Hq * D]
     scale = 1 / math.sqrt(D)
     args = (q.to(dev), pool, bt.to(dev), cached.to(dev), out, ns, chunk, ws, scale * math.log2(math.e), kv_start, G)
-    kw = dict(ring=ring.to(dev), tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), T=T)
+    kw = dict(ring=ring.to(dev), tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), T=T, f8=f8)
     ringf = Q.bf16_to_f32(bits(ring)).astype(np.float64).reshape(R + 1, T, 2 * Hkv, D)
     qf = Q.bf16_to_f32(bits(q)).astype(np.float64)
     for rep in range(2):
@@ -305,23 +322,22 @@ def test_attn_without_tail_and_rejects(dev):
     assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
     with pytest.raises(RuntimeError, match="chunk"):
         KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 100, ws, 0.1, 0, G)
-    with pytest.raises(RuntimeError, match="FP8"):
-        KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 256, ws, 0.1, 0, G, f8=True)
     with pytest.raises(RuntimeError, match="M is not built"):
         KV.v_write(torch.zeros(1, 2 * Hkv, D, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
                    torch.ones(Hkv, D, device=dev), torch.ones(Hkv, D, D, device=dev), pool, Hkv, D)
 
 
-def test_dequant_and_torch_parser(dev):
+@F8
+def test_dequant_and_torch_parser(dev, f8):
     from flagrot_releaser_amd import kivi as KV
     g = torch.Generator().manual_seed(11)
     Hkv = 4
-    pool, bt, Ks, Vs = _filled_cache(dev, [416], Hkv, g)
+    pool, bt, Ks, Vs = _filled_cache(dev, [416], Hkv, g, f8=f8)
     row = bt[0].contiguous().to(dev)
     for a, n in ((0, 416), (40, 300), (64, 65)):
-        k32, v32 = KV.dequant_cuda(pool, row, a, n, Hkv, D, dtype=torch.float32)
-        kb, vb = KV.dequant_cuda(pool, row, a, n, Hkv, D)
-        kt, vt = KV.dequant(pool, row, a, n, Hkv, D)
+        k32, v32 = KV.dequant_cuda(pool, row, a, n, Hkv, D, dtype=torch.float32, f8=f8)
+        kb, vb = KV.dequant_cuda(pool, row, a, n, Hkv, D, f8=f8)
+        kt, vt = KV.dequant(pool, row, a, n, Hkv, D, f8=f8)
         torch.cuda.synchronize()
         for got, gotb, gott, ref in ((k32, kb, kt, Ks[0][a:n]), (v32, vb, vt, Vs[0][a:n])):
             assert got.shape == ref.shape == gotb.shape == gott.shape
@@ -331,6 +347,55 @@ def test_dequant_and_torch_parser(dev):
             assert (gotb.float().cpu() - got.cpu()).abs().max() <= 2 ** -8 * sc
             back = got.bfloat16()
             assert ((gotb.view(torch.int16).int() - back.view(torch.int16).int()).abs() <= 1).all()
+
+
+def test_f8_value_flags_survive_interleaved_key_encoding(dev):
+    """FP8-meta pages keep the value rows' whole-head flags in bit 7 of key scale bytes (slot 3 of the row's cell); the
+    key encoder writes those bytes later, or earlier, or twice, and must keep the bit, and a value write must keep the
+    key scale around it (the order of integrations/vllm_flagrot/tests/test_kivi.py:358-401: V of group 0, K of group
+    0, V of the middle groups, K of the middle groups, K of group 0 again, V of the last group, K of the last group).
+    The pool must end byte-equal to the one written values first, keys after."""
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(21)
+    NG, Hkv, S = 6, 4, 4
+    T = NG * 32
+    kv = _kv(T, Hkv, g).to(dev)
+    qs, lz, co = (x.to(dev) for x in _calib(Hkv, 16, g))
+    perm = torch.randperm(2 * NG, generator=g)
+    pos = torch.arange(T)
+    slots = (perm[pos // 16] * 16 + pos % 16).long().to(dev)
+    gp = pos.view(NG, 32)
+    sid = torch.where(gp < S, -1, gp).contiguous().to(dev)           # the first S tokens stay out of their group
+    ds = slots.view(NG, 32).contiguous()
+    # frozen choices: the test is about byte ownership, not about ties of the selection
+    vfix = torch.tensor([1 << 16, 0b0110, 1 << 16, 0], dtype=torch.int32, device=dev)
+    kfix = torch.tensor([0b1001, 1 << 16, 0, 0b1111], dtype=torch.int32, device=dev)
+
+    def venc(pool, a, b):
+        KV.v_write(kv[a:b], slots[a:b].contiguous(), co, None, pool, Hkv, D, fix=vfix, f8=True)
+
+    def kenc(pool, gs):
+        KV.k_encode(kv, sid[gs].contiguous(), ds[gs].contiguous(), qs, lz, 0.09, pool, Hkv, D, fix=kfix, f8=True)
+
+    pool = torch.zeros(2 * NG, Hkv, _cb(True), dtype=torch.uint8, device=dev)
+    venc(pool, 0, 32)
+    kenc(pool, [0])
+    venc(pool, 32, T - 32)
+    kenc(pool, list(range(1, NG - 1)))
+    kenc(pool, [0])
+    venc(pool, T - 32, T)
+    kenc(pool, [NG - 1])
+    ref = torch.zeros_like(pool)
+    venc(ref, 0, T)
+    kenc(ref, list(range(NG)))
+    torch.cuda.synchronize()
+    vf = OK.parse_chunks(ref.cpu().numpy(), D, True)[4]
+    assert vf[:, 0].all() and vf[:, 2].all() and not vf[:, 1].any() and not vf[:, 3].any()
+    assert torch.equal(pool, ref)
+    # and a late value write over finished pages changes value fields and that one bit only
+    venc(pool, 0, T)
+    torch.cuda.synchronize()
+    assert torch.equal(pool, ref)
 
 
 def test_lse_merge(dev):

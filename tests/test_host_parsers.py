@@ -58,3 +58,22 @@ def test_torch_parser_head_256_and_rejects():
         K.dequant_cb_pages(torch.from_numpy(a), 16, "nf4")
     h = K.hadamard(32, "cpu", torch.float64)
     assert torch.allclose(h @ h, torch.eye(32, dtype=torch.float64)) and torch.equal(h, h.T)
+
+
+@pytest.mark.parametrize("f8", [False, True], ids=["f16meta", "f8meta"])
+def test_kivi_torch_parser_matches_reference_vectors(f8):
+    """flagrot_releaser_amd.kivi.dequant_groups (torch, here on the CPU) on the random chunk bytes of
+    tests/golden/kivi_layout.npz against what the reference's parser returned for them, both bases."""
+    import os
+
+    from flagrot_releaser_amd import kivi as KV
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "kivi_layout.npz"))
+    tag = "f8" if f8 else "f16"
+    ch = torch.from_numpy(g[f"{tag}_chunks"])
+    vf = KV.parse_chunks(ch, 128, f8)[4]
+    assert np.array_equal(vf.numpy() != 0, g[f"{tag}_vf"] != 0)
+    for basis in ("orig", "stored"):
+        k, v = KV.dequant_groups(ch, 128, basis, f8)
+        for a, ref in ((k, g[f"{tag}_k_{basis}"]), (v, g[f"{tag}_v_{basis}"])):
+            assert tuple(a.shape) == ref.shape
+            assert np.abs(a.numpy() - ref).max() <= 3e-6 * np.abs(ref).max(), (tag, basis)
