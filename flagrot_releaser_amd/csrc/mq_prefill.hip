@@ -15,8 +15,8 @@
 // reference's selectors 1 - 3) and k_mq8 (256 rows, selector 4: eight wavefronts in two groups half a block apart, the
 // matrix instructions of one group under the vector instructions of the other; described at its definition).
 // Causal rule: key j is visible to the row at position p iff kmin <= j <= max(p - shift, ext), j < nk.
-// Partials (unnormalised O, running maximum in log2 units, sum) per (item, KV head, row); k_merge combines the items
-// of a tile.  Semantics follow integrations/vllm_flagrot/csrc/mq_prefill.cu:345-498 (k_mq), :716-772 (merge),
+// Partials (unnormalised O, running maximum in log2 units, sum) per (item, KV head, row); k_fold_items combines the
+// items of a tile.  Semantics follow integrations/vllm_flagrot/csrc/mq_prefill.cu:345-498 (k_mq), :716-772 (merge),
 // :789-823 (q preparation), :1350-1465 (BF16 window gather / sink merge), :1469-1601 (C ABI).
 #include <cstdio>
 #include <cstring>
@@ -61,6 +61,34 @@ struct Params {
   int Hkv, G, shift, kmin;
   float* opart;
   float* ml;
+};
+
+// What one workgroup (item, KV head) has to do, read from its item record (tile, first block, end block, 0) and the tile
+// record that names (block-table row, first compact query row, first output row, tokens, position of the first token,
+// page keys of the request, first item, items, reach).  `reach`: a key index every row may see on top of its causal
+// range (a large negative number when there is none).
+struct Work {
+  const int* block_table;
+  int compact_row, tokens, first_pos, reach;
+  int key_end;              // keys at or past it are invisible to the whole tile or belong to a later item
+  int block0, block1;       // 64-key blocks [block0, block1) to read (empty when the item starts past key_end)
+  int rows_used;            // query rows of the tile that hold a token's head: whole tokens only
+  int shift;
+
+  DEVI Work(const Params& p, int item, int rows) {
+    const int* irec = p.items + ITEM_INTS * item;
+    const int* trec = p.tiles + TILE_INTS * irec[0];
+    block_table = p.bt + static_cast<long long>(trec[0]) * p.bt_stride;
+    compact_row = trec[1]; tokens = trec[3]; first_pos = trec[4]; reach = trec[8];
+    shift = p.shift;
+    const int causal_end = max(first_pos + tokens - shift, reach + 1);      // what the tile's last token sees
+    key_end = min(min(trec[5], irec[2] * BN), causal_end);
+    block0 = irec[1];
+    block1 = key_end > block0 * BN ? (key_end + BN - 1) / BN : block0;
+    rows_used = min(rows / p.G, tokens) * p.G;
+  }
+  DEVI bool has_row(int row) const { return row < rows_used; }
+  DEVI int last_key(int token) const { return min(key_end - 1, max(first_pos + token - shift, reach)); }
 };
 
 char g_err[512] = "";
@@ -457,20 +485,16 @@ __global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
   Smem& S = *reinterpret_cast<Smem*>(lds);
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
   const int item = blockIdx.x, h = blockIdx.y;
-  const int* it = p.items + ITEM_INTS * item;
-  const int* tl = p.tiles + TILE_INTS * it[0];
-  const int req = tl[0], crow0 = tl[1], ntok = tl[3], pos0 = tl[4], nk = tl[5], ext = tl[8];
-  const int G = p.G, Hq = p.Hkv * G, TQ = ROWS / G;
-  const int* bt = p.bt + static_cast<long long>(req) * p.bt_stride;
-  const int kend = min(min(nk, it[2] * BN), max(pos0 + ntok - p.shift, ext + 1));
-  const int kb0 = it[1];
-  const int kb1 = kend > kb0 * BN ? (kend + BN - 1) / BN : kb0;
+  const Work work(p, item, ROWS);
+  const int G = p.G, Hq = p.Hkv * G;
+  const int* bt = work.block_table;
+  const int kend = work.key_end, kb0 = work.block0, kb1 = work.block1;
   const Consts cst = make_consts();
 
   // this lane's query row
-  const int r = 32 * wv + l32, rt = r / G;
-  const bool rvalid = r < TQ * G && rt < ntok;
-  const int lim = rvalid ? min(kend - 1, max(pos0 + rt - p.shift, ext)) : -1;   // last visible key
+  const int r = 32 * wv + l32;
+  const bool rvalid = work.has_row(r);
+  const int lim = rvalid ? work.last_key(r / G) : -1;
 
   // page ids of the first blocks (published by the barriers of the q staging below)
   int cb = kb0;
@@ -487,7 +511,7 @@ __global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
   for (int row = tid >> 5; row < ROWS; row += NT / 32) {
     const int t = row / G, lq = tid & 31;
     u32x2 raw = {0u, 0u};
-    if (row < TQ * G && t < ntok) raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
+    if (work.has_row(row)) raw = gload<u32x2>(p.q + (static_cast<long long>(work.compact_row + t) * Hq + h * G + row % G) * D + 4 * lq);
     *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = raw;
   }
   __syncthreads();
@@ -762,19 +786,15 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
   const int grp = __builtin_amdgcn_readfirstlane(wv >> 2);
   const int item = blockIdx.x, h = blockIdx.y;
-  const int* it = p.items + ITEM_INTS * item;
-  const int* tl = p.tiles + TILE_INTS * it[0];
-  const int req = tl[0], crow0 = tl[1], ntok = tl[3], pos0 = tl[4], nk = tl[5], ext = tl[8];
-  const int G = p.G, Hq = p.Hkv * G, TQ = ROWS / G;
-  const int* bt = p.bt + static_cast<long long>(req) * p.bt_stride;
-  const int kend = min(min(nk, it[2] * BN), max(pos0 + ntok - p.shift, ext + 1));
-  const int kb0 = it[1];
-  const int kb1 = kend > kb0 * BN ? (kend + BN - 1) / BN : kb0;
+  const Work work(p, item, ROWS);
+  const int G = p.G, Hq = p.Hkv * G;
+  const int* bt = work.block_table;
+  const int kend = work.key_end, kb0 = work.block0, kb1 = work.block1;
   const Consts cst = make_consts();
 
-  const int r = 32 * wv + l32, rt = r / G;
-  const bool rvalid = r < TQ * G && rt < ntok;
-  const int lim = rvalid ? min(kend - 1, max(pos0 + rt - p.shift, ext)) : -1;   // last visible key
+  const int r = 32 * wv + l32;
+  const bool rvalid = work.has_row(r);
+  const int lim = rvalid ? work.last_key(r / G) : -1;
 
   int cb = kb0;
   auto fill_pages = [&]() {
@@ -789,7 +809,7 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   for (int row = tid >> 5; row < ROWS; row += NT / 32) {
     const int t = row / G, lq = tid & 31;
     u32x2 raw = {0u, 0u};
-    if (row < TQ * G && t < ntok) raw = gload<u32x2>(p.q + (static_cast<long long>(crow0 + t) * Hq + h * G + row % G) * D + 4 * lq);
+    if (work.has_row(row)) raw = gload<u32x2>(p.q + (static_cast<long long>(work.compact_row + t) * Hq + h * G + row % G) * D + 4 * lq);
     *reinterpret_cast<u32x2*>(lds + row * QROW + 8 * lq) = raw;
   }
   __syncthreads();
@@ -910,166 +930,206 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   }
 }
 
-// ------------------------------------------------------------------------------------------------ merge of a tile's items
-__global__ void __launch_bounds__(256) k_merge(const int* __restrict__ tiles, const float* __restrict__ opart,
-                                               const float* __restrict__ ml, int Hkv, int G, int rows, void* out,
-                                               long long o_ts, int out_fp32, float* lse, long long lse_ts) {
-  const int* tl = tiles + TILE_INTS * blockIdx.x;
-  const int h = blockIdx.y;
-  const int crow0 = tl[1], orow0 = tl[2], ntok = tl[3], item0 = tl[6], nitem = tl[7];
-  const int l32 = threadIdx.x & 31;
-  const int r = blockIdx.z * 8 + (threadIdx.x >> 5);
-  const int TQ = rows / G, Hq = Hkv * G, t = r / G;
-  if (r >= TQ * G || t >= ntok) return;
-  const int hq = h * G + r % G;
-  const long long b0 = (static_cast<long long>(item0) * Hkv + h) * rows + r, bs = static_cast<long long>(Hkv) * rows;
-  float M = -INFINITY;
-  for (int s = 0; s < nitem; ++s) M = fmaxf(M, ml[2 * (b0 + s * bs)]);
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  float L = 0.f;
-  if (M != -INFINITY) {
-    for (int s = 0; s < nitem; ++s) {
-      const long long b = b0 + s * bs;
-      const float2 v = *reinterpret_cast<const float2*>(ml + 2 * b);
-      if (v.x == -INFINITY) continue;
-      const float w = fexp2(v.x - M);
-      L += w * v.y;
-      const float4 x = *reinterpret_cast<const float4*>(opart + b * D + 4 * l32);
-      acc.x += w * x.x; acc.y += w * x.y; acc.z += w * x.z; acc.w += w * x.w;
+// ------------------------------------------------------------------------------------------------ items of a tile, folded
+// One wavefront per (query row of a tile, KV head), a lane per channel pair.  The items' (maximum, sum) pairs are read
+// one item per lane (64 at a time), so the common maximum, every item's weight 2^(m - M) and the total sum come from
+// three wave reductions instead of two serial passes; the accumulation loop then takes each weight from its lane.
+template <bool FP32_OUT>
+__global__ void __launch_bounds__(256) k_fold_items(const int* __restrict__ tiles, const float* __restrict__ opart,
+                                                    const float* __restrict__ ml, int Hkv, int G, int rows,
+                                                    void* __restrict__ out, long long out_stride, float* __restrict__ lse,
+                                                    long long lse_stride) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.z * 4 + (threadIdx.x >> 6), head = blockIdx.y;
+  const int* rec = tiles + TILE_INTS * blockIdx.x;
+  const int token = row / G;
+  if (row >= (rows / G) * G || token >= rec[3]) return;                  // rec[3]: tokens of the tile (wave uniform)
+  const int first = rec[6], count = rec[7];
+  const long long per_item = static_cast<long long>(Hkv) * rows;         // partial rows from one item to the next
+  const long long at = (static_cast<long long>(first) * Hkv + head) * rows + row;
+  float2 sum = make_float2(0.f, 0.f);
+  float top = -INFINITY, total = 0.f;
+  for (int s0 = 0; s0 < count; s0 += 64) top = fmaxf(top, wave_max64(s0 + lane < count ? ml[2 * (at + (s0 + lane) * per_item)] : -INFINITY));
+  if (top != -INFINITY) {
+    for (int s0 = 0; s0 < count; s0 += 64) {
+      float weight = 0.f, mass = 0.f;
+      if (s0 + lane < count) {
+        const float2 st = *reinterpret_cast<const float2*>(ml + 2 * (at + (s0 + lane) * per_item));
+        weight = st.x == -INFINITY ? 0.f : fexp2(st.x - top);
+        mass = weight * st.y;
+      }
+      total += wave_sum64(mass);
+      const int n = min(64, count - s0);
+      for (int s = 0; s < n; ++s) {
+        const float w = __shfl(weight, s, 64);
+        if (w == 0.f) continue;                                          // an item that saw no key: nothing to read
+        const float2 x = *reinterpret_cast<const float2*>(opart + (at + (s0 + s) * per_item) * D + 2 * lane);
+        sum.x += w * x.x; sum.y += w * x.y;
+      }
     }
-    const float inv = 1.f / L;
-    acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+    const float inv = 1.f / total;
+    sum.x *= inv; sum.y *= inv;
   }
-  if (out_fp32) {
-    *reinterpret_cast<float4*>(static_cast<float*>(out) + (static_cast<long long>(crow0 + t) * Hq + hq) * D + 4 * l32) = acc;
-  } else {
-    uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(orow0 + t) * o_ts + hq * D + 4 * l32;
-    *reinterpret_cast<uint2*>(dst) = make_uint2(bf16_rn(acc.x) | (bf16_rn(acc.y) << 16), bf16_rn(acc.z) | (bf16_rn(acc.w) << 16));
+  const int qhead = head * G + row % G;
+  if (FP32_OUT) {                                                        // compact rows, dense [m, Hq, D]
+    float* dst = static_cast<float*>(out) + (static_cast<long long>(rec[1] + token) * Hkv * G + qhead) * D;
+    *reinterpret_cast<float2*>(dst + 2 * lane) = sum;
+  } else {                                                               // rows of the layer output
+    uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(rec[2] + token) * out_stride + qhead * D;
+    *reinterpret_cast<uint32_t*>(dst + 2 * lane) = bf16_rn(sum.x) | (bf16_rn(sum.y) << 16);
   }
-  if (lse != nullptr && l32 == 0)
-    lse[hq * lse_ts + crow0 + t] = M == -INFINITY ? -INFINITY : (M + log2f(L)) * 0.6931471805599453f;
+  if (lse != nullptr && lane == 0)
+    lse[qhead * lse_stride + rec[1] + token] = top == -INFINITY ? -INFINITY : (top + log2f(total)) * 0.6931471805599453f;
 }
 
-// ------------------------------------------------------------------------------------------------ q preparation
-// one half wave per (row, q head): whole-head unnormalised H128 / 8 when kfull[kv head], then orthonormal H32 on the
-// kmask[kv head] groups, times qscale, rounded to fp16 (every operation in fp32, rounded on its own)
-__global__ void __launch_bounds__(256) k_prep(const void* q, int q_fp32, long long q_ts, const int* idx, int m, int Hq, int G,
-                                              const uint8_t* kfull, const uint8_t* kmask, float qscale, uint16_t* q16) {
-  const long long w = (static_cast<long long>(blockIdx.x) * 256 + threadIdx.x) >> 5;
-  const int l32 = threadIdx.x & 31;
-  if (w >= static_cast<long long>(m) * Hq) return;
-  const int t = static_cast<int>(w / Hq), hq = static_cast<int>(w % Hq), hk = hq / G;
-  const long long row = idx != nullptr ? idx[t] : t;
-  float x[4];
-  if (q_fp32) {
-    const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(q) + row * q_ts + hq * D + 4 * l32);
-    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-  } else {
-    const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(q) + row * q_ts + hq * D + 4 * l32);
-    x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
-  }
-  if (kfull != nullptr && kfull[hk]) {
-    butterflies<128>(x, l32);
+// ------------------------------------------------------------------------------------------------ query rows for the kernel
+// A workgroup takes one query row and walks its heads, eight at a time: a half wave per head, four channels per lane
+// (the shape the Hadamard helpers work on).  Where the head's keys are stored whole-head rotated the row becomes
+// H128 x / 8 (unnormalised butterflies, then one multiply), then the groups stored H32-rotated get the orthonormal H32,
+// then the softmax factor, then one rounding to fp16 -- each step rounded to fp32 on its own, in this order.
+template <typename T> DEVI void read4(const T* p, float (&x)[4]);
+template <> DEVI void read4<float>(const float* p, float (&x)[4]) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+}
+template <> DEVI void read4<uint16_t>(const uint16_t* p, float (&x)[4]) {     // bf16
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  x[0] = bf16_lo(v.x); x[1] = bf16_hi(v.x); x[2] = bf16_lo(v.y); x[3] = bf16_hi(v.y);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) k_query_rows(const T* __restrict__ q, long long q_stride, const int* __restrict__ pick,
+                                                    int Hq, int G, const uint8_t* __restrict__ whole,
+                                                    const uint8_t* __restrict__ rotated, float factor,
+                                                    uint16_t* __restrict__ q16) {
+  const int l32 = threadIdx.x & 31, sub = l32 >> 3;
+  const long long src = pick != nullptr ? pick[blockIdx.x] : blockIdx.x;
+  for (int head = threadIdx.x >> 5; head < Hq; head += 8) {
+    const int kv = head / G;
+    float x[4];
+    read4<T>(q + src * q_stride + head * D + 4 * l32, x);
+    if (whole != nullptr && whole[kv]) {
+      butterflies<128>(x, l32);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) x[i] *= 0.125f;
+      for (int i = 0; i < 4; ++i) x[i] *= 0.125f;
+    }
+    if (rotated != nullptr) {                    // every lane takes part in the exchange; the flagged groups keep the result
+      float y[4] = {x[0], x[1], x[2], x[3]};
+      fwht<32>(y, l32);
+      if (rotated[kv * 4 + sub]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = y[i];
+      }
+    }
+    uint32_t h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = f16_bits_rn(x[i] * factor);
+    *reinterpret_cast<uint2*>(q16 + (static_cast<long long>(blockIdx.x) * Hq + head) * D + 4 * l32) =
+        make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
   }
-  if (kmask != nullptr) {
-    float y[4] = {x[0], x[1], x[2], x[3]};
-    fwht<32>(y, l32);
-    if (kmask[hk * 4 + (l32 >> 3)]) { x[0] = y[0]; x[1] = y[1]; x[2] = y[2]; x[3] = y[3]; }
-  }
-  const float a = x[0] * qscale, b = x[1] * qscale, c = x[2] * qscale, d = x[3] * qscale;
-  *reinterpret_cast<uint2*>(q16 + (static_cast<long long>(t) * Hq + hq) * D + 4 * l32) =
-      make_uint2(f16_bits_rn(a) | (f16_bits_rn(b) << 16), f16_bits_rn(c) | (f16_bits_rn(d) << 16));
 }
 
-// ------------------------------------------------------------------------------------------------ BF16 window / sink parts
-__global__ void __launch_bounds__(128) k_win_gather(const long long* map, const uint16_t* sinkb, const uint16_t* preb,
-                                                    const uint16_t* kch, long long k_ts, const uint16_t* vch,
-                                                    long long v_ts, int Hkv, uint16_t* kw, uint16_t* vw) {
-  const int d = blockIdx.x;
+// ------------------------------------------------------------------------------------------------ BF16 window / sink rows
+// Collects the K and V rows of the window call: a flat grid over the 16-byte pieces of all rows (a row is Hkv x 128 bf16
+// = 16 Hkv pieces per tensor), so the launch fills the GPU whatever Hkv is.  map[d] = (source << 32) | row.
+__global__ void __launch_bounds__(256) k_collect_rows(const long long* __restrict__ map, int nrows, const uint4* __restrict__ sinks,
+                                                      const uint4* __restrict__ earlier, const uint16_t* __restrict__ kbatch,
+                                                      long long k_stride, const uint16_t* __restrict__ vbatch, long long v_stride,
+                                                      int pieces, uint4* __restrict__ kdst, uint4* __restrict__ vdst) {
+  const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= static_cast<long long>(nrows) * pieces) return;
+  const long long d = e / pieces;
+  const int i = static_cast<int>(e - d * pieces);
   const long long code = map[d];
-  const int kind = static_cast<int>(code >> 32);
+  const unsigned from = static_cast<unsigned>(code >> 32);
   const long long row = code & 0xffffffffLL;
-  const int nvec = Hkv * D / 8;
-  const uint4 *ks, *vs;
-  if (kind == 2) {
-    ks = reinterpret_cast<const uint4*>(kch + row * k_ts);
-    vs = reinterpret_cast<const uint4*>(vch + row * v_ts);
-  } else {
-    const uint16_t* b = (kind == 0 ? sinkb : preb) + row * 2LL * Hkv * D;
-    ks = reinterpret_cast<const uint4*>(b);
-    vs = reinterpret_cast<const uint4*>(b + Hkv * D);
+  uint4 k, v;
+  if (from == 2u) {                              // this batch's own rows: K and V in separate tensors
+    k = reinterpret_cast<const uint4*>(kbatch + row * k_stride)[i];
+    v = reinterpret_cast<const uint4*>(vbatch + row * v_stride)[i];
+  } else {                                       // kept rows: [K heads | V heads] side by side
+    const uint4* both = (from == 0u ? sinks : earlier) + row * 2 * pieces;
+    k = both[i];
+    v = both[pieces + i];
   }
-  uint4* kd = reinterpret_cast<uint4*>(kw + static_cast<long long>(d) * Hkv * D);
-  uint4* vd = reinterpret_cast<uint4*>(vw + static_cast<long long>(d) * Hkv * D);
-  for (int i = threadIdx.x; i < nvec; i += 128) { kd[i] = ks[i]; vd[i] = vs[i]; }
+  kdst[e] = k;
+  vdst[e] = v;
 }
 
-// per (compact row, q head) half wave: page part (fp32 o, natural-log lse) + window part (bf16 o, lse) + sink part
-// (keys j < min(S, len), j <= pos - W; fp32 softmax over bf16 rows) merged by LSE -> bf16 output row idx[c]
-__global__ void __launch_bounds__(256) k_bf_merge(int m, int Hq, int Hkv, const uint16_t* q, long long q_ts,
-                                                  const long long* idx, const float* o_p, const float* lse_p,
-                                                  const uint16_t* o_w, const float* lse_w, const uint16_t* sk,
-                                                  const long long* row_req, const long long* row_pos,
-                                                  const long long* sk_len, int S, int W, float scale, uint16_t* out,
-                                                  long long o_ts) {
-  const int c = blockIdx.x, hq = blockIdx.y * 8 + (threadIdx.x >> 5), l32 = threadIdx.x & 31;
-  if (hq >= Hq) return;
-  const int G = Hq / Hkv, kvh = hq / G;
-  const long long brow = idx[c];
-  float acc[4] = {0.f, 0.f, 0.f, 0.f}, M = -INFINITY, L = 0.f;
-  {
-    const float l = lse_p[static_cast<long long>(hq) * m + c];
-    if (l != -INFINITY && l != INFINITY && l == l) {
-      const float4 v = *reinterpret_cast<const float4*>(o_p + (static_cast<long long>(c) * Hq + hq) * D + 4 * l32);
-      acc[0] = v.x; acc[1] = v.y; acc[2] = v.z; acc[3] = v.w;
-      M = l; L = 1.f;
+// Mixes the parts of a compact row's attention by their log-sum-exps and writes the bf16 output row: one wavefront per
+// (row, query head), a lane per channel pair.  Page part fp32 (o, lse); window part bf16 (o, lse) or absent; sink part
+// computed here over the keys j < min(S, length of the request's sinks), j <= position - W: first every key's score
+// (one wave reduction each, key j's score parked in lane j), then the softmax across lanes, then the weighted rows.
+// An lse of +-inf or NaN means the part is empty.  S <= 64.
+DEVI bool usable(float lse) { return lse == lse && lse != INFINITY && lse != -INFINITY; }
+
+__global__ void __launch_bounds__(256) k_mix_parts(int m, int Hq, int Hkv, const uint16_t* __restrict__ q, long long q_stride,
+                                                   const long long* __restrict__ out_row, const float* __restrict__ o_pages,
+                                                   const float* __restrict__ lse_pages, const uint16_t* __restrict__ o_win,
+                                                   const float* __restrict__ lse_win, const uint16_t* __restrict__ sinks,
+                                                   const long long* __restrict__ req_of, const long long* __restrict__ pos_of,
+                                                   const long long* __restrict__ sink_len, int S, int W, float scale,
+                                                   uint16_t* __restrict__ out, long long out_stride) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (head >= Hq) return;
+  const int kv = head / (Hq / Hkv);
+  const long long dst_row = out_row[c], flat = (static_cast<long long>(c) * Hq + head) * D + 2 * lane;
+
+  float lp = lse_pages[static_cast<long long>(head) * m + c];
+  float2 vp = make_float2(0.f, 0.f);
+  if (usable(lp)) vp = *reinterpret_cast<const float2*>(o_pages + flat); else lp = -INFINITY;
+
+  float lw = -INFINITY;
+  float2 vw = make_float2(0.f, 0.f);
+  if (o_win != nullptr) {
+    const float l = lse_win[static_cast<long long>(head) * m + c];
+    if (usable(l)) {
+      const uint32_t raw = *reinterpret_cast<const uint32_t*>(o_win + flat);
+      lw = l; vw = make_float2(bf16_lo(raw), bf16_hi(raw));
     }
   }
-  auto merge = [&](float l, const float (&x)[4]) {
-    if (l == -INFINITY || l == INFINITY) return;
-    const float nm = fmaxf(M, l);
-    const float a = M == -INFINITY ? 0.f : expf(M - nm), b = expf(l - nm);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] = acc[e] * a + x[e] * b;
-    L = L * a + b;
-    M = nm;
-  };
-  if (o_w != nullptr) {
-    const uint2 raw = *reinterpret_cast<const uint2*>(o_w + (static_cast<long long>(c) * Hq + hq) * D + 4 * l32);
-    const float x[4] = {bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)};
-    merge(lse_w[static_cast<long long>(hq) * m + c], x);
-  }
-  if (sk != nullptr) {
-    const long long rq = row_req[c], lim = row_pos[c] - W, nsk = sk_len[rq];
-    const uint2 qr = *reinterpret_cast<const uint2*>(q + brow * q_ts + static_cast<long long>(hq) * D + 4 * l32);
-    const float qv[4] = {bf16_lo(qr.x), bf16_hi(qr.x), bf16_lo(qr.y), bf16_hi(qr.y)};
-    float sm = -INFINITY, sl = 0.f, so[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int j = 0; j < S; ++j) {
-      if (j >= nsk || j > lim) break;
-      const uint16_t* kr = sk + ((rq * S + j) * 2LL * Hkv + kvh) * D + 4 * l32;
-      const uint2 kk = *reinterpret_cast<const uint2*>(kr);
-      const uint2 vv = *reinterpret_cast<const uint2*>(kr + static_cast<long long>(Hkv) * D);
-      float dot = qv[0] * bf16_lo(kk.x) + qv[1] * bf16_hi(kk.x) + qv[2] * bf16_lo(kk.y) + qv[3] * bf16_hi(kk.y);
-#pragma unroll
-      for (int o = 16; o >= 1; o >>= 1) dot += hx(dot, o);
-      const float s = dot * scale, nm = fmaxf(sm, s);
-      const float a = sm == -INFINITY ? 0.f : expf(sm - nm), b = expf(s - nm);
-      so[0] = so[0] * a + bf16_lo(vv.x) * b; so[1] = so[1] * a + bf16_hi(vv.x) * b;
-      so[2] = so[2] * a + bf16_lo(vv.y) * b; so[3] = so[3] * a + bf16_hi(vv.y) * b;
-      sl = sl * a + b;
-      sm = nm;
-    }
-    if (sm != -INFINITY) {
-      const float inv = 1.f / sl;
-      const float x[4] = {so[0] * inv, so[1] * inv, so[2] * inv, so[3] * inv};
-      merge(sm + logf(sl), x);
+
+  float ls = -INFINITY;
+  float2 vs = make_float2(0.f, 0.f);
+  if (sinks != nullptr) {
+    const long long req = req_of[c];
+    const int n = static_cast<int>(min(min(static_cast<long long>(S), sink_len[req]), pos_of[c] - W + 1));
+    if (n > 0) {
+      const uint32_t qraw = *reinterpret_cast<const uint32_t*>(q + dst_row * q_stride + static_cast<long long>(head) * D + 2 * lane);
+      const float q0 = bf16_lo(qraw), q1 = bf16_hi(qraw);
+      const uint16_t* base = sinks + (req * S * 2 * Hkv + kv) * D + 2 * lane;       // K head kv of sink row 0
+      const long long step = 2LL * Hkv * D, to_v = static_cast<long long>(Hkv) * D;
+      float mine = -INFINITY;                                                      // lane j: score of key j
+      for (int j = 0; j < n; ++j) {
+        const uint32_t kraw = *reinterpret_cast<const uint32_t*>(base + j * step);
+        const float sc = wave_sum64(q0 * bf16_lo(kraw) + q1 * bf16_hi(kraw)) * scale;
+        if (lane == j) mine = sc;
+      }
+      const float top = wave_max64(mine);
+      const float p = lane < n ? expf(mine - top) : 0.f;
+      const float mass = wave_sum64(p);
+      for (int j = 0; j < n; ++j) {
+        const float w = __shfl(p, j, 64);
+        const uint32_t vraw = *reinterpret_cast<const uint32_t*>(base + j * step + to_v);
+        vs.x += w * bf16_lo(vraw); vs.y += w * bf16_hi(vraw);
+      }
+      vs.x /= mass; vs.y /= mass;
+      ls = top + logf(mass);
     }
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  *reinterpret_cast<uint2*>(out + brow * o_ts + static_cast<long long>(hq) * D + 4 * l32) =
-      make_uint2(bf16_rn(acc[0] * inv) | (bf16_rn(acc[1] * inv) << 16), bf16_rn(acc[2] * inv) | (bf16_rn(acc[3] * inv) << 16));
+
+  const float top = fmaxf(lp, fmaxf(lw, ls));
+  float2 o = make_float2(0.f, 0.f);
+  if (top != -INFINITY) {
+    const float wp = lp == -INFINITY ? 0.f : expf(lp - top), ww = lw == -INFINITY ? 0.f : expf(lw - top),
+                wsk = ls == -INFINITY ? 0.f : expf(ls - top);
+    const float inv = 1.f / (wp + ww + wsk);
+    o.x = (wp * vp.x + ww * vw.x + wsk * vs.x) * inv;
+    o.y = (wp * vp.y + ww * vw.y + wsk * vs.y) * inv;
+  }
+  *reinterpret_cast<uint32_t*>(out + dst_row * out_stride + static_cast<long long>(head) * D + 2 * lane) =
+      bf16_rn(o.x) | (bf16_rn(o.y) << 16);
 }
 
 template <int QM, bool K2, int NW> int launch_mq(const Params& p, int nitems, hipStream_t st) {
@@ -1118,9 +1178,12 @@ int frmq_prep_q(const void* q, int q_fp32, long long q_ts, const int* idx, int m
                 const uint8_t* kmask, float qscale, void* q16, int Dh, void* stream) {
   if (m <= 0) return 0;
   if (Dh != D) return bad(-4, "frmq_prep_q: head dim 128 only");
-  const long long hw = static_cast<long long>(m) * Hq;
-  hipLaunchKernelGGL(k_prep, dim3(static_cast<unsigned>((hw + 7) / 8)), dim3(256), 0, static_cast<hipStream_t>(stream), q,
-                     q_fp32, q_ts, idx, m, Hq, G, kfull, kmask, qscale, static_cast<uint16_t*>(q16));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint16_t* dst = static_cast<uint16_t*>(q16);
+  if (q_fp32) hipLaunchKernelGGL(k_query_rows<float>, dim3(m), dim3(256), 0, st, static_cast<const float*>(q), q_ts, idx, Hq, G,
+                                 kfull, kmask, qscale, dst);
+  else hipLaunchKernelGGL(k_query_rows<uint16_t>, dim3(m), dim3(256), 0, st, static_cast<const uint16_t*>(q), q_ts, idx, Hq, G,
+                          kfull, kmask, qscale, dst);
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_prep_q");
 }
 
@@ -1155,8 +1218,10 @@ int frmq_merge(const int* tiles, int ntiles, const float* opart, const float* ml
                long long o_ts, int out_fp32, float* lse, long long lse_ts, int Dh, void* stream) {
   if (ntiles <= 0) return 0;
   if (Dh != D) return bad(-4, "frmq_merge: head dim 128 only");
-  hipLaunchKernelGGL(k_merge, dim3(ntiles, Hkv, (rows + 7) / 8), dim3(256), 0, static_cast<hipStream_t>(stream), tiles, opart,
-                     ml, Hkv, G, rows, out, o_ts, out_fp32, lse, lse_ts);
+  const dim3 grid(ntiles, Hkv, (rows + 3) / 4);            // four wavefronts = four rows of the tile per workgroup
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_fp32) hipLaunchKernelGGL(k_fold_items<true>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
+  else hipLaunchKernelGGL(k_fold_items<false>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_merge");
 }
 
@@ -1164,10 +1229,12 @@ int frmq_win_gather(const long long* map, int nk, const void* sinkb, const void*
                     const void* vch, long long v_ts, int Hkv, void* kw, void* vw, int Dh, void* stream) {
   if (nk <= 0) return 0;
   if (Dh != D) return bad(-4, "frmq_win_gather: head dim 128 only");
-  using U = uint16_t;
-  hipLaunchKernelGGL(k_win_gather, dim3(nk), dim3(128), 0, static_cast<hipStream_t>(stream), map, static_cast<const U*>(sinkb),
-                     static_cast<const U*>(preb), static_cast<const U*>(kch), k_ts, static_cast<const U*>(vch), v_ts, Hkv,
-                     static_cast<U*>(kw), static_cast<U*>(vw));
+  const int pieces = Hkv * D / 8;                          // 16-byte pieces of one K (or V) row
+  const long long total = static_cast<long long>(nk) * pieces;
+  hipLaunchKernelGGL(k_collect_rows, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), map, nk, static_cast<const uint4*>(sinkb), static_cast<const uint4*>(preb),
+                     static_cast<const uint16_t*>(kch), k_ts, static_cast<const uint16_t*>(vch), v_ts, pieces,
+                     static_cast<uint4*>(kw), static_cast<uint4*>(vw));
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_win_gather");
 }
 
@@ -1177,8 +1244,9 @@ int frmq_bf_merge(int m, int Hq, int Hkv, const void* q, long long q_ts, const l
                   int Dh, void* stream) {
   if (m <= 0) return 0;
   if (Dh != D) return bad(-4, "frmq_bf_merge: head dim 128 only");
+  if (sk != nullptr && S > 64) return bad(-5, "frmq_bf_merge: at most 64 sink tokens");
   using U = uint16_t;
-  hipLaunchKernelGGL(k_bf_merge, dim3(m, (Hq + 7) / 8), dim3(256), 0, static_cast<hipStream_t>(stream), m, Hq, Hkv,
+  hipLaunchKernelGGL(k_mix_parts, dim3(m, (Hq + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), m, Hq, Hkv,
                      static_cast<const U*>(q), q_ts, idx, o_p, lse_p, static_cast<const U*>(o_w), lse_w,
                      static_cast<const U*>(sk), row_req, row_pos, sk_len, S, W, scale, static_cast<U*>(out), o_ts);
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_bf_merge");

@@ -1,29 +1,28 @@
-"""ctypes front end of libflagrot_kernels.so (gfx950): paged FlagRot KV-cache writers + paged decode attention.
+"""Front end of libflagrot_kernels.so (gfx950): the paged FlagRot KV-cache writers and the paged decode attention.
 
-Host-side mirror of the reference plugin's front end (integrations/vllm_flagrot/vllm_flagrot/kernels.py of the
-reference): same function names, argument meaning and error behaviour, so callers written against it
-(`v2_write`, `v2_attn`, `cb_write`, `cb_write3`, `w3_static_write`, `cb_attn`, `head_fwht`, `plan_v2`, `plan_cb`,
-`Workspace`) run unchanged.  PyTorch-ROCm only supplies device memory and the current HIP stream; every launch is
-asynchronous on that stream and allocates nothing.
+What a caller of the reference plugin's front end (integrations/vllm_flagrot/vllm_flagrot/kernels.py) finds here under
+the same names and with the same arguments: the static-format writer and decode (`v2_write`, `v2_attn`), the selecting
+writers of the key-only kinds (`cb_write`, `cb_write3`, `w3_static_write`, `head_fwht`) and their decode (`cb_attn`), the
+split planners (`plan_v2`, `plan_cb`) and the split-K `Workspace`.  `cb_attn_noalloc` exists on this build only.
 
-The shared library is built in-tree by `flagrot_releaser_amd.build` (hipcc, --offload-arch=gfx950).  It is rebuilt on
-first use when it is missing or older than a source (file lock; set FLAGROT_NO_REBUILD=1 to forbid), and a missing
-compiler or a failed build raises: there is no fallback path.
+PyTorch lends device memory and the current HIP stream; each call is one or two asynchronous kernel launches on that
+stream, and none of them allocates.  The library is built in-tree by flagrot_releaser_amd.build (hipcc,
+--offload-arch=gfx950) and rebuilt on first use when a source is newer (FLAGROT_NO_REBUILD=1 forbids that); when it
+cannot be had the call raises -- there is no other path to a result.
 """
 from __future__ import annotations
 
 import ctypes
-import fcntl
 import math
 import os
-from pathlib import Path
 
 import torch
 
-from . import build as _build
+from .native import Library, as_arg, current_stream
 
 ABI = 9
 D, RB, NG = 128, 32, 4
+# numbers the C ABI shares with the reference: format ids, kind ids, variant bits
 V2_FMT = {"int4": 4, "int4a": 5, "konly": 6, "konlya": 7, "int2a": 8, "konlya2": 9}
 INT2_FMTS = ("int2a", "konlya2")
 GEN, GT8, HD256 = 1024, 2048, 4096
@@ -33,134 +32,82 @@ STAGES = 4
 MAX_CHUNK, MAX_SPLITS = 8192, 512
 SEEDS = (0,) + tuple(range(2, 16))
 W3_SPLIT_T = int(os.environ.get("W3_SPLIT_T", "256"))
+NOALLOC_MAX_PARTS = 8192     # FR_NOALLOC_MAX_PARTS of include/flagrot_kernels.h
 
-
-# ------------------------------------------------------------------------------------------------ library
-def _lib_path() -> Path:
-    return Path(os.environ.get("FLAGROT_LIB", _build.lib_path("kernels")))
-
-
-def _stale(lib: Path) -> bool:
-    if not lib.exists():
-        return True
-    if os.environ.get("FLAGROT_NO_REBUILD") or "FLAGROT_LIB" in os.environ:
-        return False
-    t = lib.stat().st_mtime
-    return any(s.exists() and s.stat().st_mtime > t for s in _build.sources("kernels"))
-
-
-_LIB = None
+NATIVE = Library("kernels", "FLAGROT_LIB", "fr_abi_version", ABI, "fr_last_error", {
+    "fr_v2_attn": "i p l p p i p i i i i i f p p i i i i i p p p p l p p p l l p i i",
+    "fr_v2_write": "i p l p i i i p i p p i p",
+    "fr_v2_occupancy": "i i i i",
+    "fr_v2_chunk_bytes": "i i",
+    "fr_cb_nsg": "",
+    "fr_cb_write": "p l p i i i i i p p p i p p i p",
+    "fr_cb_write3": "p l p i i i i p p p p p i p i i p p",
+    "fr_w3_static_write": "p l p i i i p p i p i p p",
+    "fr_cb_attn": "p l p p i p i i i i i f p i i i p p p p l p p p l l p i",
+    "fr_cb_occupancy": "i i i i",
+    "fr_cb_chunk_bytes": "i i",
+    "fr_cb_write_smem": "i i i",
+    "fr_last_error": "->s",
+    "fr_head_fwht": "p l p l i i p f p i",
+    "fr_cb_attn_noalloc": "p l p p i p i i i i i f i p l p p p l l p i i",
+})
+EXPORTS = NATIVE.exports
 
 
 def lib():
-    """the loaded library (built first when missing or out of date); raises when it cannot be had."""
-    global _LIB
-    if _LIB is not None:
-        return _LIB
-    path = _lib_path()
-    if _stale(path):
-        if os.environ.get("FLAGROT_NO_REBUILD"):
-            raise RuntimeError(f"{path} is missing and FLAGROT_NO_REBUILD is set")
-        path.parent.mkdir(parents=True, exist_ok=True)
-        with open(str(path) + ".lock", "w") as lk:
-            fcntl.flock(lk, fcntl.LOCK_EX)
-            try:
-                if _stale(path):
-                    _build.build("kernels", verbose=False)
-            finally:
-                fcntl.flock(lk, fcntl.LOCK_UN)
-    L = ctypes.CDLL(str(path))
-    P, I, LL, F = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong, ctypes.c_float
-    L.fr_abi_version.restype = I
-    if L.fr_abi_version() != ABI:
-        raise RuntimeError(f"libflagrot_kernels ABI {L.fr_abi_version()} != {ABI}: rebuild ({path})")
-    sig = {
-        "fr_v2_attn": [I, P, LL, P, P, I, P, I, I, I, I, I, F, P, P, I, I, I, I, I, P, P, P, P, LL, P, P, P, LL, LL, P,
-                       I, I],
-        "fr_v2_write": [I, P, LL, P, I, I, I, P, I, P, P, I, P],
-        "fr_v2_occupancy": [I, I, I, I],
-        "fr_v2_chunk_bytes": [I, I],
-        "fr_cb_nsg": [],
-        "fr_cb_write": [P, LL, P, I, I, I, I, I, P, P, P, I, P, P, I, P],
-        "fr_cb_write3": [P, LL, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P],
-        "fr_w3_static_write": [P, LL, P, I, I, I, P, P, I, P, I, P, P],
-        "fr_cb_attn": [P, LL, P, P, I, P, I, I, I, I, I, F, P, I, I, I, P, P, P, P, LL, P, P, P, LL, LL, P, I],
-        "fr_cb_occupancy": [I, I, I, I],
-        "fr_cb_chunk_bytes": [I, I],
-        "fr_cb_write_smem": [I, I, I],
-        "fr_head_fwht": [P, LL, P, LL, I, I, P, F, P, I],
-        "fr_cb_attn_noalloc": [P, LL, P, P, I, P, I, I, I, I, I, F, I, P, LL, P, P, P, LL, LL, P, I, I],
-    }
-    for name, args in sig.items():
-        fn = getattr(L, name)
-        fn.argtypes, fn.restype = args, I
-    L.fr_last_error.restype = ctypes.c_char_p
-    _LIB = L
-    return L
+    """the ctypes handle (the library is built first when it is missing or older than its sources)"""
+    return NATIVE.dll
 
 
-EXPORTS = ("fr_abi_version", "fr_v2_attn", "fr_v2_write", "fr_v2_occupancy", "fr_v2_chunk_bytes", "fr_cb_nsg",
-           "fr_cb_write", "fr_cb_write3", "fr_w3_static_write", "fr_cb_attn", "fr_cb_occupancy", "fr_cb_chunk_bytes",
-           "fr_cb_write_smem", "fr_last_error", "fr_head_fwht", "fr_cb_attn_noalloc")
-NOALLOC_MAX_PARTS = 8192     # FR_NOALLOC_MAX_PARTS of include/flagrot_kernels.h
-
-
-def _check(rc: int, what: str):
-    if rc != 0:
-        raise RuntimeError(f"{what}: launch failed (code {rc}, {lib().fr_last_error().decode()})")
-
-
-def _ptr(t):
-    return None if t is None else t.data_ptr()
-
-
-_DEV_IDX: list = []
-
-
-def _stream():
-    """raw hipStream_t of torch's current stream (the device index is cached: one device per process)."""
-    if not _DEV_IDX:
-        _DEV_IDX.append(torch.cuda.current_device())
-    return torch._C._cuda_getCurrentRawStream(_DEV_IDX[0])
-
-
-_SG = None
+_SIGN_TABLE = (ctypes.c_uint * (len(SEEDS) * 4))()
 
 
 def sign_words():
-    """uint32[15 * 4] sign table argument of the codebook entry points.  The key-only kinds never read it; it is
-    passed as zeros to keep the reference signature."""
-    global _SG
-    if _SG is None:
-        _SG = (ctypes.c_uint * (len(SEEDS) * 4))()
-    return _SG
+    """The sign-table argument (uint32 [15 * 4]) of the codebook entry points.  Only codebook kinds that this build
+    does not have read it; the key-only kinds get zeros, so that the reference's signatures stay as they are."""
+    return _SIGN_TABLE
 
 
 # ------------------------------------------------------------------------------------------------ shapes / variants
 def qtile(G: int, Dh: int = 128) -> int:
-    return 8 if Dh == 128 and 5 <= G <= 8 else 4
+    """query heads one decode workgroup serves: 8 for GQA groups of 5 .. 8 at head dim 128, else 4"""
+    return 8 if (Dh == 128 and 4 < G <= 8) else 4
 
 
 def v2_variant(fmt: str, G: int = 4, Dh: int = 128) -> int:
-    if G == 4 and Dh == 128 and fmt in ("int4", "int4a", "int2a"):
+    """the `variant` argument of fr_v2_attn: 264 = the GQA-4, head-128 kernels of the static formats; every other shape
+    (and every key-only kind) adds GEN, plus GT8 for 8-head tiles and HD256 for head dim 256"""
+    if (G, Dh) == (4, 128) and fmt not in K2:
         return 264
-    return 264 | GEN | (GT8 if qtile(G, Dh) == 8 else 0) | (HD256 if Dh == 256 else 0)
+    bits = GEN
+    if qtile(G, Dh) == 8:
+        bits |= GT8
+    if Dh == 256:
+        bits |= HD256
+    return 264 | bits
 
 
 def tile_of(variant: int) -> int:
-    return 8 if (variant & GEN) and (variant & GT8) else 4
+    """query heads per partial slot of a variant"""
+    return 8 if variant & GEN and variant & GT8 else 4
 
 
 def vheads(Hkv: int, G: int, Dh: int = 128, fmt: str = "int4") -> int:
-    return Hkv * -(-G // tile_of(v2_variant(fmt, G, Dh)))
+    """workgroups per (sequence, split): one per (KV head, tile of query heads)"""
+    tile = tile_of(v2_variant(fmt, G, Dh))
+    return Hkv * ((G + tile - 1) // tile)
+
+
+def _token_bytes(fmt: str) -> int:
+    return 80 if fmt in INT2_FMTS else 144                    # codes + scale words of K and V of one 128-d token
 
 
 def v2_chunk_bytes(page: int, Dh: int = 128, fmt: str = "int4") -> int:
-    return page * (80 if fmt in INT2_FMTS else 144) * Dh // 128
+    return page * _token_bytes(fmt) * Dh // 128
 
 
 def cb_chunk_bytes(kind: str, page: int, Dh: int = 128) -> int:
-    return page * (80 if kind in INT2_FMTS else 144) * Dh // 128
+    return page * _token_bytes(kind) * Dh // 128
 
 
 # ------------------------------------------------------------------------------------------------ split planner
@@ -208,203 +155,214 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
 
 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
-    HV = Hkv * -(-G // 4)                                  # workgroups per (row, split): q tiles of 4 heads
-    s = _slots(fmt)
-    return plan_splits(B, Lmax, HV, page, s, nsplit, ncu=_NUM_CU)
+    """(nsplit, chunk) of a static-format decode: a workgroup per (KV head, tile of 4 query heads)"""
+    tiles = Hkv * ((G + 3) // 4)
+    return plan_splits(B, Lmax, tiles, page, _slots(fmt), nsplit, ncu=_NUM_CU)
 
 
 def plan_cb(B, Lmax, Hkv, page, kind, nsplit=None, G=4, Dh=128):
-    if kind in K2 and (G != 4 or Dh != 128):
+    """(nsplit, chunk) of a key-only-kind decode (shapes other than GQA 4 / head 128 run the general kernels)"""
+    if kind in K2 and (G, Dh) != (4, 128):
         return plan_v2(B, Lmax, Hkv, page, nsplit, fmt=kind, G=G, Dh=Dh)
-    s = _slots(kind)
-    return plan_splits(B, Lmax, Hkv, page, s, nsplit, ncu=_NUM_CU)
+    return plan_splits(B, Lmax, Hkv, page, _slots(kind), nsplit, ncu=_NUM_CU)
 
 
 class Workspace:
-    """split-K partials for up to `parts` (row, kv head / q tile, split) partials of GT q heads x Dh dims, plus the
-    per-(row, kv head / q tile) merge tickets (zeroed once, self-resetting).  Allocate before graph capture."""
+    """Device memory of the split-K decode: unnormalised partial outputs and (maximum, sum) pairs for `parts`
+    (sequence, KV head or head tile, split) workgroups of GT query heads x Dh channels, and one arrival counter per
+    (sequence, KV head or head tile) that the kernels leave at zero.  Create it before capturing a graph."""
 
     def __init__(self, rows: int, Hkv: int, parts: int, device, GT: int = 4, Dh: int = 128):
         self.rows, self.parts, self.HV, self.GT, self.Dh = rows, parts, Hkv, GT, Dh
-        self.opart = torch.empty(parts * GT * Dh, device=device, dtype=torch.float32)
-        self.mlpart = torch.empty(parts * GT * 2, device=device, dtype=torch.float32)
-        self.counter = torch.zeros(rows * Hkv, device=device, dtype=torch.int32)
+        fp32 = dict(dtype=torch.float32, device=device)
+        self.opart = torch.empty(parts * GT * Dh, **fp32)
+        self.mlpart = torch.empty(parts * GT * 2, **fp32)
+        self.counter = torch.zeros(rows * Hkv, dtype=torch.int32, device=device)
 
     def fits(self, B, Hkv, nsplit_total, GT=4, Dh=128):
-        return (B <= self.rows and B * Hkv * nsplit_total <= self.parts and Hkv <= self.HV
-                and GT * Dh <= self.GT * self.Dh
-                and B * Hkv * nsplit_total * GT * Dh <= self.parts * self.GT * self.Dh)
+        """whether a launch of B sequences x Hkv (head, tile) pairs x nsplit_total splits has room"""
+        need = B * Hkv * nsplit_total
+        return (B <= self.rows and Hkv <= self.HV and need <= self.parts and GT * Dh <= self.GT * self.Dh
+                and need * GT * Dh <= self.parts * self.GT * self.Dh)
 
 
 # ------------------------------------------------------------------------------------------------ launches
-def _kmu(kmu, kv):
-    if kmu is None:
-        return None
-    Hkv, Dh = kv.shape[1] // 2, kv.shape[2]
-    assert kmu.dtype == torch.float32 and kmu.is_contiguous() and tuple(kmu.shape) == (Hkv, Dh) \
-        and kmu.device == kv.device, (kmu.dtype, tuple(kmu.shape), (Hkv, Dh))
-    return kmu.data_ptr()
+def _centre(kmu, kv):
+    """the optional per-(KV head, channel) key centring vector, checked against the rows it will be subtracted from"""
+    if kmu is not None:
+        want = (kv.shape[1] // 2, kv.shape[2])
+        assert kmu.dtype == torch.float32 and kmu.device == kv.device and kmu.is_contiguous(), "kmu: fp32, contiguous, on the rows' device"
+        assert tuple(kmu.shape) == want, (tuple(kmu.shape), want)
+    return kmu
 
 
-def _rows_ok(kv):
-    """bf16 rows contiguous over (head, dim) and 8-byte aligned (the kernels load 4 elements at a time)."""
-    Dh = kv.shape[2]
-    if kv.stride(2) != 1 or kv.stride(1) != Dh or kv.stride(0) % 4 or kv.data_ptr() % 8:
-        kv = kv.contiguous()
-    return kv
+def _loadable(kv):
+    """the writers read four bf16 at a time: heads and channels of a row must be dense, rows 8-byte aligned"""
+    dense = kv.stride(2) == 1 and kv.stride(1) == kv.shape[2]
+    aligned = kv.stride(0) % 4 == 0 and kv.data_ptr() % 8 == 0
+    return kv if dense and aligned else kv.contiguous()
+
+
+def _new_rows(kv, slots):
+    """common checks of the writers' inputs: bf16 rows [T, 2 Hkv, Dh] and int64 slots; returns (rows to read, Hkv, Dh)"""
+    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
+    return _loadable(kv), kv.shape[1] // 2, kv.shape[2]
 
 
 def v2_write(kv, slots, mask, rb, pool, page, fmt="int4", kmu=None):
-    """kv bf16 [T, 2*Hkv, Dh] (Dh 128 | 256) -> pool [num_pages, Hkv, chunk] at slots int64 [T] (< 0 skipped);
-    mask uint8 [2*Hkv, Dh/rb] (K rows first); fmt "int4" | "int4a" | "int2a"."""
-    T = kv.shape[0]
-    if T == 0:
+    """Static formats ("int4" | "int4a" | "int2a"): quantise the rows kv bf16 [T, 2 Hkv, Dh] (K heads, then V heads;
+    Dh 128 or 256) into pool uint8 [pages, Hkv, chunk bytes] at the page slots `slots` int64 [T] (negative: skip).
+    mask uint8 [2 Hkv, Dh / rb] marks the rb-channel groups stored Hadamard-rotated."""
+    if kv.shape[0] == 0:
         return
-    Dh = kv.shape[2]
-    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
-    kv = _rows_ok(kv)
-    _check(lib().fr_v2_write(V2_FMT[fmt], kv.data_ptr(), kv.stride(0), slots.data_ptr(), T, kv.shape[1] // 2, page,
-                             mask.data_ptr(), rb, pool.data_ptr(), _stream(), Dh, _kmu(kmu, kv)), "fr_v2_write")
+    rows, Hkv, Dh = _new_rows(kv, slots)
+    NATIVE.run("fr_v2_write", V2_FMT[fmt], rows, rows.stride(0), slots, rows.shape[0], Hkv, page, mask, rb, pool,
+               current_stream(), Dh, _centre(kmu, rows))
 
 
-def _launcher(fn, args, what, bound):
-    """launch now, or (bound) return a zero-argument callable that launches with these very arguments: the checks and
-    the pointer marshalling are done once, as under graph capture; the tensors must stay alive and in place"""
-    if not bound:
-        _check(fn(*args), what)
-        return None
+class _Bound:
+    """A decode launch with every argument already marshalled: calling it launches again with the very same pointers
+    (what a captured graph would replay), so the tensors have to stay alive and in place."""
 
-    def launch():
-        rc = fn(*args)
-        if rc:
-            _check(rc, what)
-    return launch
+    def __init__(self, entry: str, args: tuple):
+        self.entry, self.args = entry, args
+        self.fn = getattr(NATIVE.dll, entry)
+
+    def __call__(self):
+        if self.fn(*self.args):
+            raise RuntimeError(f"{self.entry}: launch failed ({NATIVE.last_error()})")
+
+
+def _decode(entry: str, args: tuple, bound: bool):
+    if bound:
+        return _Bound(entry, tuple(map(as_arg, args)))
+    NATIVE.run(entry, *args)
+    return None
+
+
+def _tail_args(tail, tail_len, tail_idx, tail_bs, tail_ts):
+    """(rows, lengths, block per sequence, block stride, row stride) of the BF16 window; strides are 0 without one"""
+    if tail is None:
+        return None, tail_len, tail_idx, 0, 0
+    return tail, tail_len, tail_idx, tail_bs, tail_ts
 
 
 def v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kmask=None, vmask=None, rb=32,
             tail=None, tail_len=None, tail_idx=None, tail_bs=None, tail_ts=None, page=16, fmt="int4", kv_start=0,
             bound=False):
-    """q bf16 [B, G*Hkv, Dh] -> out bf16 [B, G*Hkv*Dh].  block_table int32 [B, *] (row stride may be 0), seq_lens int32
-    [B]; tail: bf16 window rows (strides tail_bs / tail_ts elements) with tail_len int32 [B] (+ tail_idx int32 [B]).
-    qscale = softmax scale * log2(e).  kv_start: tokens [0, kv_start) are masked in the paged body."""
+    """Paged decode attention of B one-token queries: q bf16 [B, G Hkv, Dh] -> out bf16 [B, G Hkv Dh] (any row stride).
+    block_table int32 [B, pages] (row stride 0 shares one row) and seq_lens int32 [B] describe the cached tokens, of
+    which [0, kv_start) are skipped; the newest tokens may sit in BF16 rows `tail` (block / row strides tail_bs /
+    tail_ts in elements, tail_len int32 [B] rows used, tail_idx int32 [B] the block of each sequence).  qscale = softmax
+    scale x log2 e; (nsplit, chunk) from plan_v2 / plan_cb; ws a Workspace.  kmask / vmask uint8 [Hkv, Dh / rb] tell the
+    static formats which groups are stored rotated.  bound: return a callable that repeats the launch."""
     B, Hq, Dh = q.shape
     Hkv = pool.shape[1]
     G = Hq // Hkv
-    assert Hq == G * Hkv and q.stride(2) == 1 and q.stride(1) == Dh and out.stride(1) == 1
-    v = v2_variant(fmt, G, Dh)
-    GT = tile_of(v)
-    assert ws.fits(B, vheads(Hkv, G, Dh, fmt), nsplit + (tail is not None), GT, Dh), "split-K workspace too small"
-    args = (V2_FMT[fmt], q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(),
-            block_table.stride(0), seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale,
-            _ptr(kmask), _ptr(vmask), rb, int(kmask is not None), int(vmask is not None), v, STAGES,
-            ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
-            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
-            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), G, int(kv_start))
-    return _launcher(lib().fr_v2_attn, args, "fr_v2_attn", bound)
+    assert G * Hkv == Hq and q.stride(2) == 1 and q.stride(1) == Dh and out.stride(1) == 1
+    variant = v2_variant(fmt, G, Dh)
+    splits = nsplit + (tail is not None)
+    assert ws.fits(B, vheads(Hkv, G, Dh, fmt), splits, tile_of(variant), Dh), "split-K workspace too small"
+    args = (V2_FMT[fmt], q, q.stride(0), pool, block_table, block_table.stride(0), seq_lens, B, Hkv, page, nsplit, chunk,
+            qscale, kmask, vmask, rb, kmask is not None, vmask is not None, variant, STAGES, ws.opart, ws.mlpart,
+            ws.counter, out, out.stride(0), *_tail_args(tail, tail_len, tail_idx, tail_bs, tail_ts), current_stream(), G,
+            int(kv_start))
+    return _decode("fr_v2_attn", args, bound)
 
 
 def cb_write(kv, slots, CT, co, kind, pool, page, tg=None, kmu=None):
-    """kv bf16 [T, 2*Hkv, 128] -> pool at slots int64 [T]; CT fp32 [Hkv, 128, 128] = C_q^T, co fp32 [Hkv, 128]."""
-    T = kv.shape[0]
-    if T == 0:
+    """Key-only kinds: choose per token and KV head between the stored bases (as is / H32 per group / whole-head
+    Hadamard), quantise and pack.  kv bf16 [T, 2 Hkv, 128] at slots int64 [T]; the choice minimises the key error as
+    seen through CT fp32 [Hkv, 128, 128] (the transposed query covariance factor) and the value error weighted by co
+    fp32 [Hkv, 128].  tg: token-group size hint of the reference's launch (1 | 2 | 4), chosen from T when None."""
+    if kv.shape[0] == 0:
         return
-    Dh = kv.shape[2]
-    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
-    kv = _rows_ok(kv)
+    rows, Hkv, Dh = _new_rows(kv, slots)
+    T = rows.shape[0]
     if tg is None:
-        tg = 1 if T <= 16 else (2 if T <= 64 or kind not in K2 else 4)
-    _check(lib().fr_cb_write(kv.data_ptr(), kv.stride(0), slots.data_ptr(), 0, T, kv.shape[1] // 2, page, tg,
-                             CT.data_ptr(), co.data_ptr(), sign_words(), CB_KINDS[kind], pool.data_ptr(), _stream(),
-                             Dh, _kmu(kmu, kv)), "fr_cb_write")
+        tg = 1 if T <= 16 else 4 if (T > 64 and kind in K2) else 2
+    NATIVE.run("fr_cb_write", rows, rows.stride(0), slots, 0, T, Hkv, page, tg, CT, co, sign_words(), CB_KINDS[kind], pool,
+               current_stream(), Dh, _centre(kmu, rows))
 
 
-_SIDE: dict = {}
+_SECOND: dict = {}
 
 
 def side_stream(device=None):
-    """second stream of the two-pass writer (one per device, default priority; create before graph capture)."""
-    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
-    if dev not in _SIDE:
-        _SIDE[dev] = torch.cuda.Stream(dev)
-    return _SIDE[dev]
+    """the stream the value pass of the two-pass writer runs on: one per device, ordinary priority; ask for it before
+    capturing a graph"""
+    where = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if where not in _SECOND:
+        _SECOND[where] = torch.cuda.Stream(where)
+    return _SECOND[where]
 
 
 def w3_nchunk(Hkv, per_cu):
-    global _NUM_CU
-    if _NUM_CU is None:
-        _NUM_CU = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-    return max(1, (per_cu * _NUM_CU) // Hkv)
+    """token chunks per KV head that give `per_cu` workgroups per CU"""
+    _slots(None)
+    return max(1, per_cu * _NUM_CU // Hkv)
 
 
 def w3_calib(Cq, kappa=None, nd=8):
-    """the reference's writer v3 takes tensor-core screening constants (C1 fp16 [H, 168, 128], aux fp32 [H, 48]).
-    This library's writer evaluates the exact fp32 criterion directly and ignores them; zero tensors of the reference
-    shapes keep callers unchanged."""
-    H = Cq.shape[0]
-    return (torch.zeros(H, 168, 128, dtype=torch.float16, device=Cq.device),
-            torch.zeros(H, 48, dtype=torch.float32, device=Cq.device))
+    """The reference's third writer screens candidates with tensor-core products and wants constants for that (C1 fp16
+    [H, 168, 128], aux fp32 [H, 48]).  This build evaluates the selection criterion itself in fp32 and never reads
+    them: zeros of those shapes are returned so that calling code needs no change."""
+    heads = Cq.shape[0]
+    return Cq.new_zeros((heads, 168, 128), dtype=torch.float16), Cq.new_zeros((heads, 48), dtype=torch.float32)
 
 
 def cb_write3(kv, slots, CT, co, C1, beta, kind, pool, page, split=None, kmu=None):
-    """= cb_write (same pool bytes).  split (default: T <= W3_SPLIT_T): key pass on the current stream, value pass on
-    the side stream (fork / join by stream waits, graph capturable), else both in one launch."""
-    T = kv.shape[0]
-    if T == 0:
+    """Writes the same pool bytes as cb_write.  split (default: up to W3_SPLIT_T tokens): the key pass launches on the
+    current stream and the value pass on side_stream(), forked and joined by stream waits, which a graph capture
+    records; otherwise one launch does both."""
+    if kv.shape[0] == 0:
         return
-    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
     assert kv.shape[2] == D, f"writer v3: head dim {D} only (got {kv.shape[2]}; use cb_write)"
-    kv = _rows_ok(kv)
-    slots = slots.contiguous()
-    Hkv = kv.shape[1] // 2
-    L = lib()
-    nk, nv = w3_nchunk(Hkv, 2), w3_nchunk(Hkv, 3)
-    km = _kmu(kmu, kv)
-    args = (kv.data_ptr(), kv.stride(0), slots.data_ptr(), 0, T, Hkv, page, CT.data_ptr(), co.data_ptr(),
-            _ptr(C1), _ptr(beta), sign_words(), CB_KINDS[kind], pool.data_ptr())
+    rows, Hkv, _ = _new_rows(kv, slots)
+    T = rows.shape[0]
+    common = (rows, rows.stride(0), slots.contiguous(), 0, T, Hkv, page, CT, co, C1, beta, sign_words(), CB_KINDS[kind],
+              pool)
+    key_chunks, value_chunks = w3_nchunk(Hkv, 2), w3_nchunk(Hkv, 3)
+    centre = _centre(kmu, rows)
     if split is None:
         split = T <= W3_SPLIT_T
     if not split:
-        _check(L.fr_cb_write3(*args, nk, nv, _stream(), km), "fr_cb_write3")
+        NATIVE.run("fr_cb_write3", *common, key_chunks, value_chunks, current_stream(), centre)
         return
-    cur = torch.cuda.current_stream()
-    side = side_stream(kv.device)
-    side.wait_stream(cur)
-    _check(L.fr_cb_write3(*args, nk, -1, cur.cuda_stream, km), "fr_cb_write3 (keys)")
-    _check(L.fr_cb_write3(*args, -1, nv, side.cuda_stream, None), "fr_cb_write3 (values)")
-    cur.wait_stream(side)
+    main, other = torch.cuda.current_stream(), side_stream(rows.device)
+    other.wait_stream(main)
+    NATIVE.run("fr_cb_write3", *common, key_chunks, -1, main.cuda_stream, centre)           # keys
+    NATIVE.run("fr_cb_write3", *common, -1, value_chunks, other.cuda_stream, None)          # values
+    main.wait_stream(other)
 
 
 def w3_static_write(kv, slots, mask, hfull, pool, page, fmt="int4", path=0, kmu=None):
-    """= head_fwht(kv, hfull, 1/16) + v2_write(.., mask, rb 32, ..) in one launch (same pool bytes)."""
-    T = kv.shape[0]
-    if T == 0:
+    """One launch for head_fwht(kv, hfull, 1 / 16) followed by v2_write(.., mask, rb = 32, ..): same pool bytes."""
+    if kv.shape[0] == 0:
         return
-    assert kv.dtype == torch.bfloat16 and slots.dtype == torch.int64
     assert kv.shape[2] == D, f"writer v3: head dim {D} only (got {kv.shape[2]}; use v2_write)"
-    kv = _rows_ok(kv)
-    slots = slots.contiguous()
-    _check(lib().fr_w3_static_write(kv.data_ptr(), kv.stride(0), slots.data_ptr(), T, kv.shape[1] // 2, page,
-                                    _ptr(mask), _ptr(hfull), {"int4": 0, "int4a": 1, "int2a": 2}[fmt],
-                                    pool.data_ptr(), path, _stream(), _kmu(kmu, kv)), "fr_w3_static_write")
+    rows, Hkv, _ = _new_rows(kv, slots)
+    NATIVE.run("fr_w3_static_write", rows, rows.stride(0), slots.contiguous(), rows.shape[0], Hkv, page, mask, hfull,
+               ("int4", "int4a", "int2a").index(fmt), pool, path, current_stream(), _centre(kmu, rows))
 
 
 def cb_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kind, tail=None, tail_len=None,
             tail_idx=None, tail_bs=None, tail_ts=None, page=16, kv_start=0, bound=False):
+    """v2_attn for the key-only kinds (arguments as there).  GQA 4 at head dim 128 has its own kernels; other shapes
+    go through the general ones."""
     B, Hq, Dh = q.shape
-    if kind in K2 and (Hq != 4 * pool.shape[1] or Dh != 128):
+    Hkv = pool.shape[1]
+    if kind in K2 and (Hq, Dh) != (4 * Hkv, 128):
         return v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, tail=tail, tail_len=tail_len,
                        tail_idx=tail_idx, tail_bs=tail_bs, tail_ts=tail_ts, page=page, fmt=kind, kv_start=kv_start,
                        bound=bound)
-    Hkv = Hq // 4
-    assert Hq == 4 * pool.shape[1] and Dh == D, f"codebook {kind}: GQA 4, head dim 128 only"
+    assert (Hq, Dh) == (4 * Hkv, D), f"codebook {kind}: GQA 4, head dim 128 only"
     assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
     assert ws.fits(B, Hkv, nsplit + (tail is not None)), "split-K workspace too small"
-    args = (q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
-            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, sign_words(), CB_KINDS[kind], 0,
-            STAGES, ws.opart.data_ptr(), ws.mlpart.data_ptr(), ws.counter.data_ptr(), out.data_ptr(),
-            out.stride(0), _ptr(tail), _ptr(tail_len), _ptr(tail_idx),
-            0 if tail is None else tail_bs, 0 if tail is None else tail_ts, _stream(), int(kv_start))
-    return _launcher(lib().fr_cb_attn, args, "fr_cb_attn", bound)
+    args = (q, q.stride(0), pool, block_table, block_table.stride(0), seq_lens, B, Hkv, page, nsplit, chunk, qscale,
+            sign_words(), CB_KINDS[kind], 0, STAGES, ws.opart, ws.mlpart, ws.counter, out, out.stride(0),
+            *_tail_args(tail, tail_len, tail_idx, tail_bs, tail_ts), current_stream(), int(kv_start))
+    return _decode("fr_cb_attn", args, bound)
 
 
 def cb_attn_noalloc(q, pool, block_table, seq_lens, out, nsplit, chunk, qscale, kind, tail=None, tail_len=None,
@@ -417,24 +375,23 @@ def cb_attn_noalloc(q, pool, block_table, seq_lens, out, nsplit, chunk, qscale, 
     G = Hq // Hkv
     assert kind in K2 and Hq == G * Hkv and Dh == D, f"{kind}: key-only 2x2 kinds, head dim 128 only"
     assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
-    args = (q.data_ptr(), q.stride(0), pool.data_ptr(), block_table.data_ptr(), block_table.stride(0),
-            seq_lens.data_ptr(), B, Hkv, page, nsplit, chunk, qscale, CB_KINDS[kind], out.data_ptr(), out.stride(0),
-            _ptr(tail), _ptr(tail_len), _ptr(tail_idx), 0 if tail is None else tail_bs,
-            0 if tail is None else tail_ts, _stream(), G, int(kv_start))
-    return _launcher(lib().fr_cb_attn_noalloc, args, "fr_cb_attn_noalloc", bound)
+    args = (q, q.stride(0), pool, block_table, block_table.stride(0), seq_lens, B, Hkv, page, nsplit, chunk, qscale,
+            CB_KINDS[kind], out, out.stride(0), *_tail_args(tail, tail_len, tail_idx, tail_bs, tail_ts), current_stream(),
+            G, int(kv_start))
+    return _decode("fr_cb_attn_noalloc", args, bound)
 
 
 def head_fwht(x, flags, scale, out=None):
-    """x bf16 [T, H, Dh] (Dh 128 | 256) -> scale * H_Dh x (unnormalised +-1 Sylvester) for heads with flags[h] != 0,
-    a copy otherwise; out may alias x."""
+    """scale x H x per head of x bf16 [T, H, Dh] (Dh 128 or 256; H the +-1 Sylvester matrix, not normalised) where
+    flags[h] is set, a plain copy of the head where it is not.  out may be x itself."""
     T, H, Dh = x.shape
-    assert x.dtype == torch.bfloat16 and x.stride(2) == 1 and x.stride(1) == Dh
+    dense = lambda t: t.stride(2) == 1 and t.stride(1) == Dh            # noqa: E731
+    assert x.dtype == torch.bfloat16 and dense(x)
     if out is None:
-        out = torch.empty(T, H, Dh, dtype=x.dtype, device=x.device)
-    assert out.stride(2) == 1 and out.stride(1) == Dh
+        out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    assert dense(out)
     if T:
-        _check(lib().fr_head_fwht(x.data_ptr(), x.stride(0), out.data_ptr(), out.stride(0), T, H, flags.data_ptr(),
-                                  scale, _stream(), Dh), "fr_head_fwht")
+        NATIVE.run("fr_head_fwht", x, x.stride(0), out, out.stride(0), T, H, flags, scale, current_stream(), Dh)
     return out
 
 
