@@ -196,7 +196,9 @@ def test_mq_attention_against_fp64(dev, case):
             c += nq
         fin = ~empty
         lerr = np.abs(gl[fin] - ref_lse[fin]).max() if fin.any() else 0.0
-        print(f"case {case} rep {rep}: lse abs err {lerr:.2e}, worst rel l2 {worst:.2e}")
+        el = float((np.abs(got - ref) / (2e-3 + 1e-2 * np.abs(ref))).max())
+        print(f"case {case} rep {rep}: lse abs err {lerr:.2e}, worst rel l2 {worst:.2e}, element-wise "
+              f"|err| / (2e-3 + 1e-2 |ref|) = {el:.2f} (fp32 output)")
         assert lerr <= (1e-2 if k2 else 5e-3), (case, rep, lerr)
         # bf16 rows of the layer output
         ob = outbuf.float().cpu()
