@@ -931,55 +931,73 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
 }
 
 // ------------------------------------------------------------------------------------------------ items of a tile, folded
-// One wavefront per (query row of a tile, KV head), a lane per channel pair.  The items' (maximum, sum) pairs are read
-// one item per lane (64 at a time), so the common maximum, every item's weight 2^(m - M) and the total sum come from
-// three wave reductions instead of two serial passes; the accumulation loop then takes each weight from its lane.
+// A wavefront folds FOLD_ROWS consecutive query rows of a tile for one KV head, a lane per channel pair.  The items'
+// (maximum, sum) pairs are read one item per lane (64 at a time), so the common maximum, every item's weight
+// 2^(m - M) and the total sum come from three wave reductions instead of two serial passes; the accumulation loop then
+// takes each weight from its lane.  A tile with a single item (the common case when the requests fill the GPU) needs
+// neither: its partial is divided by its own sum.
+constexpr int FOLD_ROWS = 4;
+
 template <bool FP32_OUT>
 __global__ void __launch_bounds__(256) k_fold_items(const int* __restrict__ tiles, const float* __restrict__ opart,
                                                     const float* __restrict__ ml, int Hkv, int G, int rows,
                                                     void* __restrict__ out, long long out_stride, float* __restrict__ lse,
                                                     long long lse_stride) {
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.z * 4 + (threadIdx.x >> 6), head = blockIdx.y;
+  const int lane = threadIdx.x & 63, head = blockIdx.y;
   const int* rec = tiles + TILE_INTS * blockIdx.x;
-  const int token = row / G;
-  if (row >= (rows / G) * G || token >= rec[3]) return;                  // rec[3]: tokens of the tile (wave uniform)
   const int first = rec[6], count = rec[7];
+  const int used = min(rows / G, rec[3]) * G;                            // rows of the tile that hold a token's head
   const long long per_item = static_cast<long long>(Hkv) * rows;         // partial rows from one item to the next
-  const long long at = (static_cast<long long>(first) * Hkv + head) * rows + row;
-  float2 sum = make_float2(0.f, 0.f);
-  float top = -INFINITY, total = 0.f;
-  for (int s0 = 0; s0 < count; s0 += 64) top = fmaxf(top, wave_max64(s0 + lane < count ? ml[2 * (at + (s0 + lane) * per_item)] : -INFINITY));
-  if (top != -INFINITY) {
-    for (int s0 = 0; s0 < count; s0 += 64) {
-      float weight = 0.f, mass = 0.f;
-      if (s0 + lane < count) {
-        const float2 st = *reinterpret_cast<const float2*>(ml + 2 * (at + (s0 + lane) * per_item));
-        weight = st.x == -INFINITY ? 0.f : fexp2(st.x - top);
-        mass = weight * st.y;
-      }
-      total += wave_sum64(mass);
-      const int n = min(64, count - s0);
-      for (int s = 0; s < n; ++s) {
-        const float w = __shfl(weight, s, 64);
-        if (w == 0.f) continue;                                          // an item that saw no key: nothing to read
-        const float2 x = *reinterpret_cast<const float2*>(opart + (at + (s0 + s) * per_item) * D + 2 * lane);
-        sum.x += w * x.x; sum.y += w * x.y;
+  const int row0 = (blockIdx.z * 4 + (threadIdx.x >> 6)) * FOLD_ROWS;
+#pragma unroll
+  for (int i = 0; i < FOLD_ROWS; ++i) {
+    const int row = row0 + i;
+    if (row >= used) break;                                              // wave uniform
+    const long long at = (static_cast<long long>(first) * Hkv + head) * rows + row;
+    float2 sum = make_float2(0.f, 0.f);
+    float top, total;
+    if (count == 1) {
+      const float2 st = *reinterpret_cast<const float2*>(ml + 2 * at);
+      top = st.x; total = st.y;
+      if (top != -INFINITY) sum = *reinterpret_cast<const float2*>(opart + at * D + 2 * lane);
+    } else {
+      top = -INFINITY; total = 0.f;
+      for (int s0 = 0; s0 < count; s0 += 64)
+        top = fmaxf(top, wave_max64(s0 + lane < count ? ml[2 * (at + (s0 + lane) * per_item)] : -INFINITY));
+      if (top != -INFINITY) {
+        for (int s0 = 0; s0 < count; s0 += 64) {
+          float weight = 0.f, mass = 0.f;
+          if (s0 + lane < count) {
+            const float2 st = *reinterpret_cast<const float2*>(ml + 2 * (at + (s0 + lane) * per_item));
+            weight = st.x == -INFINITY ? 0.f : fexp2(st.x - top);
+            mass = weight * st.y;
+          }
+          total += wave_sum64(mass);
+          const int n = min(64, count - s0);
+          for (int s = 0; s < n; ++s) {
+            const float w = __shfl(weight, s, 64);
+            if (w == 0.f) continue;                                      // an item that saw no key: nothing to read
+            const float2 x = *reinterpret_cast<const float2*>(opart + (at + (s0 + s) * per_item) * D + 2 * lane);
+            sum.x += w * x.x; sum.y += w * x.y;
+          }
+        }
       }
     }
-    const float inv = 1.f / total;
-    sum.x *= inv; sum.y *= inv;
+    if (top != -INFINITY) {
+      const float inv = 1.f / total;
+      sum.x *= inv; sum.y *= inv;
+    }
+    const int token = row / G, qhead = head * G + row % G;
+    if (FP32_OUT) {                                                      // compact rows, dense [m, Hq, D]
+      float* dst = static_cast<float*>(out) + (static_cast<long long>(rec[1] + token) * Hkv * G + qhead) * D;
+      *reinterpret_cast<float2*>(dst + 2 * lane) = sum;
+    } else {                                                             // rows of the layer output
+      uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(rec[2] + token) * out_stride + qhead * D;
+      *reinterpret_cast<uint32_t*>(dst + 2 * lane) = bf16_rn(sum.x) | (bf16_rn(sum.y) << 16);
+    }
+    if (lse != nullptr && lane == 0)
+      lse[qhead * lse_stride + rec[1] + token] = top == -INFINITY ? -INFINITY : (top + log2f(total)) * 0.6931471805599453f;
   }
-  const int qhead = head * G + row % G;
-  if (FP32_OUT) {                                                        // compact rows, dense [m, Hq, D]
-    float* dst = static_cast<float*>(out) + (static_cast<long long>(rec[1] + token) * Hkv * G + qhead) * D;
-    *reinterpret_cast<float2*>(dst + 2 * lane) = sum;
-  } else {                                                               // rows of the layer output
-    uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(rec[2] + token) * out_stride + qhead * D;
-    *reinterpret_cast<uint32_t*>(dst + 2 * lane) = bf16_rn(sum.x) | (bf16_rn(sum.y) << 16);
-  }
-  if (lse != nullptr && lane == 0)
-    lse[qhead * lse_stride + rec[1] + token] = top == -INFINITY ? -INFINITY : (top + log2f(total)) * 0.6931471805599453f;
 }
 
 // ------------------------------------------------------------------------------------------------ query rows for the kernel
@@ -1218,7 +1236,7 @@ int frmq_merge(const int* tiles, int ntiles, const float* opart, const float* ml
                long long o_ts, int out_fp32, float* lse, long long lse_ts, int Dh, void* stream) {
   if (ntiles <= 0) return 0;
   if (Dh != D) return bad(-4, "frmq_merge: head dim 128 only");
-  const dim3 grid(ntiles, Hkv, (rows + 3) / 4);            // four wavefronts = four rows of the tile per workgroup
+  const dim3 grid(ntiles, Hkv, (rows + 4 * FOLD_ROWS - 1) / (4 * FOLD_ROWS));      // four wavefronts x FOLD_ROWS rows per workgroup
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (out_fp32) hipLaunchKernelGGL(k_fold_items<true>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
   else hipLaunchKernelGGL(k_fold_items<false>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
