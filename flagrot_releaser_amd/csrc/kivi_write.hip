@@ -62,10 +62,17 @@ template <int C> DEVI void to_basis(float (&y)[4], int l32) {   // candidate 0 i
 }
 
 // ------------------------------------------------------------------------------------------------ value writer
-template <bool F8>
+// WMAT: the selection weighs the reconstruction error e (original basis) by a full matrix per head, e^T M e, instead of
+// the diagonal sum co . e^2 (kivi.cu:213-287): per sub-vector only the diagonal 32-block of M counts, the whole-head
+// candidate and the combination of the chosen sub-vector candidates use all of M.  The error vectors of a row sit in
+// LDS (one strip per half wave) and every lane forms the products of its four rows of M.
+template <bool F8, bool WMAT>
 __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv, long long kv_rs, int n, int Hkv,
                                                  const long long* __restrict__ slots, const float* __restrict__ co,
-                                                 uint8_t* __restrict__ pool, int ident, const int* __restrict__ vfix) {
+                                                 const float* __restrict__ M, uint8_t* __restrict__ pool, int ident,
+                                                 const int* __restrict__ vfix) {
+  constexpr int EW = WMAT ? 128 : 1;                    // the strips exist only in the matrix-weighted kernel
+  __shared__ float esh[WMAT ? 8 : 1][3][EW];
   const int l32 = threadIdx.x & 31;
   const long long item = static_cast<long long>(blockIdx.x) * 8 + (threadIdx.x >> 5);
   if (item >= static_cast<long long>(n) * Hkv) return;
@@ -76,7 +83,7 @@ __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv
   const float x[4] = {bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)};
   const float4 cw = *reinterpret_cast<const float4*>(co + h * 128 + 4 * l32);
   const float cwv[4] = {cw.x, cw.y, cw.z, cw.w};
-  float sc[3], mnv[3], err[3];
+  float sc[3], mnv[3], err[3], dv[3][4];
   int code[3][4];
 #pragma unroll
   for (int c = 0; c < 3; ++c) {
@@ -94,14 +101,52 @@ __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv
     if (c == 2) fwht<128>(y, l32);
     float e = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { const float d = y[i] - x[i]; e += d * d * cwv[i]; }
+    for (int i = 0; i < 4; ++i) { const float d = y[i] - x[i]; dv[c][i] = d; e += d * d * cwv[i]; }
     err[c] = e;
   }
   const int j = l32 >> 3;
   bool useH, useF;
   if (ident) { useH = false; useF = false; }
   else if (vfix != nullptr) { useF = (vfix[h] >> 16) & 1; useH = (vfix[h] >> j) & 1; }
-  else {
+  else if constexpr (WMAT) {
+    float (*E)[EW] = esh[threadIdx.x >> 5];
+    const float* Mh = M + static_cast<long long>(h) * 128 * 128;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) E[c][4 * l32 + i] = dv[c][i];
+    wave_lds_sync();
+    float eI = 0.f, eH = 0.f, eF = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float* row = Mh + (4 * l32 + i) * 128;
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+      for (int k = 32 * j; k < 32 * j + 32; ++k) { const float m = row[k]; a0 += m * E[0][k]; a1 += m * E[1][k]; }
+      for (int k = 0; k < 128; ++k) a2 += row[k] * E[2][k];
+      eI += dv[0][i] * a0; eH += dv[1][i] * a1; eF += dv[2][i] * a2;
+    }
+    eI += hx(eI, 1); eI += hx(eI, 2); eI += hx(eI, 4);
+    eH += hx(eH, 1); eH += hx(eH, 2); eH += hx(eH, 4);
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
+    useH = eH < eI;                                      // identity on ties
+    wave_lds_sync();                                     // every lane has read the strips
+    if (useH)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) E[0][4 * l32 + i] = dv[1][i];
+    wave_lds_sync();
+    float eB = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float* row = Mh + (4 * l32 + i) * 128;
+      float a = 0.f;
+      for (int k = 0; k < 128; ++k) a += row[k] * E[0][k];
+      eB += (useH ? dv[1][i] : dv[0][i]) * a;
+    }
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
+    useF = eF < eB;                                      // base on ties
+  } else {
     float eI = err[0], eH = err[1], eF = err[2];
     eI += hx(eI, 1); eI += hx(eI, 2); eI += hx(eI, 4);
     eH += hx(eH, 1); eH += hx(eH, 2); eH += hx(eH, 4);
@@ -443,11 +488,12 @@ __global__ void k_lse_merge(const uint16_t* __restrict__ oa, const float* __rest
 }  // namespace
 
 int v_write_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
-                   int ident, const int* vfix, int f8, hipStream_t st) {
+                   const float* M, int ident, const int* vfix, int f8, hipStream_t st) {
   const long long items = static_cast<long long>(n) * Hkv;
-  const auto kern = f8 ? k_v_write<true> : k_v_write<false>;
+  const bool wmat = M != nullptr && !ident && vfix == nullptr;
+  const auto kern = wmat ? (f8 ? k_v_write<true, true> : k_v_write<false, true>) : (f8 ? k_v_write<true, false> : k_v_write<false, false>);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((items + 7) / 8)), dim3(256), 0, st,
-                     static_cast<const uint16_t*>(kv), kv_rs, n, Hkv, slots, co, pool, ident, vfix);
+                     static_cast<const uint16_t*>(kv), kv_rs, n, Hkv, slots, co, M, pool, ident, vfix);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 

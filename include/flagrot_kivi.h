@@ -7,8 +7,8 @@
  * `stream` is a hipStream_t, asynchronous, no allocation.  Return codes: 0 ok, 1 launch failure, 2 bad / unsupported
  * argument (message from kv_last_error()).  Built for head dim 128, FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3
  * scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes computed from the stored values, the value rows' whole-head
- * flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88, 123-128); head dim 256 and the matrix value weighting M
- * return 2.
+ * flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88, 123-128), diagonal (co) and matrix (M) value weighting;
+ * head dim 256 returns 2.
  */
 #ifndef FLAGROT_KIVI_H
 #define FLAGROT_KIVI_H

@@ -115,9 +115,14 @@ def _back(y, c):
 
 
 # --------------------------------------------------------------------------------------------------- value encoder
-def v_encode(x_bits, co, ident=False, fix=None, f8=False, true_div=False):
+def v_encode(x_bits, co, ident=False, fix=None, f8=False, true_div=False, M=None):
     """x_bits uint16 [T, H, D] bf16 V rows; co fp32 [H, D].  Returns dict: codes uint8 [3, T, H, D] per candidate,
-    s, mn fp32 [3, T, H, NV], useH bool [T, H, NV], useF bool [T, H] (fp64 decision), margins (relative gaps)."""
+    s, mn fp32 [3, T, H, NV], useH bool [T, H, NV], useF bool [T, H] (fp64 decision), margins (relative gaps).
+    M fp32 [H, D, D] (kivi.cu:213-287; ignored with ident / fix, like the reference): the error e of a candidate, in the
+    original basis, counts as e^T M e instead of sum co e^2 -- per sub-vector with the diagonal 32-block of M only, for
+    the whole-head candidate and for the combination of the chosen sub-vector candidates with all of M.
+    Parity of the M form: pinned by its reduction to the diagonal form for M = diag(co) and by a brute-force
+    evaluation of the quadratic forms (tests/test_oracle_kivi.py); no reference-written vector covers it."""
     x = Q.bf16_to_f32(x_bits)
     T, H, D = x.shape
     NV = D // 32
@@ -126,13 +131,20 @@ def v_encode(x_bits, co, ident=False, fix=None, f8=False, true_div=False):
     s, mn = kivi_params(g.min(-1), g.max(-1), f8, true_div)
     codes = kivi_code(g, mn[..., None], s[..., None])
     rec = kivi_rec(codes, mn[..., None], s[..., None]).reshape(3, T, H, D)
-    err = []
-    for c in range(3):
-        d = (_back(rec[c], c) - x).astype(np.float64)
-        err.append((d * d * np.asarray(co, np.float64)[None]).reshape(T, H, NV, 32).sum(-1))
-    eI, eH, eF = err[0], err[1], err[2].sum(-1)
-    useH = eH < eI
-    eB = np.where(useH, eH, eI).sum(-1)
+    ds = [(_back(rec[c], c) - x).astype(np.float64) for c in range(3)]
+    if M is None or ident or fix is not None:
+        err = [(d * d * np.asarray(co, np.float64)[None]).reshape(T, H, NV, 32).sum(-1) for d in ds]
+        eI, eH, eF = err[0], err[1], err[2].sum(-1)
+        useH = eH < eI
+        eB = np.where(useH, eH, eI).sum(-1)
+    else:
+        Mh = np.asarray(M, np.float64)                                              # [H, D, D]
+        Mb = np.stack([Mh[:, 32 * j:32 * j + 32, 32 * j:32 * j + 32] for j in range(NV)], 1)     # [H, NV, 32, 32]
+        local = lambda d: np.einsum("thji,hjik,thjk->thj", d.reshape(T, H, NV, 32), Mb, d.reshape(T, H, NV, 32))  # noqa: E731
+        whole = lambda d: np.einsum("thi,hik,thk->th", d, Mh, d)                                # noqa: E731
+        eI, eH, eF = local(ds[0]), local(ds[1]), whole(ds[2])
+        useH = eH < eI
+        eB = whole(np.where(np.repeat(useH, 32, -1), ds[1], ds[0]))
     useF = eF < eB
     mH = np.abs(eH - eI) / np.maximum(eH + eI, 1e-300)
     mF = np.abs(eF - eB) / np.maximum(eF + eB, 1e-300)

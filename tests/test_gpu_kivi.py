@@ -96,6 +96,51 @@ def test_v_write_given_flags(dev, seed, T, Hkv, f8):
 
 
 @F8
+def test_v_write_matrix_weight(dev, f8):
+    """the value selection weighted by a full matrix per head (e^T M e): bytes equal to the oracle's given the stored
+    flags, a different choice only inside the fp64 margin; M = diag(co) writes the pool the diagonal criterion writes
+    (up to choices inside the margin); ident ignores M"""
+    from flagrot_releaser_amd import kivi as KV
+    g = torch.Generator().manual_seed(13)
+    T, Hkv = 150, 3
+    kv = _kv(T, Hkv, g)
+    _, _, co = _calib(Hkv, 8, g)
+    A = torch.randn(Hkv, D, D, generator=g) * 0.2
+    M = (A @ A.transpose(1, 2) + torch.diag_embed(co)).contiguous()
+    npg = (T + 15) // 16 + 1
+    slots = torch.randperm(npg * 16, generator=g)[:T].long()
+    xb = bits(kv)[:, Hkv:]
+    for Mx, name in ((M, "dense"), (torch.diag_embed(co).contiguous(), "diagonal")):
+        pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
+        KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), Mx.to(dev), pool, Hkv, D, f8=f8)
+        torch.cuda.synchronize()
+        got = pool.cpu().numpy()
+        enc = OK.v_encode(xb, co.numpy(), f8=f8, M=Mx.numpy())
+        sH, sF = _stored_value_flags(got, f8)
+        sl = slots.numpy()
+        useH, useF = sH[sl // 16, :, sl % 16], sF[sl // 16, :, sl % 16]
+        want = np.zeros_like(got)
+        OK.pack_values(want, sl, *OK.v_stored(enc, useH, useF, f8=f8), f8=f8)
+        assert np.array_equal(got, want), name
+        badF = useF != enc["useF"]
+        badH = (useH != enc["useH"]) & ~useF[..., None] & ~enc["useF"][..., None]
+        assert (enc["marginF"][badF] < 1e-3).all() and (enc["marginH"][badH] < 1e-3).all(), name
+        assert badF.mean() < 0.02 and badH.mean() < 0.02
+        if name == "diagonal":
+            ref = torch.zeros_like(pool)
+            KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, ref, Hkv, D, f8=f8)
+            assert (ref != pool).any(dim=-1).float().mean().item() < 0.05
+        else:
+            dg = OK.v_encode(xb, co.numpy(), f8=f8)
+            assert (dg["useH"] != enc["useH"]).any()               # the dense matrix does change choices
+    pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
+    ref = torch.zeros_like(pool)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), M.to(dev), pool, Hkv, D, ident=True, f8=f8)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, ref, Hkv, D, ident=True, f8=f8)
+    assert torch.equal(pool, ref)
+
+
+@F8
 @pytest.mark.parametrize("mode", ["ident", "fix"])
 def test_v_write_pinned_modes(dev, mode, f8):
     from flagrot_releaser_amd import kivi as KV
@@ -328,9 +373,9 @@ def test_attn_without_tail_and_rejects(dev):
     assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
     with pytest.raises(RuntimeError, match="chunk"):
         KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 100, ws, 0.1, 0, G)
-    with pytest.raises(RuntimeError, match="M is not built"):
-        KV.v_write(torch.zeros(1, 2 * Hkv, D, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
-                   torch.ones(Hkv, D, device=dev), torch.ones(Hkv, D, D, device=dev), pool, Hkv, D)
+    with pytest.raises(RuntimeError, match="head dim"):
+        KV.v_write(torch.zeros(1, 2 * Hkv, 256, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
+                   torch.ones(Hkv, 256, device=dev), None, pool, Hkv, 256)
 
 
 @F8

@@ -125,3 +125,42 @@ def test_lse_merge_matches_single_softmax():
     full, _ = part(np.concatenate([s1, s2], -1), np.concatenate([v1, v2], -2))
     got = Q.bf16_to_f32(KV.lse_merge(Q.bf16_bits(oa.astype(F32)), la.astype(F32), Q.bf16_bits(ob.astype(F32)), lb.astype(F32)))
     assert np.abs(got - full).max() < 0.03
+
+
+def test_value_selection_with_matrix_weight():
+    """the M form of the value criterion: equals the diagonal form for M = diag(co); the quadratic forms agree with
+    explicit loops; a rotation-mixing M changes some choices"""
+    rng = np.random.default_rng(11)
+    T, H, D = 24, 2, 128
+    x = (rng.standard_normal((T, H, D)) * (0.3 + rng.random((H, D))) + rng.standard_normal((H, D))).astype(np.float32)
+    xb = Q.f32_to_bf16_bits(x) if hasattr(Q, "f32_to_bf16_bits") else (x.view(np.uint32) >> 16).astype(np.uint16)
+    co = (rng.random((H, D)) + 0.1).astype(np.float32)
+    base = KV.v_encode(xb, co)
+    Md = np.stack([np.diag(co[h]) for h in range(H)]).astype(np.float32)
+    same = KV.v_encode(xb, co, M=Md)
+    assert np.array_equal(base["useH"], same["useH"]) and np.array_equal(base["useF"], same["useF"])
+    assert np.allclose(base["marginH"], same["marginH"], rtol=1e-9, atol=1e-12)
+    A = rng.standard_normal((H, D, D)).astype(np.float32) * 0.2
+    M = (np.einsum("hik,hjk->hij", A, A) + Md).astype(np.float32)                   # SPD, couples the sub-vectors
+    enc = KV.v_encode(xb, co, M=M)
+    # brute force of one (token, head): reconstruct the three candidates' errors and evaluate the forms by loops
+    t, h = 5, 1
+    xf = Q.bf16_to_f32(xb)[t, h].astype(np.float64)
+    recs = []
+    for c in range(3):
+        codes = enc["codes"][c, t, h].reshape(4, 32).astype(np.float64)
+        y = (codes * enc["s"][c, t, h][:, None].astype(np.float64) + enc["mn"][c, t, h][:, None].astype(np.float64)).astype(np.float32)
+        y = y.reshape(D)
+        back = y if c == 0 else Q.fwht(y, 32 if c == 1 else D)
+        recs.append(back.astype(np.float64) - xf)
+    Mh = M[h].astype(np.float64)
+    quad = lambda e, lo, hi: sum(e[i] * Mh[i, k] * e[k] for i in range(lo, hi) for k in range(lo, hi))   # noqa: E731
+    eI = [quad(recs[0], 32 * j, 32 * j + 32) for j in range(4)]
+    eH = [quad(recs[1], 32 * j, 32 * j + 32) for j in range(4)]
+    uH = [eH[j] < eI[j] for j in range(4)]
+    assert uH == enc["useH"][t, h].tolist()
+    comb = np.concatenate([recs[1][32 * j:32 * j + 32] if uH[j] else recs[0][32 * j:32 * j + 32] for j in range(4)])
+    assert (quad(recs[2], 0, D) < quad(comb, 0, D)) == bool(enc["useF"][t, h])
+    assert (enc["useH"] != base["useH"]).any() or (enc["useF"] != base["useF"]).any()
+    # ident / fix ignore M
+    assert not KV.v_encode(xb, co, M=M, ident=True)["useH"].any()
