@@ -141,10 +141,10 @@ int fr_cb_write(const void* kv, long long kv_ts, const long long* slots, int slo
                 const float* kmu) {
   (void)tg; (void)co; (void)sg;
   if (T <= 0) return 0;
-  if (hd != 0 && hd != 128) return fail(-8, "fr_cb_write: head dim 128 only");
+  if (hd != 0 && hd != 128 && hd != 256) return fail(-8, "fr_cb_write: head dim 128 | 256");
   K2WriteParams p{};
   p.kv = kv; p.kv_ts = kv_ts; p.slots = slots; p.slot_ph = slot_ph; p.T = T; p.Hkv = Hkv; p.page = page;
-  p.CT = CT; p.kmu = kmu; p.pool = pool; p.passes = 3;
+  p.CT = CT; p.kmu = kmu; p.pool = pool; p.passes = 3; p.hd = hd == 256 ? 256 : 128;
   return launched(k2_write_launch(kind, p, static_cast<hipStream_t>(stream)), "fr_cb_write");
 }
 

@@ -23,11 +23,12 @@ struct K2WriteParams {
   const long long* slots;
   int slot_ph;
   int T, Hkv, page;
-  const float* CT;         // [Hkv, 128 (k), 128 (i)] = C_q[h][i][k]
+  const float* CT;         // [Hkv, hd (k), hd (i)] = C_q[h][i][k]
   const float* kmu;
   uint8_t* pool;
   int passes;              // bit 0: key rows, bit 1: value rows
   int screen;              // 1: large key passes may run the screened kernel (same bytes; fr_cb_write3)
+  int hd;                  // head dim: 0 | 128, or 256 (fr_cb_write only)
 };
 int k2_write_launch(int kind, const K2WriteParams& p, hipStream_t st);
 int k2_write_lds_bytes();

@@ -318,6 +318,182 @@ __global__ void __launch_bounds__(256) k_k2_write(const K2WriteParams p, int tok
 }
 
 
+// ------------------------------------------------------------------------------------------------ head dim 256
+// Selecting writer of the key-only kinds for 256-d heads (attn_codebook.cu:384-392, 432; codebook_ref.encode with
+// Dq = 256).  A half wave owns a (token, head): lane l holds dims 4 l + i of BOTH 128-d halves, so the transforms of a
+// half are the 128-d ones and H256 adds one stage between the two registers of a lane (distance 128) and the exact
+// factor 1/16.  The eight key 32-groups choose I / H32 by their diagonal block of C_q, the head chooses between that
+// combination and H256 by all of C_q (the eight column blocks folded left to right, every product and sum rounded on
+// its own: the order of codebook_ref.key_head_err).  C_q^T (256 KB per head) does not fit in LDS: its rows come from
+// L2; the error vectors sit in an LDS strip per half wave.  The page chunk is two 128-d half chunks, half s = dims
+// [128 s, 128 s + 128), each in the 128-d layout; H32 flag of group g = sign bit of its K scale word, H256 flag = sign
+// bit of the token's group-0 V scale word of half 0.  Values are quantised as they are.
+template <int QM>
+DEVI void h256(float (&y)[2][4], int l32) {
+  butterflies<128>(y[0], l32);
+  butterflies<128>(y[1], l32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a = y[0][i], b = y[1][i];
+    y[0][i] = (a + b) * 0.0625f;
+    y[1][i] = (a - b) * 0.0625f;
+  }
+}
+
+template <int QM, int P>
+__global__ void __launch_bounds__(256) k_k2_write256(const K2WriteParams p) {
+  using L = Lay<QM, P>;
+  __shared__ __align__(16) float strips[8][2][256];
+  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31, g = l32 >> 3;
+  const int h = blockIdx.x;
+  const long long t = static_cast<long long>(blockIdx.y) * 8 + hw;
+  if (t >= p.T) return;                                          // (no workgroup barrier below)
+  const long long slot = p.slots[t * (p.slot_ph ? p.Hkv : 1) + (p.slot_ph ? h : 0)];
+  if (slot < 0) return;
+  float (*es)[256] = strips[hw];
+  const float* CT = p.CT + static_cast<size_t>(h) * 256 * 256;   // CT[k][i] = C_q[i][k]
+  float x[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    load_row(p.kv, t * p.kv_ts + h * 256 + 128 * s + 4 * l32, x[s]);
+    if (p.kmu != nullptr) {
+      const float4 m = *reinterpret_cast<const float4*>(p.kmu + h * 256 + 128 * s + 4 * l32);
+      x[s][0] = x[s][0] - m.x; x[s][1] = x[s][1] - m.y; x[s][2] = x[s][2] - m.z; x[s][3] = x[s][3] - m.w;
+    }
+  }
+  // ---- local candidates of the eight groups: identity and H32
+  float qb[2][4], eb[2][4];
+  uint32_t wb[2];
+  bool use_h[2];
+  {
+    float qi[2][4], ei[2][4], qh[2][4], eh[2][4];
+    uint32_t wi[2], wh[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      float y[4];
+      wi[s] = quant_group<QM, true>(x[s], qi[s], ei[s]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { ei[s][i] = ei[s][i] - x[s][i]; y[i] = x[s][i]; }
+      fwht<32>(y, l32);
+      wh[s] = quant_group<QM, true>(y, qh[s], eh[s]);
+      fwht<32>(eh[s], l32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) eh[s][i] = eh[s][i] - x[s][i];
+      *reinterpret_cast<float4*>(&es[0][128 * s + 4 * l32]) = make_float4(ei[s][0], ei[s][1], ei[s][2], ei[s][3]);
+      *reinterpret_cast<float4*>(&es[1][128 * s + 4 * l32]) = make_float4(eh[s][0], eh[s][1], eh[s][2], eh[s][3]);
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int c0 = 128 * s + 32 * g;                           // first channel of this lane's group
+      const float* crow = CT + static_cast<size_t>(c0) * 256 + 128 * s + 4 * l32;
+      float ui[4], uh[4];
+#pragma unroll 4
+      for (int k = 0; k < 32; ++k) {
+        const float4 cv = *reinterpret_cast<const float4*>(crow + static_cast<size_t>(k) * 256);
+        const float a = es[0][c0 + k], b = es[1][c0 + k];
+        const float c[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pa = c[i] * a, pb = c[i] * b;
+          ui[i] = k == 0 ? pa : ui[i] + pa;
+          uh[i] = k == 0 ? pb : uh[i] + pb;
+        }
+      }
+      float pi[4], ph[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { pi[i] = ei[s][i] * ui[i]; ph[i] = eh[s][i] * uh[i]; }
+      use_h[s] = tree32(ph) < tree32(pi);                        // strict: ties keep the identity
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { qb[s][i] = use_h[s] ? qh[s][i] : qi[s][i]; eb[s][i] = use_h[s] ? eh[s][i] : ei[s][i]; }
+      wb[s] = use_h[s] ? wh[s] : wi[s];
+    }
+  }
+  // ---- whole-head candidate: H256
+  float qf[2][4], ef[2][4];
+  uint32_t wf[2];
+  {
+    float y[2][4];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[s][i] = x[s][i];
+    h256<QM>(y, l32);
+    wf[0] = quant_group<QM, true>(y[0], qf[0], ef[0]);
+    wf[1] = quant_group<QM, true>(y[1], qf[1], ef[1]);
+    h256<QM>(ef, l32);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ef[s][i] = ef[s][i] - x[s][i];
+  }
+  wave_lds_sync();                                               // the local pass has read its strips
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    *reinterpret_cast<float4*>(&es[0][128 * s + 4 * l32]) = make_float4(eb[s][0], eb[s][1], eb[s][2], eb[s][3]);
+    *reinterpret_cast<float4*>(&es[1][128 * s + 4 * l32]) = make_float4(ef[s][0], ef[s][1], ef[s][2], ef[s][3]);
+  }
+  wave_lds_sync();
+  float tb[2][4], tf[2][4];
+#pragma unroll 1
+  for (int b = 0; b < 8; ++b) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      float ub[4], uf[4];
+      const float* crow = CT + static_cast<size_t>(32 * b) * 256 + 128 * s + 4 * l32;
+#pragma unroll 4
+      for (int k = 0; k < 32; ++k) {
+        const float4 cv = *reinterpret_cast<const float4*>(crow + static_cast<size_t>(k) * 256);
+        const float a = es[0][32 * b + k], f = es[1][32 * b + k];
+        const float c[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pa = c[i] * a, pf = c[i] * f;
+          ub[i] = k == 0 ? pa : ub[i] + pa;
+          uf[i] = k == 0 ? pf : uf[i] + pf;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        tb[s][i] = b == 0 ? ub[i] : tb[s][i] + ub[i];
+        tf[s][i] = b == 0 ? uf[i] : tf[s][i] + uf[i];
+      }
+    }
+  }
+  bool key_full;
+  {
+    // halving tree of 256 products: dims d and d + 128 first (the two registers of a lane), then the 128-tree
+    float pb[4], pf[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pb[i] = eb[0][i] * tb[0][i] + eb[1][i] * tb[1][i];
+      pf[i] = ef[0][i] * tf[0][i] + ef[1][i] * tf[1][i];
+    }
+    key_full = tree128(pf) < tree128(pb);
+  }
+  const int pos = static_cast<int>(slot % P);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    uint8_t* chunk = p.pool + ((slot / P) * (2 * p.Hkv) + 2 * h + s) * L::CHUNK;
+    uint32_t code[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) code[i] = code_bits(key_full ? qf[s][i] : qb[s][i], QM == QM_SYM4);
+    uint32_t word = key_full ? wf[s] : wb[s];
+    if (!key_full && use_h[s]) word |= 0x8000u;
+    store_row<QM, P>(chunk, pos, false, code, word, l32, false);
+    // the value half row, as it is
+    float v[4], q[4], deq[4];
+    load_row(p.kv, t * p.kv_ts + (p.Hkv + h) * 256 + 128 * s + 4 * l32, v);
+    uint32_t vword = quant_group<QM, false>(v, q, deq);
+    if (s == 0 && g == 0 && key_full) vword |= 0x8000u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) code[i] = code_bits(q[i], QM == QM_SYM4);
+    store_v_word<QM, P>(chunk, pos, vword, l32, false);
+    store_v_codes<QM, P>(chunk, pos, code, l32);
+  }
+}
+
+
 // Low-latency form of k_k2_write for a handful of tokens (a decode step): four half waves per (token, head) instead of
 // one, two tokens per workgroup.  Every half wave repeats the cheap part (quantised candidates, transforms); the
 // weighted error sums are shared out without touching the order of any sum: in the local pass half wave r carries the
@@ -949,6 +1125,14 @@ int k2_write_p(const K2WriteParams& p, hipStream_t st) {
 }
 template <int QM>
 int k2_write_qm(const K2WriteParams& p, hipStream_t st) {
+  if (p.hd == 256) {
+    if (p.passes != 3) return -8;                          // the two-pass forms exist for 128-d heads only
+    const dim3 grid(p.Hkv, (p.T + 7) / 8);
+    if (p.page == 16) hipLaunchKernelGGL((k_k2_write256<QM, 16>), grid, dim3(256), 0, st, p);
+    else if (p.page == 32) hipLaunchKernelGGL((k_k2_write256<QM, 32>), grid, dim3(256), 0, st, p);
+    else return -5;
+    return hipPeekAtLastError() == hipSuccess ? 0 : -1;
+  }
   if (p.page == 16) return k2_write_p<QM, 16>(p, st);
   if (p.page == 32) return k2_write_p<QM, 32>(p, st);
   return -5;

@@ -51,8 +51,10 @@ int fr_v2_chunk_bytes(int fmt, int page);
 /* flagrot_capi.cu:84 -- == 15 (rows of the sign table `sg`; unused by the key-only kinds) */
 int fr_cb_nsg(void);
 
-/* flagrot_capi.cu:86-98.  Selecting writer.  CT fp32 [Hkv, 128, 128] = C_q transposed; co fp32 [Hkv, 128] (unused by
- * the key-only kinds: values carry no transform); sg uint32 [15*4] (unused); tg: scheduling hint (ignored). */
+/* flagrot_capi.cu:86-98.  Selecting writer.  CT fp32 [Hkv, hd, hd] = C_q transposed; co fp32 [Hkv, hd] (unused by
+ * the key-only kinds: values carry no transform); sg uint32 [15*4] (unused); tg: scheduling hint (ignored).
+ * hd 0 | 128, or 256 (kernels/csrc/attn_codebook.cu:384-392, 432: eight key groups, whole-head H256, the page chunk two
+ * 128-d half chunks, the H256 flag in the group-0 V scale word of half 0). */
 int fr_cb_write(const void* kv, long long kv_ts, const long long* slots, int slot_ph, int T, int Hkv, int page, int tg,
                 const float* CT, const float* co, const unsigned* sg, int kind, uint8_t* pool, void* stream, int hd,
                 const float* kmu);

@@ -2,10 +2,12 @@
 inputs.  Only data is stored (inputs and the reference's outputs): nothing of the reference's source travels.
 
 Run once in the build container (the reference tree does not exist anywhere else):
-    python tests/golden/make_golden.py [/root/reference] [k2|pages|static|kivi_layout|kivi_select ...]
+    python tests/golden/make_golden.py [/root/reference] [k2|k2d256|pages|static|kivi_layout|kivi_select ...]
 
 Files and the reference functions that wrote them:
   k2_encode_<kind>.npz     kernels/codebook_ref.encode                                     (selecting writer, below)
+  k2_encode_d256_<kind>.npz  the same at head dim 256 (eight 32-groups, whole-head H256; 24 tokens, one dense SPD C_q
+                           [Hkv, 256, 256]; konly and konlya)
   pages_<fmt>_p<P>.npz     vllm_flagrot/kernels.py parse_pages / dequant_v2_pages / dequant_cb_pages on a pool of random
                            bytes into which oracle.pages.pack_tokens has packed seeded tokens (six formats x pages of 16
                            and 32 tokens): pins the oracle's parser on arbitrary bytes and its packer through the
@@ -85,6 +87,38 @@ def write_k2():
             kmode=k["mode"].numpy().astype(np.uint8), kherr=k["head_errs"].numpy(),
             vq=v["q"].numpy(), vs=v["s"].numpy(), vmode=v["mode"].numpy().astype(np.uint8))
         print(kind, "local H32 fraction", float(k["local"].float().mean()), "F fraction",
+              float((k["mode"] == 2).float().mean()))
+
+
+def write_k2_d256():
+    import codebook_ref as CR
+
+    for n, kind in enumerate(("konly", "konlya")):
+        g = torch.Generator().manual_seed(300 + n)
+        Tn, Dn = 24, 256
+        x = torch.randn(Tn, 2 * HKV, Dn, generator=g)
+        for h in range(HKV):
+            x[:, h, torch.randint(0, Dn, (6,), generator=g)] *= 6
+        x = x * (0.5 + torch.rand(Tn, 1, 1, generator=g))
+        x[0, :, 0:32] = x[0, :, 0:32].abs() + 0.1
+        x[1, :, 160:192] *= 300.0
+        x[2, :, 224:256] = 0.0
+        x[3] = 0.0
+        x = x.bfloat16()
+        qs = torch.randn(HKV, 512, Dn, generator=g)
+        qs[:, :, :8] *= 4
+        qs[:, :, 130:136] *= 3
+        C = torch.einsum("hnd,hne->hde", qs, qs).contiguous()
+        co = torch.rand(HKV, Dn, generator=g) + 0.1
+        k = CR.encode(x[:, :HKV], C, co, "k", cfg=kind, qk=QK[kind])
+        v = CR.encode(x[:, HKV:], C, co, "v", cfg=kind, qk=QK[kind])
+        np.savez_compressed(
+            OUT / f"k2_encode_d256_{kind}.npz",
+            x_bits=x.view(torch.int16).numpy().view(np.uint16), C=C.numpy(), co=co.numpy(),
+            kq=k["q"].numpy(), ks=k["s"].numpy(), klocal=k["local"].numpy().astype(np.uint8),
+            kmode=k["mode"].numpy().astype(np.uint8), kherr=k["head_errs"].numpy(),
+            vq=v["q"].numpy(), vs=v["s"].numpy(), vmode=v["mode"].numpy().astype(np.uint8))
+        print(kind, "D=256 local H32 fraction", float(k["local"].float().mean()), "F fraction",
               float((k["mode"] == 2).float().mean()))
 
 
@@ -247,7 +281,7 @@ def write_kivi_select():
     np.savez_compressed(OUT / "kivi_select.npz", **out)
 
 
-WRITERS = {"k2": write_k2, "pages": write_pages, "static": write_static, "kivi_layout": write_kivi_layout,
+WRITERS = {"k2": write_k2, "k2d256": write_k2_d256, "pages": write_pages, "static": write_static, "kivi_layout": write_kivi_layout,
            "kivi_select": write_kivi_select}
 
 

@@ -265,6 +265,47 @@ def test_static_writer_head_dim_256(dev):
     assert np.array_equal(dpool.cpu().numpy().reshape(want.shape), want)
 
 
+@pytest.mark.parametrize("kind,P", [("konly", 16), ("konlya", 16), ("konlya2", 16), ("konlya", 32)])
+def test_selecting_writer_head_dim_256(dev, kind, P):
+    """fr_cb_write at head dim 256 (eight key groups, whole-head H256, C_q [Hkv, 256, 256]; two 128-d half chunks per
+    (page, head); attn_codebook.cu:384-392,432): whole-pool bytes against the oracle (which reproduces the reference's
+    own encoder at this head dim bit for bit, tests/golden/k2_encode_d256_*.npz), garbage pool, holes, centring"""
+    from flagrot_releaser_amd import kernels as K
+    g = torch.Generator().manual_seed(900 + len(kind) + P)
+    Hkv, T, Dh = 2, 75, 256
+    npg = T // P + 3
+    cb = PG.chunk_bytes(kind, P)
+    pool = torch.randint(0, 256, (npg, Hkv, 2 * cb), dtype=torch.uint8, generator=g)
+    kv = torch.randn(T, 2 * Hkv, Dh, generator=g)
+    kv[:, :Hkv, 7] *= 6
+    kv[:, :Hkv, 200] *= 5
+    kv = (kv * (0.5 + torch.rand(T, 1, 1, generator=g)))
+    kv[3, :, 32:64] *= 300.0
+    kv[4] = 0.0
+    kv[5, :, 128:160] = 1.25
+    kv = kv.bfloat16()
+    qs = torch.randn(Hkv, 512, Dh, generator=g)
+    qs[:, :, :8] *= 4
+    Cq = torch.einsum("hnd,hne->hde", qs, qs).contiguous()
+    co = torch.rand(Hkv, Dh, generator=g) + 0.1
+    kmu = torch.randn(Hkv, Dh, generator=g) * 0.5
+    slots = torch.randperm(npg * P, generator=g)[:T].long()
+    slots[11] = -1
+    for use_mu in (False, True):
+        dpool = pool.to(dev)
+        K.cb_write(kv.to(dev), slots.to(dev), Cq.transpose(1, 2).contiguous().to(dev), co.to(dev), kind, dpool, P,
+                   kmu=kmu.to(dev) if use_mu else None)
+        torch.cuda.synchronize()
+        codes, words, info = Q.k2_encode(bits(kv), Cq.numpy(), kind, kmu.numpy() if use_mu else None)
+        want = pool.numpy().copy().reshape(npg, 2 * Hkv, cb)
+        PG.pack_tokens(want, slots.numpy(), codes.reshape(T, 4 * Hkv, 128), words.reshape(T, 4 * Hkv, 4), kind, P)
+        assert np.array_equal(dpool.cpu().numpy().reshape(want.shape), want), (kind, P, use_mu)
+        assert info["full"].any() and (~info["full"]).any() and info["local"].any()
+    # the two-pass writer has no 256-d form
+    with pytest.raises(AssertionError, match="head dim"):
+        K.cb_write3(kv.to(dev), slots.to(dev), Cq.to(dev), co.to(dev), None, None, kind, pool.to(dev), P)
+
+
 def test_centring_exact_grid_all_writers(dev):
     """writer(k, kmu) == writer(bf16(k - mu)) byte for byte when k and mu sit on a 2^-6 grid."""
     from flagrot_releaser_amd import kernels as K

@@ -27,6 +27,25 @@ def test_k2_encode_matches_reference_vectors(kind):
     assert info["local"].any() and info["full"].any() and (~info["full"]).any()
 
 
+@pytest.mark.parametrize("kind", ["konly", "konlya"])
+def test_k2_encode_head_dim_256_matches_reference_vectors(kind):
+    """codebook_ref.encode at Dq = 256: eight 32-groups, whole-head H256, head error over eight column blocks"""
+    g = np.load(os.path.join(GOLD, f"k2_encode_d256_{kind}.npz"))
+    Hkv = g["C"].shape[0]
+    assert g["x_bits"].shape[-1] == 256
+    codes, words, info = Q.k2_encode(g["x_bits"], g["C"], kind, true_div=True)
+    assert np.array_equal(codes[:, :Hkv], g["kq"]) and np.array_equal(codes[:, Hkv:], g["vq"])
+    assert np.array_equal(Q.word_scale(words[:, :Hkv]), g["ks"]) and np.array_equal(Q.word_scale(words[:, Hkv:]), g["vs"])
+    assert np.array_equal(info["local"], g["klocal"])
+    assert np.array_equal(info["full"].astype(np.uint8) * 2, g["kmode"])
+    assert np.array_equal(info["err_head"], g["kherr"])
+    assert info["local"].any() and info["full"].any() and (~info["full"]).any()
+    # flags: H32 bit of group g in K word g, H256 bit in V word 0
+    kw, vw = words[:, :Hkv], words[:, Hkv:]
+    assert np.array_equal((kw >> 15) & 1, info["local"].astype(np.int64))
+    assert np.array_equal((vw[..., 0] >> 15) & 1, info["full"].astype(np.int64)) and not ((vw[..., 1:] >> 15) & 1).any()
+
+
 @pytest.mark.parametrize("kind", ["konlya", "konlya2"])
 def test_kernel_form_differs_only_in_the_step(kind):
     """true_div=False (reciprocal multiply, the kernels' form) may move a step by one ulp: stored scale words stay
