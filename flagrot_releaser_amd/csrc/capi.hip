@@ -66,7 +66,7 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
                int gqa, int kv_start) {
   if (B <= 0) return 0;
   if (fmt < FMT_INT4 || fmt > FMT_KONLYA2) return fail(-4, "fr_v2_attn: unknown format");
-  if (variant & HD256) return fail(-8, "fr_v2_attn: head dim 256 is not built");
+  if ((variant & HD256) && (variant & GT8)) return fail(-3, "fr_v2_attn: head dim 256 takes q tiles of 4 heads");
   if ((variant & ~(GEN | GT8 | HD256)) != 264 && (variant & ~(GEN | GT8 | HD256)) != 0)
     return fail(-3, "fr_v2_attn: unsupported variant");
   if (stages < 1 || stages > 8) return fail(-3, "fr_v2_attn: unsupported stages");
@@ -106,6 +106,7 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   const bool can_draw = !force_static && counter != nullptr && p.counter_div == 1 && nparts <= 1023;
   p.wg_waves = big ? decode_waves(1 << 30) : 4;
   p.dyn = (can_draw && (!big || env_waves > 4)) ? 1 : 0;
+  if (variant & HD256) return launched(decode_wide_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_attn (head dim 256)");
   return launched(decode_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_attn");
 }
 

@@ -64,6 +64,7 @@ struct DecodeParams {
   int wg_waves;            // wavefronts per workgroup: 4, or the large workgroup that fills a CU
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
+int decode_wide_launch(int fmt, const DecodeParams& p, hipStream_t st);   // head dim 256 (decode_wide.hip)
 int decode_occupancy(int fmt, int waves);   // resident workgroups per CU of the 4- or 16-wavefront kernel
 int decode_big_chunk();                     // tokens per split from which the large workgroup is worth launching
 int decode_waves(int chunk_tokens);          // wavefronts per workgroup the launcher picks for a split of that many tokens

@@ -20,38 +20,50 @@ from . import pages as PG
 from . import quant as Q
 
 
-def dequant_pages(pool: np.ndarray, fmt: str, page: int, dtype=np.float64):
-    """pool uint8 [Np, Hkv, CHUNK] -> K, V [Np, P, Hkv, 128].
+def dequant_pages(pool: np.ndarray, fmt: str, page: int, dtype=np.float64, Dh: int = 128):
+    """pool uint8 [Np, Hkv, CHUNK] -> K, V [Np, P, Hkv, Dh].
     static formats (int4 / int4a / int2a): values in the STORED (rotated) basis;
     key-only kinds (konly / konlya / konlya2): keys in the ORIGINAL basis (inverse transform per flag bits), values as
-    stored (they carry no transform)."""
-    codes, words = PG.parse_pages(pool, fmt, page)
+    stored (they carry no transform).
+    Dh = 256 (vllm_flagrot/kernels.py:598-603, 662-667): the chunk is two 128-d half chunks, half s = dims
+    [128 s, 128 s + 128), each in the 128-d layout; key flags: H32 of group g (0..7) in its K scale word, whole-head
+    H256 in the token's group-0 V scale word of half 0."""
+    ng = Dh // 32
+    if Dh == 256:
+        Np, H, CB2 = pool.shape
+        halves = pool.reshape(Np, 2 * H, CB2 // 2)                                # half chunks as heads 2 h + s
+        codes, words = PG.parse_pages(halves, fmt, page)                          # [Np, 2 H, P, 2, 128], [.., 2, 4]
+        join = lambda a: np.moveaxis(a.reshape(Np, H, 2, *a.shape[2:]), 2, 4).reshape(Np, H, *a.shape[2:4], -1)  # noqa: E731
+        codes, words = join(codes), join(words)                                   # [Np, H, P, 2, 256], [.., 2, 8]
+    else:
+        assert Dh == 128
+        codes, words = PG.parse_pages(pool, fmt, page)
     qk = Q.QK_OF_KIND[fmt]
-    c = codes.astype(dtype)                                                       # [Np, H, P, 2, 128]
+    c = codes.astype(dtype)                                                       # [Np, H, P, 2, Dh]
     w = words.astype(np.int64)
     if qk != "sym":
         zmask = 15 if qk == "asym4" else 3
         c = c - np.repeat(w & zmask, 32, -1).astype(dtype)
     mag = Q.word_scale(w).astype(dtype)
-    x = (c.reshape(*c.shape[:-1], 4, 32) * mag[..., None])                        # [Np, H, P, 2, 4, 32]
+    x = (c.reshape(*c.shape[:-1], ng, 32) * mag[..., None])                       # [Np, H, P, 2, ng, 32]
     k, v = x[..., 0, :, :], x[..., 1, :, :]
     if fmt in ("konly", "konlya", "konlya2"):
-        flag_h = ((w[..., 0, :] >> 15) & 1).astype(bool)                          # [Np, H, P, 4]
+        flag_h = ((w[..., 0, :] >> 15) & 1).astype(bool)                          # [Np, H, P, ng]
         flag_f = ((w[..., 1, 0] >> 15) & 1).astype(bool)                          # [Np, H, P]
-        H32, H128 = Q.sylvester(32).astype(dtype), Q.sylvester(128).astype(dtype)
-        kl = np.where(flag_h[..., None], k @ H32, k).reshape(*k.shape[:-2], 128)
-        kf = k.reshape(*k.shape[:-2], 128) @ H128
+        H32, HD = Q.sylvester(32).astype(dtype), Q.sylvester(Dh).astype(dtype)
+        kl = np.where(flag_h[..., None], k @ H32, k).reshape(*k.shape[:-2], Dh)
+        kf = k.reshape(*k.shape[:-2], Dh) @ HD
         k = np.where(flag_f[..., None], kf, kl)
     else:
-        k = k.reshape(*k.shape[:-2], 128)
-    v = v.reshape(*v.shape[:-2], 128)
+        k = k.reshape(*k.shape[:-2], Dh)
+    v = v.reshape(*v.shape[:-2], Dh)
     return np.swapaxes(k, 1, 2), np.swapaxes(v, 1, 2)
 
 
 def rot_blocks(x: np.ndarray, mask: np.ndarray) -> np.ndarray:
-    """x [..., H, 128] fp64; mask [H, 4]: orthonormal H32 on flagged 32-blocks (its own inverse)."""
+    """x [..., H, Dh] fp64; mask [H, Dh / 32]: orthonormal H32 on flagged 32-blocks (its own inverse)."""
     H32 = Q.sylvester(32)
-    xb = x.reshape(*x.shape[:-1], 4, 32)
+    xb = x.reshape(*x.shape[:-1], x.shape[-1] // 32, 32)
     return np.where(np.asarray(mask).astype(bool)[..., None], xb @ H32, xb).reshape(x.shape)
 
 
@@ -92,14 +104,14 @@ def gather_cache(Kp: np.ndarray, Vp: np.ndarray, block_table: np.ndarray, Lmax: 
 
 def decode_reference(q_bits, pool, fmt, page, block_table, lens, scale, kmask=None, vmask=None, tail=None,
                      tail_len=None, tail_idx=None, kv_start=0):
-    """the full oracle of one decode launch: q_bits uint16 [B, Hq, 128] bf16 patterns; tail uint16
-    [R, W, 2*Hkv, 128] bf16 patterns (original basis).  Static formats: q is rotated by kmask, tails by kmask / vmask,
-    and the result is rotated back by vmask.  Returns fp64 [B, Hq, 128]."""
+    """the full oracle of one decode launch: q_bits uint16 [B, Hq, Dh] bf16 patterns (Dh 128 | 256); tail uint16
+    [R, W, 2*Hkv, Dh] bf16 patterns (original basis).  Static formats: q is rotated by kmask, tails by kmask / vmask,
+    and the result is rotated back by vmask.  Returns fp64 [B, Hq, Dh]."""
     q = Q.bf16_to_f32(q_bits).astype(np.float64)
     B, Hq, Dh = q.shape
     Hkv = pool.shape[1]
     G = Hq // Hkv
-    Kp, Vp = dequant_pages(pool, fmt, page)
+    Kp, Vp = dequant_pages(pool, fmt, page, Dh=Dh)
     Lmax = max(int(max(lens)) if len(lens) else 1, 1)
     Kc, Vc = gather_cache(Kp, Vp, block_table, Lmax, page)
     tails = None

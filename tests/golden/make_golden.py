@@ -2,7 +2,7 @@
 inputs.  Only data is stored (inputs and the reference's outputs): nothing of the reference's source travels.
 
 Run once in the build container (the reference tree does not exist anywhere else):
-    python tests/golden/make_golden.py [/root/reference] [k2|k2d256|pages|static|kivi_layout|kivi_select ...]
+    python tests/golden/make_golden.py [/root/reference] [k2|k2d256|pages|pages256|static|kivi_layout|kivi_select ...]
 
 Files and the reference functions that wrote them:
   k2_encode_<kind>.npz     kernels/codebook_ref.encode                                     (selecting writer, below)
@@ -12,6 +12,8 @@ Files and the reference functions that wrote them:
                            bytes into which oracle.pages.pack_tokens has packed seeded tokens (six formats x pages of 16
                            and 32 tokens): pins the oracle's parser on arbitrary bytes and its packer through the
                            reference's parser
+  pages_d256.npz           vllm_flagrot/kernels.py dequant_v2_pages / dequant_cb_pages with Dh = 256 on random chunk bytes
+                           (two 128-d half chunks per page and head; six formats, 16-token pages)
   static_writer.npz        kernels/ref.py kv_selrot_quant(fmt="int4") and int4a_quant (and formats.quant_asym_dep with
                            2 bits + scale_word_b for int2a) on seeded rows with a random rotation mask
   kivi_layout.npz          vllm_flagrot/kivi.py _kcodes / _codes / parse_chunks / dequant_groups on random chunk bytes
@@ -164,6 +166,32 @@ def write_pages():
             print("pages", fmt, P, tuple(c.shape), tuple(k.shape))
 
 
+def write_pages_d256():
+    """head dim 256 (two 128-d half chunks per page and head): the reference's parsers on random chunk bytes"""
+    from vllm_flagrot import kernels as RK
+    PG, _ = _here_oracle()
+    out = {}
+    for n, fmt in enumerate(("int4", "int4a", "int2a", "konly", "konlya", "konlya2")):
+        rng = np.random.default_rng(4000 + n)
+        P, Np, H = 16, 2, 2
+        pool = rng.integers(0, 256, (Np, H, 2 * PG.chunk_bytes(fmt, P)), dtype=np.uint8)
+        # keep every scale word's FP16 exponent finite (random bytes would make infinities / NaNs)
+        half = PG.chunk_bytes(fmt, P)
+        for s0 in (0, half):
+            sw = pool[..., s0 + half - 16 * P:s0 + half].view(np.uint16)
+            sw &= np.uint16(0xBBFF)
+        ch = torch.from_numpy(pool.copy())
+        if fmt in QK:
+            k, v = RK.dequant_cb_pages(ch, P, fmt, dtype=torch.float32, Dh=256)
+        else:
+            k, v = RK.dequant_v2_pages(ch, P, dtype=torch.float32, fmt=fmt, Dh=256)
+        out[f"{fmt}_pool"] = pool
+        out[f"{fmt}_k"] = k.contiguous().numpy()
+        out[f"{fmt}_v"] = v.contiguous().numpy()
+        print("pages d256", fmt, tuple(k.shape))
+    np.savez_compressed(OUT / "pages_d256.npz", **out)
+
+
 # ------------------------------------------------------------------------------------------------ static writers
 def write_static():
     import ref as R
@@ -281,7 +309,7 @@ def write_kivi_select():
     np.savez_compressed(OUT / "kivi_select.npz", **out)
 
 
-WRITERS = {"k2": write_k2, "k2d256": write_k2_d256, "pages": write_pages, "static": write_static, "kivi_layout": write_kivi_layout,
+WRITERS = {"k2": write_k2, "k2d256": write_k2_d256, "pages": write_pages, "pages256": write_pages_d256, "static": write_static, "kivi_layout": write_kivi_layout,
            "kivi_select": write_kivi_select}
 
 

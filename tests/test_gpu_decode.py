@@ -200,3 +200,72 @@ def test_decode_error_codes(dev):
     assert L.fr_cb_attn(zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, K.sign_words(), 3, 0, 4, zp, zp, zp, zp, 512, None,
                         None, None, 0, 0, None, 0) == -4
     assert L.fr_v2_attn(5, *(base[:6] + [0] + base[7:]), 4, 0) == 0     # B = 0: nothing to do
+
+
+@pytest.mark.parametrize("fmt", ["konly", "konlya", "konlya2", "int4", "int4a", "int2a"])
+@pytest.mark.parametrize("P", [16, 32])
+def test_head_dim_256(dev, fmt, P):
+    """head dim 256 (`variant | 4096`; the reference's shape (G, D, Hkv) = (6, 256, 4), test_kernels.py:366-374): pages
+    of two 128-d half chunks written by the 256-d writers, q tiles of 4 + 2 heads, splits, BF16 window rows, kv_start,
+    ragged lengths; against the oracle's dequantise-then-attend at that head dim, element-wise bar."""
+    from flagrot_releaser_amd import kernels as K
+    Dh, G, Hkv = 256, 6, 4
+    static = fmt in ("int4", "int4a", "int2a")
+    g = torch.Generator().manual_seed(600 + len(fmt) + P)
+    lens = [1, 17, 64, 65, 333, 700, 0]
+    B, HQ = len(lens), G * Hkv
+    num_pages = sum((n + P - 1) // P for n in lens) + 5
+    pool = torch.randint(0, 256, (num_pages, Hkv, 2 * PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g).to(dev)
+    bt = alloc_tables(lens, num_pages, g, P)
+    mask = (torch.rand(2 * Hkv, 8, generator=g) < 0.5).to(torch.uint8)
+    qs = torch.randn(Hkv, 384, Dh, generator=g)
+    qs[:, :, :8] *= 4
+    CT = torch.einsum("hnd,hne->hde", qs, qs).transpose(1, 2).contiguous().to(dev)
+    co = torch.ones(Hkv, Dh, device=dev)
+    for b, n in enumerate(lens):
+        if n == 0:
+            continue
+        kv = torch.randn(n, 2 * Hkv, Dh, generator=g)
+        kv[:, :Hkv, 9] *= 6
+        kv[:, :Hkv, 130] *= 5
+        kv[:, :Hkv] *= (0.5 + torch.rand(n, 1, 1, generator=g))
+        kv = kv.bfloat16().to(dev)
+        sl = slots_of(bt, b, n, P).to(dev)
+        if static:
+            K.v2_write(kv, sl, mask.to(dev), 32, pool, P, fmt=fmt)
+        else:
+            K.cb_write(kv, sl, CT, co, fmt, pool, P)
+    q = (torch.randn(B, HQ, Dh, generator=g) * 0.8).bfloat16()
+    scale = 1 / math.sqrt(Dh)
+    W, R, kv_start = 20, B + 1, 3
+    tail = torch.randn(R, W, 2 * Hkv, Dh, generator=g).bfloat16()
+    tail_idx = torch.randperm(R, generator=g)[:B].int()
+    tail_len = torch.randint(0, W + 1, (B,), generator=g).int()
+    tail_len[-1] = 0                                   # the empty sequence has no window rows either: output 0
+    seq = torch.tensor(lens, dtype=torch.int32)
+    ref = A.decode_reference(bits(q), pool.cpu().numpy(), fmt, P, bt.numpy(), lens, scale,
+                             kmask=mask[:Hkv].numpy() if static else None, vmask=mask[Hkv:].numpy() if static else None,
+                             tail=bits(tail), tail_len=tail_len.numpy(), tail_idx=tail_idx.numpy(), kv_start=kv_start)
+    dt = tail.to(dev)
+    tkw = dict(tail=dt, tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), tail_bs=dt.stride(0), tail_ts=dt.stride(1))
+    for nsplit in (1, 3):
+        ns, ch = (K.plan_v2 if static else K.plan_cb)(B, max(lens), Hkv, P, *((fmt,) if not static else ()), nsplit=nsplit,
+                                                     **({"fmt": fmt} if static else {}), G=G, Dh=Dh)
+        HV, GT = K.vheads(Hkv, G, Dh, fmt), K.tile_of(K.v2_variant(fmt, G, Dh))
+        assert (HV, GT) == (2 * Hkv, 4)
+        ws = K.Workspace(B, HV, B * HV * (ns + 1), dev, GT, Dh)
+        out = torch.full((B, HQ * Dh), float("nan"), dtype=torch.bfloat16, device=dev)
+        if static:
+            K.v2_attn(q.to(dev), pool, bt.to(dev), seq.to(dev), out, ns, ch, ws, scale * LOG2E, kmask=mask[:Hkv].to(dev),
+                      vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, page=P, **tkw)
+        else:
+            K.cb_attn(q.to(dev), pool, bt.to(dev), seq.to(dev), out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start,
+                      page=P, **tkw)
+        torch.cuda.synchronize()
+        got = out.view(B, HQ, Dh).float().cpu().numpy().astype(np.float64)
+        assert not np.isnan(got).any()
+        strict = np.abs(got - ref) / (ATOL + RTOL * np.abs(ref))
+        print(f"\n{fmt} P={P} D=256 G={G} ns={ns}: worst |err| / (2e-3 + 1e-2 |ref|) = {strict.max():.3f}", flush=True)
+        assert strict.max() <= 1.0, (fmt, P, ns, np.unravel_index(np.argmax(strict), strict.shape))
+        assert not got[-1].any()
+        assert int(ws.counter.abs().sum()) == 0

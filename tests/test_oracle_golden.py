@@ -224,3 +224,16 @@ def test_kivi_selection_matches_simulator(f8):
     r = _rel_groups(rec, g[f"{tag}_v_rec"].astype(np.float64), xvf, (2,))
     assert int((r > 0.2).sum()) <= max(1, r.size // 200), int((r > 0.2).sum())
     assert np.median(r) < (1e-4 if f8 else 5e-3), np.median(r)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_page_dequantiser_head_dim_256_matches_reference(fmt):
+    """vllm_flagrot/kernels.py dequant_v2_pages / dequant_cb_pages with Dh = 256 on random chunk bytes: two 128-d half
+    chunks per (page, head), eight key groups, the whole-head H256 flag in the group-0 V scale word of half 0"""
+    g = np.load(os.path.join(GOLD, "pages_d256.npz"))
+    pool = g[f"{fmt}_pool"]
+    K, V = A.dequant_pages(pool, fmt, 16, dtype=np.float64, Dh=256)
+    for a, ref in ((K, g[f"{fmt}_k"]), (V, g[f"{fmt}_v"])):
+        assert a.shape == ref.shape == (2, 16, 2, 256)
+        assert np.isfinite(ref).all()
+        assert np.abs(a - ref).max() <= 3e-6 * np.abs(ref).max(), fmt          # the reference multiplies in fp32
