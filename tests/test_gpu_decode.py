@@ -195,8 +195,8 @@ def test_decode_error_codes(dev):
     bad_page = list(base); bad_page[8] = 64
     assert L.fr_v2_attn(5, *bad_page, 4, 0) == -5
     assert L.fr_v2_attn(5, *base, 8, 0) == -7            # gqa 8 without the generalised variant bits
-    hd = list(base); hd[17] = 264 | 1024 | 4096
-    assert L.fr_v2_attn(5, *hd, 4, 0) == -8
+    hd = list(base); hd[17] = 264 | 1024 | 2048 | 4096
+    assert L.fr_v2_attn(5, *hd, 4, 0) == -3              # head dim 256 takes q tiles of 4 heads, not 8
     assert L.fr_cb_attn(zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, K.sign_words(), 3, 0, 4, zp, zp, zp, zp, 512, None,
                         None, None, 0, 0, None, 0) == -4
     assert L.fr_v2_attn(5, *(base[:6] + [0] + base[7:]), 4, 0) == 0     # B = 0: nothing to do
