@@ -4,13 +4,21 @@
 // Workgroup = 4 wavefronts per (sequence, KV head with its whole GQA group of up to 8 query heads, split); a wavefront
 // owns whole 32-token groups (two pages) and keeps its own running maxima, sums and accumulators; the wavefronts are
 // merged through LDS at the end.  Per group:
-//   q' * scale   lane = channel pair: the group's channel scales (and mins) times the query rotation the group's flags
-//                select (identity / H32 per sub-vector / H128; the three rotations are made once per workgroup and
-//                kept as fp16 pairs), packed fp16 products written to LDS strips.
-//   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads, 128 channels in four steps:
-//                a 2-bit code field masked in place is an fp16 DENORMAL whose value is code * 2^(shift - 24) (the
-//                matrix pipe keeps denormal inputs); the power of two is folded into the query operand.  The bias
-//                sum q' * min enters through the same accumulators (A = 2^-24 in every slot, B = q' * min).
+//   q' * scale   lane = channel pair: the group's channel scales times the query rotation the group's flags select
+//                (identity / H32 per sub-vector / H128; the three rotations are made once per workgroup and kept as
+//                fp16 value + fp16 remainder: 22 bits).  The product enters the matrix pipe as TWO fp16 operands per
+//                channel: the rounded product and its exact remainder (one packed fused multiply-add gives it: the
+//                product of two fp16 numbers has 22 bits, the rounded product takes the upper 11), plus the
+//                remainder part of the query -- so the scores carry no 2^-11 rounding of terms that can be a hundred
+//                times larger than their sum (heavy outlier channels).  Written to LDS strips as (value, remainder).
+//   bias         sum q' * min per (group, head): eight more matrix products whose A operand is the channel mins (the
+//                same for every token row, from a 256-byte LDS strip) and whose B operand is the query rotation
+//                itself, value and remainder, straight from the workgroup's table -- exact fp16 x fp16 products summed
+//                in fp32, no per-head vector work; added to the scores as one term per lane.
+//   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads, 128 channels in eight steps
+//                (each code pair twice: against value and remainder): a 2-bit code field masked in place is an fp16
+//                DENORMAL whose value is code * 2^(shift - 24) (the matrix pipe keeps denormal inputs); the power of
+//                two is folded into the query operand.
 //   softmax      exp2-domain, lane = (head, 8 tokens); the running maximum is re-reduced only when some token beats it.
 //   values       v_mfma_f32_32x32x16_f16, rows = the 32 channels of a sub-vector, columns = (class, head) with class =
 //                stored as is / H32 / H128, 32 tokens in two steps.  B = p * scale of the token if it belongs to the
@@ -41,6 +49,10 @@ DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 DEVI uint32_t pk_mul(uint32_t a, uint32_t b) {
   return __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, a) * __builtin_bit_cast(half2_t, b));
 }
+DEVI uint32_t pk_fma(uint32_t a, uint32_t b, uint32_t c) {      // a * b + c per half, one rounding
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b),
+                                                                __builtin_bit_cast(half2_t, c)));
+}
 DEVI uint32_t pack_rn(float a, float b) {
   half2_t v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
   return __builtin_bit_cast(uint32_t, v);
@@ -55,7 +67,8 @@ template <bool F8> constexpr int VC_OFF = F8 ? 640 : 768;
 template <bool F8> constexpr int VM_OFF = F8 ? 1152 : 1280;
 constexpr uint32_t X256 = 0x5C005C00u;                                         // fp16 pair (256, 256)
 constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
-constexpr int QROW = 68;                        // words per row of the query strips: 64 + 4 pad (conflict-free 128-bit rows)
+constexpr int QROW = 68;                        // (value, remainder) entries per row of the query strip: 64 + 4 pad
+constexpr int QHROW = 66;                       // entries per row of the rotation table: 64 + 2 pad (rows 16 bytes apart in the banks)
 constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad
 constexpr int OROW = 132;                       // floats per row of the merged accumulators: 128 + 4 pad
 
@@ -64,8 +77,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct Scr {                                    // per wavefront, rewritten for every 32-token group
-  alignas(16) uint32_t qs[GT][QROW];            // fp16 pairs of q' * scale * 2^-shift per (head, channel pair)
-  alignas(16) uint32_t qm[GT][QROW];            // fp16 pairs of q' * min
+  alignas(16) u32x2 q2[GT][QROW];               // per (head, channel pair): fp16 pair of q' * scale * 2^-shift, fp16 pair of its remainder
+  alignas(16) uint32_t mn[64];                  // fp16 pair of the channel mins per channel pair
   // rows and blocks padded so that the 128-bit rows one instruction reads fall into different banks
   alignas(16) _Float16 pst[GT][PROW];           // p per (head, token)
   alignas(16) uint16_t vsm[3][4 * 32 + 8];      // value scale (fp16 bits) per (class, sub-vector * 32 + token), 0 off its class
@@ -73,7 +86,7 @@ struct Scr {                                    // per wavefront, rewritten for 
   alignas(16) uint16_t vt[4][8 * PROW + 16];    // value code bytes (zero-extended) per (sub-vector, byte * PROW + token)
 };
 struct Smem {
-  uint32_t qh[3][GT][64];                       // query rotations as fp16 pairs per (variant, head, channel pair)
+  alignas(16) u32x2 qh[3][GT][QHROW];           // query rotations per (variant, head, channel pair): fp16 pair, fp16 pair of the remainder
   union {
     Scr w[4];
     float ob[3][GT][OROW];                      // merged accumulators per class (after the page loop)
@@ -213,7 +226,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     }
     if (var == 1) fwht<32>(x, lq);
     if (var == 2) fwht<128>(x, lq);
-    *reinterpret_cast<u32x2*>(&S.qh[var][g][2 * lq]) = u32x2{pack_rn(x[0], x[1]), pack_rn(x[2], x[3])};
+    {
+      const uint32_t h01 = pack_rn(x[0], x[1]), h23 = pack_rn(x[2], x[3]);
+      const uint32_t l01 = pack_rn(x[0] - f16_value(h01 & 0xFFFFu), x[1] - f16_value(h01 >> 16));
+      const uint32_t l23 = pack_rn(x[2] - f16_value(h23 & 0xFFFFu), x[3] - f16_value(h23 >> 16));
+      S.qh[var][g][2 * lq] = u32x2{h01, l01};
+      S.qh[var][g][2 * lq + 1] = u32x2{h23, l23};
+    }
   }
   __syncthreads();
 
@@ -238,7 +257,6 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
   const float qfold = __uint_as_float((127u - 2u * static_cast<uint32_t>(kq < 5 ? kq : kq - 5)) << 23);
   const uint32_t vmask = 0x00030003u << (2 * (l32 & 3));      // value layout row = channel l32: field l32 & 3 of byte l32 >> 2
   const uint32_t qfold8 = pack_rn(256.f * qfold, 256.f * qfold);
-  const half8 tiny = __builtin_bit_cast(half8, u32x4{0x00010001u, 0x00010001u, 0x00010001u, 0x00010001u});   // 2^-24 in every slot
 
   GroupRegs cur;
   int gi = g_first + wv;
@@ -255,7 +273,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       load_group<F8>(nxt, pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNK<F8>,
                      pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNK<F8>, lane);
     }
-    // ---- group flags; q' * scale and q' * min strips: lane = channel pair
+    // ---- group flags; q' * scale strip and the channel mins: lane = channel pair
+    int wkc;                                    // the rotation this lane's B operands of the bias product come from
     {
       // flag channels: 0 .. 3 and 4 (F8: 0, 4, 8, 12 and 16, the first byte of lanes 0, 2, 4, 6 and 8)
       const uint32_t s0 = __builtin_amdgcn_readlane(cur.km.x, 0), s1 = F8 ? __builtin_amdgcn_readlane(cur.km.x, 2) : __builtin_amdgcn_readlane(cur.km.y, 0),
@@ -275,12 +294,15 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
         spair = pack_rn(f16_value(cur.km.x & 0x7FFFu) * qfold, f16_value(cur.km.y & 0x7FFFu) * qfold);
         mpair = (cur.km.x >> 16) | (cur.km.y & 0xFFFF0000u);
       }
+      wkc = useF ? 2 : static_cast<int>((lmask >> kc) & 1u);               // sub-vector kc = channel pairs 16 kc .. 16 kc + 15
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const uint32_t qq = S.qh[which][g][lane];
-        W.qs[g][lane] = pk_mul(qq, spair);
-        W.qm[g][lane] = pk_mul(qq, mpair);
+        const u32x2 qq = S.qh[which][g][lane];
+        const uint32_t b1 = pk_mul(qq.x, spair);
+        const uint32_t rem = pk_fma(qq.x, spair, b1 ^ 0x80008000u);      // exact: what the rounding of b1 dropped
+        W.q2[g][lane] = u32x2{b1, pk_fma(qq.y, spair, rem)};
       }
+      W.mn[lane] = mpair;
     }
     // ---- value strips: lane = (token l32, half hh) serves sub-vectors 2 hh, 2 hh + 1.  Scale and min go to the strip of
     //      the token's class (0 in the other two; tokens outside the range have no class), the code bytes to byte rows.
@@ -314,21 +336,28 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       }
     }
     wave_lds_sync();
+    // ---- bias: sum q' * min of head sh (every row of the product is that sum)
+    float bq;
+    {
+      f32x4 bacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 m4 = *reinterpret_cast<const u32x4*>(&W.mn[16 * kc + 4 * s]);
+        const u32x4 q0 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][16 * kc + 4 * s]);
+        const u32x4 q1 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][16 * kc + 4 * s + 2]);
+        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{m4.x, m4.x, m4.y, m4.y}), __builtin_bit_cast(half8, q0), bacc, 0, 0, 0);
+        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{m4.z, m4.z, m4.w, m4.w}), __builtin_bit_cast(half8, q1), bacc, 0, 0, 0);
+      }
+      bq = bacc[0] * qscale;
+    }
     // ---- scores on the matrix pipe: rows = the 16 tokens of a page, columns = heads, 128 channels in four steps of 32.
     //      A code field masked in place is an fp16 denormal (code * 2^(shift - 24)); the bias sum q' * min enters as
     //      2^-24 * (q' * min) through the same accumulators.
     f32x4 sa0, sa1;
     {
-      f32x4 bias = {0.f, 0.f, 0.f, 0.f};
+      sa0 = f32x4{0.f, 0.f, 0.f, 0.f}; sa1 = sa0;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const u32x4 bm = *reinterpret_cast<const u32x4*>(&W.qm[sh][16 * kc + 4 * s]);
-        bias = __builtin_amdgcn_mfma_f32_16x16x32_f16(tiny, __builtin_bit_cast(half8, bm), bias, 0, 0, 0);
-      }
-      sa0 = bias; sa1 = bias;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4 bq = *reinterpret_cast<const u32x4*>(&W.qs[sh][16 * kc + 4 * s]);
         const uint32_t wa = (s >> 1) ? cur.ka.y : cur.ka.x, wb = (s >> 1) ? cur.kb.y : cur.kb.x;
         u32x4 xa, xb;
         if (s & 1) {
@@ -339,8 +368,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
           xa = u32x4{wa & 0x00030003u, wa & 0x000C000Cu, wa & 0x00300030u, wa & 0x00C000C0u};
           xb = u32x4{wb & 0x00030003u, wb & 0x000C000Cu, wb & 0x00300030u, wb & 0x00C000C0u};
         }
-        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, bq), sa0, 0, 0, 0);
-        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, bq), sa1, 0, 0, 0);
+        // a 16-byte strip read = (value, remainder) of two channel pairs: each code pair meets both
+        const u32x4 b0 = *reinterpret_cast<const u32x4*>(&W.q2[sh][16 * kc + 4 * s]);
+        const u32x4 b1 = *reinterpret_cast<const u32x4*>(&W.q2[sh][16 * kc + 4 * s + 2]);
+        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xa.x, xa.x, xa.y, xa.y}), __builtin_bit_cast(half8, b0), sa0, 0, 0, 0);
+        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xb.x, xb.x, xb.y, xb.y}), __builtin_bit_cast(half8, b0), sa1, 0, 0, 0);
+        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xa.z, xa.z, xa.w, xa.w}), __builtin_bit_cast(half8, b1), sa0, 0, 0, 0);
+        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xb.z, xb.z, xb.w, xb.w}), __builtin_bit_cast(half8, b1), sa1, 0, 0, 0);
       }
     }
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
@@ -356,7 +390,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
           sc[i] = (pos >= t0 && pos < t1) ? sc[i] : -INFINITY;
         }
       }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))) * up;
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))) * up + bq;
       if (__any(mx > m_run)) {
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -377,7 +411,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       float p[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        p[i] = fexp2(__builtin_fmaf(sc[i], up, -m_run));
+        p[i] = fexp2(__builtin_fmaf(sc[i], up, bq - m_run));
         l_run += p[i];
       }
       if (sn < 8) {
