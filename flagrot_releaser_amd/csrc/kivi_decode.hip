@@ -10,13 +10,13 @@
 //                channel: the rounded product and its exact remainder (one packed fused multiply-add gives it: the
 //                product of two fp16 numbers has 22 bits, the rounded product takes the upper 11), plus the
 //                remainder part of the query -- so the scores carry no 2^-11 rounding of terms that can be a hundred
-//                times larger than their sum (heavy outlier channels).  Written to LDS strips as (value, remainder).
+//                times larger than their sum (heavy outlier channels).  Written to two LDS strips (values, remainders).
 //   bias         sum q' * min per (group, head): eight more matrix products whose A operand is the channel mins (the
 //                same for every token row, from a 256-byte LDS strip) and whose B operand is the query rotation
 //                itself, value and remainder, straight from the workgroup's table -- exact fp16 x fp16 products summed
 //                in fp32, no per-head vector work; added to the scores as one term per lane.
 //   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads, 128 channels in eight steps
-//                (each code pair twice: against value and remainder): a 2-bit code field masked in place is an fp16
+//                (every code operand twice: against the values and against the remainders): a 2-bit code field masked in place is an fp16
 //                DENORMAL whose value is code * 2^(shift - 24) (the matrix pipe keeps denormal inputs); the power of
 //                two is folded into the query operand.
 //   softmax      exp2-domain, lane = (head, 8 tokens); the running maximum is re-reduced only when some token beats it.
@@ -67,8 +67,7 @@ template <bool F8> constexpr int VC_OFF = F8 ? 640 : 768;
 template <bool F8> constexpr int VM_OFF = F8 ? 1152 : 1280;
 constexpr uint32_t X256 = 0x5C005C00u;                                         // fp16 pair (256, 256)
 constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
-constexpr int QROW = 68;                        // (value, remainder) entries per row of the query strip: 64 + 4 pad
-constexpr int QHROW = 66;                       // entries per row of the rotation table: 64 + 2 pad (rows 16 bytes apart in the banks)
+constexpr int QROW = 68;                        // words per row of the query strips and tables: 64 + 4 pad (conflict-free 128-bit rows)
 constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad
 constexpr int OROW = 132;                       // floats per row of the merged accumulators: 128 + 4 pad
 
@@ -77,7 +76,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct Scr {                                    // per wavefront, rewritten for every 32-token group
-  alignas(16) u32x2 q2[GT][QROW];               // per (head, channel pair): fp16 pair of q' * scale * 2^-shift, fp16 pair of its remainder
+  alignas(16) uint32_t qs[GT][QROW];            // fp16 pairs of q' * scale * 2^-shift per (head, channel pair)
+  alignas(16) uint32_t ql[GT][QROW];            // fp16 pairs of what the rounding of those products dropped
   alignas(16) uint32_t mn[64];                  // fp16 pair of the channel mins per channel pair
   // rows and blocks padded so that the 128-bit rows one instruction reads fall into different banks
   alignas(16) _Float16 pst[GT][PROW];           // p per (head, token)
@@ -86,7 +86,8 @@ struct Scr {                                    // per wavefront, rewritten for 
   alignas(16) uint16_t vt[4][8 * PROW + 16];    // value code bytes (zero-extended) per (sub-vector, byte * PROW + token)
 };
 struct Smem {
-  alignas(16) u32x2 qh[3][GT][QHROW];           // query rotations per (variant, head, channel pair): fp16 pair, fp16 pair of the remainder
+  alignas(16) uint32_t qh[3][GT][QROW];         // query rotations as fp16 pairs per (variant, head, channel pair)
+  alignas(16) uint32_t qr[3][GT][QROW];         // their remainders (rotation - fp16 value) as fp16 pairs
   union {
     Scr w[4];
     float ob[3][GT][OROW];                      // merged accumulators per class (after the page loop)
@@ -230,8 +231,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       const uint32_t h01 = pack_rn(x[0], x[1]), h23 = pack_rn(x[2], x[3]);
       const uint32_t l01 = pack_rn(x[0] - f16_value(h01 & 0xFFFFu), x[1] - f16_value(h01 >> 16));
       const uint32_t l23 = pack_rn(x[2] - f16_value(h23 & 0xFFFFu), x[3] - f16_value(h23 >> 16));
-      S.qh[var][g][2 * lq] = u32x2{h01, l01};
-      S.qh[var][g][2 * lq + 1] = u32x2{h23, l23};
+      *reinterpret_cast<u32x2*>(&S.qh[var][g][2 * lq]) = u32x2{h01, h23};
+      *reinterpret_cast<u32x2*>(&S.qr[var][g][2 * lq]) = u32x2{l01, l23};
     }
   }
   __syncthreads();
@@ -297,10 +298,11 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       wkc = useF ? 2 : static_cast<int>((lmask >> kc) & 1u);               // sub-vector kc = channel pairs 16 kc .. 16 kc + 15
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const u32x2 qq = S.qh[which][g][lane];
-        const uint32_t b1 = pk_mul(qq.x, spair);
-        const uint32_t rem = pk_fma(qq.x, spair, b1 ^ 0x80008000u);      // exact: what the rounding of b1 dropped
-        W.q2[g][lane] = u32x2{b1, pk_fma(qq.y, spair, rem)};
+        const uint32_t qv = S.qh[which][g][lane], qrem = S.qr[which][g][lane];
+        const uint32_t b1 = pk_mul(qv, spair);
+        const uint32_t rem = pk_fma(qv, spair, b1 ^ 0x80008000u);        // exact: what the rounding of b1 dropped
+        W.qs[g][lane] = b1;
+        W.ql[g][lane] = pk_fma(qrem, spair, rem);
       }
       W.mn[lane] = mpair;
     }
@@ -344,9 +346,9 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
       for (int s = 0; s < 4; ++s) {
         const u32x4 m4 = *reinterpret_cast<const u32x4*>(&W.mn[16 * kc + 4 * s]);
         const u32x4 q0 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][16 * kc + 4 * s]);
-        const u32x4 q1 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][16 * kc + 4 * s + 2]);
-        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{m4.x, m4.x, m4.y, m4.y}), __builtin_bit_cast(half8, q0), bacc, 0, 0, 0);
-        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{m4.z, m4.z, m4.w, m4.w}), __builtin_bit_cast(half8, q1), bacc, 0, 0, 0);
+        const u32x4 q1 = *reinterpret_cast<const u32x4*>(&S.qr[wkc][sh][16 * kc + 4 * s]);
+        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q0), bacc, 0, 0, 0);
+        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q1), bacc, 0, 0, 0);
       }
       bq = bacc[0] * qscale;
     }
@@ -368,13 +370,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
           xa = u32x4{wa & 0x00030003u, wa & 0x000C000Cu, wa & 0x00300030u, wa & 0x00C000C0u};
           xb = u32x4{wb & 0x00030003u, wb & 0x000C000Cu, wb & 0x00300030u, wb & 0x00C000C0u};
         }
-        // a 16-byte strip read = (value, remainder) of two channel pairs: each code pair meets both
-        const u32x4 b0 = *reinterpret_cast<const u32x4*>(&W.q2[sh][16 * kc + 4 * s]);
-        const u32x4 b1 = *reinterpret_cast<const u32x4*>(&W.q2[sh][16 * kc + 4 * s + 2]);
-        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xa.x, xa.x, xa.y, xa.y}), __builtin_bit_cast(half8, b0), sa0, 0, 0, 0);
-        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xb.x, xb.x, xb.y, xb.y}), __builtin_bit_cast(half8, b0), sa1, 0, 0, 0);
-        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xa.z, xa.z, xa.w, xa.w}), __builtin_bit_cast(half8, b1), sa0, 0, 0, 0);
-        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, u32x4{xb.z, xb.z, xb.w, xb.w}), __builtin_bit_cast(half8, b1), sa1, 0, 0, 0);
+        // the same code operands against the products and against their remainders
+        const u32x4 b0 = *reinterpret_cast<const u32x4*>(&W.qs[sh][16 * kc + 4 * s]);
+        const u32x4 b1 = *reinterpret_cast<const u32x4*>(&W.ql[sh][16 * kc + 4 * s]);
+        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b0), sa0, 0, 0, 0);
+        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b0), sa1, 0, 0, 0);
+        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b1), sa0, 0, 0, 0);
+        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b1), sa1, 0, 0, 0);
       }
     }
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)

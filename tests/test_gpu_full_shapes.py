@@ -9,9 +9,10 @@ planner, through the C-ABI), each checked on sampled sequences against the oracl
 
 Bars (the worst element-wise ratio |err| / (2e-3 + 1e-2 |ref|) is printed for every case):
   FlagRot decode   element-wise: |out - ref| <= 2e-3 + 1e-2 |ref| on every element of the sampled sequences;
-  KIVI decode      max |err| <= 1e-2 max |ref| (the reference's own bar, integrations/vllm_flagrot/tests/test_kivi.py:243);
-                   the scores are sums of fp16 products q' * scale * code and q' * min, whose rounding shifts the weight
-                   of whole 32-token groups by up to ~1 %, so single elements near zero miss the element-wise bar;
+  KIVI decode      element-wise as well (the score operands carry value + remainder, 22 bits; with single fp16
+                   products the rounding of q' * scale * code and q' * min moved the weight of whole 32-token groups
+                   by up to ~1 % and the worst ratio was 6.7); the reference's own bar is max |err| <= 1e-2 max |ref|
+                   (integrations/vllm_flagrot/tests/test_kivi.py:243);
   MQ prefill       relative L2 <= 3e-3, the error of BF16 FlashAttention, which is what the reference measures its
                    kernel against (scripts/bench_mq_prefill.py:221-235); the bf16 rounding of the output alone is 1.1e-3.
 """
@@ -61,8 +62,8 @@ def test_configs2_int2_centred_sink_window_b64_l16384(dev):
 def test_configs3_kivi_b16_l32768(dev, f8):
     r = bench.run_kivi(_args(f8=f8), torch, dev, 3, 2)
     _report("configs[3]" + (" FP8 meta" if f8 else ""), r)
-    assert r["checked"] and r["errors"]["max_over_max"] <= 1e-2, r["check"]
-    assert r["errors"]["rel_l2"] <= 5e-3, r["check"]
+    assert r["checked"] and r["errors"]["elementwise"] <= 1.0, r["check"]
+    assert r["errors"]["max_over_max"] <= 1e-2 and r["errors"]["rel_l2"] <= 3e-3, r["check"]
 
 
 @pytest.mark.parametrize("fmt", ["int4a", "konlya"])
