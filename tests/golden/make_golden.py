@@ -17,7 +17,7 @@ Files and the reference functions that wrote them:
   static_writer.npz        kernels/ref.py kv_selrot_quant(fmt="int4") and int4a_quant (and formats.quant_asym_dep with
                            2 bits + scale_word_b for int2a) on seeded rows with a random rotation mask
   kivi_layout.npz          vllm_flagrot/kivi.py _kcodes / _codes / parse_chunks / dequant_groups on random chunk bytes
-                           (FP16 meta and FP8 meta chunks; both bases)
+                           (FP16 meta and FP8 meta chunks; both bases); kivi_layout_d256.npz: the same at head dim 256
   kivi_select.npz          blockflag.qattention.dyn_quant("kivi2:32" and "kivi2f8:32", att + F rule) reconstructions and
                            the per-group / per-token choices (the internals test_kivi.py's sim_choice_k uses) for keys
                            (token axis, with 4 sink tokens excluded from the first group) and values (head axis)
@@ -216,9 +216,9 @@ def write_static():
 
 
 # ------------------------------------------------------------------------------------------------ KIVI page layout
-def write_kivi_layout():
+def write_kivi_layout(D=128, name="kivi_layout.npz"):
     from vllm_flagrot import kivi as RKV     # top level imports ctypes, fcntl, torch only; lib() is never called
-    D, H, npg = 128, 2, 4
+    H, npg = 2, 4
     NV = D // 32
     rng = np.random.default_rng(77)
     out = {}
@@ -249,7 +249,11 @@ def write_kivi_layout():
             k, v = RKV.dequant_groups(t, D, basis=basis, f8=f8)
             out[f"{tag}_k_{basis}"], out[f"{tag}_v_{basis}"] = k.numpy(), v.numpy()
         print("kivi layout", tag, tuple(kc.shape), tuple(km.shape), tuple(vf.shape))
-    np.savez_compressed(OUT / "kivi_layout.npz", **out)
+    np.savez_compressed(OUT / name, **out)
+
+
+def write_kivi_layout_d256():
+    write_kivi_layout(256, "kivi_layout_d256.npz")
 
 
 # ------------------------------------------------------------------------------------------------ KIVI selection
@@ -309,7 +313,7 @@ def write_kivi_select():
     np.savez_compressed(OUT / "kivi_select.npz", **out)
 
 
-WRITERS = {"k2": write_k2, "k2d256": write_k2_d256, "pages": write_pages, "pages256": write_pages_d256, "static": write_static, "kivi_layout": write_kivi_layout,
+WRITERS = {"k2": write_k2, "k2d256": write_k2_d256, "pages": write_pages, "pages256": write_pages_d256, "kivi_layout256": write_kivi_layout_d256, "static": write_static, "kivi_layout": write_kivi_layout,
            "kivi_select": write_kivi_select}
 
 

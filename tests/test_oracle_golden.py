@@ -126,11 +126,12 @@ def test_static_writers_match_reference_vectors():
 
 # ------------------------------------------------------------------------------------------------ KIVI pages
 @pytest.mark.parametrize("f8", [False, True])
-def test_kivi_layout_matches_reference_parser(f8):
-    """vllm_flagrot/kivi.py parse_chunks / _kcodes / _codes / dequant_groups on random chunk bytes"""
-    g = np.load(os.path.join(GOLD, "kivi_layout.npz"))
+@pytest.mark.parametrize("D", [128, 256])
+def test_kivi_layout_matches_reference_parser(f8, D):
+    """vllm_flagrot/kivi.py parse_chunks / _kcodes / _codes / dequant_groups on random chunk bytes, head dim 128 and 256"""
+    g = np.load(os.path.join(GOLD, "kivi_layout.npz" if D == 128 else "kivi_layout_d256.npz"))
     tag = "f8" if f8 else "f16"
-    ch, D = g[f"{tag}_chunks"], 128
+    ch = g[f"{tag}_chunks"]
     kc, km, vc, vm, vf = KV.parse_chunks(ch, D, f8)
     assert np.array_equal(kc, g[f"{tag}_kcodes"]) and np.array_equal(vc, g[f"{tag}_vcodes"])
     assert np.array_equal(vf != 0, g[f"{tag}_vf"] != 0)
