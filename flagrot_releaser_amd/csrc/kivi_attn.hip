@@ -1,5 +1,5 @@
 // extern "C" surface of libflagrot_kivi.so (declared in include/flagrot_kivi.h) and the split merge of the decode
-// attention.  The writers, the dequantiser and the LSE merge are in kivi_write.hip, the decode splits in kivi_decode.hip.
+// attention.  The writers, the dequantiser and the LSE merge are in kivi_write.hip, the decode splits in kivi_decode.hip, everything of head dim 256 in kivi_wide.hip.
 // Semantics follow integrations/vllm_flagrot/csrc/kivi.cu:1908-1931 (k_merge) and :1933-2342 (C ABI).
 #include <cstdio>
 #include <cstring>
@@ -58,7 +58,13 @@ int kv_chunk_bytes8(int D) { return 10 * D; }
 int kv_v_write(const void* kv, long long kv_rs, int n, int Hkv, int D, const void* slots, const void* co, const void* M,
                void* pool, int ident, const void* vfix, int f8, void* stream) {
   if (n <= 0) return 0;
-  if (D != 128) return bad("kv_v_write: head dim 128 only");
+  if (D != 128 && D != 256) return bad("kv_v_write: head dim 128 or 256");
+  if (D == 256) {
+    if (M != nullptr && !ident && vfix == nullptr) return bad("kv_v_write: the matrix weight M is built for head dim 128 only");
+    return launched(v_write256_launch(kv, kv_rs, n, Hkv, static_cast<const long long*>(slots), static_cast<const float*>(co),
+                                      static_cast<uint8_t*>(pool), ident, static_cast<const int*>(vfix), f8 & 1,
+                                      static_cast<hipStream_t>(stream)), "kv_v_write");
+  }
   return launched(v_write_launch(kv, kv_rs, n, Hkv, static_cast<const long long*>(slots), static_cast<const float*>(co),
                                  static_cast<uint8_t*>(pool), static_cast<const float*>(M), ident, static_cast<const int*>(vfix), f8 & 1,
                                  static_cast<hipStream_t>(stream)), "kv_v_write");
@@ -68,7 +74,12 @@ int kv_k_encode(const void* src, long long src_rs, const void* src2, long long s
                 const void* dslot, int N, int Hkv, int D, const void* qs, const void* lz, int NQ, float qsc, void* pool,
                 int ident, const void* kfix, int f8, void* stream) {
   if (N <= 0) return 0;
-  if (D != 128) return bad("kv_k_encode: head dim 128 only");
+  if (D != 128 && D != 256) return bad("kv_k_encode: head dim 128 or 256");
+  if (D == 256)
+    return launched(k_encode256_launch(src, src_rs, src2, src2_rs, static_cast<const long long*>(sidx),
+                                       static_cast<const long long*>(dslot), N, Hkv, static_cast<const float*>(qs),
+                                       static_cast<const float*>(lz), NQ, qsc, static_cast<uint8_t*>(pool), ident,
+                                       static_cast<const int*>(kfix), f8 & 1, static_cast<hipStream_t>(stream)), "kv_k_encode");
   return launched(k_encode_launch(src, src_rs, src2, src2_rs, static_cast<const long long*>(sidx),
                                   static_cast<const long long*>(dslot), N, Hkv, static_cast<const float*>(qs),
                                   static_cast<const float*>(lz), NQ, qsc, static_cast<uint8_t*>(pool), ident,
@@ -81,8 +92,11 @@ int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, lon
             void* stream) {
   if (B <= 0) return 0;
   if (G > 8 || G < 1 || chunk % 32 || chunk <= 0) { std::snprintf(g_err, sizeof(g_err), "kv_attn: G %d chunk %d", G, chunk); return 2; }
-  if (D != 128) return bad("kv_attn: head dim 128 only");
+  if (D != 128 && D != 256) return bad("kv_attn: head dim 128 or 256");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (D == 256)
+    return launched(attn256_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
+                                   tail_idx, T, opart, ml, out, out_rs, f8 & 1, st), "kv_attn");
   const int rc = attn_splits_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
                                     tail_idx, T, opart, ml, f8 & 1, st);
   if (rc) return launched(rc, "kv_attn");
@@ -94,7 +108,10 @@ int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, lon
 int kv_dequant(const void* pool, const void* bt, int g0, int g1, int nvalid, int Hkv, int D, int fp32, void* ok, void* ov,
                int f8, void* stream) {
   if (g1 <= g0) return 0;
-  if (D != 128) return bad("kv_dequant: head dim 128 only");
+  if (D != 128 && D != 256) return bad("kv_dequant: head dim 128 or 256");
+  if (D == 256)
+    return launched(dequant256_launch(static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), g0, g1, nvalid, Hkv, fp32,
+                                      ok, ov, f8 & 1, static_cast<hipStream_t>(stream)), "kv_dequant");
   return launched(dequant_launch(static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), g0, g1, nvalid, Hkv, fp32, ok,
                                  ov, f8 & 1, static_cast<hipStream_t>(stream)), "kv_dequant");
 }

@@ -1,4 +1,5 @@
-// Launcher prototypes shared by the translation units of libflagrot_kivi.so (head dim 128; f8: FP8-meta pages).
+// Launcher prototypes shared by the translation units of libflagrot_kivi.so (f8: FP8-meta pages).  The plain names are
+// the 128-d kernels (kivi_write.hip, kivi_decode.hip), the *256 ones the 256-d kernels (kivi_wide.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -19,5 +20,18 @@ int lse_merge_launch(const void* oa, const float* la, long long la_hs, const voi
 int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
                        const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
                        const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st);
+
+
+int v_write256_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
+                      int ident, const int* vfix, int f8, hipStream_t st);
+int k_encode256_launch(const void* src, long long src_rs, const void* src2, long long src2_rs, const long long* sidx,
+                       const long long* dslot, int N, int Hkv, const float* qs, const float* lz, int NQ, float qsc,
+                       uint8_t* pool, int ident, const int* kfix, int f8, hipStream_t st);
+int dequant256_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nvalid, int Hkv, int fp32, void* ok, void* ov,
+                      int f8, hipStream_t st);
+// splits and merge in one call: out bf16 rows of Hkv G 256 values
+int attn256_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
+                   int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring, const void* tail_len,
+                   const void* tail_idx, int T, void* opart, void* ml, void* out, long long out_rs, int f8, hipStream_t st);
 
 }  // namespace frkv

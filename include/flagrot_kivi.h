@@ -5,10 +5,11 @@
  * Drop-in for the entry points the reference plugin binds with ctypes (integrations/vllm_flagrot/vllm_flagrot/kivi.py:
  * 49-77 of the reference; definitions in integrations/vllm_flagrot/csrc/kivi.cu:1933-2342).  Raw device pointers,
  * `stream` is a hipStream_t, asynchronous, no allocation.  Return codes: 0 ok, 1 launch failure, 2 bad / unsupported
- * argument (message from kv_last_error()).  Built for head dim 128, FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3
- * scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes computed from the stored values, the value rows' whole-head
- * flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88, 123-128), diagonal (co) and matrix (M) value weighting;
- * head dim 256 returns 2.
+ * argument (message from kv_last_error()).  Built for head dim 128 and 256 (kivi.cu's <128> and <256> instantiations;
+ * at 256 a chunk has eight sub-vectors and key cells of eight channels, and kv_attn serves G <= 8 with a plain fp32
+ * kernel), FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3 scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes
+ * computed from the stored values, the value rows' whole-head flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88,
+ * 123-128), diagonal (co) value weighting at both head dims and matrix (M) weighting at head dim 128 (M at 256: 2).
  */
 #ifndef FLAGROT_KIVI_H
 #define FLAGROT_KIVI_H

@@ -28,15 +28,15 @@ D, PAGE = 128, 16
 F8 = pytest.mark.parametrize("f8", [False, True], ids=["f16meta", "f8meta"])
 
 
-def _cb(f8):
-    return OK.chunk_bytes(D, f8)
+def _cb(f8, hd=D):
+    return OK.chunk_bytes(hd, f8)
 
 
-def _kv(T, Hkv, g, shift=2.0, big=200.0):
+def _kv(T, Hkv, g, shift=2.0, big=200.0, hd=D):
     """rows with per-channel offsets (what makes rotated bases win or lose per group), a few outlier channels, a zero
     row, a constant sub-vector, a tiny row and a row scaled by `big`."""
-    mu = torch.randn(2 * Hkv, D, generator=g) * shift
-    x = mu[None] + torch.randn(T, 2 * Hkv, D, generator=g) * (0.3 + torch.rand(2 * Hkv, D, generator=g))
+    mu = torch.randn(2 * Hkv, hd, generator=g) * shift
+    x = mu[None] + torch.randn(T, 2 * Hkv, hd, generator=g) * (0.3 + torch.rand(2 * Hkv, hd, generator=g))
     x[:, :, 5] *= 6
     if T >= 8:
         x[3] = 0.0
@@ -46,15 +46,15 @@ def _kv(T, Hkv, g, shift=2.0, big=200.0):
     return x.bfloat16()
 
 
-def _calib(Hkv, NQ, g):
-    qs = (torch.randn(Hkv, NQ, D, generator=g) * 0.4).contiguous()
+def _calib(Hkv, NQ, g, hd=D):
+    qs = (torch.randn(Hkv, NQ, hd, generator=g) * 0.4).contiguous()
     lz = (3.0 + torch.rand(Hkv, NQ, generator=g) * 4).contiguous()
-    co = (torch.rand(Hkv, D, generator=g) + 0.1).contiguous()
+    co = (torch.rand(Hkv, hd, generator=g) + 0.1).contiguous()
     return qs, lz, co
 
 
-def _stored_value_flags(pool_np, f8=False):
-    _, _, _, vm, vf = OK.parse_chunks(pool_np, D, f8)
+def _stored_value_flags(pool_np, f8=False, hd=D):
+    _, _, _, vm, vf = OK.parse_chunks(pool_np, hd, f8)
     return (vm[..., 0] >> (7 if f8 else 15)).astype(bool), vf.astype(bool)          # [np, H, 16, NV], [np, H, 16]
 
 
@@ -161,10 +161,10 @@ def test_v_write_pinned_modes(dev, mode, f8):
     assert np.array_equal(pool.cpu().numpy(), want)
 
 
-def _groups(NG, Hkv, g, ragged=True):
+def _groups(NG, Hkv, g, ragged=True, hd=D):
     """NG groups of 32 tokens from two source tensors; returns kv rows, src2 rows, sidx, dslot, valid."""
-    rows = _kv(NG * 32 + 5, Hkv, g)
-    rows2 = _kv(40, Hkv, g, shift=1.0)
+    rows = _kv(NG * 32 + 5, Hkv, g, hd=hd)
+    rows2 = _kv(40, Hkv, g, shift=1.0, hd=hd)
     sidx = torch.arange(NG * 32).reshape(NG, 32).long() + 5
     if ragged and NG >= 3:
         sidx[1, 20:] = -1                      # a short group
@@ -175,7 +175,7 @@ def _groups(NG, Hkv, g, ragged=True):
 
 
 def _group_rows(rows, rows2, sidx_row, Hkv):
-    xb = np.zeros((32, Hkv, D), np.uint16)
+    xb = np.zeros((32, Hkv, rows.shape[-1]), np.uint16)
     rb, rb2 = bits(rows), bits(rows2)
     for t, r in enumerate(sidx_row.tolist()):
         if r >= 0:
@@ -185,13 +185,14 @@ def _group_rows(rows, rows2, sidx_row, Hkv):
     return xb, (sidx_row.numpy() != -1)
 
 
-def _stored_key_flags(pool_np, dslot_row, h, f8=False):
+def _stored_key_flags(pool_np, dslot_row, h, f8=False, hd=D):
     pg0 = int(dslot_row[0]) // 16
     pg1 = int(dslot_row[16]) // 16
-    _, km, *_ = OK.parse_chunks(pool_np[[pg0, pg1]][:, h:h + 1], D, f8)
-    s = km[:, 0, :, :, 0].reshape(-1)                                 # 128 channel scales, cell-major
-    st, fb = (4, 7) if f8 else (1, 15)                                # flag channels 0, st, 2 st, 3 st and 4 st
-    return (s[0:4 * st:st] >> fb).astype(bool), bool(s[4 * st] >> fb)
+    _, km, *_ = OK.parse_chunks(pool_np[[pg0, pg1]][:, h:h + 1], hd, f8)
+    s = km[:, 0, :, :, 0].reshape(-1)                                 # the channel scales, cell-major
+    NV = hd // 32
+    st, fb = (NV, 7) if f8 else (1, 15)                               # flag channels 0, st, .., (NV - 1) st and NV st
+    return (s[0:NV * st:st] >> fb).astype(bool), bool(s[NV * st] >> fb)
 
 
 @F8
@@ -258,7 +259,7 @@ def test_k_encode_pinned_modes_keep_value_fields(dev, mode, f8):
     assert np.array_equal(pool.cpu().numpy(), want)
 
 
-def _filled_cache(dev, lens, Hkv, g, tail_T=0, f8=False):
+def _filled_cache(dev, lens, Hkv, g, tail_T=0, f8=False, hd=D):
     """pages of B sequences written by the GPU writers (whole groups), block table, and the fp64 K / V the oracle
     reads back from the same bytes."""
     from flagrot_releaser_amd import kivi as KV
@@ -267,24 +268,24 @@ def _filled_cache(dev, lens, Hkv, g, tail_T=0, f8=False):
     npg = 2 * sum(ngs) + 1
     perm = torch.randperm(npg, generator=g)
     bt = torch.zeros(B, 2 * max(ngs), dtype=torch.int32)
-    pool = torch.zeros(npg, Hkv, _cb(f8), dtype=torch.uint8, device=dev)
-    qs, lz, co = _calib(Hkv, 24, g)
+    pool = torch.zeros(npg, Hkv, _cb(f8, hd), dtype=torch.uint8, device=dev)
+    qs, lz, co = _calib(Hkv, 24, g, hd=hd)
     o = 0
     Ks, Vs = [], []
     for b in range(B):
         n = ngs[b] * 32
         bt[b, :2 * ngs[b]] = perm[o:o + 2 * ngs[b]].int()
         o += 2 * ngs[b]
-        kv = _kv(n, Hkv, g).to(dev)
+        kv = _kv(n, Hkv, g, hd=hd).to(dev)
         slots = (bt[b].long()[torch.arange(n) // 16] * 16 + torch.arange(n) % 16)
-        KV.v_write(kv, slots.to(dev), co.to(dev), None, pool, Hkv, D, f8=f8)
+        KV.v_write(kv, slots.to(dev), co.to(dev), None, pool, Hkv, hd, f8=f8)
         sidx = torch.arange(n).reshape(-1, 32).long()
-        KV.k_encode(kv, sidx.to(dev), slots.reshape(-1, 32).to(dev), qs.to(dev), lz.to(dev), 1 / math.sqrt(D), pool, Hkv, D,
-                    f8=f8)
+        KV.k_encode(kv, sidx.to(dev), slots.reshape(-1, 32).to(dev), qs.to(dev), lz.to(dev), 1 / math.sqrt(hd), pool, Hkv,
+                    hd, f8=f8)
     torch.cuda.synchronize()
     pnp = pool.cpu().numpy()
     for b in range(B):
-        k, v = OK.dequant_groups(pnp[bt[b, :2 * ngs[b]].numpy()], D, f8=f8)
+        k, v = OK.dequant_groups(pnp[bt[b, :2 * ngs[b]].numpy()], hd, f8=f8)
         Ks.append(k)
         Vs.append(v)
     return pool, bt, Ks, Vs
@@ -374,8 +375,8 @@ def test_attn_without_tail_and_rejects(dev):
     with pytest.raises(RuntimeError, match="chunk"):
         KV.attn(q.to(dev), pool, bt.to(dev), cached, out, 2, 100, ws, 0.1, 0, G)
     with pytest.raises(RuntimeError, match="head dim"):
-        KV.v_write(torch.zeros(1, 2 * Hkv, 256, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
-                   torch.ones(Hkv, 256, device=dev), None, pool, Hkv, 256)
+        KV.v_write(torch.zeros(1, 2 * Hkv, 64, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
+                   torch.ones(Hkv, 64, device=dev), None, pool, Hkv, 64)
 
 
 @F8
