@@ -29,7 +29,7 @@ STRICT = ["-ffp-contract=off", "-fno-fast-math"]
 LIBS = {
     "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("capi.hip", [])]),
     "kivi": ("libflagrot_kivi.so", [("kivi_write.hip", STRICT), ("kivi_wide.hip", STRICT), ("kivi_attn.hip", []), ("kivi_decode.hip", [])]),
-    "mq": ("libflagrot_mq.so", [("mq_prefill.hip", [])]),
+    "mq": ("libflagrot_mq.so", [("mq_prefill.hip", []), ("mq_wide.hip", [])]),
 }
 
 

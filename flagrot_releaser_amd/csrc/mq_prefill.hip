@@ -24,458 +24,14 @@
 #include "../../include/flagrot_mq.h"
 #include "fr_common.hpp"
 #include "fr_unpack.hpp"
+#include "mq_launch.hpp"
+#include "mq_tiles.hpp"
 
 namespace frmq {
 using namespace fr;
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-constexpr int D = 128, PAGE = 16, BN = 64, TILE_INTS = 9, ITEM_INTS = 4;
-constexpr int KROW = 272;                    // bytes per K tile row: 256 + 16 pad
-constexpr int VROW = 144;                    // bytes per V^T tile row: 128 + 16 pad
-constexpr int KT_BYTES = BN * KROW, VT_BYTES = D * VROW;
-constexpr int QROW = 264;                    // bytes per staged q row (natural order)
-constexpr int PG_CACHE = 1024;               // page ids kept in LDS (256 blocks of 64 keys)
-
-struct Smem {
-  alignas(16) uint8_t kt[KT_BYTES];
-  alignas(16) uint8_t vt[VT_BYTES];
-  alignas(16) uint32_t vsc[4][8][4];         // per (group, run): scale pairs (t0,t4) (t1,t5) (t2,t6) (t3,t7)
-  alignas(16) uint32_t vnz[4][8][4];         // per (group, run): -(1024 + zero point) pairs
-  int pages[PG_CACHE];                       // page ids of the blocks [cb, cb + PG_CACHE / 4) of the item
-};
-static_assert(128 * QROW <= KT_BYTES + VT_BYTES, "q staging aliases the tiles");
-
-struct Params {
-  const uint16_t* q;
-  const uint8_t* pool;
-  long long page_stride;
-  const int* bt;
-  long long bt_stride;
-  const int* tiles;
-  const int* items;
-  int Hkv, G, shift, kmin;
-  float* opart;
-  float* ml;
-};
-
-// What one workgroup (item, KV head) has to do, read from its item record (tile, first block, end block, 0) and the tile
-// record that names (block-table row, first compact query row, first output row, tokens, position of the first token,
-// page keys of the request, first item, items, reach).  `reach`: a key index every row may see on top of its causal
-// range (a large negative number when there is none).
-struct Work {
-  const int* block_table;
-  int compact_row, tokens, first_pos, reach;
-  int key_end;              // keys at or past it are invisible to the whole tile or belong to a later item
-  int block0, block1;       // 64-key blocks [block0, block1) to read (empty when the item starts past key_end)
-  int rows_used;            // query rows of the tile that hold a token's head: whole tokens only
-  int shift;
-
-  DEVI Work(const Params& p, int item, int rows) {
-    const int* irec = p.items + ITEM_INTS * item;
-    const int* trec = p.tiles + TILE_INTS * irec[0];
-    block_table = p.bt + static_cast<long long>(trec[0]) * p.bt_stride;
-    compact_row = trec[1]; tokens = trec[3]; first_pos = trec[4]; reach = trec[8];
-    shift = p.shift;
-    const int causal_end = max(first_pos + tokens - shift, reach + 1);      // what the tile's last token sees
-    key_end = min(min(trec[5], irec[2] * BN), causal_end);
-    block0 = irec[1];
-    block1 = key_end > block0 * BN ? (key_end + BN - 1) / BN : block0;
-    rows_used = min(rows / p.G, tokens) * p.G;
-  }
-  DEVI bool has_row(int row) const { return row < rows_used; }
-  DEVI int last_key(int token) const { return min(key_end - 1, max(first_pos + token - shift, reach)); }
-};
-
 char g_err[512] = "";
-
-template <typename T> DEVI T gload(const void* p) {
-  return *reinterpret_cast<const __attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p));
-}
-DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
-DEVI half8 as_h8(u32x4 v) { return __builtin_bit_cast(half8, v); }
-DEVI uint32_t pack_h2(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-DEVI uint32_t pack_h2_rn(float a, float b) {
-  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-  h2 v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
-  return __builtin_bit_cast(uint32_t, v);
-}
-
-// token (0..31 inside a 32-key tile) -> K tile row, and accumulator index -> token
-DEVI int krow_of_token(int tk) {
-  const int run = tk >> 3, t8 = tk & 7, e = 2 * (t8 & 3) + (t8 >> 2);
-  return 16 * (run >> 1) + 8 * (e >> 2) + 4 * (run & 1) + (e & 3);
-}
-DEVI constexpr int token_of_acc(int i, int hh) {   // accumulator i of the lane half hh
-  const int s = i >> 3, e = i & 7;
-  const int t8 = (e >> 1) + 4 * (e & 1);           // run order t0 t4 t1 t5 t2 t6 t3 t7
-  return 8 * (2 * s + hh) + t8;
-}
-
-template <int QM> struct Fmt {
-  static constexpr int CB = QM == QM_ASYM2 ? 32 : 64;
-  static constexpr int V_OFF = CB * PAGE, KS_OFF = 2 * CB * PAGE, VS_OFF = KS_OFF + 8 * PAGE, CHUNK = VS_OFF + 8 * PAGE;
-  static constexpr uint32_t ZM = QM == QM_ASYM2 ? 3u : 15u;
-};
-
-// ------------------------------------------------------------------------------------------------ key-only pages
-// Inverse transform of one token's keys while they are fp16 pairs in registers.  A thread holds, per 32-group, the 8
-// elements d = 4 tg + i (A_i) and 16 + 4 tg + i (B_i) as (A0 A2) (B0 B2) (A1 A3) (B1 B3); the four threads of a quad
-// (tg = lane & 3) hold the group.  Index bits of d: bit 0 = registers 0,1 <-> 2,3; bit 1 = low <-> high half; bits 2,3 =
-// the quad lanes (DPP); bit 4 = registers 0 <-> 1, 2 <-> 3; the two group bits of the whole-head transform = registers of
-// different groups.  The five stages inside a group run on the integers code - zero point (exact in fp16), then the
-// group scale times an exact power of two (2^-2 per group, 2^-3 whole head) is applied, then the two whole-head stages;
-// the remaining 2^-0.5 is one multiply at the end.
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-DEVI h2_t h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
-DEVI uint32_t u2(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
-DEVI void bfly(uint32_t& a, uint32_t& b) {
-  const h2_t x = h2(a), y = h2(b);
-  a = u2(x + y); b = u2(x - y);
-}
-DEVI uint32_t bfly_halves(uint32_t a) {                       // (lo, hi) -> (lo + hi, lo - hi)
-  const uint32_t sw = (a >> 16) | (a << 16);
-  const h2_t sg = h2(0xBC003C00u);                            // (1, -1)
-  return u2(__builtin_elementwise_fma(h2(a), sg, h2(sw)));
-}
-template <int CTRL> DEVI uint32_t bfly_lanes(uint32_t a, uint32_t sgn) {   // sgn = (1,1) on the lower lane, (-1,-1) on the upper
-  const uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(a), CTRL, 0xF, 0xF, true));
-  return u2(__builtin_elementwise_fma(h2(a), h2(sgn), h2(o)));
-}
-DEVI void h32_group(uint32_t (&x)[4], uint32_t sgn1, uint32_t sgn2) {
-  bfly(x[0], x[2]); bfly(x[1], x[3]);                          // d bit 0
-#pragma unroll
-  for (int r = 0; r < 4; ++r) x[r] = bfly_halves(x[r]);        // d bit 1
-#pragma unroll
-  for (int r = 0; r < 4; ++r) x[r] = bfly_lanes<0xB1>(x[r], sgn1);   // d bit 2: quad lanes xor 1
-#pragma unroll
-  for (int r = 0; r < 4; ++r) x[r] = bfly_lanes<0x4E>(x[r], sgn2);   // d bit 3: quad lanes xor 2
-  bfly(x[0], x[1]); bfly(x[2], x[3]);                          // d bit 4
-}
-
-// ------------------------------------------------------------------------------------------------ tile converters
-// The raw page words of a 64-key block are fetched into registers one block ahead (load_raw) and turned into the
-// fp16 tiles after the previous block's matrix work (convert_k, v_tables, convert_v).
-template <int NT> struct Raw {
-  static constexpr int NI = 256 / NT;
-  u32x4 kc[NI];      // K code words of (token, tg): INT4 four groups, INT2 two words in .x .y
-  u32x2 ks[NI];      // the token's four K scale words
-  uint32_t vf[NI];   // the token's group-0 V scale word (whole-head flag of key-only pages)
-  u32x4 vc[NI];      // V^T entry (e, c8) of a page
-  u32x4 vs;          // threads < 32: V scale words of (group, run)
-};
-
-template <int QM, bool K2, int NT>
-DEVI void load_raw(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, int kend) {   // pg[0] = first page of block kb
-  using F = Fmt<QM>;
-#pragma unroll
-  for (int it = 0; it < Raw<NT>::NI; ++it) {
-    const int idx = threadIdx.x + it * NT;
-    {
-      const int tk = idx >> 2, tg = idx & 3, j = kb * BN + tk;
-      if (j < kend) {
-        const uint8_t* ch = p.pool + static_cast<long long>(pg[tk >> 4]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
-        const int pos = j & 15;
-        if constexpr (QM == QM_ASYM2) {
-          const u32x2 c = gload<u32x2>(ch + 32 * (pos ^ ((pos >> 1) & 2)) + 8 * tg);
-          R.kc[it] = u32x4{c.x, c.y, 0u, 0u};
-        } else {
-          R.kc[it] = gload<u32x4>(ch + 64 * pos + 16 * tg);
-        }
-        R.ks[it] = gload<u32x2>(ch + F::KS_OFF + 8 * pos);
-        if constexpr (K2) R.vf[it] = gload<uint16_t>(ch + F::VS_OFF + (8 * (pos >> 3) + vs_slot8(pos)) * 2);
-      }
-    }
-    {
-      const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, j0 = kb * BN + PAGE * pgi;
-      if (j0 < kend) {
-        const uint8_t* ch = p.pool + static_cast<long long>(pg[pgi]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
-        if constexpr (QM == QM_ASYM2) {
-          const u32x2 c = gload<u32x2>(ch + F::V_OFF + (e * 2 + c8) * 8);
-          R.vc[it] = u32x4{c.x, c.y, 0u, 0u};
-        } else {
-          R.vc[it] = gload<u32x4>(ch + F::V_OFF + (e * 2 + c8) * 16);
-        }
-      }
-    }
-  }
-  if (threadIdx.x < 32) {
-    const int g = threadIdx.x >> 3, run = threadIdx.x & 7, j0 = kb * BN + 8 * run;
-    if (j0 < kend) {
-      const uint8_t* ch = p.pool + static_cast<long long>(pg[run >> 1]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
-      R.vs = gload<u32x4>(ch + F::VS_OFF + (g * PAGE + 8 * (run & 1)) * 2);   // t0 t2 | t4 t6 | t1 t3 | t5 t7
-    }
-  }
-}
-
-// K tile entry idx = (token tk = idx >> 2 of the block, quarter tg = idx & 3) from the token's raw words
-template <int QM, bool K2>
-DEVI void convert_k_entry(uint8_t* kt, int idx, const u32x4 kc, const u32x2 sw, uint32_t vf, int kb, int kend, const Consts& cst) {
-  using F = Fmt<QM>;
-  {
-    const int tk = idx >> 2, tg = idx & 3;
-    const int j = kb * BN + tk;
-    const int row = 32 * (tk >> 5) + krow_of_token(tk & 31);
-    u32x4* dst = reinterpret_cast<u32x4*>(kt + row * KROW);
-    if (j >= kend) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) dst[4 * g + tg] = u32x4{0u, 0u, 0u, 0u};
-      return;
-    }
-    uint32_t w[4];
-    if constexpr (QM == QM_ASYM2) {
-      w[0] = kc.x; w[1] = kc.x >> 4; w[2] = kc.y; w[3] = kc.y >> 4;
-    } else {
-      w[0] = kc.x; w[1] = kc.y; w[2] = kc.z; w[3] = kc.w;
-    }
-    const uint32_t s16[4] = {sw.x & 0xFFFFu, sw.x >> 16, sw.y & 0xFFFFu, sw.y >> 16};
-    if constexpr (!K2) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
-        const uint32_t nz[4] = {z, z, z, z};
-        uint32_t x[4];
-        Unpack<QM>::run(w[g], nz, cst, x);
-        dst[4 * g + tg] = u32x4{pk_mul(x[0], sc), pk_mul(x[1], sc), pk_mul(x[2], sc), pk_mul(x[3], sc)};
-      }
-    } else {
-      // key-only pages: the token's flags select identity / H32 per group / whole-head H128 (the quad of a token agrees)
-      const bool ff = (vf >> 15) & 1u;
-      const uint32_t sgn1 = (tg & 1) ? 0xBC00BC00u : 0x3C003C00u, sgn2 = (tg & 2) ? 0xBC00BC00u : 0x3C003C00u;
-      uint32_t x[4][4], y[4][4];
-      bool rot[4];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        rot[g] = ff || ((s16[g] >> 15) & 1u);
-        const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
-        const uint32_t pre = ff ? 0x30003000u : 0x34003400u;                                 // 2^-3, 2^-2 (exact)
-        const uint32_t sce = pk_mul(sc, pre);
-        const uint32_t nz[4] = {z, z, z, z};
-        uint32_t c[4];
-        Unpack<QM>::run(w[g], nz, cst, c);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) { x[g][r] = pk_mul(c[r], sc); y[g][r] = c[r]; }
-        h32_group(y[g], sgn1, sgn2);              // on the integers code - zero point: exact (|sum| <= 32 * 15)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) y[g][r] = pk_mul(y[g][r], sce);
-      }
-      if (__any(ff)) {                                           // the two group bits of the whole-head transform
-        uint32_t f[4][4];
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) f[g][r] = y[g][r];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) { bfly(f[0][r], f[1][r]); bfly(f[2][r], f[3][r]); }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) { bfly(f[0][r], f[2][r]); bfly(f[1][r], f[3][r]); }
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) y[g][r] = ff ? f[g][r] : y[g][r];
-      }
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x4 v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = rot[g] ? pk_mul(y[g][r], 0x39A839A8u) : x[g][r];   // 2^-0.5
-        dst[4 * g + tg] = v;
-      }
-    }
-  }
-}
-
-template <int QM, bool K2, int NT>
-DEVI void convert_k(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
-#pragma unroll
-  for (int it = 0; it < Raw<NT>::NI; ++it)
-    convert_k_entry<QM, K2>(S.kt, threadIdx.x + it * NT, R.kc[it], R.ks[it], K2 ? R.vf[it] : 0u, kb, kend, cst);
-}
-
-// per (group, run) scale / zero point pairs in the run order; tokens at or beyond kend get scale 0
-template <int QM, int NT>
-DEVI void v_tables(Smem& S, const Raw<NT>& R, int kb, int kend) {
-  using F = Fmt<QM>;
-  if (threadIdx.x < 32) {
-    const int g = threadIdx.x >> 3, run = threadIdx.x & 7;
-    const int j0 = kb * BN + 8 * run;
-    u32x4 sc = {0u, 0u, 0u, 0u}, nz = {0u, 0u, 0u, 0u};
-    if (j0 < kend) {
-      const u32x4 w = R.vs;
-      const uint32_t t[8] = {w.x & 0xFFFFu, w.z & 0xFFFFu, w.x >> 16, w.z >> 16, w.y & 0xFFFFu, w.w & 0xFFFFu, w.y >> 16, w.w >> 16};
-      uint32_t s[8], z[8];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        s[k] = j0 + k < kend ? (t[k] & 0x7FFFu) : 0u;
-        z[k] = negz16(t[k] & F::ZM);
-      }
-      sc = u32x4{s[0] | (s[4] << 16), s[1] | (s[5] << 16), s[2] | (s[6] << 16), s[3] | (s[7] << 16)};
-      nz = u32x4{z[0] | (z[4] << 16), z[1] | (z[5] << 16), z[2] | (z[6] << 16), z[3] | (z[7] << 16)};
-    }
-    *reinterpret_cast<u32x4*>(S.vsc[g][run]) = sc;
-    *reinterpret_cast<u32x4*>(S.vnz[g][run]) = nz;
-  }
-}
-
-template <int QM, int NT>
-DEVI void convert_v(Smem& S, const Raw<NT>& R, int kb, int kend, const Consts& cst) {
-#pragma unroll
-  for (int it = 0; it < Raw<NT>::NI; ++it) {
-    const int idx = threadIdx.x + it * NT;
-    const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, run = 2 * pgi + c8;
-    const int j0 = kb * BN + PAGE * pgi;
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
-    if (j0 < kend) {
-      if constexpr (QM == QM_ASYM2) {
-        w[0] = R.vc[it].x; w[1] = R.vc[it].x >> 4; w[2] = R.vc[it].y; w[3] = R.vc[it].y >> 4;
-      } else {
-        w[0] = R.vc[it].x; w[1] = R.vc[it].y; w[2] = R.vc[it].z; w[3] = R.vc[it].w;
-      }
-    }
-#pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
-      const int d = 64 * (sub >> 1) + 16 * (e >> 3) + 8 * (sub & 1) + (e & 7), g = d >> 5;
-      const u32x4 sc = *reinterpret_cast<const u32x4*>(S.vsc[g][run]);
-      const u32x4 z = *reinterpret_cast<const u32x4*>(S.vnz[g][run]);
-      const uint32_t nz[4] = {z.x, z.y, z.z, z.w};
-      uint32_t x[4];
-      Unpack<QM>::run(w[sub], nz, cst, x);
-      *reinterpret_cast<u32x4*>(S.vt + d * VROW + 16 * run) =
-          u32x4{pk_mul(x[0], sc.x), pk_mul(x[1], sc.y), pk_mul(x[2], sc.z), pk_mul(x[3], sc.w)};
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------------ one 64-key block
-// scores, mask, online softmax and values of the wavefront's 32 rows against the tiles in LDS, in three parts
-// S^T = K q^T: two 32-key tiles (two independent accumulator chains), eight 16-element steps; the K operands of four
-// steps are requested ahead, and the scheduler is told to keep the reads that far in front of the matrix instructions
-DEVI void qk_block(const uint8_t* kt, const u32x4 (&qf)[8], f32x16 (&sacc)[2], int l32, int hh) {
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[t][i] = 0.f;
-  const uint8_t* k0 = kt + l32 * KROW + 16 * hh;
-  const uint8_t* k1 = k0 + 32 * KROW;
-  u32x4 a0[8], a1[8];
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    a0[s] = *reinterpret_cast<const u32x4*>(k0 + 64 * (s >> 1) + 32 * (s & 1));
-    a1[s] = *reinterpret_cast<const u32x4*>(k1 + 64 * (s >> 1) + 32 * (s & 1));
-  }
-#pragma unroll
-  for (int s = 0; s < 8; ++s) {
-    if (s + 4 < 8) {
-      a0[s + 4] = *reinterpret_cast<const u32x4*>(k0 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
-      a1[s + 4] = *reinterpret_cast<const u32x4*>(k1 + 64 * ((s + 4) >> 1) + 32 * (s & 1));
-    }
-    sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a0[s]), as_h8(qf[s]), sacc[0], 0, 0, 0);
-    sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(a1[s]), as_h8(qf[s]), sacc[1], 0, 0, 0);
-  }
-  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // 8 LDS reads
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     // 2 MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);     // 2 LDS reads
-  }
-  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-}
-
-// max over lanes l and l + 32, in both: one v_permlane32_swap, no trip through the LDS queue (which the other group's
-// matrix operand reads keep full)
-DEVI float max_halves(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);   // (lo, lo), (hi, hi)
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-
-// mask + online softmax (lane = row; lanes l and l + 32 hold the two halves of its keys); the probabilities leave as the
-// fp16 B operands of the value product, in the V^T token order
-DEVI void softmax_block(f32x16 (&sacc)[2], u32x4 (&pb)[4], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
-                        bool rvalid, int kmin, int hh) {
-  const int jb = kb * BN;
-  const bool full = __all(rvalid && jb + BN - 1 <= lim) && jb >= kmin;
-  if (!full) {
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int j = jb + 32 * kt + token_of_acc(i, hh);
-        if (!(j <= lim && j >= kmin)) sacc[kt][i] = -INFINITY;
-      }
-  }
-  float mx = -INFINITY;
-#pragma unroll
-  for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kt][i]);
-  mx = max_halves(mx);
-  const float mnew = fmaxf(mrow, mx);
-  const float base = mnew == -INFINITY ? 0.f : mnew;
-  const float alpha = fexp2(mrow - base);
-  float sum = 0.f;
-#pragma unroll
-  for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sacc[kt][i] = fexp2(sacc[kt][i] - base);
-      sum += sacc[kt][i];
-    }
-  lrow = lrow * alpha + sum;
-  if (!__all(mnew == mrow)) {
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-  }
-  mrow = mnew;
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {      // ks = 2 kt + s
-    const int kt = ks >> 1, s2 = ks & 1;
-    pb[ks] = u32x4{pack_h2_rn(sacc[kt][8 * s2], sacc[kt][8 * s2 + 1]), pack_h2_rn(sacc[kt][8 * s2 + 2], sacc[kt][8 * s2 + 3]),
-                   pack_h2_rn(sacc[kt][8 * s2 + 4], sacc[kt][8 * s2 + 5]), pack_h2_rn(sacc[kt][8 * s2 + 6], sacc[kt][8 * s2 + 7])};
-  }
-}
-
-// O^T += V^T P^T: four independent accumulator chains (the 32-dim blocks); V^T operands requested two steps ahead
-DEVI void pv_block(const uint8_t* vt, const u32x4 (&pb)[4], f32x16 (&o)[4], int l32, int hh) {
-  u32x4 va[4][4];
-  const uint8_t* v0 = vt + l32 * VROW + 16 * hh;
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-    for (int db = 0; db < 4; ++db) va[ks][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * ks);
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    if (ks + 2 < 4) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db) va[ks + 2][db] = *reinterpret_cast<const u32x4*>(v0 + 32 * db * VROW + 32 * (ks + 2));
-    }
-#pragma unroll
-    for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_h8(va[ks][db]), as_h8(pb[ks]), o[db], 0, 0, 0);
-  }
-  __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 1);
-  }
-  __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
-}
-
-DEVI void attend_block(const Smem& S, const u32x4 (&qf)[8], f32x16 (&o)[4], float& mrow, float& lrow, int kb, int lim,
-                       bool rvalid, int kmin, int l32, int hh) {
-  f32x16 sacc[2];
-  u32x4 pb[4];
-  qk_block(S.kt, qf, sacc, l32, hh);
-  softmax_block(sacc, pb, o, mrow, lrow, kb, lim, rvalid, kmin, hh);
-  pv_block(S.vt, pb, o, l32, hh);
-}
 
 // ------------------------------------------------------------------------------------------------ main kernel
 template <int QM, bool K2, int NW>
@@ -938,7 +494,25 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
 // neither: its partial is divided by its own sum.
 constexpr int FOLD_ROWS = 4;
 
-template <bool FP32_OUT>
+// W consecutive floats per lane: W = 2 covers a 128-d row with one wavefront, W = 4 a 256-d row
+template <int W> DEVI void ldw(const float* p, float (&x)[W]) {
+  if constexpr (W == 2) { const float2 v = *reinterpret_cast<const float2*>(p); x[0] = v.x; x[1] = v.y; }
+  else { const float4 v = *reinterpret_cast<const float4*>(p); x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w; }
+}
+template <int W> DEVI void stw(float* p, const float (&x)[W]) {
+  if constexpr (W == 2) *reinterpret_cast<float2*>(p) = make_float2(x[0], x[1]);
+  else *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+}
+template <int W> DEVI void ldw_bf16(const uint16_t* p, float (&x)[W]) {
+  if constexpr (W == 2) { const uint32_t v = *reinterpret_cast<const uint32_t*>(p); x[0] = bf16_lo(v); x[1] = bf16_hi(v); }
+  else { const uint2 v = *reinterpret_cast<const uint2*>(p); x[0] = bf16_lo(v.x); x[1] = bf16_hi(v.x); x[2] = bf16_lo(v.y); x[3] = bf16_hi(v.y); }
+}
+template <int W> DEVI void stw_bf16(uint16_t* p, const float (&x)[W]) {
+  if constexpr (W == 2) *reinterpret_cast<uint32_t*>(p) = bf16_rn(x[0]) | (bf16_rn(x[1]) << 16);
+  else *reinterpret_cast<uint2*>(p) = make_uint2(bf16_rn(x[0]) | (bf16_rn(x[1]) << 16), bf16_rn(x[2]) | (bf16_rn(x[3]) << 16));
+}
+
+template <bool FP32_OUT, int W>
 __global__ void __launch_bounds__(256) k_fold_items(const int* __restrict__ tiles, const float* __restrict__ opart,
                                                     const float* __restrict__ ml, int Hkv, int G, int rows,
                                                     void* __restrict__ out, long long out_stride, float* __restrict__ lse,
@@ -953,13 +527,16 @@ __global__ void __launch_bounds__(256) k_fold_items(const int* __restrict__ tile
   for (int i = 0; i < FOLD_ROWS; ++i) {
     const int row = row0 + i;
     if (row >= used) break;                                              // wave uniform
+    constexpr int DW = 64 * W;                                           // the head dim
     const long long at = (static_cast<long long>(first) * Hkv + head) * rows + row;
-    float2 sum = make_float2(0.f, 0.f);
+    float sum[W];
+#pragma unroll
+    for (int k = 0; k < W; ++k) sum[k] = 0.f;
     float top, total;
     if (count == 1) {
       const float2 st = *reinterpret_cast<const float2*>(ml + 2 * at);
       top = st.x; total = st.y;
-      if (top != -INFINITY) sum = *reinterpret_cast<const float2*>(opart + at * D + 2 * lane);
+      if (top != -INFINITY) ldw<W>(opart + at * DW + W * lane, sum);
     } else {
       top = -INFINITY; total = 0.f;
       for (int s0 = 0; s0 < count; s0 += 64)
@@ -977,23 +554,26 @@ __global__ void __launch_bounds__(256) k_fold_items(const int* __restrict__ tile
           for (int s = 0; s < n; ++s) {
             const float w = __shfl(weight, s, 64);
             if (w == 0.f) continue;                                      // an item that saw no key: nothing to read
-            const float2 x = *reinterpret_cast<const float2*>(opart + (at + (s0 + s) * per_item) * D + 2 * lane);
-            sum.x += w * x.x; sum.y += w * x.y;
+            float x[W];
+            ldw<W>(opart + (at + (s0 + s) * per_item) * DW + W * lane, x);
+#pragma unroll
+            for (int k = 0; k < W; ++k) sum[k] += w * x[k];
           }
         }
       }
     }
     if (top != -INFINITY) {
       const float inv = 1.f / total;
-      sum.x *= inv; sum.y *= inv;
+#pragma unroll
+      for (int k = 0; k < W; ++k) sum[k] *= inv;
     }
     const int token = row / G, qhead = head * G + row % G;
     if (FP32_OUT) {                                                      // compact rows, dense [m, Hq, D]
-      float* dst = static_cast<float*>(out) + (static_cast<long long>(rec[1] + token) * Hkv * G + qhead) * D;
-      *reinterpret_cast<float2*>(dst + 2 * lane) = sum;
+      float* dst = static_cast<float*>(out) + (static_cast<long long>(rec[1] + token) * Hkv * G + qhead) * DW;
+      stw<W>(dst + W * lane, sum);
     } else {                                                             // rows of the layer output
-      uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(rec[2] + token) * out_stride + qhead * D;
-      *reinterpret_cast<uint32_t*>(dst + 2 * lane) = bf16_rn(sum.x) | (bf16_rn(sum.y) << 16);
+      uint16_t* dst = static_cast<uint16_t*>(out) + static_cast<long long>(rec[2] + token) * out_stride + qhead * DW;
+      stw_bf16<W>(dst + W * lane, sum);
     }
     if (lse != nullptr && lane == 0)
       lse[qhead * lse_stride + rec[1] + token] = top == -INFINITY ? -INFINITY : (top + log2f(total)) * 0.6931471805599453f;
@@ -1081,47 +661,50 @@ __global__ void __launch_bounds__(256) k_collect_rows(const long long* __restric
 // An lse of +-inf or NaN means the part is empty.  S <= 64.
 DEVI bool usable(float lse) { return lse == lse && lse != INFINITY && lse != -INFINITY; }
 
+template <int W>
 __global__ void __launch_bounds__(256) k_mix_parts(int m, int Hq, int Hkv, const uint16_t* __restrict__ q, long long q_stride,
                                                    const long long* __restrict__ out_row, const float* __restrict__ o_pages,
                                                    const float* __restrict__ lse_pages, const uint16_t* __restrict__ o_win,
                                                    const float* __restrict__ lse_win, const uint16_t* __restrict__ sinks,
                                                    const long long* __restrict__ req_of, const long long* __restrict__ pos_of,
-                                                   const long long* __restrict__ sink_len, int S, int W, float scale,
+                                                   const long long* __restrict__ sink_len, int S, int W_keep, float scale,
                                                    uint16_t* __restrict__ out, long long out_stride) {
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6);
   if (head >= Hq) return;
+  constexpr int DW = 64 * W;                     // the head dim: W channels per lane
   const int kv = head / (Hq / Hkv);
-  const long long dst_row = out_row[c], flat = (static_cast<long long>(c) * Hq + head) * D + 2 * lane;
+  const long long dst_row = out_row[c], flat = (static_cast<long long>(c) * Hq + head) * DW + W * lane;
 
   float lp = lse_pages[static_cast<long long>(head) * m + c];
-  float2 vp = make_float2(0.f, 0.f);
-  if (usable(lp)) vp = *reinterpret_cast<const float2*>(o_pages + flat); else lp = -INFINITY;
+  float vp[W], vw[W], vs[W];
+#pragma unroll
+  for (int k = 0; k < W; ++k) vp[k] = vw[k] = vs[k] = 0.f;
+  if (usable(lp)) ldw<W>(o_pages + flat, vp); else lp = -INFINITY;
 
   float lw = -INFINITY;
-  float2 vw = make_float2(0.f, 0.f);
   if (o_win != nullptr) {
     const float l = lse_win[static_cast<long long>(head) * m + c];
-    if (usable(l)) {
-      const uint32_t raw = *reinterpret_cast<const uint32_t*>(o_win + flat);
-      lw = l; vw = make_float2(bf16_lo(raw), bf16_hi(raw));
-    }
+    if (usable(l)) { lw = l; ldw_bf16<W>(o_win + flat, vw); }
   }
 
   float ls = -INFINITY;
-  float2 vs = make_float2(0.f, 0.f);
   if (sinks != nullptr) {
     const long long req = req_of[c];
-    const int n = static_cast<int>(min(min(static_cast<long long>(S), sink_len[req]), pos_of[c] - W + 1));
+    const int n = static_cast<int>(min(min(static_cast<long long>(S), sink_len[req]), pos_of[c] - W_keep + 1));
     if (n > 0) {
-      const uint32_t qraw = *reinterpret_cast<const uint32_t*>(q + dst_row * q_stride + static_cast<long long>(head) * D + 2 * lane);
-      const float q0 = bf16_lo(qraw), q1 = bf16_hi(qraw);
-      const uint16_t* base = sinks + (req * S * 2 * Hkv + kv) * D + 2 * lane;       // K head kv of sink row 0
-      const long long step = 2LL * Hkv * D, to_v = static_cast<long long>(Hkv) * D;
+      float qv[W];
+      ldw_bf16<W>(q + dst_row * q_stride + static_cast<long long>(head) * DW + W * lane, qv);
+      const uint16_t* base = sinks + (req * S * 2 * Hkv + kv) * DW + W * lane;      // K head kv of sink row 0
+      const long long step = 2LL * Hkv * DW, to_v = static_cast<long long>(Hkv) * DW;
       float mine = -INFINITY;                                                      // lane j: score of key j
       for (int j = 0; j < n; ++j) {
-        const uint32_t kraw = *reinterpret_cast<const uint32_t*>(base + j * step);
-        const float sc = wave_sum64(q0 * bf16_lo(kraw) + q1 * bf16_hi(kraw)) * scale;
+        float kk[W];
+        ldw_bf16<W>(base + j * step, kk);
+        float dot = 0.f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) dot += qv[k] * kk[k];
+        const float sc = wave_sum64(dot) * scale;
         if (lane == j) mine = sc;
       }
       const float top = wave_max64(mine);
@@ -1129,25 +712,29 @@ __global__ void __launch_bounds__(256) k_mix_parts(int m, int Hq, int Hkv, const
       const float mass = wave_sum64(p);
       for (int j = 0; j < n; ++j) {
         const float w = __shfl(p, j, 64);
-        const uint32_t vraw = *reinterpret_cast<const uint32_t*>(base + j * step + to_v);
-        vs.x += w * bf16_lo(vraw); vs.y += w * bf16_hi(vraw);
+        float vv[W];
+        ldw_bf16<W>(base + j * step + to_v, vv);
+#pragma unroll
+        for (int k = 0; k < W; ++k) vs[k] += w * vv[k];
       }
-      vs.x /= mass; vs.y /= mass;
+#pragma unroll
+      for (int k = 0; k < W; ++k) vs[k] /= mass;
       ls = top + logf(mass);
     }
   }
 
   const float top = fmaxf(lp, fmaxf(lw, ls));
-  float2 o = make_float2(0.f, 0.f);
+  float o[W];
+#pragma unroll
+  for (int k = 0; k < W; ++k) o[k] = 0.f;
   if (top != -INFINITY) {
     const float wp = lp == -INFINITY ? 0.f : expf(lp - top), ww = lw == -INFINITY ? 0.f : expf(lw - top),
                 wsk = ls == -INFINITY ? 0.f : expf(ls - top);
     const float inv = 1.f / (wp + ww + wsk);
-    o.x = (wp * vp.x + ww * vw.x + wsk * vs.x) * inv;
-    o.y = (wp * vp.y + ww * vw.y + wsk * vs.y) * inv;
+#pragma unroll
+    for (int k = 0; k < W; ++k) o[k] = (wp * vp[k] + ww * vw[k] + wsk * vs[k]) * inv;
   }
-  *reinterpret_cast<uint32_t*>(out + dst_row * out_stride + static_cast<long long>(head) * D + 2 * lane) =
-      bf16_rn(o.x) | (bf16_rn(o.y) << 16);
+  stw_bf16<W>(out + dst_row * out_stride + static_cast<long long>(head) * DW + W * lane, o);
 }
 
 template <int QM, bool K2, int NW> int launch_mq(const Params& p, int nitems, hipStream_t st) {
@@ -1190,13 +777,17 @@ extern "C" {
 
 int frmq_abi_version(void) { return 7; }
 const char* frmq_last_error(void) { return g_err; }
-int frmq_smem_bytes(void) { return static_cast<int>(sizeof(Smem8) > sizeof(Smem) ? sizeof(Smem8) : sizeof(Smem)); }
+int frmq_smem_bytes(void) {
+  const int a = static_cast<int>(sizeof(Smem8) > sizeof(Smem) ? sizeof(Smem8) : sizeof(Smem)), b = wide_smem_bytes();
+  return a > b ? a : b;
+}
 
 int frmq_prep_q(const void* q, int q_fp32, long long q_ts, const int* idx, int m, int Hq, int G, const uint8_t* kfull,
                 const uint8_t* kmask, float qscale, void* q16, int Dh, void* stream) {
   if (m <= 0) return 0;
-  if (Dh != D) return bad(-4, "frmq_prep_q: head dim 128 only");
+  if (Dh != D && Dh != 256) return bad(-4, "frmq_prep_q: head dim 128 or 256");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (Dh == 256) return done(wide_query_rows_launch(q, q_fp32, q_ts, idx, m, Hq, G, kfull, kmask, qscale, q16, st), "frmq_prep_q");
   uint16_t* dst = static_cast<uint16_t*>(q16);
   if (q_fp32) hipLaunchKernelGGL(k_query_rows<float>, dim3(m), dim3(256), 0, st, static_cast<const float*>(q), q_ts, idx, Hq, G,
                                  kfull, kmask, qscale, dst);
@@ -1209,9 +800,9 @@ int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const
               const int* tiles, const int* items, int nitems, int Hkv, int G, int shift, int konly, float* opart,
               float* ml, int kernel, int Dh, void* stream, int kmin) {
   if (nitems <= 0) return 0;
-  const int rows = kernel == 1 ? 64 : kernel == 4 ? 256 : 128;
+  if (Dh != D && Dh != 256) return bad(-4, "frmq_attn: head dim 128 or 256");
+  const int rows = Dh == 256 ? 128 : kernel == 1 ? 64 : kernel == 4 ? 256 : 128;     // head dim 256: one kernel, 128 rows
   if (G < 1 || G > rows) return bad(-3, "frmq_attn: G out of range");
-  if (Dh != D) return bad(-4, "frmq_attn: head dim 128 only");
   if (kernel < 1 || kernel > 4) return bad(-2, "frmq_attn: kernel must be 1, 2, 3 or 4");
   Params p{};
   p.q = static_cast<const uint16_t*>(q16); p.pool = pool; p.page_stride = page_stride; p.bt = bt; p.bt_stride = bt_stride;
@@ -1219,7 +810,9 @@ int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool k2 = konly & 1, i2 = konly & 2;
   int rc;
-  if (rows == 256) {
+  if (Dh == 256) {
+    rc = wide_attn_launch(p, nitems, konly, st);
+  } else if (rows == 256) {
     rc = i2 ? (k2 ? launch_mq8<QM_ASYM2, true>(p, nitems, st) : launch_mq8<QM_ASYM2, false>(p, nitems, st))
             : (k2 ? launch_mq8<QM_ASYM4, true>(p, nitems, st) : launch_mq8<QM_ASYM4, false>(p, nitems, st));
   } else if (rows == 64) {
@@ -1235,19 +828,20 @@ int frmq_attn(const void* q16, const uint8_t* pool, long long page_stride, const
 int frmq_merge(const int* tiles, int ntiles, const float* opart, const float* ml, int Hkv, int G, int rows, void* out,
                long long o_ts, int out_fp32, float* lse, long long lse_ts, int Dh, void* stream) {
   if (ntiles <= 0) return 0;
-  if (Dh != D) return bad(-4, "frmq_merge: head dim 128 only");
+  if (Dh != D && Dh != 256) return bad(-4, "frmq_merge: head dim 128 or 256");
   const dim3 grid(ntiles, Hkv, (rows + 4 * FOLD_ROWS - 1) / (4 * FOLD_ROWS));      // four wavefronts x FOLD_ROWS rows per workgroup
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (out_fp32) hipLaunchKernelGGL(k_fold_items<true>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
-  else hipLaunchKernelGGL(k_fold_items<false>, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
+  const auto kern = Dh == 256 ? (out_fp32 ? k_fold_items<true, 4> : k_fold_items<false, 4>)
+                              : (out_fp32 ? k_fold_items<true, 2> : k_fold_items<false, 2>);
+  hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, tiles, opart, ml, Hkv, G, rows, out, o_ts, lse, lse_ts);
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_merge");
 }
 
 int frmq_win_gather(const long long* map, int nk, const void* sinkb, const void* preb, const void* kch, long long k_ts,
                     const void* vch, long long v_ts, int Hkv, void* kw, void* vw, int Dh, void* stream) {
   if (nk <= 0) return 0;
-  if (Dh != D) return bad(-4, "frmq_win_gather: head dim 128 only");
-  const int pieces = Hkv * D / 8;                          // 16-byte pieces of one K (or V) row
+  if (Dh != D && Dh != 256) return bad(-4, "frmq_win_gather: head dim 128 or 256");
+  const int pieces = Hkv * Dh / 8;                         // 16-byte pieces of one K (or V) row
   const long long total = static_cast<long long>(nk) * pieces;
   hipLaunchKernelGGL(k_collect_rows, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), map, nk, static_cast<const uint4*>(sinkb), static_cast<const uint4*>(preb),
@@ -1261,10 +855,11 @@ int frmq_bf_merge(int m, int Hq, int Hkv, const void* q, long long q_ts, const l
                   const long long* row_pos, const long long* sk_len, int S, int W, float scale, void* out, long long o_ts,
                   int Dh, void* stream) {
   if (m <= 0) return 0;
-  if (Dh != D) return bad(-4, "frmq_bf_merge: head dim 128 only");
+  if (Dh != D && Dh != 256) return bad(-4, "frmq_bf_merge: head dim 128 or 256");
   if (sk != nullptr && S > 64) return bad(-5, "frmq_bf_merge: at most 64 sink tokens");
   using U = uint16_t;
-  hipLaunchKernelGGL(k_mix_parts, dim3(m, (Hq + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), m, Hq, Hkv,
+  const auto kern = Dh == 256 ? k_mix_parts<4> : k_mix_parts<2>;
+  hipLaunchKernelGGL(kern, dim3(m, (Hq + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), m, Hq, Hkv,
                      static_cast<const U*>(q), q_ts, idx, o_p, lse_p, static_cast<const U*>(o_w), lse_w,
                      static_cast<const U*>(sk), row_req, row_pos, sk_len, S, W, scale, static_cast<U*>(out), o_ts);
   return done(hipPeekAtLastError() == hipSuccess ? 0 : -1, "frmq_bf_merge");

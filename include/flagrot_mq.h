@@ -4,7 +4,8 @@
  * Drop-in for the entry points the reference plugin binds with ctypes (integrations/vllm_flagrot/vllm_flagrot/
  * prefill_mq.py:57-86 of the reference; definitions in integrations/vllm_flagrot/csrc/mq_prefill.cu:1469-1601).  Raw
  * device pointers, `stream` is a hipStream_t, asynchronous, no allocation.  Return codes: 0 ok, -1 launch failure,
- * -2 bad kernel selector, -3 bad G, -4 unsupported head dim (128 only).  frmq_last_error() returns this library's
+ * -2 bad kernel selector, -3 bad G, -4 unsupported head dim (128 and 256 are built; at 256 one kernel
+ * with 128-row tiles serves every selector, like the reference's k_mq3).  frmq_last_error() returns this library's
  * last message.
  *
  * Plan buffers (host planner, prefill_mq.py:128-210): tiles int32 [nt][9] = (block-table row, compact row0, output

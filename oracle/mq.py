@@ -41,9 +41,10 @@ def _butterflies(x: np.ndarray, n: int) -> np.ndarray:
 
 
 def prep_q(q, G: int, qscale: float, idx=None, kfull=None, kmask=None) -> np.ndarray:
-    """q fp32 values [n, Hq, 128] (bf16 inputs are passed as their exact fp32 values) -> fp16 bit patterns
-    [m, Hq, 128]: rows idx; whole-head unnormalised H128 times 0.125 where kfull[kv head]; orthonormal H32 on the
-    groups kmask[kv head, g]; times fp32(qscale); every step rounded to fp32, one final rounding to fp16."""
+    """q fp32 values [n, Hq, D] (bf16 inputs are passed as their exact fp32 values) -> fp16 bit patterns
+    [m, Hq, D]: rows idx; whole-head unnormalised H_D times 0.125 (D = 128) or 0.0625 (D = 256; mq_prefill.cu:1319-1323)
+    where kfull[kv head]; orthonormal H32 on the groups kmask[kv head, g]; times fp32(qscale); every step rounded to
+    fp32, one final rounding to fp16."""
     x = np.asarray(q, dtype=F32)
     if idx is not None:
         x = x[np.asarray(idx, dtype=np.int64)]
@@ -51,7 +52,7 @@ def prep_q(q, G: int, qscale: float, idx=None, kfull=None, kmask=None) -> np.nda
     hk = np.arange(Hq) // G
     if kfull is not None:
         f = np.asarray(kfull).astype(bool)[hk]
-        full = (_butterflies(x, D) * F32(0.125)).astype(F32)
+        full = (_butterflies(x, D) * F32(0.125 if D == 128 else 0.0625)).astype(F32)
         x = np.where(f[None, :, None], full, x)
     if kmask is not None:
         km = np.asarray(kmask).astype(bool).reshape(-1, D // 32)[hk]                # [Hq, 4]

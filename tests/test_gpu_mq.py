@@ -223,7 +223,7 @@ def test_prep_q_fp32_rows_and_rejects(dev):
     got = MQ.prep_q(q.to(dev), 1.7, G).cpu().view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(got, OM.prep_q(q.numpy(), G, 1.7))
     L = MQ.lib()
-    assert L.frmq_attn(None, None, 0, None, 0, None, None, 1, 2, 4, 0, 0, None, None, 3, 256, None, 0) == -4
+    assert L.frmq_attn(None, None, 0, None, 0, None, None, 1, 2, 4, 0, 0, None, None, 3, 64, None, 0) == -4
     assert L.frmq_attn(None, None, 0, None, 0, None, None, 1, 2, 200, 0, 0, None, None, 3, 128, None, 0) == -3
     assert b"head dim" in L.frmq_last_error() or b"G out" in L.frmq_last_error()
     assert L.frmq_smem_bytes() > 0
