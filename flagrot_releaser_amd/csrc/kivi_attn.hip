@@ -59,12 +59,10 @@ int kv_v_write(const void* kv, long long kv_rs, int n, int Hkv, int D, const voi
                void* pool, int ident, const void* vfix, int f8, void* stream) {
   if (n <= 0) return 0;
   if (D != 128 && D != 256) return bad("kv_v_write: head dim 128 or 256");
-  if (D == 256) {
-    if (M != nullptr && !ident && vfix == nullptr) return bad("kv_v_write: the matrix weight M is built for head dim 128 only");
+  if (D == 256)
     return launched(v_write256_launch(kv, kv_rs, n, Hkv, static_cast<const long long*>(slots), static_cast<const float*>(co),
-                                      static_cast<uint8_t*>(pool), ident, static_cast<const int*>(vfix), f8 & 1,
-                                      static_cast<hipStream_t>(stream)), "kv_v_write");
-  }
+                                      static_cast<uint8_t*>(pool), static_cast<const float*>(M), ident,
+                                      static_cast<const int*>(vfix), f8 & 1, static_cast<hipStream_t>(stream)), "kv_v_write");
   return launched(v_write_launch(kv, kv_rs, n, Hkv, static_cast<const long long*>(slots), static_cast<const float*>(co),
                                  static_cast<uint8_t*>(pool), static_cast<const float*>(M), ident, static_cast<const int*>(vfix), f8 & 1,
                                  static_cast<hipStream_t>(stream)), "kv_v_write");

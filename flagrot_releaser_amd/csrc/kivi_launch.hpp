@@ -23,7 +23,7 @@ int attn_splits_launch(int G, const void* q, long long q_rs, const void* pool, c
 
 
 int v_write256_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
-                      int ident, const int* vfix, int f8, hipStream_t st);
+                      const float* M, int ident, const int* vfix, int f8, hipStream_t st);
 int k_encode256_launch(const void* src, long long src_rs, const void* src2, long long src2_rs, const long long* sidx,
                        const long long* dslot, int N, int Hkv, const float* qs, const float* lz, int NQ, float qsc,
                        uint8_t* pool, int ident, const int* kfix, int f8, hipStream_t st);

@@ -70,10 +70,17 @@ template <bool F8> DEVI bool value_whole(const uint8_t* chunk, int cell) {
 }
 
 // ------------------------------------------------------------------------------------------------ value writer
-template <bool F8>
+// WMAT: the selection weighs the error vectors by a full matrix per head (e^T M e; kivi.cu:213-287) as the 128-d
+// writer's matrix form does: the diagonal 32-block for a sub-vector's choice, all of M for the whole-head candidate and
+// for the combination.  The three error vectors of a row sit in an LDS strip per half wave; a lane forms the products
+// of its eight rows of M.
+template <bool F8, bool WMAT>
 __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__ kv, long long kv_rs, int n, int Hkv,
                                                     const long long* __restrict__ slots, const float* __restrict__ co,
-                                                    uint8_t* __restrict__ pool, int ident, const int* __restrict__ vfix) {
+                                                    const float* __restrict__ M, uint8_t* __restrict__ pool, int ident,
+                                                    const int* __restrict__ vfix) {
+  constexpr int EW = WMAT ? D2 : 1;                       // the strips exist only in the matrix-weighted kernel
+  __shared__ float esh[WMAT ? 8 : 1][3][EW];
   const int l32 = threadIdx.x & 31;
   const long long item = static_cast<long long>(blockIdx.x) * 8 + (threadIdx.x >> 5);
   if (item >= static_cast<long long>(n) * Hkv) return;
@@ -87,7 +94,7 @@ __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__
     const float4 c4 = *reinterpret_cast<const float4*>(co + h * D2 + 128 * s + 4 * l32);
     cw[s][0] = c4.x; cw[s][1] = c4.y; cw[s][2] = c4.z; cw[s][3] = c4.w;
   }
-  float sc[3][2], mnv[3][2], err[3][2];
+  float sc[3][2], mnv[3][2], err[3][2], dv[3][2][4];
   int code[3][2][4];
 #pragma unroll
   for (int c = 0; c < 3; ++c) {
@@ -114,7 +121,7 @@ __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__
     for (int s = 0; s < 2; ++s) {
       float e = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { const float d = y[s][i] - x[s][i]; e += d * d * cw[s][i]; }
+      for (int i = 0; i < 4; ++i) { const float d = y[s][i] - x[s][i]; dv[c][s][i] = d; e += d * d * cw[s][i]; }
       err[c][s] = e;
     }
   }
@@ -122,7 +129,57 @@ __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__
   bool useH0, useH1, useF;
   if (ident) { useH0 = useH1 = useF = false; }
   else if (vfix != nullptr) { useF = (vfix[h] >> 16) & 1; useH0 = (vfix[h] >> j) & 1; useH1 = (vfix[h] >> (4 + j)) & 1; }
-  else {
+  else if constexpr (WMAT) {
+    float (*E)[EW] = esh[threadIdx.x >> 5];
+    const float* Mh = M + static_cast<long long>(h) * D2 * D2;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) E[c][128 * s + 4 * l32 + i] = dv[c][s][i];
+    wave_lds_sync();
+    float eI[2] = {0.f, 0.f}, eH[2] = {0.f, 0.f}, eF = 0.f;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
+        const int k0 = 128 * s + 32 * j;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+        for (int k = k0; k < k0 + 32; ++k) { const float m = row[k]; a0 += m * E[0][k]; a1 += m * E[1][k]; }
+        for (int k = 0; k < D2; ++k) a2 += row[k] * E[2][k];
+        eI[s] += dv[0][s][i] * a0; eH[s] += dv[1][s][i] * a1; eF += dv[2][s][i] * a2;
+      }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      eI[s] += hx(eI[s], 1); eI[s] += hx(eI[s], 2); eI[s] += hx(eI[s], 4);
+      eH[s] += hx(eH[s], 1); eH[s] += hx(eH[s], 2); eH[s] += hx(eH[s], 4);
+    }
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
+    useH0 = eH[0] < eI[0]; useH1 = eH[1] < eI[1];          // identity on ties
+    wave_lds_sync();                                       // every lane has read the strips
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+      if (s ? useH1 : useH0)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) E[0][128 * s + 4 * l32 + i] = dv[1][s][i];
+    wave_lds_sync();
+    float eB = 0.f;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
+        float a = 0.f;
+        for (int k = 0; k < D2; ++k) a += row[k] * E[0][k];
+        eB += ((s ? useH1 : useH0) ? dv[1][s][i] : dv[0][s][i]) * a;
+      }
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
+    useF = eF < eB;                                        // base on ties
+  } else {
     float eI0 = err[0][0], eI1 = err[0][1], eH0 = err[1][0], eH1 = err[1][1], eF = err[2][0] + err[2][1];
     eI0 += hx(eI0, 1); eI0 += hx(eI0, 2); eI0 += hx(eI0, 4);
     eI1 += hx(eI1, 1); eI1 += hx(eI1, 2); eI1 += hx(eI1, 4);
@@ -720,11 +777,13 @@ template <typename K> bool carve(K kern, size_t bytes) {
 }  // namespace
 
 int v_write256_launch(const void* kv, long long kv_rs, int n, int Hkv, const long long* slots, const float* co, uint8_t* pool,
-                      int ident, const int* vfix, int f8, hipStream_t st) {
+                      const float* M, int ident, const int* vfix, int f8, hipStream_t st) {
   const long long items = static_cast<long long>(n) * Hkv;
-  const auto kern = f8 ? k_v_write256<true> : k_v_write256<false>;
+  const bool wmat = M != nullptr && !ident && vfix == nullptr;
+  const auto kern = wmat ? (f8 ? k_v_write256<true, true> : k_v_write256<false, true>)
+                         : (f8 ? k_v_write256<true, false> : k_v_write256<false, false>);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>((items + 7) / 8)), dim3(256), 0, st, static_cast<const uint16_t*>(kv),
-                     kv_rs, n, Hkv, slots, co, pool, ident, vfix);
+                     kv_rs, n, Hkv, slots, co, M, pool, ident, vfix);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 

@@ -9,7 +9,7 @@
  * at 256 a chunk has eight sub-vectors and key cells of eight channels, and kv_attn serves G <= 8 with a plain fp32
  * kernel), FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3 scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes
  * computed from the stored values, the value rows' whole-head flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88,
- * 123-128), diagonal (co) value weighting at both head dims and matrix (M) weighting at head dim 128 (M at 256: 2).
+ * 123-128), diagonal (co) and matrix (M) value weighting at both head dims.
  */
 #ifndef FLAGROT_KIVI_H
 #define FLAGROT_KIVI_H

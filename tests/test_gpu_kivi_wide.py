@@ -79,20 +79,49 @@ def test_v_write_pinned_modes(dev, mode, f8):
     assert np.array_equal(pool.cpu().numpy(), want)
 
 
-def test_v_write_matrix_weight_is_refused(dev):
-    """the full-matrix selection weight exists at head dim 128 only: asked for at 256 the library says so instead of
-    falling back to the diagonal weight; with ident or fix the matrix is ignored, as at 128"""
+@F8
+def test_v_write_matrix_weight(dev, f8):
+    """the value selection weighted by a full 256 x 256 matrix per head (e^T M e; kivi.cu:213-287): bytes equal to the
+    oracle's given the stored flags, a different choice only inside the fp64 margin; M = diag(co) writes what the
+    diagonal criterion writes (up to choices inside the margin); ident ignores M"""
     from flagrot_releaser_amd import kivi as KV
-    Hkv = 2
-    kv = torch.zeros(4, 2 * Hkv, D, dtype=torch.bfloat16, device=dev)
-    slots = torch.arange(4, device=dev)
-    co = torch.ones(Hkv, D, device=dev)
-    M = torch.eye(D, device=dev).repeat(Hkv, 1, 1).contiguous()
-    pool = torch.zeros(1, Hkv, _cb(False, D), dtype=torch.uint8, device=dev)
-    with pytest.raises(RuntimeError, match="matrix weight"):
-        KV.v_write(kv, slots, co, M, pool, Hkv, D)
-    KV.v_write(kv, slots, co, M, pool, Hkv, D, ident=True)
-    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(17)
+    T, Hkv = 120, 3
+    kv = _kv(T, Hkv, g, hd=D)
+    _, _, co = _calib(Hkv, 8, g, hd=D)
+    A = torch.randn(Hkv, D, D, generator=g) * 0.15
+    M = (A @ A.transpose(1, 2) + torch.diag_embed(co)).contiguous()
+    npg = (T + 15) // 16 + 1
+    slots = torch.randperm(npg * 16, generator=g)[:T].long()
+    xb = bits(kv)[:, Hkv:]
+    for Mx, name in ((M, "dense"), (torch.diag_embed(co).contiguous(), "diagonal")):
+        pool = torch.zeros(npg, Hkv, _cb(f8, D), dtype=torch.uint8, device=dev)
+        KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), Mx.to(dev), pool, Hkv, D, f8=f8)
+        torch.cuda.synchronize()
+        got = pool.cpu().numpy()
+        enc = OK.v_encode(xb, co.numpy(), f8=f8, M=Mx.numpy())
+        sH, sF = _stored_value_flags(got, f8, hd=D)
+        sl = slots.numpy()
+        useH, useF = sH[sl // 16, :, sl % 16], sF[sl // 16, :, sl % 16]
+        want = np.zeros_like(got)
+        OK.pack_values(want, sl, *OK.v_stored(enc, useH, useF, f8=f8), f8=f8)
+        assert np.array_equal(got, want), name
+        badF = useF != enc["useF"]
+        badH = (useH != enc["useH"]) & ~useF[..., None] & ~enc["useF"][..., None]
+        assert (enc["marginF"][badF] < 1e-3).all() and (enc["marginH"][badH] < 1e-3).all(), name
+        assert badF.mean() < 0.02 and badH.mean() < 0.02
+        if name == "diagonal":
+            ref = torch.zeros_like(pool)
+            KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, ref, Hkv, D, f8=f8)
+            assert (ref != pool).any(dim=-1).float().mean().item() < 0.05
+        else:
+            dg = OK.v_encode(xb, co.numpy(), f8=f8)
+            assert (dg["useH"] != enc["useH"]).any()               # the dense matrix does change choices
+    pool = torch.zeros(npg, Hkv, _cb(f8, D), dtype=torch.uint8, device=dev)
+    ref = torch.zeros_like(pool)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), M.to(dev), pool, Hkv, D, ident=True, f8=f8)
+    KV.v_write(kv.to(dev), slots.to(dev), co.to(dev), None, ref, Hkv, D, ident=True, f8=f8)
+    assert torch.equal(pool, ref)
 
 
 @F8
