@@ -392,6 +392,16 @@ def run_kivi(args, torch, dev, steps, warmup):
     ref = OK.attention_reference(qf, Kd, Vd, 0, Lp, rg[:, :HKV], rg[:, HKV:], Gq, 1 / math.sqrt(DH))
     got = out[b].view(Gq * HKV, DH).float().cpu().numpy().astype(np.float64)
     st = error_stats(got, ref)
+    # the prefill support path: one sequence's whole paged prefix back to bf16 K and V (kv_dequant), eager launches
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(13):
+        if i == 3:
+            e0.record()
+        KV.dequant_cuda(pools[i % ncopy], bt[i % B], 0, Lp, HKV, DH, f8=f8)
+    e1.record()
+    torch.cuda.synchronize()
+    dq_us = e0.elapsed_time(e1) / 10 * 1e3
+    dq_bytes = Lp * HKV * (CB // P) + 2 * Lp * HKV * DH * 2
     return {"workload": name, "us_per_layer_step": round(us, 2), "GBps": round(gbps, 1),
             "frac": round(gbps / PEAK_HBM_GBPS, 4), "nsplit": ns, "chunk": ch,
             "graph_min_us": round(t["graph_min_us"], 2), "graph_max_us": round(t["graph_max_us"], 2),
@@ -401,6 +411,9 @@ def run_kivi(args, torch, dev, steps, warmup):
             "errors": st, "check": f"sequence {b} x all {Gq * HKV} heads vs fp64 attention over the oracle's dequantised "
                                    "pages: " + describe(st),
             "note": "one step = kv_attn = the split kernel + the merge kernel",
+            "dequant": {"tokens": Lp, "us": round(dq_us, 1), "GBps": round(dq_bytes / (dq_us * 1e-6) / 1e9, 1),
+                        "note": "kv_dequant of one sequence's paged prefix to bf16 K and V (page bytes read + rows "
+                                "written), eager, includes torch's allocation of the two outputs"},
             "writer": {"prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * Lp,
                        "note": f"value writer + key group encoder ({NQ} calibration queries), includes synthetic input generation"}}
 
@@ -557,8 +570,9 @@ def main():
                             "avg_launch_us": r["us_per_layer_step"], "graph_min_us": r["graph_min_us"],
                             "graph_max_us": r["graph_max_us"], "eager_us": r["eager_us"]},
                "checked": r["checked"], "bar": r["bar"], "errors": r["errors"], "check": r["check"]}
-        if "writer" in r:
-            res["writer"] = r["writer"]
+        for extra in ("writer", "dequant"):
+            if extra in r:
+                res[extra] = r[extra]
         if workload == "int4" and extras:
             ref = rr["reference"]
             res["reference_planner"] = {k: ref[k] for k in ("nsplit", "chunk", "us_per_layer_step", "frac", "eager_us", "checked")}
