@@ -51,7 +51,7 @@ def decode_plan(kind: str, B: int, max_len: int, Hkv: int, G: int = 4, Dh: int =
     """(nsplit, chunk) of a decode batch of B rows: fixed per (batch bucket, longest context), no device sync."""
     Bp = plan_bucket(B)
     if kind == "kivi2":
-        return KIVI.plan(Bp, max_len, Hkv)
+        return KIVI.plan(Bp, max_len, Hkv, D=Dh)
     if is_static(kind):
         return K.plan_v2(Bp, max_len, Hkv, PAGE, fmt=kind, G=G, Dh=Dh)
     return K.plan_cb(Bp, max_len, Hkv, PAGE, kind, G=G, Dh=Dh)

@@ -1,0 +1,44 @@
+// Pieces shared by the two matrix-pipe decode kernels over KIVI-style pages (head dim 128: kivi_decode.hip, head dim
+// 256: kivi_decode_wide.hip): packed-fp16 helpers, global loads through the global address space, and the strip
+// geometry (a strip row serves 128 channels = 64 fp16 pairs; the 256-d kernel works through its head in two halves).
+#pragma once
+#include "fr_common.hpp"
+
+namespace frkv {
+namespace mma {
+using namespace fr;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+DEVI float dot2(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+}
+DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+DEVI uint32_t pk_mul(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, a) * __builtin_bit_cast(half2_t, b));
+}
+DEVI uint32_t pk_fma(uint32_t a, uint32_t b, uint32_t c) {      // a * b + c per half, one rounding
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b),
+                                                                __builtin_bit_cast(half2_t, c)));
+}
+DEVI uint32_t pack_rn(float a, float b) {
+  half2_t v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <class T> DEVI T gload(const uint8_t* p) {
+  typedef const __attribute__((address_space(1))) T* gp;
+  return *(gp)(p);
+}
+constexpr uint32_t X256 = 0x5C005C00u;                                         // fp16 pair (256, 256)
+constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
+constexpr int QROW = 68;                        // words per row of the query strips and tables: 64 + 4 pad (conflict-free 128-bit rows)
+constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+}  // namespace mma
+}  // namespace frkv

@@ -6,8 +6,7 @@
  * 49-77 of the reference; definitions in integrations/vllm_flagrot/csrc/kivi.cu:1933-2342).  Raw device pointers,
  * `stream` is a hipStream_t, asynchronous, no allocation.  Return codes: 0 ok, 1 launch failure, 2 bad / unsupported
  * argument (message from kv_last_error()).  Built for head dim 128 and 256 (kivi.cu's <128> and <256> instantiations;
- * at 256 a chunk has eight sub-vectors and key cells of eight channels, and kv_attn serves G <= 8 with a plain fp32
- * kernel), FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3 scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes
+ * at 256 a chunk has eight sub-vectors and key cells of eight channels; kv_attn serves G <= 8 at both head dims), FP16 scale / min pages (f8 bit 0 clear) and FP8 E4M3 scale / min pages (f8 bit 0 set: 10 D-byte chunks, codes
  * computed from the stored values, the value rows' whole-head flags in bit 7 of key scale bytes; kivi.cu:28-35, 84-88,
  * 123-128), diagonal (co) and matrix (M) value weighting at both head dims.
  */

@@ -240,6 +240,40 @@ def test_attn_against_fp64(dev, case, f8):
     assert (outbuf[:, Hq * D:] == 7.0).all()
 
 
+def test_attn_plain_kernel_switch(dev, monkeypatch):
+    """FLAGROT_KIVI_WIDE_PLAIN=1 (read at every call) sends the page splits through the plain fp32 kernel as well: same
+    partial format, same merge, outputs within the bar of each other and of the fp64 reference"""
+    from flagrot_releaser_amd import kivi as KV
+    lens, Hkv, G, kv_start, (ns, chunk), tails = CASES[2]
+    g = torch.Generator().manual_seed(77)
+    B, Hq = len(lens), Hkv * G
+    pool, bt, Ks, Vs = _filled_cache(dev, lens, Hkv, g, hd=D)
+    T = 128
+    ring = (torch.randn((B + 2) * T, 2 * Hkv, D, generator=g) * 1.5).bfloat16()
+    tail_idx = torch.arange(B, dtype=torch.int32)
+    tail_len = torch.tensor(tails, dtype=torch.int32)
+    cached = torch.tensor(lens, dtype=torch.int32)
+    q = (torch.randn(B, Hq, D, generator=g) * 1.2).bfloat16()
+    ws = KV.Workspace(B * Hkv * (ns + 1), G, D, dev)
+    scale = 1 / math.sqrt(D)
+    outs = []
+    for plain in ("0", "1"):
+        monkeypatch.setenv("FLAGROT_KIVI_WIDE_PLAIN", plain)
+        out = torch.zeros(B, Hq * D, dtype=torch.bfloat16, device=dev)
+        KV.attn(q.to(dev), pool, bt.to(dev), cached.to(dev), out, ns, chunk, ws, scale * math.log2(math.e), kv_start, G,
+                ring=ring.to(dev), tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), T=T)
+        torch.cuda.synchronize()
+        outs.append(Q.bf16_to_f32(bits(out)).astype(np.float64).reshape(B, Hq, D))
+    ringf = Q.bf16_to_f32(bits(ring)).astype(np.float64).reshape(B + 2, T, 2 * Hkv, D)
+    for b in range(B):
+        tb = ringf[b, :tails[b]]
+        ref = _ref_attn(Q.bf16_to_f32(bits(q)).astype(np.float64)[b], Ks[b], Vs[b], min(kv_start, lens[b]), lens[b],
+                        tb[:, :Hkv], tb[:, Hkv:], G, scale)
+        for o in outs:
+            assert (np.abs(o[b] - ref) / (2e-3 + 1e-2 * np.abs(ref))).max() <= 1.0
+
+
+
 @F8
 def test_dequant_and_torch_parser(dev, f8):
     from flagrot_releaser_amd import kivi as KV
