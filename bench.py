@@ -50,15 +50,15 @@ REPLAYS = 7
 TRAFFIC_FILE = "profiles/decode_traffic.json"
 
 
-def synth_kv(T, g, dev, torch, outliers=4, gain=8.0, mu=None):
+def synth_kv(T, g, dev, torch, outliers=4, gain=8.0, mu=None, hkv=HKV, dh=DH):
     """K ~ N(0,1) with `outliers` channels per head x gain and per-token norms ~ lognormal(0, 0.5); V ~ N(0,1)."""
-    kv = torch.randn(T, 2 * HKV, DH, generator=g, device=dev)
-    for h in range(HKV):
-        ch = torch.randint(0, DH, (outliers,), generator=g, device=dev)
+    kv = torch.randn(T, 2 * hkv, dh, generator=g, device=dev)
+    for h in range(hkv):
+        ch = torch.randint(0, dh, (outliers,), generator=g, device=dev)
         kv[:, h, ch] *= gain
-    kv[:, :HKV] *= torch.exp(0.5 * torch.randn(T, 1, 1, generator=g, device=dev))
+    kv[:, :hkv] *= torch.exp(0.5 * torch.randn(T, 1, 1, generator=g, device=dev))
     if mu is not None:
-        kv[:, :HKV] += mu[None]
+        kv[:, :hkv] += mu[None]
     return kv.bfloat16()
 
 
@@ -333,8 +333,13 @@ def run_kivi(args, torch, dev, steps, warmup):
     KV.lib()
     f8 = bool(args.f8)
     B, L, Gq, W, NQ, outl, gain = 16, 32768, 8, 128, 64, 8, 12.0
+    HKV, DH = globals()["HKV"], globals()["DH"]
     name = ("configs[3]: KIVI-style FlagRot INT2 paged decode (per-channel keys over 32-token groups, per-token values"
             + (", FP8 meta" if f8 else "") + "), 128-token BF16 residual, Qwen-32B GQA 64q/8kv d=128, B=16 L=32768 page=16")
+    if args.head_dim == 256:       # not a configuration of the baseline: the head dim 256 kernels on the reference's test shape class
+        B, L, Gq, HKV, DH = 16, 8192 + W, 6, 4, 256
+        name = ("KIVI-style FlagRot INT2 paged decode at head dim 256" + (", FP8 meta" if f8 else "") +
+                f", 128-token BF16 residual, GQA 24q/4kv d=256, B={B} L={L} page=16 (no baseline configuration)")
     CB = KV.chunk_bytes(DH, f8)
     g = torch.Generator(device=dev).manual_seed(3)
     Lp = L - W
@@ -348,7 +353,7 @@ def run_kivi(args, torch, dev, steps, warmup):
     for b in range(B):
         for s0 in range(0, Lp, 8192):
             n = min(8192, Lp - s0)
-            kv = synth_kv(n, g, dev, torch, outliers=outl, gain=gain)
+            kv = synth_kv(n, g, dev, torch, outliers=outl, gain=gain, hkv=HKV, dh=DH)
             pos = torch.arange(s0, s0 + n, device=dev)
             slots = bt[b].long()[pos // P] * P + pos % P
             KV.v_write(kv, slots, co, None, pool, HKV, DH, f8=f8)
@@ -364,7 +369,7 @@ def run_kivi(args, torch, dev, steps, warmup):
     tail_len = torch.full((B,), W, dtype=torch.int32, device=dev)
     tail_idx = torch.arange(B, dtype=torch.int32, device=dev)
     cached = torch.full((B,), Lp, dtype=torch.int32, device=dev)
-    ns, ch = KV.plan(B, Lp, HKV)
+    ns, ch = KV.plan(B, Lp, HKV, D=DH)
     if args.nsplit:
         ns = args.nsplit
         ch = -(-Lp // ns // 32) * 32
@@ -515,6 +520,7 @@ def main():
     ap.add_argument("--workload", default=None, choices=["int4", "int2", "kivi", "mq"])
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
+    ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="kivi: 256 = the head dim 256 kernels")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", action="store_true", help="the chosen workload only (no extra legs)")
@@ -563,7 +569,7 @@ def main():
                           "cache_copies_cycled": r["cache_copies_cycled"], "timing": timing, "sink": r["sink"],
                           "window": r["window"]},
                "roofline": {"bound": "hbm", "achieved": r["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": r["frac"],
-                            "traffic": traffic_of("kivi" if workload == "kivi" else workload),
+                            "traffic": traffic_of("kivi" if workload == "kivi" else workload) if args.head_dim == 128 else None,
                             "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this launch in "
                                               "separate runs, scaled by a device copy; not measured in this run)",
                             "algorithmic_bytes_per_launch": r["algorithmic_bytes_per_launch"],

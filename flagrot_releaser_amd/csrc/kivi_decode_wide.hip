@@ -1,5 +1,5 @@
 // Paged split-K decode attention over KIVI-style FlagRot INT2 pages at head dim 256 for gfx950, both products on the
-// matrix pipe: the page splits (the BF16 ring rows stay with the plain kernel of kivi_wide.hip, one more split).
+// matrix pipe: the page splits, and the BF16 ring rows as one more split (plain fp32, a wavefront per row).
 //
 // The design is the 128-d kernel's (kivi_decode.hip) worked through a head in halves, so that the per-wavefront LDS
 // strips and the register sets keep the 128-d size and two workgroups of 4 wavefronts stay resident per CU:
@@ -93,12 +93,96 @@ DEVI void h256(float (&y)[2][4], int l32) {                     // orthonormal H
   }
 }
 
+// The BF16 ring rows of one sequence (split index NS): rows [0, tail_len) of ring block tail_idx, K row h, V row Hkv + h,
+// original basis.  A wavefront takes every fourth row, lanes own 4 dims; same partial format as the page splits.
+template <int G>
+DEVI void tail_split256(SmemW& S, const uint16_t* __restrict__ q, long long q_rs, const uint16_t* __restrict__ ring,
+                        const int* __restrict__ tail_len, const int* __restrict__ tail_idx, int T, int Hkv, int Gq, int b, int h,
+                        float qscale, float* __restrict__ op, float* __restrict__ mlp) {
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+  const int n = tail_len != nullptr ? tail_len[b] : 0;
+  if (n <= 0) {
+    if (tid < Gq) { mlp[2 * tid] = -INFINITY; mlp[2 * tid + 1] = 0.f; }
+    return;
+  }
+  float qa[G][4], m[G], l[G], oa[G][4];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qa[g][i] = oa[g][i] = 0.f;
+    if (g < Gq) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(q + static_cast<long long>(b) * q_rs + (static_cast<long long>(h) * Gq + g) * 256 + 4 * lane);
+      qa[g][0] = bf16_lo(raw.x) * qscale; qa[g][1] = bf16_hi(raw.x) * qscale;
+      qa[g][2] = bf16_lo(raw.y) * qscale; qa[g][3] = bf16_hi(raw.y) * qscale;
+    }
+    m[g] = -INFINITY; l[g] = 0.f;
+  }
+  const uint16_t* rbase = ring + static_cast<long long>(tail_idx != nullptr ? tail_idx[b] : 0) * T * 2 * Hkv * 256;
+  // eight rows of the wavefront in flight at a time (past the end: the last row again, skipped): a row's work is
+  // short against the latency of its loads
+  for (int tb = wv; tb < n; tb += 32) {
+    uint2 kr[8], vr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint16_t* row = rbase + static_cast<long long>(min(tb + 4 * i, n - 1)) * 2 * Hkv * 256;
+      kr[i] = *reinterpret_cast<const uint2*>(row + h * 256 + 4 * lane);
+      vr[i] = *reinterpret_cast<const uint2*>(row + (Hkv + h) * 256 + 4 * lane);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (tb + 4 * i >= n) break;
+      const float k[4] = {bf16_lo(kr[i].x), bf16_hi(kr[i].x), bf16_lo(kr[i].y), bf16_hi(kr[i].y)};
+      const float v[4] = {bf16_lo(vr[i].x), bf16_hi(vr[i].x), bf16_lo(vr[i].y), bf16_hi(vr[i].y)};
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float sc = wave_sum64(qa[g][0] * k[0] + qa[g][1] * k[1] + qa[g][2] * k[2] + qa[g][3] * k[3]);
+        const float mn = fmaxf(m[g], sc);
+        const float alpha = m[g] == -INFINITY ? 0.f : fexp2(m[g] - mn), p = fexp2(sc - mn);
+        l[g] = l[g] * alpha + p;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) oa[g][c] = oa[g][c] * alpha + p * v[c];
+        m[g] = mn;
+      }
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) { S.mw[wv][g] = m[g]; S.lw[wv][g] = l[g]; }
+  }
+  __syncthreads();
+  for (int r = 0; r < 4; ++r) {
+    if (wv == r) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float M = fmaxf(fmaxf(S.mw[0][g], S.mw[1][g]), fmaxf(S.mw[2][g], S.mw[3][g]));
+        const float f = m[g] == -INFINITY ? 0.f : fexp2(m[g] - M);
+        float4* dst = reinterpret_cast<float4*>(&S.ob[0][g][4 * lane]);
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r) acc = *dst;
+        *dst = make_float4(acc.x + f * oa[g][0], acc.y + f * oa[g][1], acc.z + f * oa[g][2], acc.w + f * oa[g][3]);
+      }
+    }
+    __syncthreads();
+  }
+  for (int g = wv; g < G && g < Gq; g += 4) {
+    *reinterpret_cast<float4*>(op + g * 256 + 4 * lane) = *reinterpret_cast<const float4*>(&S.ob[0][g][4 * lane]);
+    if (lane == 0) {
+      const float M = fmaxf(fmaxf(S.mw[0][g], S.mw[1][g]), fmaxf(S.mw[2][g], S.mw[3][g]));
+      float L = 0.f;
+      for (int w = 0; w < 4; ++w) L += S.mw[w][g] == -INFINITY ? 0.f : fexp2(S.mw[w][g] - M) * S.lw[w][g];
+      mlp[2 * g] = M; mlp[2 * g + 1] = L;
+    }
+  }
+}
+
 template <bool F8>
 __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __restrict__ q, long long q_rs,
                                                        const uint8_t* __restrict__ pool, const int* __restrict__ bt,
                                                        long long bt_rs, const int* __restrict__ cached, int kv_start,
                                                        int Hkv, int NS, int chunk, float qscale,
-                                                       float* __restrict__ opart, float* __restrict__ ml, int Gq) {
+                                                       float* __restrict__ opart, float* __restrict__ ml, int Gq,
+                                                       const uint16_t* __restrict__ ring, const int* __restrict__ tail_len,
+                                                       const int* __restrict__ tail_idx, int T) {
   constexpr int G = GT;
   extern __shared__ __align__(16) uint8_t lds[];
   SmemW& S = *reinterpret_cast<SmemW*>(lds);
@@ -107,6 +191,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
   const long long pidx = (static_cast<long long>(b) * Hkv + h) * (NS + 1) + sp;
   float* op = opart + pidx * Gq * 256;
   float* mlp = ml + pidx * Gq * 2;
+  if (sp == NS) {
+    tail_split256<G>(S, q, q_rs, ring, tail_len, tail_idx, T, Hkv, Gq, b, h, qscale, op, mlp);
+    return;
+  }
   const int t0 = max(sp * chunk, kv_start), t1 = min((sp + 1) * chunk, cached[b]);
   if (t1 <= t0) {
     if (tid < Gq) { mlp[2 * tid] = -INFINITY; mlp[2 * tid + 1] = 0.f; }
@@ -425,10 +513,9 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
 }  // namespace
 
 int attn_pages256_launch(int Gq, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
-                         const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, void* opart,
-                         void* ml, int f8, hipStream_t st) {
+                         const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
+                         const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st) {
   if (Gq < 1 || Gq > GT) return 2;
-  if (NS <= 0) return 0;
   static bool attr = false;
   if (!attr) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_pages256<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -438,9 +525,10 @@ int attn_pages256_launch(int Gq, const void* q, long long q_rs, const void* pool
     attr = true;
   }
   const auto kern = f8 ? k_attn_pages256<true> : k_attn_pages256<false>;
-  hipLaunchKernelGGL(kern, dim3(B, Hkv, NS), dim3(256), sizeof(SmemW), st, static_cast<const uint16_t*>(q), q_rs,
+  hipLaunchKernelGGL(kern, dim3(B, Hkv, NS + 1), dim3(256), sizeof(SmemW), st, static_cast<const uint16_t*>(q), q_rs,
                      static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), bt_rs, static_cast<const int*>(cached),
-                     kv_start, Hkv, NS, chunk, qscale, static_cast<float*>(opart), static_cast<float*>(ml), Gq);
+                     kv_start, Hkv, NS, chunk, qscale, static_cast<float*>(opart), static_cast<float*>(ml), Gq,
+                     static_cast<const uint16_t*>(ring), static_cast<const int*>(tail_len), static_cast<const int*>(tail_idx), T);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
 

@@ -31,8 +31,8 @@ int dequant256_launch(const uint8_t* pool, const int* bt, int g0, int g1, int nv
                       int f8, hipStream_t st);
 // splits and merge in one call: out bf16 rows of Hkv G 256 values
 int attn_pages256_launch(int Gq, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs,
-                         const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, void* opart,
-                         void* ml, int f8, hipStream_t st);
+                         const void* cached, int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring,
+                         const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, int f8, hipStream_t st);
 int attn256_launch(int G, const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
                    int kv_start, int B, int Hkv, int NS, int chunk, float qscale, const void* ring, const void* tail_len,
                    const void* tail_idx, int T, void* opart, void* ml, void* out, long long out_rs, int f8, hipStream_t st);

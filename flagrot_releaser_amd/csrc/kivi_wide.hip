@@ -20,9 +20,9 @@
 //
 // The attention kernel here is the plain fp32 form (no matrix cores): per 32-token group, scores by (token, sub-vector)
 // threads against the three rotated queries, one softmax per head in a half wave, values by channel threads into one
-// accumulator per (head, basis), the two inverse transforms once at the end.  It serves the BF16 ring rows (the last
-// split) of every launch; the page splits go through the matrix-pipe kernel of kivi_decode_wide.hip unless
-// FLAGROT_KIVI_WIDE_PLAIN=1 asks for this one.  Same partials either way, one merge kernel.
+// accumulator per (head, basis), the two inverse transforms once at the end.  It runs only when
+// FLAGROT_KIVI_WIDE_PLAIN=1 asks for it: the launches go through the matrix-pipe kernel of kivi_decode_wide.hip.
+// Same partials either way, one merge kernel.
 #include <cstdlib>
 
 #include "fr_common.hpp"
@@ -573,10 +573,10 @@ __global__ void __launch_bounds__(256) k_attn256(const uint16_t* __restrict__ q,
                                                  const int* __restrict__ cached, int kv_start, int Hkv, int G, int NS,
                                                  int chunk, float qscale, const uint16_t* __restrict__ ring,
                                                  const int* __restrict__ tail_len, const int* __restrict__ tail_idx, int T,
-                                                 float* __restrict__ opart, float* __restrict__ ml, int sp0) {
+                                                 float* __restrict__ opart, float* __restrict__ ml) {
   extern __shared__ __align__(16) uint8_t lds[];
   WideAttn& S = *reinterpret_cast<WideAttn*>(lds);
-  const int b = blockIdx.x, h = blockIdx.y, sp = sp0 + blockIdx.z;
+  const int b = blockIdx.x, h = blockIdx.y, sp = blockIdx.z;
   const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
   const long long pidx = (static_cast<long long>(b) * Hkv + h) * (NS + 1) + sp;
   float* op = opart + pidx * G * D2;
@@ -827,21 +827,21 @@ int attn256_launch(int G, const void* q, long long q_rs, const void* pool, const
     if (!carve(&k_attn256<false>, sizeof(WideAttn)) || !carve(&k_attn256<true>, sizeof(WideAttn))) return 1;
     attr = true;
   }
-  // page splits on the matrix pipe (kivi_decode_wide.hip), the ring rows (split NS) through the plain kernel;
-  // FLAGROT_KIVI_WIDE_PLAIN=1 (read at every call) sends every split through the plain kernel
+  // every split through the matrix-pipe kernel file (kivi_decode_wide.hip) unless FLAGROT_KIVI_WIDE_PLAIN=1 (read at
+  // every call) asks for the plain kernel of this file
   const char* env = std::getenv("FLAGROT_KIVI_WIDE_PLAIN");
-  const bool plain = env != nullptr && env[0] == '1';
-  if (!plain) {
-    const int rc = attn_pages256_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, opart, ml, f8, st);
+  if (env != nullptr && env[0] == '1') {
+    const auto kern = f8 ? k_attn256<true> : k_attn256<false>;
+    hipLaunchKernelGGL(kern, dim3(B, Hkv, NS + 1), dim3(256), sizeof(WideAttn), st, static_cast<const uint16_t*>(q), q_rs,
+                       static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), bt_rs, static_cast<const int*>(cached),
+                       kv_start, Hkv, G, NS, chunk, qscale, static_cast<const uint16_t*>(ring), static_cast<const int*>(tail_len),
+                       static_cast<const int*>(tail_idx), T, static_cast<float*>(opart), static_cast<float*>(ml));
+    if (hipPeekAtLastError() != hipSuccess) return 1;
+  } else {
+    const int rc = attn_pages256_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
+                                        tail_idx, T, opart, ml, f8, st);
     if (rc) return rc;
   }
-  const int sp0 = plain ? 0 : NS;
-  const auto kern = f8 ? k_attn256<true> : k_attn256<false>;
-  hipLaunchKernelGGL(kern, dim3(B, Hkv, NS + 1 - sp0), dim3(256), sizeof(WideAttn), st, static_cast<const uint16_t*>(q), q_rs,
-                     static_cast<const uint8_t*>(pool), static_cast<const int*>(bt), bt_rs, static_cast<const int*>(cached),
-                     kv_start, Hkv, G, NS, chunk, qscale, static_cast<const uint16_t*>(ring), static_cast<const int*>(tail_len),
-                     static_cast<const int*>(tail_idx), T, static_cast<float*>(opart), static_cast<float*>(ml), sp0);
-  if (hipPeekAtLastError() != hipSuccess) return 1;
   hipLaunchKernelGGL(k_merge256, dim3(B, Hkv * G), dim3(256), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
                      Hkv, G, NS, static_cast<uint16_t*>(out), out_rs);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
