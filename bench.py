@@ -140,24 +140,27 @@ def describe(st):
             f"relative L2 = {st['rel_l2']:.2e}")
 
 
-def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192):
+def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192, hkv=HKV, dh=DH):
     """fills one pool with B sequences of L tokens through the selecting writer; returns pool, block table, calib."""
     g = torch.Generator(device=dev).manual_seed(seed)
     npages = B * ((L + P - 1) // P)
-    pool = torch.zeros(npages + 16, HKV, K.cb_chunk_bytes(kind, P), dtype=torch.uint8, device=dev)
+    pool = torch.zeros(npages + 16, hkv, K.cb_chunk_bytes(kind, P) * (dh // 128), dtype=torch.uint8, device=dev)
     perm = torch.randperm(npages + 16, generator=g, device=dev)[:npages].int()
     bt = perm.view(B, -1).contiguous()
-    w = 0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)
+    w = 0.5 + 1.5 * torch.rand(hkv, dh, generator=g, device=dev)
     CT = torch.diag_embed(w).contiguous()                      # C_q = diag(w) (symmetric: C^T = C)
     co = w.contiguous()
     t0 = time.perf_counter()
     for b in range(B):
         for s in range(0, L, chunk_tokens):
             n = min(chunk_tokens, L - s)
-            kv = synth_kv(n, g, dev, torch, mu=kmu)
+            kv = synth_kv(n, g, dev, torch, mu=kmu, hkv=hkv, dh=dh)
             pos = torch.arange(s, s + n, device=dev)
             slots = bt[b].long()[pos // P] * P + pos % P
-            K.cb_write3(kv, slots, CT, co, None, None, kind, pool, P, split=False, kmu=kmu)    # = cb_write bytes
+            if dh == 128:
+                K.cb_write3(kv, slots, CT, co, None, None, kind, pool, P, split=False, kmu=kmu)    # = cb_write bytes
+            else:
+                K.cb_write(kv, slots, CT, co, kind, pool, P, kmu=kmu)
     torch.cuda.synchronize()
     return pool, bt, CT, co, time.perf_counter() - t0
 
@@ -240,11 +243,17 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
         kind, B, L, S, W, cell = "konlya2", 64, 16384, 4, 128, 80
         name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
                 "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
+    HKV, DH, G = globals()["HKV"], globals()["DH"], globals()["G"]
+    if getattr(args, "head_dim", 128) == 256:     # not a configuration of the baseline: the head dim 256 kernels, same page bytes
+        HKV, DH, G = 4, 256, 6
+        name = (f"{'INT4' if workload == 'int4' else 'INT2'} FlagRot {kind} paged decode at head dim 256, GQA 24q/4kv, B={B} "
+                f"L={L} page=16" + (f", {S} sink / {W} window BF16" if S + W else "") + " (no baseline configuration)")
+        cell *= 2
     g = torch.Generator(device=dev).manual_seed(1)
     kmu = None
     if workload == "int2":
         kmu = (2.0 * torch.randn(HKV, DH, generator=g, device=dev)).contiguous()
-    pool, bt, CT, co, fill_s = build_cache(torch, K, dev, kind, B, L, seed=1, kmu=kmu)
+    pool, bt, CT, co, fill_s = build_cache(torch, K, dev, kind, B, L, seed=1, kmu=kmu, hkv=HKV, dh=DH)
     ncopy = max(1, min(8, int(6e9 // pool.numel())))
     pools = [pool] + [pool.clone() for _ in range(ncopy - 1)]
     q = torch.randn(B, G * HKV, DH, generator=g, device=dev).bfloat16()
@@ -267,11 +276,15 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
     results = {}
     for plan in plans:
         if plan == "own":
-            ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None)
+            ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None, G=G, Dh=DH)
         else:      # "reference": the reference front end's cost model fed with this library's occupancy answer
             occ = K.lib().fr_cb_occupancy(K.CB_KINDS[kind], 0, K.STAGES, P)
             ns, ch = reference_plan(B, Lpages, HKV, max(1, occ) * cus)
-        ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
+        if DH == 128:
+            ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
+        else:
+            hv = K.vheads(HKV, G, DH, kind)
+            ws = K.Workspace(B, hv, B * hv * (ns + 1), dev, K.tile_of(K.v2_variant(kind, G, DH)), DH)
 
         def step(i):
             K.cb_attn(q, pools[i % ncopy], bt, seq, out, ns, ch, ws, scale, kind, **tkw)
@@ -305,7 +318,7 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
             "check": f"sequences {rows} x all {G * HKV} heads vs the fp64 oracle: " + describe(st),
         }
     # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
-    kv_new = synth_kv(B, g, dev, torch, mu=kmu)
+    kv_new = synth_kv(B, g, dev, torch, mu=kmu, hkv=HKV, dh=DH)
     slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
     for _ in range(3):
         K.cb_write(kv_new, slots_new, CT, co, kind, pools[0], P, kmu=kmu)
@@ -336,7 +349,7 @@ def run_kivi(args, torch, dev, steps, warmup):
     HKV, DH = globals()["HKV"], globals()["DH"]
     name = ("configs[3]: KIVI-style FlagRot INT2 paged decode (per-channel keys over 32-token groups, per-token values"
             + (", FP8 meta" if f8 else "") + "), 128-token BF16 residual, Qwen-32B GQA 64q/8kv d=128, B=16 L=32768 page=16")
-    if args.head_dim == 256:       # not a configuration of the baseline: the head dim 256 kernels on the reference's test shape class
+    if getattr(args, "head_dim", 128) == 256:       # not a configuration of the baseline: the head dim 256 kernels on the reference's test shape class
         B, L, Gq, HKV, DH = 16, 8192 + W, 6, 4, 256
         name = ("KIVI-style FlagRot INT2 paged decode at head dim 256" + (", FP8 meta" if f8 else "") +
                 f", 128-token BF16 residual, GQA 24q/4kv d=256, B={B} L={L} page=16 (no baseline configuration)")
@@ -433,13 +446,20 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
     from oracle import mq as OM
     MQ.lib()
     R, NQ, PRE, Gq = 4, 512, 16384, 8
-    L = PRE + NQ
+    HKV, DH = globals()["HKV"], globals()["DH"]
     k2 = fmt == "konlya"
+    if getattr(args, "head_dim", 128) == 256:       # not a configuration of the baseline: the head dim 256 kernel on the reference's test shape class
+        assert k2, "head dim 256: key-only pages (--mq-fmt konlya)"
+        R, NQ, PRE, Gq, HKV, DH = 2, 512, 8192, 6, 4, 256
+    L = PRE + NQ
     name = (f"configs[4]: multi-query prefill over INT4 FlagRot pages ({fmt}), Qwen-32B GQA 64q/8kv d=128, {R} requests x "
             f"{NQ} new tokens over a {PRE}-token cached prefix (L={L}), page=16, causal inside the chunk")
+    if DH == 256:
+        name = (f"multi-query prefill over INT4 FlagRot pages ({fmt}) at head dim 256, GQA {Gq * HKV}q/{HKV}kv, {R} requests x "
+                f"{NQ} new tokens over a {PRE}-token cached prefix (L={L}), page=16 (no baseline configuration)")
     g = torch.Generator(device=dev).manual_seed(4)
     npg = (L + P - 1) // P
-    pool = torch.zeros(R * npg + 16, HKV, 144 * P, dtype=torch.uint8, device=dev)
+    pool = torch.zeros(R * npg + 16, HKV, 144 * P * (DH // 128), dtype=torch.uint8, device=dev)
     bt = torch.randperm(R * npg + 16, generator=g, device=dev)[:R * npg].int().view(R, npg).contiguous()
     w = 0.5 + 1.5 * torch.rand(HKV, DH, generator=g, device=dev)
     CT, co = torch.diag_embed(w).contiguous(), w.contiguous()
@@ -448,7 +468,7 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
     for r in range(R):
         for s0 in range(0, L, 8192):
             n = min(8192, L - s0)
-            kv = synth_kv(n, g, dev, torch)
+            kv = synth_kv(n, g, dev, torch, hkv=HKV, dh=DH)
             pos = torch.arange(s0, s0 + n, device=dev)
             slots = bt[r].long()[pos // P] * P + pos % P
             if k2:
@@ -457,7 +477,7 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
                 K.w3_static_write(kv, slots, mask, None, pool, P, fmt=fmt)
     torch.cuda.synchronize()
     reqs = [(r, r * NQ, (r + 1) * NQ, L, PRE) for r in range(R)]
-    plan = MQ.build_plan(reqs, Gq, HKV, 0, dev)
+    plan = MQ.build_plan(reqs, Gq, HKV, 0, dev, D=DH)
     q = (2.0 * torch.randn(R * NQ, Gq * HKV, DH, generator=g, device=dev)).bfloat16()
     out = torch.zeros(R * NQ, Gq * HKV * DH, dtype=torch.bfloat16, device=dev)
     scale = LOG2E / math.sqrt(DH)
@@ -481,7 +501,7 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
     torch.cuda.synchronize()
     r, nh = R - 1, 2
     mp = pool.index_select(0, bt[r].long())[:, :nh].contiguous().cpu().numpy()
-    Kp, Vp = A.dequant_pages(mp, fmt, P)
+    Kp, Vp = A.dequant_pages(mp, fmt, P, Dh=DH)
     Kd, Vd = Kp.reshape(-1, nh, DH)[:L], Vp.reshape(-1, nh, DH)[:L]
     q16 = keep["q16"].view(R * NQ, Gq * HKV, DH)
     gots, refs = [], []
@@ -520,7 +540,7 @@ def main():
     ap.add_argument("--workload", default=None, choices=["int4", "int2", "kivi", "mq"])
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
-    ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="kivi: 256 = the head dim 256 kernels")
+    ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="256 = the head dim 256 kernels (GQA 24q/4kv, the reference's test shape class); not a baseline configuration")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", action="store_true", help="the chosen workload only (no extra legs)")
@@ -569,7 +589,7 @@ def main():
                           "cache_copies_cycled": r["cache_copies_cycled"], "timing": timing, "sink": r["sink"],
                           "window": r["window"]},
                "roofline": {"bound": "hbm", "achieved": r["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": r["frac"],
-                            "traffic": traffic_of("kivi" if workload == "kivi" else workload) if args.head_dim == 128 else None,
+                            "traffic": traffic_of("kivi" if workload == "kivi" else workload) if getattr(args, "head_dim", 128) == 128 else None,
                             "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this launch in "
                                               "separate runs, scaled by a device copy; not measured in this run)",
                             "algorithmic_bytes_per_launch": r["algorithmic_bytes_per_launch"],

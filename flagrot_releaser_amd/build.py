@@ -27,7 +27,7 @@ STRICT = ["-ffp-contract=off", "-fno-fast-math"]
 
 # library -> [(source, extra flags)]
 LIBS = {
-    "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("capi.hip", [])]),
+    "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("decode_wide_mma.hip", []), ("capi.hip", [])]),
     "kivi": ("libflagrot_kivi.so", [("kivi_write.hip", STRICT), ("kivi_wide.hip", STRICT), ("kivi_attn.hip", []), ("kivi_decode.hip", []), ("kivi_decode_wide.hip", [])]),
     "mq": ("libflagrot_mq.so", [("mq_prefill.hip", []), ("mq_wide.hip", [])]),
 }

@@ -1,0 +1,478 @@
+// Building blocks of the matrix-pipe decode kernels over FlagRot INT4 / INT2 pages (decode.hip: head dim 128;
+// decode_wide_mma.hip: head dim 256 as two 128-d half chunks): LDS strip geometry, the query prologue, the page loaders,
+// and the three phases of a wave iteration over a quad of 64 tokens -- key phase (scores on the matrix pipe), online
+// softmax with the p * V-scale strips, value phase.  The phases take the LDS block as a template parameter: anything
+// with qhi / qlo / qz [group][lane] operand tables and pb(wave) / zb(wave) strips serves.
+#pragma once
+#include "fr_common.hpp"
+#include "fr_launch.hpp"
+#include "fr_unpack.hpp"
+
+namespace fr {
+namespace dec {
+
+DEVI float dot2(uint32_t a, uint32_t b, float c) { return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), c, false); }
+DEVI float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+
+// LDS strips are padded so that the few distinct 16-byte rows the lanes of one instruction touch (one per
+// row group) start in different banks.
+// A wave iteration covers QB blocks of 16 tokens: 4 (64 tokens) for every format.  (Measured for the 2-bit formats:
+// 8 blocks per iteration -- the bytes in flight of a 4-bit iteration -- need 155 registers, i.e. three wavefronts per
+// SIMD instead of four, and are 4 % slower on configs[2]: that loop is bound by instruction issue, not by latency.)
+template <int QM> constexpr int QBLK = 4;
+constexpr int PB_RSTRIDE = 17;                     // uint4 per row group (block, c8): 16 + 1 pad (the pad stays zero: below)
+constexpr int ZB_RSTRIDE = 5;                      // uint4 per row group: 4 + 1 pad
+template <int QM> struct Strip {
+  static constexpr int ROWS = 2 * QBLK<QM>;                    // row groups = runs of 8 tokens
+  static constexpr int PB_BYTES = ROWS * PB_RSTRIDE * 16;      // per wave: [block][c8][group][head][8 fp16]
+  static constexpr int ZB_BYTES = ROWS * ZB_RSTRIDE * 16;      // per wave: [block][c8][group][8 fp16] = zero point (x 2^SH for odd tokens)
+  static constexpr int BYTES = PB_BYTES + ZB_BYTES;            // per wave
+};
+constexpr int DRAW_BATCH = 2;                      // quads per draw from the shared (device-scope) counter
+constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
+constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
+constexpr float QPRE = 16.f;                       // the query operands carry 2^4 (fp16 range: |q| up to 127 in any rotation)
+
+template <int QM, int NW>
+struct Smem {
+  static constexpr int STRIP_BYTES = Strip<QM>::BYTES, PB_BYTES = Strip<QM>::PB_BYTES;
+  // A operands of the score products: [group j][lane of the matrix instruction = row (head, variant) + 16 x k block]
+  alignas(16) uint4 qhi[4][64];                      // fp16(q * 2^4 / element factor)
+  alignas(16) uint4 qlo[4][64];                      // fp16 of what that rounding left
+  alignas(16) uint4 qz[4][64];                       // -(sum of the group's query elements), fp16 pair in k blocks 0 / 1 (first word)
+  // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
+  alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
+  float m[NW][4], l[NW][4];
+  int btc[BT_CACHE];
+  int next;                                          // next quad of 4 pages nobody has taken yet
+  int last;
+  DEVI uint8_t* pb(int w) { return work + w * STRIP_BYTES; }
+  DEVI const uint8_t* pb(int w) const { return work + w * STRIP_BYTES; }
+  DEVI uint8_t* zb(int w) { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI const uint8_t* zb(int w) const { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI float* o(int w, int h) { return reinterpret_cast<float*>(work) + (w * 4 + h) * 128; }
+};
+
+// slot of element (isB, i) of a K word / of token r8 of a V word inside the 8-fp16 operand vector
+DEVI int kslot(int isB, int i) { return 2 * (2 * (i & 1) + isB) + (i >> 1); }
+DEVI int vslot(int r8) { return 2 * (r8 & 3) + (r8 >> 2); }
+
+// Rotates the q tile three ways and stores it as the A operands of the score products: rows = (head, variant), per
+// 32-group j and k block (= quarter tg of a code row) the eight elements in the order the masked code words give
+// them.  An element is held as an fp16 pair (value + what its rounding left), both times 2^4 and divided by the
+// factor its code field comes out of the unpacking with (2^SH for the B elements of a word, 2^4 more for the odd
+// groups of the 2-bit words).  The third operand removes the zero points: -(sum of the group's elements as held).
+// Wavefronts 0..3: one head each; half 0 writes the rows of variants 0 (identity, or the static kmask rotation) and
+// 1 (H32), half 1 those of variant 2 (H128) and the idle row 3; rows of variants a format does not use are zero.
+template <int QM, bool K2, class SM>
+DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
+  const int w = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
+  const int hq = tile * 4 + w;                       // head inside the GQA group
+  float x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (hq < p.gqa) {
+    const uint16_t* qr = static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
+                         (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 4 * l32;
+    const uint2 raw = *reinterpret_cast<const uint2*>(qr);
+    x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
+  }
+  const int g = l32 >> 3, isB = (l32 >> 2) & 1, tg = l32 & 3;   // the lane's dims 4 l32 + i: group, word half, quarter
+  float y[4] = {x[0], x[1], x[2], x[3]};
+  if (half == 0) fwht<32>(y, l32); else fwht<128>(y, l32);
+  // factor of the lane's code fields after the unpacking (the operand is divided by it)
+  const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
+  const float fold = QPRE / beta;
+#pragma unroll
+  for (int vi = 0; vi < 2; ++vi) {
+    const int var = 2 * half + vi;
+    float v[4];
+    bool live;
+    if (K2) {
+      live = var < 3;
+      const bool rot = var != 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
+    } else {
+      live = var == 0;
+      // (a bit mask and not `rot ? y[i] : x[i]`: the compiler turns that into a choice between the two arrays'
+      // addresses, which puts both into scratch memory)
+      const uint32_t rot = (p.kmask != nullptr && p.kmask[kvh * 4 + g] != 0) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = __uint_as_float((__float_as_uint(y[i]) & rot) | (__float_as_uint(x[i]) & ~rot));
+    }
+    uint32_t hb[4], lb[4];
+    float qs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = live ? v[i] * fold : 0.f;
+      const _Float16 hi = static_cast<_Float16>(a);
+      const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
+      hb[i] = __builtin_bit_cast(uint16_t, hi);
+      lb[i] = __builtin_bit_cast(uint16_t, lo);
+      qs += (static_cast<float>(hi) + static_cast<float>(lo)) * beta;
+    }
+    // elements i = 0, 2 are halves 2 isB, 2 isB + 1 of the operand (word isB), i = 1, 3 halves 4 + 2 isB, 5 + 2 isB
+    const int m = 4 * w + var, ln = m + 16 * tg;
+    uint32_t* dh = reinterpret_cast<uint32_t*>(&S.qhi[g][ln]);
+    uint32_t* dl = reinterpret_cast<uint32_t*>(&S.qlo[g][ln]);
+    dh[isB] = hb[0] | (hb[2] << 16); dh[2 + isB] = hb[1] | (hb[3] << 16);
+    dl[isB] = lb[0] | (lb[2] << 16); dl[2 + isB] = lb[1] | (lb[3] << 16);
+    if constexpr (QM != QM_SYM4) {
+      qs += hx(qs, 1); qs += hx(qs, 2); qs += hx(qs, 4);
+      if ((l32 & 7) == 0) {   // k blocks 0 / 1 carry the pair, in the half the zero point of group g is masked into
+        const _Float16 zh = static_cast<_Float16>(-qs);
+        const _Float16 zl = static_cast<_Float16>(-qs - static_cast<float>(zh));
+        const int sh = 16 * (g & 1);
+        S.qz[g][m] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zh)) << sh, 0u, 0u, 0u);
+        S.qz[g][m + 16] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zl)) << sh, 0u, 0u, 0u);
+        S.qz[g][m + 32] = make_uint4(0u, 0u, 0u, 0u);
+        S.qz[g][m + 48] = make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  }
+}
+
+// Page loads are forced into the global address space: a generic (flat) load also counts on the LDS counter, so
+// every wait for an LDS read would wait for the page data in flight as well.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T> DEVI T gload(const uint8_t* p) {
+  typedef const __attribute__((address_space(1))) T* gp;
+  return *(gp)(p);
+}
+
+// One wave iteration covers a quad = 64 consecutive tokens (four 16-token pages or two 32-token pages), as four
+// blocks of 16 tokens.  Key phase: lane = (token t = lane & 15 of a block, quarter x = lane >> 4 of its code row).
+// Value phase: lane = V^T entry `lane` of each of the 4 blocks in turn.
+template <int QM> struct KRegs {
+  static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;   // code words per 16-byte / 8-byte quarter row
+  static constexpr int QB = QBLK<QM>;
+  uint32_t kc[QB][NW];      // [block][word]: quarter x of token t's code row (word j = group j; 2-bit: groups 2 j, 2 j + 1)
+  uint2 ks[QB];             // [block]: the token's 4 K scale words
+  uint16_t vs[QB];          // [block]: the token's V scale word of group x; 16 bits wide so that the widening belongs to the use
+                            // (a widening at the load would be scheduled right behind it and wait for the keys in flight)
+};
+// The value product P' V runs on the matrix pipe: sixteen v_mfma_f32_16x16x32_f16 per quad of pages, rows = 16 V^T
+// entries, columns = (group, head), 32 tokens deep.  An entry word masked in place (eight tokens as fp16 denormal
+// pairs; the matrix pipe keeps denormal inputs) is the A operand of its lane, one 16-byte strip row (p' of a run's eight
+// tokens for a (group, head)) the B operand.  The scores stay on the vector pipe (v_dot2_f32_f16).
+template <int QM> struct VRegs {
+  static constexpr int NW = QM == QM_ASYM2 ? 2 : 4;
+  uint32_t vc[QBLK<QM>][NW];   // [2 (block pair s) + entry half][entry word] of lane (entry m = lane & 15, run kc = lane >> 4)
+};
+
+// lane offsets of the key-side loads inside a chunk (block 0 of a page; a 32-token page's second block adds constants)
+template <int QM, int P> struct KOffs { int k, ks, vs; };
+template <int QM, int P>
+DEVI KOffs<QM, P> key_offsets(int lane) {
+  using L = Lay<QM, P>;
+  const int t = lane & 15, x = lane >> 4;
+  KOffs<QM, P> o;
+  o.k = QM == QM_ASYM2 ? L::K_OFF + 32 * (t ^ ((t >> 1) & 2)) + 8 * x : L::K_OFF + 64 * t + 16 * x;
+  o.ks = L::KS_OFF + 8 * t;
+  o.vs = L::VS_OFF + (x * P + 8 * (t >> 3) + vs_slot8(t)) * 2;
+  return o;
+}
+// chunk[b]: the chunk of block b's page (wave uniform); 32-token pages: blocks 2 s, 2 s + 1 are the halves of page s
+template <int QM, int P>
+DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], const KOffs<QM, P>& o) {
+#pragma unroll
+  for (int b = 0; b < QBLK<QM>; ++b) {
+    const int hp = P == 32 ? (b & 1) : 0;            // second half of a 32-token page: 16 tokens further
+    const uint8_t* ch = chunk[b];
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 k = gload<u32x2>(ch + o.k + hp * 16 * 32);
+      r.kc[b][0] = k.x; r.kc[b][1] = k.y;
+    } else {
+      const u32x4 k = gload<u32x4>(ch + o.k + hp * 16 * 64);
+      r.kc[b][0] = k.x; r.kc[b][1] = k.y; r.kc[b][2] = k.z; r.kc[b][3] = k.w;
+    }
+    { const u32x2 t2 = gload<u32x2>(ch + o.ks + hp * 16 * 8); r.ks[b] = make_uint2(t2.x, t2.y); }
+    r.vs[b] = gload<uint16_t>(ch + o.vs + hp * 16 * 2);
+  }
+}
+
+template <int QM, int P>
+DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], int lane) {
+  using L = Lay<QM, P>;
+  // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of half s of the quad:
+  // 16-token pages 2 s, 2 s + 1 with two runs each, or the 32-token page s with four)
+  constexpr int R = P / 8;                       // runs of 8 tokens (entries per dim group) per page
+  const int m = lane & 15, kc = lane >> 4;
+#pragma unroll
+  for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {
+    const uint8_t* ch = P == 16 ? ((kc >> 1) ? chunk[2 * s2 + 1] : chunk[2 * s2]) : chunk[2 * s2];
+    const int c8 = P == 16 ? (kc & 1) : kc;
+#pragma unroll
+    for (int eh = 0; eh < 2; ++eh) {
+      if constexpr (QM == QM_ASYM2) {
+        const u32x2 v = gload<u32x2>(ch + L::V_OFF + 8 * (R * (16 * eh + m) + c8));
+        r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y;
+      } else {
+        const u32x4 v = gload<u32x4>(ch + L::V_OFF + 16 * (R * (16 * eh + m) + c8));
+        r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y; r.vc[2 * s2 + eh][2] = v.z; r.vc[2 * s2 + eh][3] = v.w;
+      }
+    }
+  }
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+struct WaveState {
+  float m;           // running maximum of head x = lane >> 4 (log2 domain; uniform over the head's 16 lanes)
+  float l;           // this lane's share of the running sum of head x
+  // 2^-24 sum p' code (zero points not yet removed), [entry word parity]: column lane & 15 = (group g, head), rows =
+  // entries 16 (g & 1) + 4 (lane >> 4) + r, entry word 2 (g >> 1) + parity
+  f32x4 ot[2];
+  float z[2];        // lane = (page, half, group, head pair): its share of sum p' zero point, heads 2 hp and 2 hp + 1
+};
+
+// exchange among the four lanes of a token (lane ^ 16, ^ 32, ^ 48): one crossbar instruction each, no vector ALU work
+// (a v_permlane32_swap costs two copies, a wait state and a select around it).  byte address of the source lane: 4 x lane
+DEVI uint32_t lane_from(uint32_t v, int src_lane4) {
+  return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(src_lane4, static_cast<int>(v)));
+}
+// all-reduce over the 16 lanes of a row (DPP: quad permutes, then the mirrors of 8 and of 16 lanes)
+DEVI float row_max16(float v) {
+  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true)));   // row_half_mirror
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true))); // row_mirror
+}
+DEVI float row_sum16(float v) {
+  v += dpp_xor1(v); v += dpp_xor2(v);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+// the 16-bit scale word `j` of a packed pair as fp32; its sign bit is a flag, which the caller drops with fabsf (a
+// source modifier of the multiply-add that uses the value).  Plain code on purpose: instructions written as inline
+// assembly are invisible to the compiler's hazard handling, and a register that a matrix instruction is still
+// writing (an unused row of its result) may be handed to them as their output.
+DEVI float word_value(uint32_t pair, int j) {
+  const uint16_t w = static_cast<uint16_t>((j & 1) ? (pair >> 16) : pair);
+  return static_cast<float>(__builtin_bit_cast(_Float16, w));
+}
+
+// Scores of the lane's (token, head) for the four blocks of the quad: raw sums 2^-20 sum_j scale_j sum (c - z) q'
+// (the factor and qscale are applied with the softmax).
+// the tokens' whole-head flags (key-only kinds; false otherwise)
+template <int QM, bool K2>
+DEVI void whole_head_flags(const KRegs<QM>& r, int lane, bool (&full)[QBLK<QM>]) {
+#pragma unroll
+  for (int b = 0; b < QBLK<QM>; ++b) {
+    // the whole-head flag is bit 15 of the token's group-0 V scale word (lane x = 0 of the token's four lanes holds it);
+    // the words of the other value groups never carry that bit (scale words are non-negative fp16 patterns), so the
+    // union over the four lanes names it
+    full[b] = false;
+    if constexpr (K2) {
+      uint32_t f = r.vs[b] & 0x8000u;
+      f |= lane_from(f, 4 * (lane ^ 16));
+      f |= lane_from(f, 4 * (lane ^ 32));
+      full[b] = f != 0u;
+    }
+  }
+}
+
+// sc += the score parts of the lane's (token, head) for the four blocks, given the tokens' whole-head flags
+template <int QM, bool K2, class SM>
+DEVI void key_scores(const SM& S, const KRegs<QM>& r, int lane, const bool (&full)[QBLK<QM>], float (&sc)[QBLK<QM>]) {
+  constexpr int QB = QBLK<QM>;
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  // the zero point of group j, masked in place (an fp16 denormal z 2^-24 in the low half of the pair word for even j,
+  // in the high half for odd j): lanes of k blocks 0 and 1 feed it (first element pair of their eight) against the pair
+  // -(sum q) of the third operand
+  const uint32_t zlane = (lane < 32) ? static_cast<uint32_t>(ZM) : 0u;
+  // group by group (one set of A operands live at a time), the four blocks of a group back to back
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const half8 qh = __builtin_bit_cast(half8, S.qhi[j][lane]), ql = __builtin_bit_cast(half8, S.qlo[j][lane]);
+    half8 qz;
+    if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[j][lane]);
+#pragma unroll
+    for (int b0 = 0; b0 < QB; b0 += 4) {
+    f32x4 acc[4];
+#pragma unroll
+    for (int bb = 0; bb < 4; ++bb) {
+      const int b = b0 + bb;
+      uint32_t x[4];
+      if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher (2^4 is in its query operand)
+        if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
+      }
+      else UnpackD<QM>::run(r.kc[b][j], x);
+      const half8 kb = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+      f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh, kb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      a = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql, kb, a, 0, 0, 0);
+      if constexpr (ZM != 0) {
+        const uint32_t kwz = (j & 2) ? r.ks[b].y : r.ks[b].x;
+        const uint32_t zz = kwz & (zlane << (16 * (j & 1)));
+        // (the same instruction as the two products before it: a chain of one kind on one accumulator)
+        a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qz, __builtin_bit_cast(half8, make_uint4(zz, 0u, 0u, 0u)), a, 0, 0, 0);
+      }
+      acc[bb] = a;
+    }
+#pragma unroll
+    for (int bb = 0; bb < 4; ++bb) {     // rows 4 x + variant of the product: the lane's head, every variant
+      const int b = b0 + bb;
+      const uint32_t kw = (j & 2) ? r.ks[b].y : r.ks[b].x;
+      float pick = acc[bb][0];
+      if constexpr (K2) {
+        const bool h32 = (kw >> (16 * (j & 1) + 15)) & 1u;
+        pick = full[b] ? acc[bb][2] : (h32 ? acc[bb][1] : acc[bb][0]);
+      }
+      sc[b] += pick * fabsf(word_value(kw, j));
+    }
+    }
+  }
+}
+
+template <int QM, bool K2, class SM>
+DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[QBLK<QM>]) {
+  bool full[QBLK<QM>];
+  whole_head_flags<QM, K2>(r, lane, full);
+#pragma unroll
+  for (int b = 0; b < QBLK<QM>; ++b) sc[b] = 0.f;
+  key_scores<QM, K2>(S, r, lane, full, sc);
+}
+
+// p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order (vs: the lane's
+// V scale words of its group x per block).
+template <int QM, class SM>
+DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
+                       int lane, int wave) {
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  constexpr int QB = QBLK<QM>;
+  // Odd tokens are unpacked from the V^T words with the factor 2^SH (UnpackD): their scores were lowered by SH (p
+  // carries 2^-SH), their zero point is raised by 2^SH; zero points are fp16 denormals like the codes.
+  const int t = lane & 15, x = lane >> 4;
+  const int sl = vslot(t & 7);
+  uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + (t >> 3) * PB_RSTRIDE * 8 + sl;   // + block * 2 rows; + (group * 4 + head) * 8
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (t >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
+  const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
+  const int c0 = ((x) * 4 + x) * 8, c1 = ((x ^ 1) * 4 + x) * 8, c2 = ((x ^ 2) * 4 + x) * 8, c3 = ((x ^ 3) * 4 + x) * 8;
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe[b], pe[b]));
+    // the token's four V scale words, sign bits stripped: own group x, then the lanes 16, 32, 48 further (groups
+    // x ^ 1, x ^ 2, x ^ 3); unwritten slots may hold any pattern: masked
+    const uint32_t v0 = valid[b] ? (vs[b] & 0x7FFFu) : 0u;
+    const uint32_t v1 = lane_from(v0, 4 * (lane ^ 16)), v2 = lane_from(v0, 4 * (lane ^ 32)), v3 = lane_from(v0, 4 * (lane ^ 48));
+    const uint32_t xa = pk_mul(pp, (v1 << 16) | v0), xb = pk_mul(pp, (v3 << 16) | v2);
+    uint16_t* row = pb + b * 2 * PB_RSTRIDE * 8;
+    row[c0] = static_cast<uint16_t>(xa);
+    row[c1] = static_cast<uint16_t>(xa >> 16);
+    row[c2] = static_cast<uint16_t>(xb);
+    row[c3] = static_cast<uint16_t>(xb >> 16);
+    if constexpr (QM != QM_SYM4) zb[b * 2 * ZB_RSTRIDE * 8] = static_cast<uint16_t>((vs[b] & ZM) << zsh);
+  }
+}
+
+// online softmax step for the quad, lane = (token, head x): the running maximum is only re-reduced when some lane
+// beats it; then p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order.
+// qs20 = qscale * 2^20 (the factor the raw score sums lack); sc0 lowers the scores of odd tokens by SH (below).
+template <int QM, class SM>
+DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
+                        float qs20, float sc0, int lane, int wave) {
+  constexpr int QB = QBLK<QM>;
+  bool beat = false;
+  float mx = -INFINITY;
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    sc[b] = valid[b] ? sc[b] * qs20 + sc0 : -INFINITY;
+    mx = fmaxf(mx, sc[b]);
+  }
+  beat = mx > st.m;
+  // The state is multiplied every time (by 1 unless the maxima moved): modifying it only inside the rare branch makes
+  // the compiler keep two copies of all its registers and move them on the common path.
+  float al = 1.f, az0 = 1.f, az1 = 1.f, am = 1.f;
+  if (__builtin_expect(__any(beat), 0)) {   // rare after the first quads
+    const float mn = fmaxf(st.m, row_max16(mx));
+    am = mn == -INFINITY ? 1.f : fexp2(st.m - mn);
+    st.m = mn;
+    // the factors of the four heads (rows of 16 lanes) for the lanes whose accumulator columns belong to them
+    const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 0));
+    const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 16));
+    const float a2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 32));
+    const float a3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am), 48));
+    al = (lane & 2) ? ((lane & 1) ? a3 : a2) : ((lane & 1) ? a1 : a0);     // accumulator column: head lane & 3
+    az0 = (lane & 1) ? a2 : a0;
+    az1 = (lane & 1) ? a3 : a1;
+  }
+  st.l *= am;
+  st.ot[0] *= al; st.ot[1] *= al;
+  st.z[0] *= az0; st.z[1] *= az1;
+  float pe[QB];
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    pe[b] = fexp2(sc[b] - st.m);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
+    st.l += pe[b];
+  }
+  write_strips<QM>(S, r.vs, pe, valid, lane, wave);
+}
+
+template <int QM, class SM>
+DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
+  // An entry word (entry half eh, word sub) holds channels of group 2 (sub >> 1) + eh only.  The products of all
+  // four groups share one accumulator per word parity: the B operand of a group is the strip row with the columns of
+  // the other groups zero (those lanes read the row group's pad entry, which nobody writes and which is zeroed once),
+  // so each column collects its own group's rows.
+  const int n = lane & 15, kc = lane >> 4;
+  const uint4* rowg = reinterpret_cast<const uint4*>(S.pb(wave)) + kc * PB_RSTRIDE;
+#pragma unroll
+  for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {   // 32 tokens: the runs (block 2 s + (kc >> 1), c8 = kc & 1) = strip row group 4 s + kc
+    half8 b[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const uint4* src = rowg + ((n >> 2) == g ? n : 16);
+      b[g] = __builtin_bit_cast(half8, src[4 * s2 * PB_RSTRIDE]);
+    }
+#pragma unroll
+    for (int eh = 0; eh < 2; ++eh)
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub) {
+        uint32_t x[4];
+        if constexpr (QM == QM_ASYM2) {   // two sub-vectors per word: the odd one's sums carry 2^4 until the fold
+          if (sub & 1) UnpackD<QM>::run_hi(r.vc[2 * s2 + eh][sub >> 1], x); else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub >> 1], x);
+        }
+        else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub], x);
+        const uint4 aq = make_uint4(x[0], x[1], x[2], x[3]);
+        st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aq), b[2 * (sub >> 1) + eh], st.ot[sub & 1], 0, 0, 0);
+      }
+  }
+  if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (block, block half, group, head pair), 8 row groups at a time
+#pragma unroll
+    for (int r8 = 0; r8 < Strip<QM>::ROWS; r8 += 8) {
+    const int rg = r8 + (lane >> 3), g = (lane >> 1) & 3, hp = lane & 1;
+    const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const uint4 pq = pp[e];
+      float a = st.z[e];
+      a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
+      st.z[e] = a;
+    }
+    }
+  }
+}
+
+// The workgroup's running maxima per head after every wavefront has put its four into S.m: lane w < NW fetches
+// wavefront w's four at once, one row reduction, one broadcast -- a single LDS round trip (a loop over the
+// wavefronts is NW dependent ones).
+template <int NW, class SM>
+DEVI void workgroup_max(const SM& S, int lane, float (&M)[4]) {
+  float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  if (lane < NW) v = *reinterpret_cast<const float4*>(&S.m[lane][0]);
+  M[0] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.x))));
+  M[1] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.y))));
+  M[2] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.z))));
+  M[3] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(v.w))));
+}
+// element i of four values held in registers (selects on values: an index into an array of locals would put the
+// array into scratch memory, and a kernel that uses scratch starts its workgroups late)
+DEVI float pick4(float v0, float v1, float v2, float v3, int i) {
+  const float lo = (i & 1) ? v1 : v0, hi = (i & 1) ? v3 : v2;
+  return (i & 2) ? hi : lo;
+}
+
+}  // namespace dec
+}  // namespace fr

@@ -16,10 +16,13 @@
 // grid.  k_wide_merge combines the splits, rotates static formats back and writes bf16.  The caller's counter words
 // are not used (they stay zero).  Byte positions follow the page layout as the writers store it (fr_common.hpp Lay,
 // place4 / store_v_codes) and as the torch parser of the front end reads it.
+#include <cstdlib>
+
 #include "fr_common.hpp"
 #include "fr_launch.hpp"
 
 namespace fr {
+int decode_wide_mma_launch(int fmt, const DecodeParams& p, int ntile, int nparts, hipStream_t st);   // decode_wide_mma.hip
 namespace {
 
 constexpr int WD = 256, WG = 8;                 // head dim, 32-channel groups per head
@@ -51,12 +54,12 @@ struct WideSmem {
 };
 
 template <int QM, bool K2, int P>
-__global__ void __launch_bounds__(256) k_wide_parts(const DecodeParams p, int ntile, int nparts) {
+__global__ void __launch_bounds__(256) k_wide_parts(const DecodeParams p, int ntile, int nparts, int split0) {
   using L = Lay<QM, P>;
   constexpr uint32_t ZMASK = QM == QM_ASYM4 ? 15u : QM == QM_ASYM2 ? 3u : 0u;
   __shared__ WideSmem S;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = blockIdx.y, b = blockIdx.z;
+  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = split0 + blockIdx.y, b = blockIdx.z;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   float* const op = p.opart + part_id * 4 * WD;
@@ -286,15 +289,26 @@ __global__ void __launch_bounds__(256) k_wide_merge(const DecodeParams p, int nt
   }
 }
 
-template <int QM, bool K2>
+template <int QM, bool K2, int FMT>
 int wide_qm(const DecodeParams& p, hipStream_t st) {
   const int ntile = (p.gqa + 3) / 4;
   const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
-  const dim3 grid(p.Hkv * ntile, nparts, p.B);
-  if (p.page == 16) hipLaunchKernelGGL((k_wide_parts<QM, K2, 16>), grid, dim3(256), 0, st, p, ntile, nparts);
-  else if (p.page == 32) hipLaunchKernelGGL((k_wide_parts<QM, K2, 32>), grid, dim3(256), 0, st, p, ntile, nparts);
-  else return -5;
-  if (hipPeekAtLastError() != hipSuccess) return -1;
+  if (p.page != 16 && p.page != 32) return -5;
+  // the body splits through the matrix-pipe kernel (decode_wide_mma.hip), the BF16 window rows through the plain one;
+  // FLAGROT_WIDE_PLAIN=1 (read at every call) sends every split through the plain kernel
+  const char* env = std::getenv("FLAGROT_WIDE_PLAIN");
+  const bool plain = env != nullptr && env[0] == '1';
+  if (!plain) {
+    const int rc = decode_wide_mma_launch(FMT, p, ntile, nparts, st);
+    if (rc) return rc;
+  }
+  const int split0 = plain ? 0 : p.nsplit;
+  if (nparts > split0) {
+    const dim3 grid(p.Hkv * ntile, nparts - split0, p.B);
+    if (p.page == 16) hipLaunchKernelGGL((k_wide_parts<QM, K2, 16>), grid, dim3(256), 0, st, p, ntile, nparts, split0);
+    else hipLaunchKernelGGL((k_wide_parts<QM, K2, 32>), grid, dim3(256), 0, st, p, ntile, nparts, split0);
+    if (hipPeekAtLastError() != hipSuccess) return -1;
+  }
   hipLaunchKernelGGL(k_wide_merge, dim3(p.Hkv * ntile, p.B), dim3(256), 0, st, p, ntile, nparts, (!K2 && p.vmask != nullptr) ? 1 : 0);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;
 }
@@ -303,12 +317,12 @@ int wide_qm(const DecodeParams& p, hipStream_t st) {
 
 int decode_wide_launch(int fmt, const DecodeParams& p, hipStream_t st) {
   switch (fmt) {
-    case FMT_INT4: return wide_qm<QM_SYM4, false>(p, st);
-    case FMT_INT4A: return wide_qm<QM_ASYM4, false>(p, st);
-    case FMT_INT2A: return wide_qm<QM_ASYM2, false>(p, st);
-    case FMT_KONLY: return wide_qm<QM_SYM4, true>(p, st);
-    case FMT_KONLYA: return wide_qm<QM_ASYM4, true>(p, st);
-    case FMT_KONLYA2: return wide_qm<QM_ASYM2, true>(p, st);
+    case FMT_INT4: return wide_qm<QM_SYM4, false, FMT_INT4>(p, st);
+    case FMT_INT4A: return wide_qm<QM_ASYM4, false, FMT_INT4A>(p, st);
+    case FMT_INT2A: return wide_qm<QM_ASYM2, false, FMT_INT2A>(p, st);
+    case FMT_KONLY: return wide_qm<QM_SYM4, true, FMT_KONLY>(p, st);
+    case FMT_KONLYA: return wide_qm<QM_ASYM4, true, FMT_KONLYA>(p, st);
+    case FMT_KONLYA2: return wide_qm<QM_ASYM2, true, FMT_KONLYA2>(p, st);
   }
   return -4;
 }

@@ -134,7 +134,7 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
     of them and about sqrt(quads of pages) per pair."""
     gran = max(64, page)
     Lmax = max(1, int(Lmax))
-    ncu = ncu or max(1, slots // 4)
+    ncu = max(1, slots // 4) if ncu is None else ncu          # 0: no large workgroups
 
     def plan(ns):
         ns = max(1, min(MAX_SPLITS, ns, math.ceil(Lmax / gran)))
@@ -157,7 +157,10 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
     """(nsplit, chunk) of a static-format decode: a workgroup per (KV head, tile of 4 query heads)"""
     tiles = Hkv * ((G + 3) // 4)
-    return plan_splits(B, Lmax, tiles, page, _slots(fmt), nsplit, ncu=_NUM_CU)
+    slots = _slots(fmt)
+    if Dh == 256:      # workgroups of 4 wavefronts only, two resident per CU (256 registers): one round of them
+        return plan_splits(B, Lmax, tiles, page, slots // 2, nsplit, ncu=0)
+    return plan_splits(B, Lmax, tiles, page, slots, nsplit, ncu=_NUM_CU)
 
 
 def plan_cb(B, Lmax, Hkv, page, kind, nsplit=None, G=4, Dh=128):

@@ -269,3 +269,11 @@ def test_head_dim_256(dev, fmt, P):
         assert strict.max() <= 1.0, (fmt, P, ns, np.unravel_index(np.argmax(strict), strict.shape))
         assert not got[-1].any()
         assert int(ws.counter.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("fmt,P", [("konlya", 16), ("int2a", 32)])
+def test_head_dim_256_plain_switch(dev, fmt, P, monkeypatch):
+    """FLAGROT_WIDE_PLAIN=1 (read at every call) sends the body splits through the plain fp32 kernel, which otherwise
+    serves the BF16 window rows only: same partial format, same bar"""
+    monkeypatch.setenv("FLAGROT_WIDE_PLAIN", "1")
+    test_head_dim_256(dev, fmt, P)
