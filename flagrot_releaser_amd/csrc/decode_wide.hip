@@ -54,12 +54,12 @@ struct WideSmem {
 };
 
 template <int QM, bool K2, int P>
-__global__ void __launch_bounds__(256) k_wide_parts(const DecodeParams p, int ntile, int nparts, int split0) {
+__global__ void __launch_bounds__(256) k_wide_parts(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
   constexpr uint32_t ZMASK = QM == QM_ASYM4 ? 15u : QM == QM_ASYM2 ? 3u : 0u;
   __shared__ WideSmem S;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = split0 + blockIdx.y, b = blockIdx.z;
+  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = blockIdx.y, b = blockIdx.z;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   float* const op = p.opart + part_id * 4 * WD;
@@ -294,20 +294,17 @@ int wide_qm(const DecodeParams& p, hipStream_t st) {
   const int ntile = (p.gqa + 3) / 4;
   const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
   if (p.page != 16 && p.page != 32) return -5;
-  // the body splits through the matrix-pipe kernel (decode_wide_mma.hip), the BF16 window rows through the plain one;
-  // FLAGROT_WIDE_PLAIN=1 (read at every call) sends every split through the plain kernel
+  // every split through the matrix-pipe kernel file (decode_wide_mma.hip) unless FLAGROT_WIDE_PLAIN=1 (read at every
+  // call) asks for the plain kernel of this file
   const char* env = std::getenv("FLAGROT_WIDE_PLAIN");
-  const bool plain = env != nullptr && env[0] == '1';
-  if (!plain) {
+  if (env != nullptr && env[0] == '1') {
+    const dim3 grid(p.Hkv * ntile, nparts, p.B);
+    if (p.page == 16) hipLaunchKernelGGL((k_wide_parts<QM, K2, 16>), grid, dim3(256), 0, st, p, ntile, nparts);
+    else hipLaunchKernelGGL((k_wide_parts<QM, K2, 32>), grid, dim3(256), 0, st, p, ntile, nparts);
+    if (hipPeekAtLastError() != hipSuccess) return -1;
+  } else {
     const int rc = decode_wide_mma_launch(FMT, p, ntile, nparts, st);
     if (rc) return rc;
-  }
-  const int split0 = plain ? 0 : p.nsplit;
-  if (nparts > split0) {
-    const dim3 grid(p.Hkv * ntile, nparts - split0, p.B);
-    if (p.page == 16) hipLaunchKernelGGL((k_wide_parts<QM, K2, 16>), grid, dim3(256), 0, st, p, ntile, nparts, split0);
-    else hipLaunchKernelGGL((k_wide_parts<QM, K2, 32>), grid, dim3(256), 0, st, p, ntile, nparts, split0);
-    if (hipPeekAtLastError() != hipSuccess) return -1;
   }
   hipLaunchKernelGGL(k_wide_merge, dim3(p.Hkv * ntile, p.B), dim3(256), 0, st, p, ntile, nparts, (!K2 && p.vmask != nullptr) ? 1 : 0);
   return hipPeekAtLastError() == hipSuccess ? 0 : -1;

@@ -9,8 +9,10 @@
 //   values   per half: p * V-scale strips of that half's four groups, then its value products into its own accumulators.
 // One workgroup of 4 wavefronts per (KV head x q tile of 4 heads, split, sequence), wavefront = head in the prologue;
 // the wavefronts draw quads of 64 tokens from a counter in LDS.  Partials go out in the format of k_wide_parts
-// (decode_wide.hip: o [4][256] relative to the part's maxima, (maximum, sum) per head), whose merge kernel and BF16
-// window split serve both.
+// (decode_wide.hip: o [4][256] relative to the part's maxima, (maximum, sum) per head), whose merge kernel serves
+// both; the BF16 sink / window rows are one more split of this grid (plain fp32, a wavefront per row).
+#include <cstddef>
+
 #include "decode_tiles.hpp"
 
 namespace fr {
@@ -125,6 +127,94 @@ DEVI void q_prologue_wide(WideMma<QM>& S, const DecodeParams& p, int b, int kvh,
   }
 }
 
+// The BF16 sink / window rows of one sequence (the split after the body splits): a wavefront takes every fourth row,
+// lanes own 4 dims (lanes 0..31 half 0, 32..63 half 1), eight rows in flight; the wavefronts are merged through LDS and
+// the partial leaves in the body splits' format.  Static formats merge in the stored basis: the rows' share is rotated
+// on the vmask groups (H32 inside the eight lanes of a group).
+template <int QM, bool K2>
+DEVI void tail_split_wide(WideMma<QM>& S, const DecodeParams& p, int b, int kvh, int tile, float* __restrict__ op,
+                          float* __restrict__ mlp) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = p.tail_len != nullptr ? p.tail_len[b] : 0;
+  if (n <= 0) {                                       // uniform
+    if (threadIdx.x < 4) { mlp[2 * threadIdx.x] = -INFINITY; mlp[2 * threadIdx.x + 1] = 0.f; }
+    return;
+  }
+  const uint16_t* base = static_cast<const uint16_t*>(p.tail) + static_cast<long long>(p.tail_idx != nullptr ? p.tail_idx[b] : b) * p.tail_bs;
+  float q[4][4], m[4], l[4], o[4][4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int hq = tile * 4 + h;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[h][i] = o[h][i] = 0.f;
+    if (hq < p.gqa) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
+                                                        (static_cast<long long>(kvh) * p.gqa + hq) * 256 + 4 * lane);
+      q[h][0] = bf16_lo(raw.x) * p.qscale; q[h][1] = bf16_hi(raw.x) * p.qscale;
+      q[h][2] = bf16_lo(raw.y) * p.qscale; q[h][3] = bf16_hi(raw.y) * p.qscale;
+    }
+    m[h] = -INFINITY; l[h] = 0.f;
+  }
+  for (int tb = wave; tb < n; tb += 4 * 8) {
+    uint2 kr[8], vr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint16_t* row = base + static_cast<long long>(min(tb + 4 * i, n - 1)) * p.tail_ts;
+      kr[i] = *reinterpret_cast<const uint2*>(row + kvh * 256 + 4 * lane);
+      vr[i] = *reinterpret_cast<const uint2*>(row + (p.Hkv + kvh) * 256 + 4 * lane);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (tb + 4 * i >= n) break;
+      const float k[4] = {bf16_lo(kr[i].x), bf16_hi(kr[i].x), bf16_lo(kr[i].y), bf16_hi(kr[i].y)};
+      const float v[4] = {bf16_lo(vr[i].x), bf16_hi(vr[i].x), bf16_lo(vr[i].y), bf16_hi(vr[i].y)};
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const float sc = wave_sum64(q[h][0] * k[0] + q[h][1] * k[1] + q[h][2] * k[2] + q[h][3] * k[3]);
+        const float mn = fmaxf(m[h], sc);
+        const float alpha = m[h] == -INFINITY ? 0.f : fexp2(m[h] - mn), pe = fexp2(sc - mn);
+        l[h] = l[h] * alpha + pe;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o[h][c] = o[h][c] * alpha + pe * v[c];
+        m[h] = mn;
+      }
+    }
+  }
+  if (lane < 4) S.m[wave][lane] = pick4(m[0], m[1], m[2], m[3], lane);
+  __syncthreads();
+  float Mwg[4];
+  workgroup_max<NWW>(S, lane, Mwg);
+  // [wave][head][256] fp32 = 16 KB in place of the operand tables (24 KB, contiguous), which this split never builds
+  static_assert(sizeof(S.qhi) + sizeof(S.qlo) >= NWW * 4 * 256 * 4 && offsetof(WideMma<QM>, qlo) == sizeof(S.qhi), "merge buffer");
+  float* buf = reinterpret_cast<float*>(&S.qhi[0][0][0]);
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const float f = m[h] == -INFINITY ? 0.f : fexp2(m[h] - Mwg[h]);
+    if (lane == 0) S.l[wave][h] = f * l[h];
+    *reinterpret_cast<float4*>(buf + (wave * 4 + h) * 256 + 4 * lane) = make_float4(f * o[h][0], f * o[h][1], f * o[h][2], f * o[h][3]);
+  }
+  __syncthreads();
+  {   // wavefront = head: sum over the wavefronts, rotate (static formats), store
+    const int h = wave;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int w = 0; w < NWW; ++w) {
+      const float4 v = *reinterpret_cast<const float4*>(buf + (w * 4 + h) * 256 + 4 * lane);
+      a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+    }
+    if (!K2 && p.vmask != nullptr) {
+      float y[4] = {a.x, a.y, a.z, a.w};
+      fwht<32>(y, lane & 31);
+      if (p.vmask[kvh * 8 + (lane >> 3)]) a = make_float4(y[0], y[1], y[2], y[3]);
+    }
+    *reinterpret_cast<float4*>(op + h * 256 + 4 * lane) = a;
+    if (lane == 0) {
+      mlp[2 * h] = pick4(Mwg[0], Mwg[1], Mwg[2], Mwg[3], h);
+      mlp[2 * h + 1] = (S.l[0][h] + S.l[1][h]) + (S.l[2][h] + S.l[3][h]);
+    }
+  }
+}
+
 template <int QM, bool K2, int P>
 __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
@@ -135,6 +225,10 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   float* const op = p.opart + part_id * 4 * 256;
   float* const mlp = p.mlpart + part_id * 8;
+  if (p.tail != nullptr && split == p.nsplit) {
+    tail_split_wide<QM, K2>(S, p, b, kvh, tile, op, mlp);
+    return;
+  }
   const int len = p.seq_lens[b];
   const int lo = max(split * p.chunk, min(p.kv_start, len)), hi = min(len, (split + 1) * p.chunk);
   if (lo >= hi) {                                     // uniform: nothing of the range is visible
@@ -324,7 +418,7 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
 
 template <int QM, bool K2>
 int wide_mma_qm(const DecodeParams& p, int ntile, int nparts, hipStream_t st) {
-  const dim3 grid(p.Hkv * ntile, p.nsplit, p.B);
+  const dim3 grid(p.Hkv * ntile, nparts, p.B);
   if (p.page == 16) hipLaunchKernelGGL((k_wide_parts_mma<QM, K2, 16>), grid, dim3(64 * NWW), 0, st, p, ntile, nparts);
   else if (p.page == 32) hipLaunchKernelGGL((k_wide_parts_mma<QM, K2, 32>), grid, dim3(64 * NWW), 0, st, p, ntile, nparts);
   else return -5;
@@ -333,9 +427,9 @@ int wide_mma_qm(const DecodeParams& p, int ntile, int nparts, hipStream_t st) {
 
 }  // namespace
 
-// the body splits (0 .. nsplit - 1) of a head dim 256 launch; nparts = nsplit (+ 1 with BF16 window rows)
+// every split of a head dim 256 launch; nparts = nsplit (+ 1 with BF16 window rows)
 int decode_wide_mma_launch(int fmt, const DecodeParams& p, int ntile, int nparts, hipStream_t st) {
-  if (p.nsplit <= 0) return 0;
+  if (nparts <= 0) return 0;
   switch (fmt) {
     case FMT_INT4: return wide_mma_qm<QM_SYM4, false>(p, ntile, nparts, st);
     case FMT_INT4A: return wide_mma_qm<QM_ASYM4, false>(p, ntile, nparts, st);
