@@ -41,16 +41,6 @@ template <int QM> struct HalfView {
   DEVI uint8_t* zb(int w) const { return work + w * Strip<QM>::BYTES + Strip<QM>::PB_BYTES; }
 };
 
-DEVI void h256(float (&y)[2][4], int l32) {                     // orthonormal H_256 of a row held as two 128-d halves
-  butterflies<128>(y[0], l32);
-  butterflies<128>(y[1], l32);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float a = y[0][i], b = y[1][i];
-    y[0][i] = (a + b) * 0.0625f;
-    y[1][i] = (a - b) * 0.0625f;
-  }
-}
 
 // The 128-d prologue per half (decode_tiles.hpp q_prologue): wavefront = head, half wave 0 writes the rows of variants
 // 0 (identity, or the static kmask rotation) and 1 (H32), half wave 1 those of variant 2 (H256) and the idle row 3.

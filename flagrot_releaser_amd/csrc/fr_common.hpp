@@ -82,6 +82,19 @@ DEVI void fwht(float (&x)[4], int l32) {  // orthonormal: butterflies, then one 
 #pragma unroll
   for (int i = 0; i < 4; ++i) x[i] = x[i] * c;
 }
+// orthonormal H_256 of a row that a half wave holds as two 128-d halves (lane l: dims 128 s + 4 l + i): the 128-d
+// butterflies per half, the stage of distance 128 inside the lane, the exact factor 1/16 -- stages in the order of the
+// smaller transforms (distance 1, 2, 4, ..), every operation rounded on its own
+DEVI void h256(float (&y)[2][4], int l32) {
+  butterflies<128>(y[0], l32);
+  butterflies<128>(y[1], l32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a = y[0][i], b = y[1][i];
+    y[0][i] = (a + b) * 0.0625f;
+    y[1][i] = (a - b) * 0.0625f;
+  }
+}
 
 // ---------------------------------------------------------------------------------------------- group statistics
 DEVI float gmax8(float a) {  // over the 8 lanes of a 32-group

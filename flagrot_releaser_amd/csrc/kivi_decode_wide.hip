@@ -82,16 +82,6 @@ DEVI void load_group(GroupRegsW& r, const uint8_t* chA, const uint8_t* chB, int 
   else r.vf = gload<uint8_t>(cht + VFW + (t & 15));
 }
 
-DEVI void h256(float (&y)[2][4], int l32) {                     // orthonormal H_256 of a row held as two 128-d halves
-  butterflies<128>(y[0], l32);
-  butterflies<128>(y[1], l32);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float a = y[0][i], b = y[1][i];
-    y[0][i] = (a + b) * 0.0625f;
-    y[1][i] = (a - b) * 0.0625f;
-  }
-}
 
 // The BF16 ring rows of one sequence (split index NS): rows [0, tail_len) of ring block tail_idx, K row h, V row Hkv + h,
 // original basis.  A wavefront takes every fourth row, lanes own 4 dims; same partial format as the page splits.

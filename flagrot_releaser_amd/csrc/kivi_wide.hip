@@ -41,16 +41,6 @@ template <bool F8> constexpr int VM2 = F8 ? 2304 : 2560;
 constexpr int VF2 = 3072;
 template <bool F8> constexpr int CELL = F8 ? 16 : 32;                 // bytes of meta per cell (8 entries)
 
-DEVI void h256(float (&y)[2][4], int l32) {
-  butterflies<128>(y[0], l32);
-  butterflies<128>(y[1], l32);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float a = y[0][i], b = y[1][i];
-    y[0][i] = (a + b) * 0.0625f;
-    y[1][i] = (a - b) * 0.0625f;
-  }
-}
 template <int C> DEVI void to_basis2(float (&y)[2][4], int l32) {     // candidate 0 identity, 1 H32, 2 H256 (involutions)
   if (C == 1) { fwht<32>(y[0], l32); fwht<32>(y[1], l32); }
   if (C == 2) h256(y, l32);

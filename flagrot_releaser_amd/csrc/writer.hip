@@ -328,17 +328,6 @@ __global__ void __launch_bounds__(256) k_k2_write(const K2WriteParams p, int tok
 // L2; the error vectors sit in an LDS strip per half wave.  The page chunk is two 128-d half chunks, half s = dims
 // [128 s, 128 s + 128), each in the 128-d layout; H32 flag of group g = sign bit of its K scale word, H256 flag = sign
 // bit of the token's group-0 V scale word of half 0.  Values are quantised as they are.
-template <int QM>
-DEVI void h256(float (&y)[2][4], int l32) {
-  butterflies<128>(y[0], l32);
-  butterflies<128>(y[1], l32);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float a = y[0][i], b = y[1][i];
-    y[0][i] = (a + b) * 0.0625f;
-    y[1][i] = (a - b) * 0.0625f;
-  }
-}
 
 template <int QM, int P>
 __global__ void __launch_bounds__(256) k_k2_write256(const K2WriteParams p) {
@@ -418,10 +407,10 @@ __global__ void __launch_bounds__(256) k_k2_write256(const K2WriteParams p) {
     for (int s = 0; s < 2; ++s)
 #pragma unroll
       for (int i = 0; i < 4; ++i) y[s][i] = x[s][i];
-    h256<QM>(y, l32);
+    h256(y, l32);
     wf[0] = quant_group<QM, true>(y[0], qf[0], ef[0]);
     wf[1] = quant_group<QM, true>(y[1], qf[1], ef[1]);
-    h256<QM>(ef, l32);
+    h256(ef, l32);
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
