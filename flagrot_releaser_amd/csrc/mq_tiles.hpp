@@ -109,8 +109,10 @@ template <int QM> struct Fmt {
 // (tg = lane & 3) hold the group.  Index bits of d: bit 0 = registers 0,1 <-> 2,3; bit 1 = low <-> high half; bits 2,3 =
 // the quad lanes (DPP); bit 4 = registers 0 <-> 1, 2 <-> 3; the two group bits of the whole-head transform = registers of
 // different groups.  The five stages inside a group run on the integers code - zero point (exact in fp16), then the
-// group scale times an exact power of two (2^-2 per group, 2^-3 whole head) is applied, then the two whole-head stages;
-// the remaining 2^-0.5 is one multiply at the end.
+// group scale times the transform's whole normalisation is applied -- as an fp16 value + remainder pair (scale x
+// 2^-2.5 is not an fp16 number; a single rounded factor would be off by up to 2^-12 for all 32 channels of the group
+// alike, which moves the group's share of every score the same way), two packed operations per register -- then the
+// whole-head stages.
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 DEVI h2_t h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
 DEVI uint32_t u2(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -208,11 +210,11 @@ DEVI void load_raw(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, in
 }
 
 // Key-only pages, one 128-d (half) chunk: the keys of (token, quarter tg) per group g as four fp16 pairs, either final
-// (rot[g] false: (code - zero point) * scale, one rounding) or rotated back up to a last factor (rot[g] true): the five
-// in-group stages on the exact integers, the group scale times 2^-2 (H32 alone) or 2^-3 (whole head: `whole`), and
-// for `whole` the two stages across the four groups.  What is left for the caller: times 2^-0.5 (head dim 128), or the
-// stage across the two halves and times 2^-1 (head dim 256).
-template <int QM>
+// (rot[g] false: (code - zero point) * scale, one rounding) or rotated back (rot[g] true): the five in-group stages on
+// the exact integers, the group scale times 2^-2.5 (H32 alone) or times the whole-head normalisation (`whole`: 2^-3.5
+// at head dim 128, 2^-4 at head dim 256), and for `whole` the two stages across the four groups.  Head dim 256 leaves
+// the stage across the two halves to the caller.
+template <int QM, int HD>
 DEVI void k2_values(const u32x4 kc, const u32x2 sw, bool whole, int tg, const Consts& cst, uint32_t (&v)[4][4], bool (&rot)[4]) {
   using F = Fmt<QM>;
   uint32_t w[4];
@@ -227,8 +229,11 @@ DEVI void k2_values(const u32x4 kc, const u32x2 sw, bool whole, int tg, const Co
   for (int g = 0; g < 4; ++g) {
     rot[g] = whole || ((s16[g] >> 15) & 1u);
     const uint32_t z = negz16(s16[g] & F::ZM) * 0x10001u, sc = (s16[g] & 0x7FFFu) * 0x10001u;
-    const uint32_t pre = whole ? 0x30003000u : 0x34003400u;                               // 2^-3, 2^-2 (exact)
-    const uint32_t sce = pk_mul(sc, pre);
+    // normalisation as fp16 value + remainder: 2^-2.5 = 0x31A8 + 0x013D, 2^-3.5 = 0x2DA8 + 0x009E, 2^-4 = 0x2C00 (exact)
+    const uint32_t ch = whole ? (HD == 128 ? 0x2DA82DA8u : 0x2C002C00u) : 0x31A831A8u;
+    const uint32_t cl = whole ? (HD == 128 ? 0x009E009Eu : 0u) : 0x013D013Du;
+    const uint32_t fh = pk_mul(sc, ch);
+    const uint32_t fl = u2(__builtin_elementwise_fma(h2(sc), h2(cl), __builtin_elementwise_fma(h2(sc), h2(ch), h2(fh ^ 0x80008000u))));
     const uint32_t nz[4] = {z, z, z, z};
     uint32_t c[4], y[4];
     Unpack<QM>::run(w[g], nz, cst, c);
@@ -236,7 +241,8 @@ DEVI void k2_values(const u32x4 kc, const u32x2 sw, bool whole, int tg, const Co
     for (int r = 0; r < 4; ++r) y[r] = c[r];
     h32_group(y, sgn1, sgn2);                 // on the integers code - zero point: exact (|sum| <= 32 * 15)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) v[g][r] = rot[g] ? pk_mul(y[r], sce) : pk_mul(c[r], sc);
+    for (int r = 0; r < 4; ++r)
+      v[g][r] = rot[g] ? u2(__builtin_elementwise_fma(h2(y[r]), h2(fl), h2(y[r]) * h2(fh))) : pk_mul(c[r], sc);
   }
   if (__any(whole)) {                                          // the two group bits of the whole-head transform
     uint32_t f[4][4];                                          // (whole: every group is rotated, v holds the y of all four)
@@ -290,14 +296,9 @@ DEVI void convert_k_entry(uint8_t* kt, int idx, const u32x4 kc, const u32x2 sw, 
       const bool ff = (vf >> 15) & 1u;
       uint32_t v[4][4];
       bool rot[4];
-      k2_values<QM>(kc, sw, ff, tg, cst, v, rot);
+      k2_values<QM, 128>(kc, sw, ff, tg, cst, v, rot);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x4 o;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = rot[g] ? pk_mul(v[g][r], 0x39A839A8u) : v[g][r];   // 2^-0.5
-        dst[4 * g + tg] = o;
-      }
+      for (int g = 0; g < 4; ++g) dst[4 * g + tg] = u32x4{v[g][0], v[g][1], v[g][2], v[g][3]};
     }
   }
 }

@@ -8,8 +8,8 @@
 //            registers more and run one wavefront per SIMD).  Price: the score product and the K conversion twice.
 // Key-only pages: the H32 flag of group g (0..7) is the sign of its K scale word in half g / 4, the whole-head H256
 // flag the sign of the token's group-0 V scale word of half 0.  A thread converts both halves of its (token, quarter):
-// the in-half stages as at 128 (k2_values), then the stage across the halves in registers and the exact factor 2^-1
-// (2^-3 before, 2^-4 = 1/16 in all).
+// the in-half stages as at 128 (k2_values, with the whole normalisation 2^-4 = 1/16 of H256 applied there), then the
+// stage across the halves in registers.
 // 128 rows per workgroup whatever the selector, like the reference at this head dim.
 #include "mq_launch.hpp"
 #include "mq_tiles.hpp"
@@ -41,8 +41,8 @@ DEVI void convert_k2_wide(uint8_t* kt0, uint8_t* kt1, int idx, const u32x4 kc0, 
   const bool ff = (vf >> 15) & 1u;
   uint32_t v0[4][4], v1[4][4];
   bool r0[4], r1[4];
-  k2_values<QM>(kc0, sw0, ff, tg, cst, v0, r0);
-  k2_values<QM>(kc1, sw1, ff, tg, cst, v1, r1);
+  k2_values<QM, 256>(kc0, sw0, ff, tg, cst, v0, r0);
+  k2_values<QM, 256>(kc1, sw1, ff, tg, cst, v1, r1);
   if (__any(ff)) {                                             // the stage across the halves
 #pragma unroll
     for (int g = 0; g < 4; ++g)
@@ -54,17 +54,10 @@ DEVI void convert_k2_wide(uint8_t* kt0, uint8_t* kt1, int idx, const u32x4 kc0, 
         v1[g][r] = ff ? b : v1[g][r];
       }
   }
-  const uint32_t last = ff ? 0x38003800u : 0x39A839A8u;       // 2^-1 (exact) after H256's eight stages, 2^-0.5 after H32's five
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    u32x4 o0, o1;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      o0[r] = r0[g] ? pk_mul(v0[g][r], last) : v0[g][r];
-      o1[r] = r1[g] ? pk_mul(v1[g][r], last) : v1[g][r];
-    }
-    d0[4 * g + tg] = o0;
-    d1[4 * g + tg] = o1;
+    d0[4 * g + tg] = u32x4{v0[g][0], v0[g][1], v0[g][2], v0[g][3]};
+    d1[4 * g + tg] = u32x4{v1[g][0], v1[g][1], v1[g][2], v1[g][3]};
   }
 }
 
