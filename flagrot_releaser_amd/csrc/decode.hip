@@ -84,10 +84,21 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
   using L = Lay<QM, P>;
   __shared__ Smem<QM, NW> S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile;
+  int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile;
   // Workgroups are dispatched in linear order and the CU's arbiter favours the older wavefronts: the splits of one
   // sequence are spread over the whole dispatch order (split slowest) so that every sequence gets the same mix.
-  const int lin = blockIdx.z * gridDim.y + blockIdx.y;
+  int lin = blockIdx.z * gridDim.y + blockIdx.y;
+  if (ntile > 1 && (p.Hkv * static_cast<int>(gridDim.y * gridDim.z)) % 8 == 0) {
+    // Workgroups go to the 8 XCDs round robin in dispatch order and each XCD has its own L2.  The q tiles of one (KV
+    // head, split, sequence) read the same pages: they are made neighbours on ONE XCD (dispatch positions 8 apart), so
+    // that the second reader finds the first one's lines in that L2 -- whoever runs ahead waits for HBM, whoever
+    // follows catches up.
+    const int pos = blockIdx.x + gridDim.x * lin;
+    const int slot = pos >> 3, t3 = (slot / ntile) * 8 + (pos & 7);
+    tile = slot % ntile;
+    kvh = t3 % p.Hkv;
+    lin = t3 / p.Hkv;
+  }
   const int split = lin / p.B, b = lin % p.B;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
   // The block-table entries of the workgroup's page range are requested before the sequence length is known (the

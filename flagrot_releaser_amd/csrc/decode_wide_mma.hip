@@ -211,7 +211,20 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
   constexpr int QB = QBLK<QM>, PPQ = 16 * QB / P;
   __shared__ WideMma<QM> S;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = blockIdx.y, b = blockIdx.z;
+  // Workgroups go to the 8 XCDs round robin in dispatch order, and each XCD has its own L2.  The q tiles of one (KV
+  // head, split, sequence) read the same pages: they are made neighbours ON ONE XCD (dispatch positions 8 apart), so
+  // that the second reader finds the first one's lines in that L2 -- whoever runs ahead waits for HBM, whoever follows
+  // catches up.  (Needs the number of (KV head, split, sequence) triples to be a multiple of 8.)
+  int kvh = blockIdx.x / ntile, tile = blockIdx.x % ntile, split = blockIdx.y, b = blockIdx.z;
+  {
+    const int triples = p.Hkv * nparts * p.B;
+    if (ntile > 1 && triples % 8 == 0) {
+      const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+      const int slot = lin >> 3, t3 = (slot / ntile) * 8 + (lin & 7);
+      tile = slot % ntile;
+      kvh = t3 % p.Hkv; split = (t3 / p.Hkv) % nparts; b = t3 / (p.Hkv * nparts);
+    }
+  }
   const long long part_id = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tile) * nparts + split;
   float* const op = p.opart + part_id * 4 * 256;
   float* const mlp = p.mlpart + part_id * 8;
