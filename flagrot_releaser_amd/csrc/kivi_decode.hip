@@ -11,12 +11,13 @@
 //                product of two fp16 numbers has 22 bits, the rounded product takes the upper 11), plus the
 //                remainder part of the query -- so the scores carry no 2^-11 rounding of terms that can be a hundred
 //                times larger than their sum (heavy outlier channels).  Written to two LDS strips (values, remainders).
-//   bias         sum q' * min per (group, head): eight more matrix products whose A operand is the channel mins (the
+//   bias         sum q' * min per (group, head): four more matrix products whose A operand is the channel mins (the
 //                same for every token row, from a 256-byte LDS strip) and whose B operand is the query rotation
 //                itself, value and remainder, straight from the workgroup's table -- exact fp16 x fp16 products summed
 //                in fp32, no per-head vector work; added to the scores as one term per lane.
-//   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads, 128 channels in eight steps
-//                (every code operand twice: against the values and against the remainders): a 2-bit code field masked in place is an fp16
+//   scores       v_mfma_f32_16x16x32_f16, rows = the 16 tokens of a page, columns = heads (0..7 against the value
+//                strips, 8..15 against the remainder strips; the two halves are added afterwards), 128 channels in
+//                four steps per page: a 2-bit code field masked in place is an fp16
 //                DENORMAL whose value is code * 2^(shift - 24) (the matrix pipe keeps denormal inputs); the power of
 //                two is folded into the query operand.
 //   softmax      exp2-domain, lane = (head, 8 tokens); the running maximum is re-reduced only when some token beats it.
@@ -312,16 +313,17 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     // ---- bias: sum q' * min of head sh (every row of the product is that sum)
     float bq;
     {
+      // columns 0..7 of the product take the rotations' values, columns 8..15 their remainders: one product where
+      // there were two, and the halves of a row of 16 lanes are added afterwards
       f32x4 bacc = {0.f, 0.f, 0.f, 0.f};
+      const uint32_t* qsel = sn < 8 ? &S.qh[wkc][sh][0] : &S.qr[wkc][sh][0];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 m4 = *reinterpret_cast<const u32x4*>(&W.mn[16 * kc + 4 * s]);
-        const u32x4 q0 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][16 * kc + 4 * s]);
-        const u32x4 q1 = *reinterpret_cast<const u32x4*>(&S.qr[wkc][sh][16 * kc + 4 * s]);
+        const u32x4 q0 = *reinterpret_cast<const u32x4*>(qsel + 16 * kc + 4 * s);
         bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q0), bacc, 0, 0, 0);
-        bacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q1), bacc, 0, 0, 0);
       }
-      bq = bacc[0] * qscale;
+      bq = (bacc[0] + ror8(bacc[0])) * qscale;
     }
     // ---- scores on the matrix pipe: rows = the 16 tokens of a page, columns = heads, 128 channels in four steps of 32.
     //      A code field masked in place is an fp16 denormal (code * 2^(shift - 24)); the bias sum q' * min enters as
@@ -329,6 +331,7 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
     f32x4 sa0, sa1;
     {
       sa0 = f32x4{0.f, 0.f, 0.f, 0.f}; sa1 = sa0;
+      const uint32_t* bsel = sn < 8 ? &W.qs[sh][0] : &W.ql[sh][0];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const uint32_t wa = (s >> 1) ? cur.ka.y : cur.ka.x, wb = (s >> 1) ? cur.kb.y : cur.kb.x;
@@ -341,14 +344,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
           xa = u32x4{wa & 0x00030003u, wa & 0x000C000Cu, wa & 0x00300030u, wa & 0x00C000C0u};
           xb = u32x4{wb & 0x00030003u, wb & 0x000C000Cu, wb & 0x00300030u, wb & 0x00C000C0u};
         }
-        // the same code operands against the products and against their remainders
-        const u32x4 b0 = *reinterpret_cast<const u32x4*>(&W.qs[sh][16 * kc + 4 * s]);
-        const u32x4 b1 = *reinterpret_cast<const u32x4*>(&W.ql[sh][16 * kc + 4 * s]);
+        // the code operands against the products (columns 0..7) and against their remainders (columns 8..15)
+        const u32x4 b0 = *reinterpret_cast<const u32x4*>(bsel + 16 * kc + 4 * s);
         sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b0), sa0, 0, 0, 0);
         sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b0), sa1, 0, 0, 0);
-        sa0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b1), sa0, 0, 0, 0);
-        sa1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b1), sa1, 0, 0, 0);
       }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { sa0[i] += ror8(sa0[i]); sa1[i] += ror8(sa1[i]); }      // value part + remainder part
     }
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
     {

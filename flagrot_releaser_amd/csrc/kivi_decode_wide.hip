@@ -293,21 +293,23 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
       wave_lds_sync();
       const int wkc = useF ? 2 : static_cast<int>((lmask >> (4 * hf + kc)) & 1u);   // sub-vector 4 hf + kc = pairs 16 kc .. 16 kc + 15 of the half
       // ---- bias: sum q' * min of head sh over the half (every row of the product is that sum)
+      // Columns 0..7 of a product take the values (of the rotation / of q' * scale), columns 8..15 the remainders: one
+      // product where there would be two; the halves of a row of 16 lanes are added at the end.  Every product starts
+      // from zero and the partial sums are added by the vector unit (round to nearest): the matrix pipe cuts addends
+      // far below the largest one of an instruction short, and with a token in the group that is hundreds of times
+      // larger than its neighbours a chain of 32 instructions through one accumulator left the scores of the whole
+      // group ~5e-3 (log2 units) low.
+      const uint32_t* qsel = sn < 8 ? &S.qh[wkc][sh][hf][0] : &S.qr[wkc][sh][hf][0];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 m4 = *reinterpret_cast<const u32x4*>(&W.mn[16 * kc + 4 * s]);
-        const u32x4 q0 = *reinterpret_cast<const u32x4*>(&S.qh[wkc][sh][hf][16 * kc + 4 * s]);
-        const u32x4 q1 = *reinterpret_cast<const u32x4*>(&S.qr[wkc][sh][hf][16 * kc + 4 * s]);
-        // every product starts from zero and the partial sums are added by the vector unit (round to nearest): the
-        // matrix pipe cuts addends far below the largest one of an instruction short, and with a token in the group
-        // that is hundreds of times larger than its neighbours a chain of 32 instructions through one accumulator
-        // left the scores of the whole group ~5e-3 (log2 units) low
+        const u32x4 q0 = *reinterpret_cast<const u32x4*>(qsel + 16 * kc + 4 * s);
         const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
         const f32x4 t0_ = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q0), z4, 0, 0, 0);
-        const f32x4 t1_ = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, m4), __builtin_bit_cast(half8, q1), z4, 0, 0, 0);
-        bacc[0] += t0_[0]; bacc[0] += t1_[0];
+        bacc[0] += t0_[0];
       }
       // ---- scores: rows = the 16 tokens of a page, columns = heads, the half's 128 channels in four steps of 32
+      const uint32_t* bsel = sn < 8 ? &W.qs[sh][0] : &W.ql[sh][0];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const uint32_t wa = (s >> 1) ? cur.ka[hf].y : cur.ka[hf].x, wb = (s >> 1) ? cur.kb[hf].y : cur.kb[hf].x;
@@ -320,17 +322,16 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
           xa = u32x4{wa & 0x00030003u, wa & 0x000C000Cu, wa & 0x00300030u, wa & 0x00C000C0u};
           xb = u32x4{wb & 0x00030003u, wb & 0x000C000Cu, wb & 0x00300030u, wb & 0x00C000C0u};
         }
-        const u32x4 b0 = *reinterpret_cast<const u32x4*>(&W.qs[sh][16 * kc + 4 * s]);
-        const u32x4 b1 = *reinterpret_cast<const u32x4*>(&W.ql[sh][16 * kc + 4 * s]);
+        const u32x4 b0 = *reinterpret_cast<const u32x4*>(bsel + 16 * kc + 4 * s);
         const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
         sa0 += __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b0), z4, 0, 0, 0);
         sa1 += __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b0), z4, 0, 0, 0);
-        sa0 += __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xa), __builtin_bit_cast(half8, b1), z4, 0, 0, 0);
-        sa1 += __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, xb), __builtin_bit_cast(half8, b1), z4, 0, 0, 0);
       }
       wave_lds_sync();                            // the strips are free for the other half / the next group
     }
-    const float bq = bacc[0] * qscale;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sa0[i] += ror8(sa0[i]); sa1[i] += ror8(sa1[i]); }      // value part + remainder part
+    const float bq = (bacc[0] + ror8(bacc[0])) * qscale;
     // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
     {
       float sc[8];                       // raw accumulators: score = sc * 2^24 * qscale (a positive factor)

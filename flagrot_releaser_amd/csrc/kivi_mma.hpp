@@ -27,6 +27,9 @@ DEVI uint32_t pack_rn(float a, float b) {
   half2_t v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
   return __builtin_bit_cast(uint32_t, v);
 }
+DEVI float ror8(float v) {      // the value of the lane 8 further in its row of 16 (row_ror:8)
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));
+}
 template <class T> DEVI T gload(const uint8_t* p) {
   typedef const __attribute__((address_space(1))) T* gp;
   return *(gp)(p);
