@@ -352,21 +352,25 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
 #pragma unroll
       for (int i = 0; i < 4; ++i) { sa0[i] += ror8(sa0[i]); sa1[i] += ror8(sa1[i]); }      // value part + remainder part
     }
-    // ---- softmax: lane = (head sh, tokens 4 kc + r of page A and of page B)
+    // ---- softmax: lane = (head sh, tokens 4 kc + r of page A (columns 0..7) or of page B (columns 8..15))
     {
-      float sc[8];                       // raw accumulators: score = sc * 2^24 * qscale (a positive factor)
+      // after the halves were added both column halves hold the totals: the lanes of columns 0..7 go on with page A's
+      // four tokens, those of columns 8..15 with page B's
+      const int pgb = sn >> 3;
+      float sc[4];                       // raw accumulators: score = sc * 2^24 * qscale (a positive factor)
       const float up = 16777216.f * qscale;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sc[i] = i < 4 ? sa0[i & 3] : sa1[i & 3];
+      for (int i = 0; i < 4; ++i) sc[i] = pgb ? sa1[i] : sa0[i];
       if (!full) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int pos = gi * 32 + 16 * (i >> 2) + 4 * kc + (i & 3);
+        for (int i = 0; i < 4; ++i) {
+          const int pos = gi * 32 + 16 * pgb + 4 * kc + i;
           sc[i] = (pos >= t0 && pos < t1) ? sc[i] : -INFINITY;
         }
       }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))) * up + bq;
+      float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])) * up + bq;
       if (__any(mx > m_run)) {
+        mx = fmaxf(mx, ror8(mx));
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m_run, mx);
@@ -383,16 +387,13 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
         for (int r = 0; r < 4; ++r) amd[r] *= __shfl(alpha, 4 * kc + r, 64);      // rows = heads 4 kc + r (8..15 repeat 0..7)
       }
       // a wavefront's group always holds a token of the range: the maximum is finite from its first group on
-      float p[8];
+      float p[4];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < 4; ++i) {
         p[i] = fexp2(__builtin_fmaf(sc[i], up, bq - m_run));
         l_run += p[i];
       }
-      if (sn < 8) {
-        *reinterpret_cast<u32x2*>(&W.pst[sh][4 * kc]) = u32x2{pack_rn(p[0], p[1]), pack_rn(p[2], p[3])};
-        *reinterpret_cast<u32x2*>(&W.pst[sh][16 + 4 * kc]) = u32x2{pack_rn(p[4], p[5]), pack_rn(p[6], p[7])};
-      }
+      *reinterpret_cast<u32x2*>(&W.pst[sh][16 * pgb + 4 * kc]) = u32x2{pack_rn(p[0], p[1]), pack_rn(p[2], p[3])};
     }
     wave_lds_sync();
     // ---- values on the matrix pipe: rows = the 32 channels of a sub-vector, columns = (class, head), 32 tokens in two
@@ -422,7 +423,8 @@ __global__ void __launch_bounds__(256, 3) k_attn_pages(const uint16_t* __restric
 
   // ---- merge of the wavefronts: maxima, sums, accumulators per class (in wavefront order), inverse transforms
   {
-    float lt = l_run + __shfl_xor(l_run, 16, 64);
+    float lt = l_run + ror8(l_run);
+    lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (lane < G) { S.mw[wv][lane] = m_run; S.lw[wv][lane] = lt; }
     if (sn < 12 && kc < 2) {
