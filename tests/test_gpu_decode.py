@@ -208,8 +208,20 @@ def test_head_dim_256(dev, fmt, P):
     """head dim 256 (`variant | 4096`; the reference's shape (G, D, Hkv) = (6, 256, 4), test_kernels.py:366-374): pages
     of two 128-d half chunks written by the 256-d writers, q tiles of 4 + 2 heads, splits, BF16 window rows, kv_start,
     ragged lengths; against the oracle's dequantise-then-attend at that head dim, element-wise bar."""
+    _head_dim_256(dev, fmt, P, 6, 4)
+
+
+@pytest.mark.parametrize("fmt", ["konlya2", "int4a"])
+@pytest.mark.parametrize("G,Hkv", [(1, 4), (4, 2), (8, 2), (12, 1), (5, 8)])
+def test_head_dim_256_groups(dev, fmt, G, Hkv):
+    """other GQA groups at head dim 256: one, two and three q tiles per KV head (with and without the placement of a
+    KV head's tiles on one XCD, which needs (KV heads x splits x sequences) to be a multiple of 8)"""
+    _head_dim_256(dev, fmt, 16, G, Hkv)
+
+
+def _head_dim_256(dev, fmt, P, G, Hkv):
     from flagrot_releaser_amd import kernels as K
-    Dh, G, Hkv = 256, 6, 4
+    Dh = 256
     static = fmt in ("int4", "int4a", "int2a")
     g = torch.Generator().manual_seed(600 + len(fmt) + P)
     lens = [1, 17, 64, 65, 333, 700, 0]
@@ -252,7 +264,7 @@ def test_head_dim_256(dev, fmt, P):
         ns, ch = (K.plan_v2 if static else K.plan_cb)(B, max(lens), Hkv, P, *((fmt,) if not static else ()), nsplit=nsplit,
                                                      **({"fmt": fmt} if static else {}), G=G, Dh=Dh)
         HV, GT = K.vheads(Hkv, G, Dh, fmt), K.tile_of(K.v2_variant(fmt, G, Dh))
-        assert (HV, GT) == (2 * Hkv, 4)
+        assert (HV, GT) == (Hkv * ((G + 3) // 4), 4)
         ws = K.Workspace(B, HV, B * HV * (ns + 1), dev, GT, Dh)
         out = torch.full((B, HQ * Dh), float("nan"), dtype=torch.bfloat16, device=dev)
         if static:
