@@ -285,7 +285,7 @@ def _head_dim_256(dev, fmt, P, G, Hkv):
 
 @pytest.mark.parametrize("fmt,P", [("konlya", 16), ("int2a", 32)])
 def test_head_dim_256_plain_switch(dev, fmt, P, monkeypatch):
-    """FLAGROT_WIDE_PLAIN=1 (read at every call) sends the body splits through the plain fp32 kernel, which otherwise
-    serves the BF16 window rows only: same partial format, same bar"""
+    """FLAGROT_WIDE_PLAIN=1 (read at every call) sends every split through the plain fp32 kernel instead of the
+    matrix-pipe one: same partial format, same bar"""
     monkeypatch.setenv("FLAGROT_WIDE_PLAIN", "1")
     test_head_dim_256(dev, fmt, P)

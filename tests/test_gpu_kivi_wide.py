@@ -241,7 +241,7 @@ def test_attn_against_fp64(dev, case, f8):
 
 
 def test_attn_plain_kernel_switch(dev, monkeypatch):
-    """FLAGROT_KIVI_WIDE_PLAIN=1 (read at every call) sends the page splits through the plain fp32 kernel as well: same
+    """FLAGROT_KIVI_WIDE_PLAIN=1 (read at every call) sends every split through the plain fp32 kernel instead: same
     partial format, same merge, outputs within the bar of each other and of the fp64 reference"""
     from flagrot_releaser_amd import kivi as KV
     lens, Hkv, G, kv_start, (ns, chunk), tails = CASES[2]
