@@ -30,7 +30,10 @@ int fr_abi_version(void);
  * caller (merge tickets and, when the body workgroups of a sequence share its page range, their page draws; the last
  * arriving workgroup leaves the word at 0).  If B*Hkv*ceil(gqa/4)*nsplit fits the CUs and chunk >= 1024, split s owns
  * tokens [s, s+1)*chunk and one large workgroup per CU runs it; otherwise nsplit only counts the workgroups per
- * (sequence, KV head, q tile); nsplit*chunk must cover the longest sequence either way. */
+ * (sequence, KV head, q tile); nsplit*chunk must cover the longest sequence either way.
+ * variant bit 4096 (kernels/csrc/attn_decode_v2g.cuh:11-25, 276): head dim 256 -- q, out and tail rows have 256 channels,
+ * the pool chunk is two 128-d half chunks per (page, KV head), kmask / vmask are [Hkv, 8], partials are GT*256 floats
+ * with GT = 4, split s owns tokens [s, s+1)*chunk and the counter words are not used. */
 int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
                const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale,
                const uint8_t* kmask, const uint8_t* vmask, int rb, int qrot, int vrot, int variant, int stages,
