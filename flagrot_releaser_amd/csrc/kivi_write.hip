@@ -423,11 +423,26 @@ __global__ void __launch_bounds__(256) k_dequant(const uint8_t* __restrict__ poo
       float x[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = static_cast<float>((byte >> (2 * i)) & 3u) * vs + vmn;
-      if (f) fwht<128>(x, l32);
-      else if (l) {
+      // The two tokens of a wavefront may differ in their flags: the stages H32 and H128 share (distance 1 .. 16 channels
+      // first, in H128's own order) run once for both, H128 adds its two stages across the sub-vectors.
+      if (f || l) {
         float y[4] = {x[0], x[1], x[2], x[3]};
-        fwht<32>(y, l32);
-        if ((l >> j) & 1u) { x[0] = y[0]; x[1] = y[1]; x[2] = y[2]; x[3] = y[3]; }
+        butterflies<32>(y, l32);
+        if (f) {
+#pragma unroll
+          for (int lm = 8; lm <= 16; lm <<= 1) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float o2 = hx(y[i], lm);
+              y[i] = (l32 & lm) ? (o2 - y[i]) : (y[i] + o2);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[i] = y[i] * kC128;
+        } else if ((l >> j) & 1u) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[i] = y[i] * kC32;
+        }
       }
       if (o < nvalid)
 #pragma unroll
