@@ -72,3 +72,17 @@ def test_configs4_mq_prefill_4x512_over_16384(dev, fmt):
     _report(f"configs[4] {fmt}", r)
     assert r["checked"] and r["errors"]["rel_l2"] <= 3e-3, r["check"]
     assert r["rows_per_tile"] == 256
+
+
+def test_head_dim_256_bench_shapes(dev):
+    """the head dim 256 workloads of bench.py (--head-dim 256; GQA 24q/4kv, no configuration of the baseline): FlagRot
+    INT4 decode, KIVI decode and the multi-query prefill at their record shapes, same bars as their 128-d workloads"""
+    r = bench.run_flagrot(_args(head_dim=256), torch, dev, "int4", 3, 2)["own"]
+    _report("INT4 decode, head dim 256", r)
+    assert r["checked"] and r["errors"]["elementwise"] <= 1.0, r["check"]
+    r = bench.run_kivi(_args(head_dim=256), torch, dev, 3, 2)
+    _report("KIVI decode, head dim 256", r)
+    assert r["checked"] and r["errors"]["elementwise"] <= 1.0, r["check"]
+    r = bench.run_mq(_args(head_dim=256), torch, dev, 2, 1, "konlya")
+    _report("MQ prefill, head dim 256", r)
+    assert r["checked"] and r["errors"]["rel_l2"] <= 3e-3 and r["rows_per_tile"] == 128, r["check"]
