@@ -99,7 +99,14 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
     kvh = t3 % p.Hkv;
     lin = t3 / p.Hkv;
   }
-  const int split = lin / p.B, b = lin % p.B;
+  // Where the body workgroups of a sequence draw from one shared range, the BF16 rows' workgroups (the last split) go
+  // first in dispatch order: short ones that start with the launch instead of trailing it, and a body workgroup that
+  // starts later for it just draws what is left.  (With fixed ranges per split a late start is a late end: there the
+  // body goes first; measured both ways.)
+  const int nsp = static_cast<int>(gridDim.y * gridDim.z) / p.B;
+  int split = lin / p.B;
+  if (p.tail != nullptr && p.dyn != 0) split = split == 0 ? nsp - 1 : split - 1;
+  const int b = lin % p.B;
   const bool is_tail = p.tail != nullptr && split == p.nsplit;
   // The block-table entries of the workgroup's page range are requested before the sequence length is known (the
   // length load and these loads are then in flight together: one memory latency less before the first page arrives).
