@@ -22,16 +22,32 @@ __global__ void __launch_bounds__(128) k_merge(const float* __restrict__ opart, 
                                                int NS, uint16_t* __restrict__ out, long long out_rs) {
   const int b = blockIdx.x, hq = blockIdx.y, h = hq / G, g = hq % G;
   const long long p0 = (static_cast<long long>(b) * Hkv + h) * (NS + 1);
+  // eight partials at a time: their loads are issued together (one after the other in a plain loop, each iteration
+  // would wait for its own)
   float M = -INFINITY;
-  for (int s = 0; s <= NS; ++s) M = fmaxf(M, ml[((p0 + s) * G + g) * 2]);
+  for (int s0 = 0; s0 <= NS; s0 += 8) {
+    float m8[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m8[i] = ml[((p0 + min(s0 + i, NS)) * G + g) * 2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) M = fmaxf(M, m8[i]);
+  }
   float o = 0.f, L = 0.f;
   if (M != -INFINITY) {
-    for (int s = 0; s <= NS; ++s) {
-      const float m = ml[((p0 + s) * G + g) * 2];
-      if (m == -INFINITY) continue;
-      const float f = exp2f(m - M);
-      L += f * ml[((p0 + s) * G + g) * 2 + 1];
-      o += f * opart[((p0 + s) * G + g) * 128 + threadIdx.x];
+    for (int s0 = 0; s0 <= NS; s0 += 8) {
+      float m8[8], l8[8], o8[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const long long at = (p0 + min(s0 + i, NS)) * G + g;
+        m8[i] = ml[at * 2]; l8[i] = ml[at * 2 + 1]; o8[i] = opart[at * 128 + threadIdx.x];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (s0 + i > NS || m8[i] == -INFINITY) continue;
+        const float f = exp2f(m8[i] - M);
+        L += f * l8[i];
+        o += f * o8[i];
+      }
     }
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
