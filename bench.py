@@ -317,6 +317,20 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
             "checked": bool(st["elementwise"] <= 1.0), "bar": "elementwise <= 1", "errors": st,
             "check": f"sequences {rows} x all {G * HKV} heads vs the fp64 oracle: " + describe(st),
         }
+    # the yardstick: a kernel that only READS the same pages through the same block table, with the decode kernel's
+    # workgroup layout (flagrot_releaser_amd/csrc/probe_read.hip), timed the same way on the same caches
+    if DH == 128:
+        from flagrot_releaser_amd import probe as PR
+        PR.lib()
+        sink_word = torch.zeros(4, dtype=torch.int32, device=dev)
+        tr = timed(torch, lambda i: PR.read_pages(pools[i % ncopy], bt, seq, sink_word, P), steps, warmup)
+        rus = tr["graph_us"]
+        first = results[plans[0]]
+        first["read_probe"] = {"us": round(rus, 2), "GBps": round(page_bytes / (rus * 1e-6) / 1e9, 1),
+                               "frac_of_peak": round(page_bytes / (rus * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4),
+                               "decode_over_read": round(first["us_per_layer_step"] / rus, 3),
+                               "note": "a kernel that only reads the launch's page chunks through the same block table "
+                                       "(16-wavefront workgroup per (sequence, KV head), 4 pages in flight per wavefront)"}
     # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
     kv_new = synth_kv(B, g, dev, torch, mu=kmu, hkv=HKV, dh=DH)
     slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
@@ -599,7 +613,7 @@ def main():
                             "avg_launch_us": r["us_per_layer_step"], "graph_min_us": r["graph_min_us"],
                             "graph_max_us": r["graph_max_us"], "eager_us": r["eager_us"]},
                "checked": r["checked"], "bar": r["bar"], "errors": r["errors"], "check": r["check"]}
-        for extra in ("writer", "dequant"):
+        for extra in ("writer", "dequant", "read_probe"):
             if extra in r:
                 res[extra] = r[extra]
         if workload == "int4" and extras:

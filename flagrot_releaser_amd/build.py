@@ -1,7 +1,7 @@
 """Builds the gfx950 shared libraries of this package with hipcc (cross-compiles without a GPU).
 
     python -m flagrot_releaser_amd.build            # all libraries
-    python -m flagrot_releaser_amd.build kernels    # one of: kernels, kivi, mq
+    python -m flagrot_releaser_amd.build kernels    # one of: kernels, kivi, mq, probe (a measurement aid for bench.py)
 
 Libraries land in flagrot_releaser_amd/lib/ (in-tree, git-ignored).  Counterpart of the reference's
 integrations/vllm_flagrot/csrc/build.sh / build_kivi.sh / build_mq.sh.
@@ -30,6 +30,7 @@ LIBS = {
     "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("decode_wide_mma.hip", []), ("capi.hip", [])]),
     "kivi": ("libflagrot_kivi.so", [("kivi_write.hip", STRICT), ("kivi_wide.hip", STRICT), ("kivi_attn.hip", []), ("kivi_decode.hip", []), ("kivi_decode_wide.hip", [])]),
     "mq": ("libflagrot_mq.so", [("mq_prefill.hip", []), ("mq_wide.hip", [])]),
+    "probe": ("libflagrot_probe.so", [("probe_read.hip", [])]),      # measurement aid (bench.py), not a boundary library
 }
 
 

@@ -64,6 +64,20 @@ def test_mq_library_exports_header_symbols():
     assert 0 < L.frmq_smem_bytes() <= 160 * 1024
 
 
+def test_probe_library_exports_header_symbols():
+    from flagrot_releaser_amd import build, probe
+    path = build.lib_path("probe")
+    if not path.exists():
+        build.build("probe", verbose=False)
+    L = ctypes.CDLL(str(path))
+    names = _declared("flagrot_probe.h")
+    assert set(names) == set(probe.EXPORTS) == {"fr_probe_abi_version", "fr_probe_last_error", "fr_probe_read"}
+    for n in names:
+        assert hasattr(L, n), n
+    L.fr_probe_abi_version.restype = ctypes.c_int
+    assert L.fr_probe_abi_version() == probe.ABI
+
+
 def test_host_planner_invariants():
     from flagrot_releaser_amd import kernels as K
     for B, L in ((1, 1), (1, 2048), (32, 8192), (64, 16384), (3, 33000), (8, 65536)):
