@@ -60,10 +60,10 @@ struct GroupRegsW {
   uint32_t vf;         // the token's whole-head flag: non-zero = H256
 };
 
+// The key words and the value words of a group are requested apart: each set as soon as the phase that read the
+// previous group's set is over, into the same registers (one register set per wavefront instead of two).
 template <bool F8>
-DEVI void load_group(GroupRegsW& r, const uint8_t* chA, const uint8_t* chB, int lane) {
-  const int t = lane & 31, hh = lane >> 5;
-  const uint8_t* cht = t < 16 ? chA : chB;
+DEVI void load_group_keys(GroupRegsW& r, const uint8_t* chA, const uint8_t* chB, int lane) {
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
     r.ka[hf] = gload<u32x2>(chA + (lane & 15) * 64 + 32 * hf + 8 * (lane >> 4));
@@ -72,6 +72,11 @@ DEVI void load_group(GroupRegsW& r, const uint8_t* chA, const uint8_t* chB, int 
     if (F8) r.km[hf] = u32x2{gload<uint32_t>((hf ? chB : chA) + KMW + lane * 4), 0u};
     else r.km[hf] = gload<u32x2>((hf ? chB : chA) + KMW + lane * 8);
   }
+}
+template <bool F8>
+DEVI void load_group_values(GroupRegsW& r, const uint8_t* chA, const uint8_t* chB, int lane) {
+  const int t = lane & 31, hh = lane >> 5;
+  const uint8_t* cht = t < 16 ? chA : chB;
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
     r.vc[p] = gload<u32x4>(cht + VCW<F8> + (t & 15) * 64 + 32 * p + 16 * hh);
@@ -239,17 +244,18 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
 
   GroupRegsW cur;
   int gi = g_first + wv;
-  if (gi < g_end) load_group<F8>(cur, pool + (static_cast<long long>(btb[2 * gi]) * Hkv + h) * CHUNKW<F8>,
-                                 pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNKW<F8>, lane);
+  if (gi < g_end) {
+    const uint8_t* chA = pool + (static_cast<long long>(btb[2 * gi]) * Hkv + h) * CHUNKW<F8>;
+    const uint8_t* chB = pool + (static_cast<long long>(btb[2 * gi + 1]) * Hkv + h) * CHUNKW<F8>;
+    load_group_keys<F8>(cur, chA, chB, lane);
+    load_group_values<F8>(cur, chA, chB, lane);
+  }
   for (; gi < g_end; gi += 4) {
     const bool full = gi * 32 >= t0 && gi * 32 + 32 <= t1;     // every token of the group is inside the range (wave uniform)
-    // the next group is requested on every path (past the range: the range's last group again, a cache hit nobody uses)
-    GroupRegsW nxt;
-    {
-      const int gn = min(gi + 4, g_end - 1);
-      load_group<F8>(nxt, pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNKW<F8>,
-                     pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNKW<F8>, lane);
-    }
+    // the next group's pages (past the range: the range's last group again, a cache hit nobody uses)
+    const int gn = min(gi + 4, g_end - 1);
+    const uint8_t* const chAn = pool + (static_cast<long long>(btb[2 * gn]) * Hkv + h) * CHUNKW<F8>;
+    const uint8_t* const chBn = pool + (static_cast<long long>(btb[2 * gn + 1]) * Hkv + h) * CHUNKW<F8>;
     // ---- group flags, all in the meta of half 0: sub-vector j = channel j (FP8: channel 8 j), whole head = channel 8 (FP8: 64)
     bool useF;
     uint32_t lmask = 0;
@@ -329,6 +335,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
       }
       wave_lds_sync();                            // the strips are free for the other half / the next group
     }
+    // the key words are read: the next group's take their registers (in flight over the softmax and the value phase)
+    __builtin_amdgcn_sched_barrier(0);
+    load_group_keys<F8>(cur, chAn, chBn, lane);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) { sa0[i] += ror8(sa0[i]); sa1[i] += ror8(sa1[i]); }      // value part + remainder part
     const float bq = (bacc[0] + ror8(bacc[0])) * qscale;
@@ -431,7 +441,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
       }
       wave_lds_sync();
     }
-    cur = nxt;
+    // ... and the value words likewise (in flight over the next group's key phase)
+    __builtin_amdgcn_sched_barrier(0);
+    load_group_values<F8>(cur, chAn, chBn, lane);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- merge of the wavefronts: maxima, sums, accumulators per class (in wavefront order), inverse transforms
