@@ -54,12 +54,7 @@ __global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
 
   // page ids of the first blocks (published by the barriers of the q staging below)
   int cb = kb0;
-  auto fill_pages = [&]() {
-    for (int i = tid; i < PG_CACHE; i += NT) {
-      const int pgx = 4 * cb + i;
-      S.pages[i] = pgx * PAGE < kend ? bt[pgx] : 0;
-    }
-  };
+  auto fill_pages = [&]() { fill_page_window<NT>(S.pages, bt, cb, kb1, kend, tid); };
   fill_pages();
 
   // q fragments: the tile through LDS (natural order), gathered in code-word order
@@ -88,26 +83,36 @@ __global__ void __launch_bounds__(64 * NW, 2) k_mq(const Params p) {
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float mrow = -INFINITY, lrow = 0.f;
 
+  // Raw words in flight: two blocks ahead in two register sets; the 64-row kernel (two entries per thread and set) has
+  // room for one set only and fetches one block ahead -- a second set there is spilled as it arrives, and a spilled
+  // register's reload waits for every fetch in flight.
+  constexpr int AHEAD = NW == 2 ? 1 : 2;
   Raw<NT> rawA, rawB;
-  if (kb0 < kb1) load_raw<QM, K2, NT>(rawA, p, S.pages, h, kb0, kend);
-  if (kb0 + 1 < kb1) load_raw<QM, K2, NT>(rawB, p, S.pages + 4, h, kb0 + 1, kend);
+  if (kb0 < kb1) load_raw<QM, K2, NT, NW == 2>(rawA, p, S.pages, h, kb0, kend);
+  if constexpr (AHEAD == 2) {
+    if (kb0 + 1 < kb1) load_raw<QM, K2, NT, NW == 2>(rawB, p, S.pages + 4, h, kb0 + 1, kend);
+  }
   auto block_step = [&](Raw<NT>& raw, int kb) {
     __syncthreads();                                   // the tiles (or the q staging) are no longer read
     convert_k<QM, K2, NT>(S, raw, kb, kend, cst);
     v_tables<QM, NT>(S, raw, kb, kend);
-    if (kb + 2 < kb1 && kb + 2 >= cb + PG_CACHE / 4) {   // the next fetch leaves the cached window: slide it
-      cb = kb + 2;
+    if (kb + AHEAD < kb1 && kb + AHEAD >= cb + PG_CACHE / 4) {   // the next fetch leaves the cached window: slide it
+      cb = kb + AHEAD;
       fill_pages();
     }
     __syncthreads();
     convert_v<QM, NT>(S, raw, kb, kend, cst);
     __syncthreads();
-    if (kb + 2 < kb1) load_raw<QM, K2, NT>(raw, p, S.pages + 4 * (kb + 2 - cb), h, kb + 2, kend);   // two blocks ahead
+    if (kb + AHEAD < kb1) load_raw<QM, K2, NT, NW == 2>(raw, p, S.pages + 4 * (kb + AHEAD - cb), h, kb + AHEAD, kend);
     attend_block(S, qf, o, mrow, lrow, kb, lim, rvalid, p.kmin, l32, hh);
   };
-  for (int kb = kb0; kb < kb1; kb += 2) {
-    block_step(rawA, kb);
-    if (kb + 1 < kb1) block_step(rawB, kb + 1);
+  if constexpr (AHEAD == 2) {
+    for (int kb = kb0; kb < kb1; kb += 2) {
+      block_step(rawA, kb);
+      if (kb + 1 < kb1) block_step(rawB, kb + 1);
+    }
+  } else {
+    for (int kb = kb0; kb < kb1; ++kb) block_step(rawA, kb);
   }
   // partials
   const float l = lrow + __shfl_xor(lrow, 32, 64);
@@ -140,15 +145,6 @@ struct Smem8 {
   int pages[PG_CACHE];
 };
 static_assert(256 * QROW <= 2 * (KT_BYTES + VT_BYTES), "q staging aliases the tiles");
-
-// The thread index as a value the compiler must take as new at every use site: what a converter derives from it (tile
-// addresses, lane offsets) is recomputed per block with a few integer operations instead of being kept in registers
-// across the whole key loop, where the accumulators leave no room for it.
-DEVI int tid_now() {
-  int t = threadIdx.x;
-  asm volatile("" : "+v"(t));
-  return t;
-}
 
 // Raw page words of a thread's tile entry, one register set for both groups (a set per group would let the compiler
 // reuse the other group's registers for LDS operands and guard them with waits on outstanding fetches):
@@ -353,12 +349,7 @@ __global__ void __launch_bounds__(512, 1) k_mq8(const Params p) {
   const int lim = rvalid ? work.last_key(r / G) : -1;
 
   int cb = kb0;
-  auto fill_pages = [&]() {
-    for (int i = tid; i < PG_CACHE; i += NT) {
-      const int pgx = 4 * cb + i;
-      S.pages[i] = pgx * PAGE < kend ? bt[pgx] : 0;
-    }
-  };
+  auto fill_pages = [&]() { fill_page_window<NT>(S.pages, bt, cb, kb1, kend, tid); };
   fill_pages();
 
   u32x4 qf[8];

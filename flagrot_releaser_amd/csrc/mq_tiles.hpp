@@ -141,6 +141,33 @@ DEVI void h32_group(uint32_t (&x)[4], uint32_t sgn1, uint32_t sgn2) {
 }
 
 // ------------------------------------------------------------------------------------------------ tile converters
+// Page ids of the blocks [cb, cb + PG_CACHE / 4) of an item into the LDS window.  Only the item's own pages are read
+// (entries past them are 0) and every load is unconditional, its index clamped to the item's last page: a thread's
+// loads are in flight together, one memory latency per fill (as loads under a condition each was waited for in turn).
+template <int NT>
+DEVI void fill_page_window(int* pages, const int* bt, int cb, int kb1, int kend, int tid) {
+  constexpr int NF = PG_CACHE / NT;
+  const int last = min(4 * kb1, (kend + PAGE - 1) / PAGE) - 1;     // the item's last page
+  int v[NF];
+#pragma unroll
+  for (int k = 0; k < NF; ++k) v[k] = 0;
+  if (last >= 4 * cb) {                                              // (uniform over the workgroup)
+#pragma unroll
+    for (int k = 0; k < NF; ++k) v[k] = bt[min(4 * cb + tid + k * NT, last)];
+  }
+#pragma unroll
+  for (int k = 0; k < NF; ++k) pages[tid + k * NT] = 4 * cb + tid + k * NT <= last ? v[k] : 0;
+}
+
+// The thread index as a value the compiler must take as new at every use site: what a converter derives from it (tile
+// addresses, lane offsets) is recomputed per block with a few integer operations instead of being kept in registers
+// across the whole key loop, where the accumulators leave no room for it.
+DEVI int tid_now() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 // The raw page words of a 64-key block are fetched into registers one block ahead (load_raw) and turned into the
 // fp16 tiles after the previous block's matrix work (convert_k, v_tables, convert_v).
 template <int NT> struct Raw {
@@ -153,12 +180,17 @@ template <int NT> struct Raw {
 };
 
 // `h` is the index of the chunk inside a page: the KV head at head dim 128, 2 head + half at head dim 256
-template <int QM, bool K2, int NT>
+// FRESH: the lane offsets are recomputed per block from the thread index (a few integer operations) instead of being
+// kept as 64-bit addresses across the key loop -- for the kernels whose registers are short (there the kept addresses
+// were spilled, and a spilled register's reload waits for every fetch in flight); where there is room, keeping them is
+// the faster form.
+template <int QM, bool K2, int NT, bool FRESH = false>
 DEVI void load_raw_k(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, int kend) {   // pg[0] = first page of block kb
   using F = Fmt<QM>;
+  const int tnow = FRESH ? tid_now() : static_cast<int>(threadIdx.x);
 #pragma unroll
   for (int it = 0; it < Raw<NT>::NI; ++it) {
-    const int idx = threadIdx.x + it * NT;
+    const int idx = tnow + it * NT;
     {
       const int tk = idx >> 2, tg = idx & 3, j = kb * BN + tk;
       if (j < kend) {
@@ -176,12 +208,13 @@ DEVI void load_raw_k(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, 
     }
   }
 }
-template <int QM, int NT>
+template <int QM, int NT, bool FRESH = false>
 DEVI void load_raw_v(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, int kend) {
   using F = Fmt<QM>;
+  const int tnow = FRESH ? tid_now() : static_cast<int>(threadIdx.x);
 #pragma unroll
   for (int it = 0; it < Raw<NT>::NI; ++it) {
-    const int idx = threadIdx.x + it * NT;
+    const int idx = tnow + it * NT;
     {
       const int pgi = idx >> 6, e = (idx & 63) >> 1, c8 = idx & 1, j0 = kb * BN + PAGE * pgi;
       if (j0 < kend) {
@@ -195,18 +228,18 @@ DEVI void load_raw_v(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, 
       }
     }
   }
-  if (threadIdx.x < 32) {
-    const int g = threadIdx.x >> 3, run = threadIdx.x & 7, j0 = kb * BN + 8 * run;
+  if (tnow < 32) {
+    const int g = tnow >> 3, run = tnow & 7, j0 = kb * BN + 8 * run;
     if (j0 < kend) {
       const uint8_t* ch = p.pool + static_cast<long long>(pg[run >> 1]) * p.page_stride + static_cast<long long>(h) * F::CHUNK;
       R.vs = gload<u32x4>(ch + F::VS_OFF + (g * PAGE + 8 * (run & 1)) * 2);   // t0 t2 | t4 t6 | t1 t3 | t5 t7
     }
   }
 }
-template <int QM, bool K2, int NT>
+template <int QM, bool K2, int NT, bool FRESH = false>
 DEVI void load_raw(Raw<NT>& R, const Params& p, const int* pg, int h, int kb, int kend) {
-  load_raw_k<QM, K2, NT>(R, p, pg, h, kb, kend);
-  load_raw_v<QM, NT>(R, p, pg, h, kb, kend);
+  load_raw_k<QM, K2, NT, FRESH>(R, p, pg, h, kb, kend);
+  load_raw_v<QM, NT, FRESH>(R, p, pg, h, kb, kend);
 }
 
 // Key-only pages, one 128-d (half) chunk: the keys of (token, quarter tg) per group g as four fp16 pairs, either final

@@ -80,12 +80,7 @@ __global__ void __launch_bounds__(256, 2) k_mq256(const Params p) {
   const int lim = rvalid ? work.last_key(r / G) : -1;
 
   int cb = kb0;
-  auto fill_pages = [&]() {
-    for (int i = tid; i < PG_CACHE; i += NT) {
-      const int pgx = 4 * cb + i;
-      S.pages[i] = pgx * PAGE < kend ? bt[pgx] : 0;
-    }
-  };
+  auto fill_pages = [&]() { fill_page_window<NT>(S.pages, bt, cb, kb1, kend, tid); };
   fill_pages();
 
   // q fragments of both halves: the tile through LDS (natural order), gathered in code-word order
@@ -124,9 +119,9 @@ __global__ void __launch_bounds__(256, 2) k_mq256(const Params p) {
   struct RawW { Raw<NT> half[2], val; };                // (K fields of half[], V fields of val are the ones used)
   RawW raw;
   auto fetch = [&](RawW& R, const int* pg, int kb) {
-    load_raw_k<QM, K2, NT>(R.half[0], p, pg, 2 * h, kb, kend);
-    load_raw_k<QM, K2, NT>(R.half[1], p, pg, 2 * h + 1, kb, kend);
-    load_raw_v<QM, NT>(R.val, p, pg, 2 * h + vz, kb, kend);
+    load_raw_k<QM, K2, NT, true>(R.half[0], p, pg, 2 * h, kb, kend);
+    load_raw_k<QM, K2, NT, true>(R.half[1], p, pg, 2 * h + 1, kb, kend);
+    load_raw_v<QM, NT, true>(R.val, p, pg, 2 * h + vz, kb, kend);
   };
   if (kb0 < kb1) fetch(raw, S.pages, kb0);
   auto block_step = [&](RawW& R, int kb) {
