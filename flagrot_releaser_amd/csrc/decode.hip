@@ -205,14 +205,22 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
       const float sc0 = (lane & 1) ? -static_cast<float>(UnpackD<QM>::SH) : 0.f;
       const float qs20 = p.qscale * (16777216.f / QPRE);         // raw score sums carry 2^-24 from the codes and QPRE from the query
       // chunk addresses of a quad's four blocks (wave uniform).  Pages past the range name the range's last page again
-      // (their tokens are masked).  The entry comes from LDS; past the cached window it is read from memory.
+      // (their tokens are masked).  The quad's entries come from LDS in ONE read (lane k < PPQ takes the k-th, the other
+      // lanes repeat them); past the cached window they are read from memory.
       auto chunks_of = [&](int quad, const uint8_t* (&ch)[QB]) {
+        const int i = min(PPQ * quad + (lane & (PPQ - 1)), npg - 1);
+        int entry = S.btc[min(i, BT_CACHE - 1)];
+        // (the value is made opaque here so that this stays an LDS read of its own: merged with the memory path below
+        // into one load through a selected pointer it becomes a flat access, and a flat access is awaited together
+        // with every fetch in flight -- the value loads of this quad, and whatever of the next keys was requested)
+        asm volatile("" : "+v"(entry));
+        if (__builtin_expect(PPQ * quad + PPQ > BT_CACHE, 0)) {
+          if (i >= BT_CACHE) entry = bt[pg0 + i];
+          asm volatile("" : "+v"(entry));      // awaited inside the branch: after the join nothing of it is pending
+        }
 #pragma unroll
         for (int k = 0; k < PPQ; ++k) {
-          const int i = min(PPQ * quad + k, npg - 1);
-          int page = S.btc[min(i, BT_CACHE - 1)];
-          if (__builtin_expect(i >= BT_CACHE, 0)) page = bt[pg0 + i];
-          page = __builtin_amdgcn_readfirstlane(page);
+          const int page = __builtin_amdgcn_readlane(entry, k);
           const uint8_t* c = (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
           if constexpr (P == 16) ch[k] = c;
           else { ch[2 * k] = c; ch[2 * k + 1] = c; }
