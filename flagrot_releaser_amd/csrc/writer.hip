@@ -797,6 +797,7 @@ DEVI float sum32(float v) {
 
 typedef float w3_f32x16 __attribute__((ext_vector_type(16)));
 
+typedef __attribute__((address_space(1))) float gfloat;      // a float in global memory: loads through it are global_load, not flat_load
 template <int QM, int P>
 __global__ void __launch_bounds__(256) k_k2_screen(const K2WriteParams p, int tile, float kappa) {
   __shared__ W3Smem S;
@@ -890,8 +891,9 @@ __global__ void __launch_bounds__(256) k_k2_screen(const K2WriteParams p, int ti
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
       const float* dcol = &S.dm[l32][32 * wv];
-      const float* alq = alp;
-      asm volatile("" : "+v"(alq));             // keeps these loads inside the step (not hoisted into 80 registers)
+      const float* alq_ = alp;
+      asm volatile("" : "+v"(alq_));            // keeps these loads inside the step (not hoisted into 80 registers)
+      const gfloat* alq = reinterpret_cast<const gfloat*>(reinterpret_cast<uintptr_t>(alq_));   // (a global, not a flat, access)
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) {
         const float4 d4 = *reinterpret_cast<const float4*>(dcol + 16 * kq + 4 * s4);
@@ -944,8 +946,9 @@ __global__ void __launch_bounds__(256) k_k2_screen(const K2WriteParams p, int ti
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
       const float* dcol = &S.dm[l32][0];
-      const float* ahq = ahp;
-      asm volatile("" : "+v"(ahq));
+      const float* ahq_ = ahp;
+      asm volatile("" : "+v"(ahq_));
+      const gfloat* ahq = reinterpret_cast<const gfloat*>(reinterpret_cast<uintptr_t>(ahq_));
 #pragma unroll 4
       for (int s4 = 0; s4 < 16; ++s4) {
         const float4 d4 = *reinterpret_cast<const float4*>(dcol + 64 * kq + 4 * s4);
