@@ -43,12 +43,30 @@ def sources(name: str) -> list:
 
 
 def _compile(args):
+    """one translation unit -> object file; the compiler's per-kernel register report goes to <object>.usage.txt"""
     src, flags, obj = args
-    cmd = [HIPCC, *COMMON, *flags, "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *COMMON, *flags, "-Rpass-analysis=kernel-resource-usage", "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stdout}\n{r.stderr}")
+    Path(str(obj) + ".usage.txt").write_text(r.stderr)
     return obj
+
+
+def spills(name: str) -> dict:
+    """kernel (mangled name) -> spilled vector registers, from the register reports of the library's last build"""
+    out = {}
+    for s, _ in LIBS[name][1]:
+        rep = LIBDIR / "obj" / (Path(s).stem + ".o.usage.txt")
+        if not rep.exists():
+            continue
+        kernel = None
+        for line in rep.read_text().splitlines():
+            if "Function Name:" in line:
+                kernel = line.split("Function Name:")[1].split()[0]
+            elif "VGPRs Spill:" in line and kernel:
+                out[kernel] = int(line.split("VGPRs Spill:")[1].split()[0])
+    return out
 
 
 def build(name: str, verbose: bool = True) -> Path:

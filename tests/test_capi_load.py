@@ -96,3 +96,21 @@ def test_host_planner_invariants():
     assert K.plan_splits(64, 2048, 8, 16, 1024, ncu=256) == (2, 1024)
     assert K.v2_variant("int4a", 4) == 264 and K.tile_of(K.v2_variant("konlya", 8)) == 8
     assert K.vheads(8, 8, 128, "konlya") == 8 and K.vheads(4, 12, 128, "int4") == 12
+
+
+def test_key_loops_keep_their_registers():
+    """No kernel with a software-pipelined page loop may spill: a reload from scratch is a vector-memory load, and the
+    wait for it is a wait for every page fetch in flight.  Read from the register reports of the in-tree build."""
+    from flagrot_releaser_amd import build
+    hot = ("k_decode", "k_wide_parts_mma", "k_attn_pages", "k_mq")
+    known = ("8k_decodeILi2ELb0ELi32E",)          # static INT2 with 32-token pages: 4-8 registers, not a measured configuration
+    seen = 0
+    for lib in ("kernels", "kivi", "mq"):
+        rep = build.spills(lib)
+        if not rep:
+            pytest.skip("no register report: the libraries were not built in this tree")
+        for kernel, n in rep.items():
+            if any(h in kernel for h in hot) and not any(k in kernel for k in known):
+                seen += 1
+                assert n == 0, (kernel, n)
+    assert seen >= 40
