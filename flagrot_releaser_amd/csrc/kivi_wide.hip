@@ -141,7 +141,10 @@ __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__
         const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
         const int k0 = 128 * s + 32 * j;
         float a0 = 0.f, a1 = 0.f, a2 = 0.f;
+        // (the sums keep their order; unrolled whole, the 256-term loops spilled some 400 registers)
+#pragma unroll 8
         for (int k = k0; k < k0 + 32; ++k) { const float m = row[k]; a0 += m * E[0][k]; a1 += m * E[1][k]; }
+#pragma unroll 8
         for (int k = 0; k < D2; ++k) a2 += row[k] * E[2][k];
         eI[s] += dv[0][s][i] * a0; eH[s] += dv[1][s][i] * a1; eF += dv[2][s][i] * a2;
       }
@@ -167,6 +170,7 @@ __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__
       for (int i = 0; i < 4; ++i) {
         const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
         float a = 0.f;
+#pragma unroll 8
         for (int k = 0; k < D2; ++k) a += row[k] * E[0][k];
         eB += ((s ? useH1 : useH0) ? dv[1][s][i] : dv[0][s][i]) * a;
       }
