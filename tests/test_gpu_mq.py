@@ -113,6 +113,9 @@ CASES = [  # (requests [(L, nq)], shift, sink, G, fmt, kernel, ext)
     # items longer than the page-id window of the kernels (256 blocks): the window slides
     ([(30000, 40)], 0, 0, 4, "int4a", 4, None, 400),
     ([(30000, 40)], 0, 0, 4, "konlya", 3, None, 400),
+    # ... and in the 64-row kernel, which fetches one block ahead (the others two)
+    ([(30000, 12)], 0, 0, 4, "konlya", 1, None, 400),
+    ([(20000, 16)], 0, 0, 4, "int2a", 1, None, 300),
 ]
 
 
