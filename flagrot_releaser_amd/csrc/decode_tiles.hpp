@@ -143,9 +143,10 @@ template <class T> DEVI T gload(const uint8_t* p) {
 // page words: read once per launch (twice where two q tiles share a KV head), never written by it -- the non-temporal
 // hint keeps them from displacing each other in the caches; a kernel that only reads the pages of a launch is 11 %
 // faster with it (46.9 vs 52.6 us for 302 MB)
-template <class T> DEVI T gload_stream(const uint8_t* p) {
+template <class T, bool STREAM = true> DEVI T gload_stream(const uint8_t* p) {
   typedef const __attribute__((address_space(1))) T* gp;
-  return __builtin_nontemporal_load((gp)(p));
+  if constexpr (STREAM) return __builtin_nontemporal_load((gp)(p));
+  else return *(gp)(p);
 }
 
 // One wave iteration covers a quad = 64 consecutive tokens (four 16-token pages or two 32-token pages), as four
@@ -181,25 +182,26 @@ DEVI KOffs<QM, P> key_offsets(int lane) {
   return o;
 }
 // chunk[b]: the chunk of block b's page (wave uniform); 32-token pages: blocks 2 s, 2 s + 1 are the halves of page s
-template <int QM, int P>
+// STREAM = false: ordinary loads, for the kernels whose q tiles of one KV head count on finding each other's lines in L2
+template <int QM, int P, bool STREAM = true>
 DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], const KOffs<QM, P>& o) {
 #pragma unroll
   for (int b = 0; b < QBLK<QM>; ++b) {
     const int hp = P == 32 ? (b & 1) : 0;            // second half of a 32-token page: 16 tokens further
     const uint8_t* ch = chunk[b];
     if constexpr (QM == QM_ASYM2) {
-      const u32x2 k = gload_stream<u32x2>(ch + o.k + hp * 16 * 32);
+      const u32x2 k = gload_stream<u32x2, STREAM>(ch + o.k + hp * 16 * 32);
       r.kc[b][0] = k.x; r.kc[b][1] = k.y;
     } else {
-      const u32x4 k = gload_stream<u32x4>(ch + o.k + hp * 16 * 64);
+      const u32x4 k = gload_stream<u32x4, STREAM>(ch + o.k + hp * 16 * 64);
       r.kc[b][0] = k.x; r.kc[b][1] = k.y; r.kc[b][2] = k.z; r.kc[b][3] = k.w;
     }
-    { const u32x2 t2 = gload_stream<u32x2>(ch + o.ks + hp * 16 * 8); r.ks[b] = make_uint2(t2.x, t2.y); }
-    r.vs[b] = gload_stream<uint16_t>(ch + o.vs + hp * 16 * 2);
+    { const u32x2 t2 = gload_stream<u32x2, STREAM>(ch + o.ks + hp * 16 * 8); r.ks[b] = make_uint2(t2.x, t2.y); }
+    r.vs[b] = gload_stream<uint16_t, STREAM>(ch + o.vs + hp * 16 * 2);
   }
 }
 
-template <int QM, int P>
+template <int QM, int P, bool STREAM = true>
 DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], int lane) {
   using L = Lay<QM, P>;
   // lane = (entry m = lane & 15 (+ 16 for the second half), run kc = lane >> 4 of the 32 tokens of half s of the quad:
@@ -213,10 +215,10 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], int lane
 #pragma unroll
     for (int eh = 0; eh < 2; ++eh) {
       if constexpr (QM == QM_ASYM2) {
-        const u32x2 v = gload_stream<u32x2>(ch + L::V_OFF + 8 * (R * (16 * eh + m) + c8));
+        const u32x2 v = gload_stream<u32x2, STREAM>(ch + L::V_OFF + 8 * (R * (16 * eh + m) + c8));
         r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y;
       } else {
-        const u32x4 v = gload_stream<u32x4>(ch + L::V_OFF + 16 * (R * (16 * eh + m) + c8));
+        const u32x4 v = gload_stream<u32x4, STREAM>(ch + L::V_OFF + 16 * (R * (16 * eh + m) + c8));
         r.vc[2 * s2 + eh][0] = v.x; r.vc[2 * s2 + eh][1] = v.y; r.vc[2 * s2 + eh][2] = v.z; r.vc[2 * s2 + eh][3] = v.w;
       }
     }

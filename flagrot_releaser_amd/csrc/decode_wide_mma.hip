@@ -277,15 +277,15 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
     chunks_of(qi, ch0);
 #pragma unroll
     for (int k = 0; k < QB; ++k) ch1[k] = ch0[k] + L::CHUNK;
-    load_k<QM, P>(k0, ch0, koff);
-    load_k<QM, P>(k1, ch1, koff);
+    load_k<QM, P, false>(k0, ch0, koff);
+    load_k<QM, P, false>(k1, ch1, koff);
   }
   while (qi < nquad) {
     int take = 0;
     if (lane == 0) take = atomicAdd(&S.next, 1);
     VRegs<QM> v0, v1;                                  // this quad's V^T entries: in flight during the key phase
-    load_v<QM, P>(v0, ch0, lane);
-    load_v<QM, P>(v1, ch1, lane);
+    load_v<QM, P, false>(v0, ch0, lane);
+    load_v<QM, P, false>(v1, ch1, lane);
     bool valid[QB];
     {
       const int tok0 = (pg0 + PPQ * qi) * P + (lane & 15);
@@ -340,8 +340,8 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
     chunks_of(qn, ch0);
 #pragma unroll
     for (int k = 0; k < QB; ++k) ch1[k] = ch0[k] + L::CHUNK;
-    load_k<QM, P>(k0, ch0, koff);
-    load_k<QM, P>(k1, ch1, koff);
+    load_k<QM, P, false>(k0, ch0, koff);
+    load_k<QM, P, false>(k1, ch1, koff);
     // ---- values, half by half through the same strips
     write_strips<QM>(H0, vs0, pe, valid, lane, wave);
     wave_lds_sync();
