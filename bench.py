@@ -330,7 +330,8 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
                                "frac_of_peak": round(page_bytes / (rus * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4),
                                "decode_over_read": round(first["us_per_layer_step"] / rus, 3),
                                "note": "a kernel that only reads the launch's page chunks through the same block table "
-                                       "(16-wavefront workgroup per (sequence, KV head), 4 pages in flight per wavefront)"}
+                                       "(16-wavefront workgroup per (sequence, KV head), 4 pages in flight per wavefront, non-temporal loads "
+                                       "as in the decode kernels)"}
     # decode-step writer (T = B new tokens) and the prefill-time writer rate, for the record
     kv_new = synth_kv(B, g, dev, torch, mu=kmu, hkv=HKV, dh=DH)
     slots_new = (bt[:, -1].long() * P + (P - 1)).contiguous()
