@@ -16,6 +16,7 @@ Workloads (BASELINE.json configs):
         batch 32, context 8192, page 16, randomly permuted page table.                       [default, headline]
   int2  configs[2]: INT2 FlagRot (kind konlya2) with static key centring, 4 sink + 128 window BF16 tokens,
         batch 64, context 16384.
+  int2_b32  INT2 FlagRot (kind konlya2) at the headline shape: batch 32, context 8192, no BF16 rows.
   kivi  configs[3]: KIVI-style FlagRot INT2 (keys per channel over 32-token groups, values per token), 128-token
         BF16 residual, Qwen-32B shape 64q/8kv, d=128, batch 16, context 32768 (libflagrot_kivi.so).
   mq    configs[4]: prefix-cached multi-query prefill over INT4 pages (libflagrot_mq.so, the MFMA path): 4 requests x
@@ -165,49 +166,124 @@ def build_cache(torch, K, dev, kind, B, L, seed, kmu=None, chunk_tokens=8192, hk
     return pool, bt, CT, co, time.perf_counter() - t0
 
 
-def host_threads():
+def cpu_model():
     try:
-        from threadpoolctl import threadpool_limits
-        return threadpool_limits(limits=1)
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
+
+
+def blas_threads(limit=None):
+    """context that pins numpy's thread pools to `limit` threads (None: as the host gives them), and the count in use"""
+    import contextlib
+    try:
+        from threadpoolctl import threadpool_info, threadpool_limits
     except Exception:      # no threadpoolctl: numpy runs with whatever its BLAS was built with
-        import contextlib
-        return contextlib.nullcontext()
+        return contextlib.nullcontext(), None
+    if limit is None:
+        n = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+        return contextlib.nullcontext(), n
+    return threadpool_limits(limits=limit), limit
 
 
-def cpu_baseline(torch, K, dev):
-    """the oracle's two legs on configs[0]'s shape (batch 1, context 2048, 32q/8kv, INT4 groups of 32, uniform
-    calibration weights), one host thread: (i) the selecting writer for the 2048 tokens x 8 KV heads (K and V),
-    (ii) one decode step = page parse + dequantise + inverse transforms + fp64 softmax attention."""
+def median_time(fn, runs=5):
+    fn()                                   # one warm-up
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2]
+
+
+def configs0(torch, K, dev, runs=5, timed_legs=True):
+    """configs[0] (batch 1, context 2048, 32q/8kv, head dim 128, page 16, INT4 key-only pages of kind konly with groups
+    of 32, uniform calibration weights C_q = I and c_o = 1, identity page order) through BOTH paths on the same seeded
+    inputs: the oracle's writer + page packer + dequantise-then-attend on the host, and the HIP writer + decode through
+    the C ABI.  Returns the comparison (pool bytes equal, attention inside the bar) and, when asked, the host timings:
+    median of `runs` after one warm-up, with one thread and with the host's own thread count."""
     import numpy as np
     from oracle import attend as A
+    from oracle import pages as PG
     from oracle import quant as Q
     kind, L = "konly", 2048
     g = torch.Generator(device=dev).manual_seed(0)
-    kv = synth_kv(L, g, dev, torch).cpu()
-    kvb = kv.view(torch.int16).numpy().view(np.uint16)
+    kv = synth_kv(L, g, dev, torch)
+    gq = torch.Generator().manual_seed(0)
+    q = torch.randn(1, G * HKV, DH, generator=gq).bfloat16()
+    kvb = kv.cpu().view(torch.int16).numpy().view(np.uint16)
+    qb = q.view(torch.int16).numpy().view(np.uint16)
     C = np.stack([np.eye(DH, dtype=np.float32)] * HKV)
-    with host_threads():
-        t0 = time.perf_counter()
-        Q.k2_encode(kvb, C, kind)
-        t_write = time.perf_counter() - t0
-        pool, bt, CT, co, _ = build_cache(torch, K, dev, kind, 1, L, seed=0)
-        gq = torch.Generator().manual_seed(0)
-        q = torch.randn(1, G * HKV, DH, generator=gq).bfloat16()
-        qb = q.view(torch.int16).numpy().view(np.uint16)
-        hp, hbt = pool.cpu().numpy(), bt.cpu().numpy()
-        ts = []
-        for _ in range(4):
-            t0 = time.perf_counter()
-            A.decode_reference(qb, hp, kind, P, hbt, [L], 1 / math.sqrt(DH))
-            ts.append(time.perf_counter() - t0)
-    t = sorted(ts[1:])[len(ts[1:]) // 2]
+    npages = L // P
+    slots = np.arange(L, dtype=np.int64)
+    hbt = np.arange(npages, dtype=np.int32)[None]
+    cb = PG.chunk_bytes(kind, P)
+
+    def write_host():
+        pool = np.zeros((npages, HKV, cb), dtype=np.uint8)
+        codes, words, _ = Q.k2_encode(kvb, C, kind)
+        PG.pack_tokens(pool, slots, codes, words, kind, P)
+        return pool
+
+    want = write_host()
+    ref = A.decode_reference(qb, want, kind, P, hbt, [L], 1 / math.sqrt(DH))
+    # the same inputs through the HIP libraries
+    dpool = torch.zeros(npages, HKV, cb, dtype=torch.uint8, device=dev)
+    CT = torch.eye(DH, device=dev).repeat(HKV, 1, 1).contiguous()
+    co = torch.ones(HKV, DH, device=dev)
+    K.cb_write(kv, torch.from_numpy(slots).to(dev), CT, co, kind, dpool, P)
+    torch.cuda.synchronize()
+    same = bool(np.array_equal(dpool.cpu().numpy(), want))
+    out = torch.zeros(1, G * HKV * DH, dtype=torch.bfloat16, device=dev)
+    ns, ch = K.plan_cb(1, L, HKV, P, kind)
+    ws = K.Workspace(1, HKV, HKV * (ns + 1), dev)
+    K.cb_attn(q.to(dev), dpool, torch.from_numpy(hbt).to(dev), torch.tensor([L], dtype=torch.int32, device=dev), out, ns, ch,
+              ws, LOG2E / math.sqrt(DH), kind)
+    torch.cuda.synchronize()
+    got = out.view(1, G * HKV, DH).float().cpu().numpy().astype(np.float64)
+    st = error_stats(got, ref)
+    res = {"pool_bytes_equal": same, "errors": st, "nsplit": ns, "chunk": ch,
+           "checked": bool(same and st["elementwise"] <= 1.0),
+           "check": f"configs[0] through the HIP path: writer pool {'byte-equal to' if same else 'DIFFERS from'} the "
+                    f"oracle's packed pool ({want.size} bytes); decode vs the oracle's dequantise-then-attend: " + describe(st)}
+    if not timed_legs:
+        return res
+    legs = {}
+    for label, limit in (("one_thread", 1), ("host_threads", None)):
+        ctx, n = blas_threads(limit)
+        with ctx:
+            tw = median_time(write_host, runs)
+            td = median_time(lambda: A.decode_reference(qb, want, kind, P, hbt, [L], 1 / math.sqrt(DH)), runs)
+        legs[label] = {"threads": n, "writer_s": tw, "decode_s": td}
+    res["legs"] = legs
+    return res
+
+
+def cpu_baseline(torch, K, dev):
+    """the oracle's two legs on configs[0], timed on this host: (i) the selecting writer for the 2048 tokens x 8 KV heads
+    (K with selection, V plain) + page packing, (ii) one decode step = page parse + dequantise + inverse transforms +
+    fp64 softmax attention for the 32 q heads.  The same inputs go through the HIP path and the two are compared."""
+    L = 2048
+    r = configs0(torch, K, dev)
+    one, full = r["legs"]["one_thread"], r["legs"]["host_threads"]
     nbytes = L * HKV * 144
+    t = one["decode_s"]
     return {"value": round(nbytes / t / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"numpy oracle on configs[0] (B=1 L={L} 32q/8kv INT4 konly, page 16), one thread of the host's "
-                      f"{os.cpu_count()} cpus: decode step (decode_reference, {nbytes} page bytes) median of 3 after 1 "
-                      f"warm-up = {t * 1e6:.0f} us per layer-step; writer (k2_encode, {L} tokens x {HKV} KV heads, K and V) "
-                      f"one run = {t_write:.2f} s = {t_write / L * 1e6:.0f} us per token",
-            "decode_us_per_layer_step": round(t * 1e6, 0), "writer_us_per_token": round(t_write / L * 1e6, 1)}
+            "sample": f"numpy oracle on configs[0] (B=1 L={L} 32q/8kv INT4 konly, C_q = I, c_o = 1, page 16), median of 5 runs "
+                      f"after one warm-up, one thread: decode step (decode_reference, {nbytes} page bytes) = {t * 1e6:.0f} us "
+                      f"per layer-step; writer (k2_encode + pack_tokens, {L} tokens x {HKV} KV heads, K and V) = "
+                      f"{one['writer_s']:.2f} s = {one['writer_s'] / L * 1e6:.0f} us per token",
+            "decode_us_per_layer_step": round(t * 1e6, 0), "writer_us_per_token": round(one["writer_s"] / L * 1e6, 1),
+            "host_threads": {"threads": full["threads"], "decode_us_per_layer_step": round(full["decode_s"] * 1e6, 0),
+                             "GBps": round(nbytes / full["decode_s"] / 1e9, 6),
+                             "writer_us_per_token": round(full["writer_s"] / L * 1e6, 1)},
+            "cpu": cpu_model(), "os_cpu_count": os.cpu_count(), "torch_num_threads": torch.get_num_threads(),
+            "checked": r["checked"], "pool_bytes_equal": r["pool_bytes_equal"], "errors": r["errors"], "check": r["check"]}
 
 
 def reference_plan(B, Lmax, Hkv, slots):
@@ -239,6 +315,10 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
     if workload == "int4":
         kind, B, L, S, W, cell = "konlya", 32, 8192, 0, 0, 144
         name = "configs[1]: INT4 FlagRot konlya paged decode, Llama-3.1-8B GQA 32q/8kv d=128, B=32 L=8192 page=16"
+    elif workload == "int2_b32":
+        kind, B, L, S, W, cell = "konlya2", 32, 8192, 0, 0, 80
+        name = ("INT2 FlagRot konlya2 paged decode at the headline shape (the metric names INT4 and INT2): Llama-3.1-8B "
+                "GQA 32q/8kv d=128, B=32 L=8192 page=16, no BF16 rows")
     else:
         kind, B, L, S, W, cell = "konlya2", 64, 16384, 4, 128, 80
         name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
@@ -555,7 +635,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=None, choices=["int4", "int2", "kivi", "mq"])
+    ap.add_argument("--workload", default=None, choices=["int4", "int2", "int2_b32", "kivi", "mq"])
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
     ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="256 = the head dim 256 kernels (GQA 24q/4kv, the reference's test shape class); not a baseline configuration")
@@ -627,6 +707,8 @@ def main():
         wl = {}
         torch.cuda.empty_cache()
         wl["int2"] = run_flagrot(args, torch, dev, "int2", short, 5)["own"]
+        torch.cuda.empty_cache()
+        wl["int2_b32_l8192"] = run_flagrot(args, torch, dev, "int2_b32", short, 5)["own"]
         torch.cuda.empty_cache()
         wl["kivi"] = run_kivi(args, torch, dev, short, 5)
         torch.cuda.empty_cache()

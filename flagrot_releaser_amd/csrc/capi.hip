@@ -104,6 +104,11 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   const long long wgs = static_cast<long long>(B) * Hkv * ntile * nsplit;
   const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && wgs <= device_cus());
   const bool can_draw = !force_static && counter != nullptr && p.counter_div == 1 && nparts <= 1023;
+  // the split merge goes through the caller's workspace: partials, their (max, sum) pairs and, at head dim 128, the ticket
+  if (nparts > 1 && (opart == nullptr || mlpart == nullptr || (!(variant & HD256) && counter == nullptr)))
+    return fail(-3, "fr_v2_attn: more than one partial per (sequence, KV head) needs opart, mlpart and counter");
+  if ((variant & HD256) && (opart == nullptr || mlpart == nullptr))
+    return fail(-3, "fr_v2_attn: the head dim 256 kernels need opart and mlpart");
   p.wg_waves = big ? decode_waves(1 << 30) : 4;
   p.dyn = (can_draw && (!big || env_waves > 4)) ? 1 : 0;
   if (variant & HD256) return launched(decode_wide_launch(fmt, p, static_cast<hipStream_t>(stream)), "fr_v2_attn (head dim 256)");
@@ -280,8 +285,8 @@ int fr_cb_occupancy(int kind, int variant, int stages, int page) {
 int fr_cb_chunk_bytes(int kind, int page) { return page * (kind == KIND_KONLYA2 ? 80 : 144); }
 int fr_cb_write_smem(int kind, int tg, int hd) {
   (void)tg;
-  if (fmt_of_kind(kind) < 0 || (hd != 0 && hd != 128)) return 0;
-  return k2_write_lds_bytes();
+  if (fmt_of_kind(kind) < 0 || (hd != 0 && hd != 128 && hd != 256)) return 0;
+  return k2_write_lds_bytes(hd);
 }
 
 const char* fr_last_error(void) { return g_err; }

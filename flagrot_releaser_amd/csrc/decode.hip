@@ -502,17 +502,6 @@ int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
   return -4;
 }
 
-template <int QM, bool K2>
-int occupancy_qm(int waves) {
-  int n = 0;
-  const void* f = waves > 4 ? reinterpret_cast<const void*>(&k_decode<QM, K2, 16, BIGW<QM>>) : reinterpret_cast<const void*>(&k_decode<QM, K2, 16, 4>);
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, 64 * (waves > 4 ? BIGW<QM> : 4), 0) != hipSuccess || n < 1) {
-    (void)hipGetLastError();
-    return waves > 4 ? 1 : 2;
-  }
-  return n;
-}
-
 }  // namespace
 
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) { return decode_dispatch(fmt, p, st); }
@@ -520,25 +509,6 @@ int decode_waves(int chunk_tokens) { return waves_for(chunk_tokens); }
 int decode_big_chunk() {      // FLAGROT_BIG_CHUNK overrides (experiments)
   static const int v = getenv("FLAGROT_BIG_CHUNK") != nullptr ? atoi(getenv("FLAGROT_BIG_CHUNK")) : BIG_CHUNK;
   return v;
-}
-
-// resident workgroups per CU the host split planner may count on (queried once per format and workgroup size)
-int decode_occupancy(int fmt, int waves) {
-  static int cache[16][2] = {{0}};
-  if (fmt < 0 || fmt >= 16) return 0;
-  const int wi = waves > 4 ? 1 : 0;
-  if (cache[fmt][wi] == 0) {
-    switch (fmt) {
-      case FMT_INT4: cache[fmt][wi] = occupancy_qm<QM_SYM4, false>(waves); break;
-      case FMT_INT4A: cache[fmt][wi] = occupancy_qm<QM_ASYM4, false>(waves); break;
-      case FMT_INT2A: cache[fmt][wi] = occupancy_qm<QM_ASYM2, false>(waves); break;
-      case FMT_KONLY: cache[fmt][wi] = occupancy_qm<QM_SYM4, true>(waves); break;
-      case FMT_KONLYA: cache[fmt][wi] = occupancy_qm<QM_ASYM4, true>(waves); break;
-      case FMT_KONLYA2: cache[fmt][wi] = occupancy_qm<QM_ASYM2, true>(waves); break;
-      default: return 0;
-    }
-  }
-  return cache[fmt][wi];
 }
 
 }  // namespace fr

@@ -31,7 +31,7 @@ struct K2WriteParams {
   int hd;                  // head dim: 0 | 128, or 256 (fr_cb_write only)
 };
 int k2_write_launch(int kind, const K2WriteParams& p, hipStream_t st);
-int k2_write_lds_bytes();
+int k2_write_lds_bytes(int hd);
 
 int head_fwht_launch(const void* x, long long x_ts, void* out, long long o_ts, int T, int H, const uint8_t* flags,
                      float scale, hipStream_t st, int D);
@@ -65,7 +65,6 @@ struct DecodeParams {
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
 int decode_wide_launch(int fmt, const DecodeParams& p, hipStream_t st);   // head dim 256 (decode_wide.hip)
-int decode_occupancy(int fmt, int waves);   // resident workgroups per CU of the 4- or 16-wavefront kernel
 int decode_big_chunk();                     // tokens per split from which the large workgroup is worth launching
 int decode_waves(int chunk_tokens);          // wavefronts per workgroup the launcher picks for a split of that many tokens
 

@@ -1149,7 +1149,9 @@ int k2_write_launch(int kind, const K2WriteParams& p, hipStream_t st) {
   }
   return -4;
 }
-int k2_write_lds_bytes() { return K2_LDS; }
+int k2_write_lds_bytes(int hd) {      // LDS a selecting-writer workgroup holds (the 256-d kernel: its error strips; C_q^T stays in L2)
+  return hd == 256 ? static_cast<int>(8 * 2 * 256 * sizeof(float)) : K2_LDS;
+}
 
 int head_fwht_launch(const void* x, long long x_ts, void* out, long long o_ts, int T, int H, const uint8_t* flags,
                      float scale, hipStream_t st, int D) {

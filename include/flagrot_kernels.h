@@ -91,7 +91,8 @@ int fr_cb_attn(const void* q, long long q_bs, const uint8_t* pool, const int* bl
  * held until the process ends); the call allocates nothing and clears its counters itself.  Limit:
  * B*Hkv*ceil(gqa/4)*(nsplit+1) <= FR_NOALLOC_MAX_PARTS, else -2 with a message in fr_last_error().  All calls on one
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are safe.
- * The first call on a device looks the array's address up (no stream work, no allocation). */
+ * The first call on a device looks the array's address up (a host-side query: no stream work, no allocation); make it
+ * outside a stream capture -- every later call on that device may be captured into a HIP graph. */
 #define FR_NOALLOC_MAX_PARTS 8192
 int fr_cb_attn_noalloc(const void* q, long long q_bs, const uint8_t* pool, const int* block_table, int bt_stride,
                        const int* seq_lens, int B, int Hkv, int page, int nsplit, int chunk, float qscale, int kind,

@@ -25,8 +25,9 @@ int kv_chunk_bytes(int D);
 int kv_chunk_bytes8(int D);
 
 /* kivi.cu:1934-1949.  kv bf16 [n, 2*Hkv, D] (row stride kv_rs elements; V rows Hkv..2Hkv-1); slots int64 [n]
- * (< 0 skipped); co fp32 [Hkv, D]; M must be null; vfix int32 [Hkv] or null (bits 0..3 = H32 per sub-vector,
- * bit 16 = H_D); ident: identity only. */
+ * (< 0 skipped); co fp32 [Hkv, D]; M fp32 [Hkv, D, D] or null (null: a candidate's error is sum d^2 co; else d^T M d,
+ * the diagonal 32-blocks of M for the sub-vector choices, kivi.cu:213-287); vfix int32 [Hkv] or null (bits 0..3 = H32
+ * per sub-vector, bit 16 = H_D); ident: identity only. */
 int kv_v_write(const void* kv, long long kv_rs, int n, int Hkv, int D, const void* slots, const void* co, const void* M,
                void* pool, int ident, const void* vfix, int f8, void* stream);
 

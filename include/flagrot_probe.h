@@ -12,7 +12,7 @@ extern "C" {
 
 int fr_probe_abi_version(void);
 const char* fr_probe_last_error(void);
-/* pool [num_pages, Hkv, chunk_bytes] (chunk_bytes a multiple of 16, at most 3072); block_table int32 [B, bt_stride];
+/* pool [num_pages, Hkv, chunk_bytes] (chunk_bytes a multiple of 16, at most 5120: a 32-token INT4 page is 4608); block_table int32 [B, bt_stride];
  * seq_lens int32 [B]; page 16 | 32; sink: one writable 32-bit word (practically never written). */
 int fr_probe_read(const uint8_t* pool, const int* block_table, int bt_stride, const int* seq_lens, int B, int Hkv, int page,
                   int chunk_bytes, uint32_t* sink, void* stream);

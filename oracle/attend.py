@@ -44,7 +44,8 @@ def dequant_pages(pool: np.ndarray, fmt: str, page: int, dtype=np.float64, Dh: i
     if qk != "sym":
         zmask = 15 if qk == "asym4" else 3
         c = c - np.repeat(w & zmask, 32, -1).astype(dtype)
-    mag = Q.word_scale(w).astype(dtype)
+    with np.errstate(invalid="ignore"):       # bytes that were never written parse as any pattern, NaN scale words among them
+        mag = Q.word_scale(w).astype(dtype)
     x = (c.reshape(*c.shape[:-1], ng, 32) * mag[..., None])                       # [Np, H, P, 2, ng, 32]
     k, v = x[..., 0, :, :], x[..., 1, :, :]
     if fmt in ("konly", "konlya", "konlya2"):
@@ -111,9 +112,14 @@ def decode_reference(q_bits, pool, fmt, page, block_table, lens, scale, kmask=No
     B, Hq, Dh = q.shape
     Hkv = pool.shape[1]
     G = Hq // Hkv
-    Kp, Vp = dequant_pages(pool, fmt, page, Dh=Dh)
     Lmax = max(int(max(lens)) if len(lens) else 1, 1)
-    Kc, Vc = gather_cache(Kp, Vp, block_table, Lmax, page)
+    # only the pages the block table names are parsed: free pages may hold any bytes (scale words that read as NaN)
+    npg = max(1, -(-Lmax // page))
+    bt = np.asarray(block_table)[:, :npg].astype(np.int64)
+    used, inv = np.unique(bt, return_inverse=True)
+    with np.errstate(invalid="ignore"):       # slots past a sequence's end inside its last page are garbage as well
+        Kp, Vp = dequant_pages(pool[used], fmt, page, Dh=Dh)
+    Kc, Vc = gather_cache(Kp, Vp, inv.reshape(bt.shape), Lmax, page)
     tails = None
     if tail is not None:
         tails = []

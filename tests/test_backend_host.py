@@ -34,42 +34,42 @@ def test_ring_slot_keeps_sinks_and_window(S, W):
 @pytest.mark.parametrize("S,W", [(0, 0), (4, 128), (4, 0), (0, 16)])
 def test_metadata_builder_rows(S, W):
     R, rows = 5, 8
-    b = BK.MetadataBuilder("konlya", 8, 4, 4096, rows, R, S, W, "cpu", plan_fn=lambda B: (3, 1408))
+    b = BK.StepPlanner("konlya", 8, 4, 4096, rows, R, S, W, "cpu", plan_fn=lambda B: (3, 1408))
     lens = torch.tensor([1, 3, 4, 5, 131, 132, 133, 1000], dtype=torch.int32)
     req = np.array([2, 0, 4, 1, 3, 2])                     # two rows more than request slots: padding rows
-    md = b.build(lens, torch.zeros(8, 4, dtype=torch.int32), torch.zeros(8, dtype=torch.int64), req_idx=req)
-    assert (md.nsplit, md.chunk, md.num_decodes) == (3, 1408, 8)
+    md = b.prepare(lens, torch.zeros(8, 4, dtype=torch.int32), torch.zeros(8, dtype=torch.int64), homes=req)
+    assert (md.nsplit, md.chunk, md.rows) == (3, 1408, 8)
     if S == 0 and W == 0:
-        assert md.dec_cached is lens and md.dec_tail_len is None
+        assert md.page_tokens is lens and md.ring_tokens is None
         return
     T = S + W
     for i, L in enumerate(lens.tolist()):
         row = int(req[i]) if i < len(req) else R
-        assert int(md.dec_tail_idx[i]) == row
-        assert int(md.dec_cached[i]) == (L - W if L - W > S else 0)
-        assert int(md.dec_tail_len[i]) == min(L, T)
+        assert int(md.ring_home[i]) == row
+        assert int(md.page_tokens[i]) == (L - W if L - W > S else 0)
+        assert int(md.ring_tokens[i]) == min(L, T)
         s = BK.ring_slot(L - 1, S, W)
-        assert int(md.dec_ring_pos[i]) == (row * T + s if s >= 0 else R * T)
+        assert int(md.ring_dest[i]) == (row * T + s if s >= 0 else R * T)
     # the buffers are persistent: a second, shorter build reuses them
-    md2 = b.build(lens[:3] + 1, md.block_table[:3], md.slot_mapping[:3], req_idx=req[:3])
-    assert md2.dec_tail_idx.data_ptr() == md.dec_tail_idx.data_ptr() and md2.dec_ring_pos.shape[0] == 3
+    md2 = b.prepare(lens[:3] + 1, md.block_table[:3], md.slots[:3], homes=req[:3])
+    assert md2.ring_home.data_ptr() == md.ring_home.data_ptr() and md2.ring_dest.shape[0] == 3
 
 
 def test_kivi_decode_groups():
     """the key group a decode step completes: ring rows of its 32 positions (sinks excluded) and their page slots"""
     S, W, R = 4, 64, 3
     T = S + W
-    b = BK.MetadataBuilder("kivi2", 2, 4, 4096, 6, R, S, W, "cpu", plan_fn=lambda B: (2, 512))
+    b = BK.StepPlanner("kivi2", 2, 4, 4096, 6, R, S, W, "cpu", plan_fn=lambda B: (2, 512))
     lens = torch.tensor([32, 33, 64, 31, 96, 128], dtype=torch.int32)
     bt = torch.arange(6 * 16, dtype=torch.int32).view(6, 16) * 3 % 97
     req = np.array([1, 0, 2, 1])                                           # rows 4, 5: padding (ring row R)
-    md = b.build(lens, bt, torch.zeros(6, dtype=torch.int64), req_idx=req)
+    md = b.prepare(lens, bt, torch.zeros(6, dtype=torch.int64), homes=req)
     for i, L in enumerate(lens.tolist()):
         act = L % 32 == 0 and L >= 32 and i < len(req)
         if not act:
-            assert int(md.kivi_dslot[i, 0]) < 0 and (md.kivi_sidx[i] == -1).all()
+            assert int(md.group_dst[i, 0]) < 0 and (md.group_src[i] == -1).all()
             continue
         for j in range(32):
             p = L - 32 + j
-            assert int(md.kivi_dslot[i, j]) == int(bt[i, p // 16]) * 16 + p % 16
-            assert int(md.kivi_sidx[i, j]) == (-1 if p < S else int(req[i]) * T + BK.ring_slot(p, S, W))
+            assert int(md.group_dst[i, j]) == int(bt[i, p // 16]) * 16 + p % 16
+            assert int(md.group_src[i, j]) == (-1 if p < S else int(req[i]) * T + BK.ring_slot(p, S, W))

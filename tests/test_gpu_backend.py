@@ -39,7 +39,7 @@ def test_decode_steps_in_graph(dev, kind, S, W, center):
         kw.update(CT=Cq.transpose(1, 2).contiguous().to(dev), co=co.to(dev))
     if center:
         kw["kmu"] = (1.5 * torch.randn(Hkv, 128, generator=g)).to(dev)
-    builder = BK.MetadataBuilder(kind, Hkv, G, max_len, rows, R, S, W, dev)
+    builder = BK.StepPlanner(kind, Hkv, G, max_len, rows, R, S, W, dev)
     layer = BK.DecodeLayer(kind, Hkv, G, pool, builder, **kw)
 
     def slot_of(b, p):
@@ -64,7 +64,7 @@ def test_decode_steps_in_graph(dev, kind, S, W, center):
         slots.copy_(torch.tensor([slot_of(b, lens[b] - 1) for b in range(nreal)] + [-1], dtype=torch.int64))
         q.copy_((torch.randn(q.shape, generator=g) * 0.8).bfloat16())
         kvn.copy_(make_kv(nrows, Hkv, g, edge=False))
-        md = builder.build(seq, dbt, slots, req_idx=req)
+        md = builder.prepare(seq, dbt, slots, homes=req)
         if graph is None:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -92,13 +92,13 @@ def test_decode_steps_in_graph(dev, kind, S, W, center):
                 s = BK.ring_slot(lens[b] - 1, S, W)
                 if s >= 0:
                     assert torch.equal(layer.ring[int(req[b]), s], want[b]), (step, b)
-        cached = md.dec_cached[:nreal].cpu().tolist() if T else lens
+        cached = md.page_tokens[:nreal].cpu().tolist() if T else lens
         ref = A.decode_reference(bits(q[:nreal]), pool.cpu().numpy(), kind, P, bt[:nreal].numpy(), cached, 1 / math.sqrt(128),
                                  kmask=kw["wmask"][:Hkv].cpu().numpy() if static else None,
                                  vmask=kw["wmask"][Hkv:].cpu().numpy() if static else None,
                                  tail=None if not T else bits(layer.ring),
-                                 tail_len=None if not T else md.dec_tail_len[:nreal].cpu().numpy(),
-                                 tail_idx=None if not T else md.dec_tail_idx[:nreal].cpu().numpy(), kv_start=S)
+                                 tail_len=None if not T else md.ring_tokens[:nreal].cpu().numpy(),
+                                 tail_idx=None if not T else md.ring_home[:nreal].cpu().numpy(), kv_start=S)
         got = out[:nreal].view(nreal, G * Hkv, 128).float().cpu().numpy().astype(np.float64)
         assert not np.isnan(got).any()
         lim = 2e-3 + 1e-2 * np.abs(ref) + 1e-5 * np.abs(ref).max(axis=(1, 2), keepdims=True)
@@ -132,7 +132,7 @@ def test_kivi_decode_steps_in_graph(dev, f8):
     bt = torch.zeros(nrows, nblk, dtype=torch.int32)
     bt[:nreal] = torch.randperm(num_pages, generator=g)[:nreal * nblk].int().view(nreal, nblk)
     qs, lz, co = _calib(Hkv, 24, g)
-    builder = BK.MetadataBuilder("kivi2", Hkv, G, max_len, rows, R, S, W, dev)
+    builder = BK.StepPlanner("kivi2", Hkv, G, max_len, rows, R, S, W, dev)
     layer = BK.KiviDecodeLayer(Hkv, G, pool, builder, qs.to(dev), lz.to(dev), co.to(dev), f8=f8)
 
     def slot_of(b, p):
@@ -156,8 +156,8 @@ def test_kivi_decode_steps_in_graph(dev, f8):
         slots.copy_(torch.tensor([slot_of(b, lens[b] - 1) for b in range(nreal)] + [-1], dtype=torch.int64))
         q.copy_((torch.randn(q.shape, generator=g) * 1.2).bfloat16())
         kvn.copy_(_kv(nrows, Hkv, g))
-        md = builder.build(seq, dbt, slots, req_idx=req)
-        encoded += int((md.kivi_dslot[:, 0] >= 0).sum())
+        md = builder.prepare(seq, dbt, slots, homes=req)
+        encoded += int((md.group_dst[:, 0] >= 0).sum())
         if graph is None:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -179,7 +179,7 @@ def test_kivi_decode_steps_in_graph(dev, f8):
         got = Q.bf16_to_f32(bits(out)).astype(np.float64).reshape(nrows, G * Hkv, 128)
         for b in range(nreal):
             L = lens[b]
-            cached, tl = int(md.dec_cached[b]), int(md.dec_tail_len[b])
+            cached, tl = int(md.page_tokens[b]), int(md.ring_tokens[b])
             assert cached == (L - W if L - W > S else 0) and tl == min(L, T) and cached <= 32 * (L // 32)
             Kp, Vp = OK.dequant_groups(pnp[bt[b, :2 * (-(-max(cached, 1) // 32))].numpy()], 128, f8=f8)
             tb = ringf[int(req[b]), :tl]

@@ -160,6 +160,18 @@ def test_block_table_beyond_the_lds_cache(dev):
     run_case(dev, "codebook", [16500], "konlya2", seed=24, Hkv=1, nsplit=3)
 
 
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("static", "int4a")])
+def test_long_contexts(dev, mode, fmt):
+    """33 000 and 65 536 tokens (the lengths of the reference's own long cases, kernels/test_attn_v2.py:144,354-382, and
+    of its decode benchmark, scripts/bench_attn_int2.py:30): 2063 and 4096 pages per sequence, so three quarters of the
+    block table is read past the workgroup's LDS window; the planner's split, the fewest splits a chunk of 8192 tokens
+    allows, and BF16 rows with a masked sink range"""
+    run_case(dev, mode, [33000], fmt, seed=50, Hkv=1)
+    run_case(dev, mode, [33000, 700], fmt, seed=51, Hkv=1, nsplit=5)
+    run_case(dev, mode, [65536, 40], fmt, seed=52, Hkv=1, win=(132, 3), kv_start=4)
+    run_case(dev, mode, [65536], fmt, seed=53, Hkv=1, nsplit=8)
+
+
 @pytest.mark.parametrize("shared", ["copy", "stride0"])
 def test_shared_block_table_row(dev, shared):
     run_case(dev, "codebook", [100, 37, 64], "konlya", bt_shared=shared, seed=9, Hkv=2)
@@ -195,6 +207,10 @@ def test_decode_error_codes(dev):
     bad_page = list(base); bad_page[8] = 64
     assert L.fr_v2_attn(5, *bad_page, 4, 0) == -5
     assert L.fr_v2_attn(5, *base, 8, 0) == -7            # gqa 8 without the generalised variant bits
+    no_ws = list(base); no_ws[9] = 2; no_ws[19] = None                # two splits, no partial buffer: an error code, not a fault
+    assert L.fr_v2_attn(5, *no_ws, 4, 0) == -3 and b"opart" in L.fr_last_error()
+    no_ctr = list(base); no_ctr[9] = 2; no_ctr[21] = None
+    assert L.fr_v2_attn(5, *no_ctr, 4, 0) == -3
     hd = list(base); hd[17] = 264 | 1024 | 2048 | 4096
     assert L.fr_v2_attn(5, *hd, 4, 0) == -3              # head dim 256 takes q tiles of 4 heads, not 8
     assert L.fr_cb_attn(zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, K.sign_words(), 3, 0, 4, zp, zp, zp, zp, 512, None,

@@ -1,6 +1,7 @@
 """The benchmark workloads at their FULL shapes, as parity tests: the very launches bench.py times (same builders, same
 planner, through the C-ABI), each checked on sampled sequences against the oracle.
 
+  configs[0]  INT4 key-only pages (konly), B=1, L=2048, uniform calibration: writer bytes and attention against the oracle
   configs[1]  INT4 key-only pages (konlya), B=32, 32q/8kv, L=8192: nsplit 1, chunk 8192, 16-wavefront workgroups; with
               the split plan of this build's planner and with the one the reference's cost model makes
   configs[2]  INT2 key-only pages (konlya2) + static key centring + 4 sink / 128 window BF16 rows, B=64, L=16384
@@ -35,6 +36,25 @@ def _args(**kw):
 
 def _report(name, r):
     print(f"\n{name}: {r['check']}  [{r['bar']}]", flush=True)
+
+
+def test_configs0_b1_l2048_konly_uniform_calibration(dev):
+    """configs[0] -- the reference's own CPU-runnable case (one decode step of the Llama-3.1-8B layer shape, batch 1,
+    context 2048, INT4 key-only pages, C_q = I, c_o = 1; kernels/codebook_ref.py:191-236 for the writer,
+    integrations/vllm_flagrot/tests/test_kernels.py:37-56 for the attention) through the HIP writer and decode: the pool
+    must be byte-equal to the oracle's packed pool and the attention inside the element-wise bar"""
+    from flagrot_releaser_amd import kernels as K
+    r = bench.configs0(torch, K, dev, timed_legs=False)
+    print("\n" + r["check"], flush=True)
+    assert r["pool_bytes_equal"], r["check"]
+    assert r["checked"] and r["errors"]["elementwise"] <= 1.0, r["check"]
+
+
+def test_int2_at_the_headline_shape_b32_l8192(dev):
+    """the metric names INT4 and INT2 at batch 32 x 8K: the INT2 key-only pages at configs[1]'s shape"""
+    r = bench.run_flagrot(_args(), torch, dev, "int2_b32", 3, 2)["own"]
+    _report("INT2 konlya2, B=32 L=8192", r)
+    assert r["checked"] and r["errors"]["elementwise"] <= 1.0, r["check"]
 
 
 def test_configs1_int4_b32_l8192_both_planners(dev):

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 MARK = 0x9E3779B9 - (1 << 32)
 
 
-@pytest.mark.parametrize("chunk,page,hkv", [(2304, 16, 8), (1280, 16, 4), (1552, 32, 2)])
+@pytest.mark.parametrize("chunk,page,hkv", [(2304, 16, 8), (1280, 16, 4), (1552, 32, 2), (4608, 32, 2)])
 def test_probe_reads_the_addressed_pages_only(chunk, page, hkv):
     from flagrot_releaser_amd import probe
     dev = torch.device("cuda:0")

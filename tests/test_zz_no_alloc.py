@@ -100,6 +100,50 @@ def test_noalloc_large_workgroups_twice(dev):
     _check(*b, "large second (smaller)")
 
 
+def test_noalloc_allocates_nothing_and_replays_from_a_graph(dev):
+    """after one warm-up call (the first call on a device looks the built-in array up and must not be made under
+    capture) a call changes neither the device's free memory nor torch's allocator; captured into a HIP graph it replays
+    with new queries and matches the eager call each time"""
+    from flagrot_releaser_amd import kernels as K
+    kind, lens, Hkv, G = "konlya", [900, 333, 1500], 2, 4
+    pool, bt, g = _cache(dev, lens, kind, Hkv, 75)
+    B, HQ = len(lens), G * Hkv
+    dq = (torch.randn(B, HQ, 128, generator=g) * 0.8).bfloat16().to(dev)
+    dbt, dseq = bt.to(dev), torch.tensor(lens, dtype=torch.int32, device=dev)
+    ns, ch = K.plan_cb(B, max(lens), Hkv, P16, kind, nsplit=3)
+    out = torch.zeros(B, HQ * 128, dtype=torch.bfloat16, device=dev)
+    scale = LOG2E / math.sqrt(128)
+    call = K.cb_attn_noalloc(dq, pool, dbt, dseq, out, ns, ch, scale, kind, bound=True)
+    call()                                                   # warm-up: address lookup, module load
+    torch.cuda.synchronize()
+    free0, held0, peak0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.max_memory_allocated()
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == held0
+    assert torch.cuda.max_memory_allocated() == peak0
+    eager = out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        K.cb_attn_noalloc(dq, pool, dbt, dseq, out, ns, ch, scale, kind)      # the capture stream's first use
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        K.cb_attn_noalloc(dq, pool, dbt, dseq, out, ns, ch, scale, kind)
+    for rep in range(3):
+        if rep:
+            dq.copy_((torch.randn(B, HQ, 128, generator=g) * 0.8).bfloat16())
+            call()                                           # eager work and a synchronisation between the replays
+            torch.cuda.synchronize()
+            eager = out.clone()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        a, b = eager.float().cpu().numpy().astype(np.float64), out.float().cpu().numpy().astype(np.float64)
+        assert (np.abs(b - a) <= ATOL + RTOL * np.abs(a)).all(), f"replay {rep} differs from the eager call"
+
+
 def test_noalloc_rejects_sizes_beyond_the_built_in_workspace(dev):
     from flagrot_releaser_amd import kernels as K
     L = K.lib()
