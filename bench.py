@@ -611,7 +611,9 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
         gots.append(got)
         refs.append(ref)
     st = error_stats(np.stack(gots), np.stack(refs))
+    probe = mfma_probe(torch, dev)
     return {"workload": name, "ms_per_layer": round(us * 1e-3, 4), "TFLOPs": round(tflops, 1),
+            "mfma_probe": {**probe, "kernel_over_lds_probe": round(tflops / max(probe["lds_operand_TFLOPs"], 1e-9), 4)},
             "frac": round(tflops / PEAK_F16_TFLOPS, 4), "bound": "mfma", "peak_TFLOPs": PEAK_F16_TFLOPS,
             "graph_min_us": round(t["graph_min_us"], 1), "graph_max_us": round(t["graph_max_us"], 1),
             "eager_us": round(t["eager_us"], 1), "algorithmic_flops_per_launch": flops, "steps": steps,
@@ -620,6 +622,32 @@ def run_mq(args, torch, dev, steps, warmup, fmt):
             "errors": st, "check": f"request {r}, rows 0-3 and {NQ - 4}-{NQ - 1}, {nh * Gq} q heads vs fp64 attention over "
                                    "the oracle's dequantised pages: " + describe(st),
             "note": "one step = frmq_prep_q + frmq_attn + frmq_merge; the attention kernel dominates"}
+
+
+def mfma_probe(torch, dev, iters=4000):
+    """the matrix pipe's reachable dense-fp16 rate on this box: a kernel of nothing but v_mfma_f32_32x32x16_f16 (one
+    workgroup of 8 wavefronts per CU), operands in registers / one operand of every instruction read from LDS"""
+    from flagrot_releaser_amd import probe as PR
+    PR.lib()
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {}
+    for mode, key in ((0, "registers_TFLOPs"), (1, "lds_operand_TFLOPs")):
+        PR.mfma_burst(mode, iters // 8, cus, sink)
+        torch.cuda.synchronize()
+        best = 0.0
+        for _ in range(3):
+            e0.record()
+            flops = PR.mfma_burst(mode, iters, cus, sink)
+            e1.record()
+            torch.cuda.synchronize()
+            best = max(best, flops / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+        out[key] = round(best, 1)
+    out["nominal_TFLOPs"] = PEAK_F16_TFLOPS
+    out["note"] = (f"{cus} workgroups x 8 wavefronts x {iters} x 4 v_mfma_f32_32x32x16_f16, best of 3 launches "
+                   "(flagrot_releaser_amd/csrc/probe_mfma.hip)")
+    return out
 
 
 def traffic_of(workload):
@@ -670,6 +698,7 @@ def main():
                             "frac": r["frac"], "traffic": None,
                             "algorithmic_flops_per_launch": r["algorithmic_flops_per_launch"],
                             "avg_launch_us": r["ms_per_layer"] * 1e3, "eager_us": r["eager_us"]},
+               "mfma_probe": r["mfma_probe"],
                "checked": r["checked"], "bar": r["bar"], "errors": r["errors"], "check": r["check"]}
     else:
         if workload == "kivi":

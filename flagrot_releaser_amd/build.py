@@ -24,13 +24,16 @@ COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-t
           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 # bit-exact translation units: every fp32 operation rounded on its own
 STRICT = ["-ffp-contract=off", "-fno-fast-math"]
+# FLAGROT_STRICT_MERGE=1 in the environment of the build: memory-model-strict split merge in the decode kernels (decode.hip)
+if os.environ.get("FLAGROT_STRICT_MERGE", "0") not in ("", "0"):
+    COMMON = COMMON + ["-DFLAGROT_STRICT_MERGE=1"]
 
 # library -> [(source, extra flags)]
 LIBS = {
     "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("decode_wide_mma.hip", []), ("capi.hip", [])]),
     "kivi": ("libflagrot_kivi.so", [("kivi_write.hip", STRICT), ("kivi_wide.hip", STRICT), ("kivi_attn.hip", []), ("kivi_decode.hip", []), ("kivi_decode_wide.hip", [])]),
     "mq": ("libflagrot_mq.so", [("mq_prefill.hip", []), ("mq_wide.hip", [])]),
-    "probe": ("libflagrot_probe.so", [("probe_read.hip", [])]),      # measurement aid (bench.py), not a boundary library
+    "probe": ("libflagrot_probe.so", [("probe_read.hip", []), ("probe_mfma.hip", [])]),      # measurement aid (bench.py), not a boundary library
 }
 
 

@@ -35,9 +35,18 @@
 #include "fr_unpack.hpp"
 #include "decode_tiles.hpp"
 
+// FLAGROT_STRICT_MERGE=1 (a build flag: `FLAGROT_STRICT_MERGE=1 python -m flagrot_releaser_amd.build kernels`) gives the
+// split-merge ticket the orders the HIP memory model asks for -- an agent-scope release on the ticket, an agent-scope
+// acquire in the last arriver -- instead of relying on what write-through stores and read-through loads do on gfx950.
+// Same results; each workgroup then pays a write-back and an invalidate of its XCD's L2.
+#ifndef FLAGROT_STRICT_MERGE
+#define FLAGROT_STRICT_MERGE 0
+#endif
+
 namespace fr {
 using namespace dec;
 namespace {
+constexpr bool STRICT_MERGE = FLAGROT_STRICT_MERGE != 0;
 
 // BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
 template <int NW>
@@ -141,7 +150,6 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
   // the (sequence, KV head, q tile)'s counter slot: merge ticket, and in the dynamic mode the quad draw counter
   const int tpc = p.counter_div;                                 // q tiles that share one counter slot
   int* const ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
-  float Mwg[4];                   // the workgroup's maxima per head (uniform)
   if (!is_tail) {
     const int lo = dyn ? min(p.kv_start, len) : max(split * p.chunk, min(p.kv_start, len));
     const int hi = dyn ? len : min(len, (split + 1) * p.chunk);
@@ -315,59 +323,49 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) st.ot[y][r4] = (st.ot[y][r4] - zg) * 16777216.f;
     }
-    // head x = lane >> 4 lives in a row of 16 lanes
+    // head x = lane >> 4 lives in a row of 16 lanes.  Every wavefront leaves its maxima, its sums and its outputs
+    // relative to its OWN maxima (its strips are dead: the outputs take their place); the output threads scale while
+    // they add -- one barrier and one LDS round trip between the last quad and the result.
     const float lsum = row_sum16(st.l * unfold);
-    if ((lane & 15) == 0) S.m[wave][lane >> 4] = st.m;
-    __syncthreads();     // every wave is done with its strip: the partial outputs may overwrite them
+    if ((lane & 15) == 0) { S.m[wave][lane >> 4] = st.m; S.l[wave][lane >> 4] = lsum; }
     {
-      workgroup_max<NW>(S, lane, Mwg);
-      // this wavefront's factors 2^(m - M) per head (uniform): its own maxima sit in lanes 0, 16, 32, 48
-      float f[4];
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const float mh = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, st.m), 16 * h));
-        f[h] = mh == -INFINITY ? 0.f : fexp2(mh - Mwg[h]);
-      }
-      if ((lane & 15) == 0) S.l[wave][lane >> 4] = pick4(f[0], f[1], f[2], f[3], lane >> 4) * lsum;
-      const float fl = pick4(f[0], f[1], f[2], f[3], hl);
       const int kc = lane >> 4;      // the lane's four entry rows: 4 kc + r
       float* o = S.o(wave, hl);
 #pragma unroll
       for (int y = 0; y < 2; ++y) {
         // entry e = 16 (gl & 1) + 4 kc + r, word sub = 2 (gl >> 1) + y: dim 64 (sub >> 1) + 16 (e >> 3) + 8 (sub & 1) + (e & 7)
         const int d = 32 * gl + 16 * (kc >> 1) + 8 * y + 4 * (kc & 1);
-        *reinterpret_cast<float4*>(o + d) = make_float4(fl * st.ot[y][0], fl * st.ot[y][1], fl * st.ot[y][2], fl * st.ot[y][3]);
+        *reinterpret_cast<float4*>(o + d) = make_float4(st.ot[y][0], st.ot[y][1], st.ot[y][2], st.ot[y][3]);
       }
     }
-    __syncthreads();
   } else {
     float m[4], l[4], o[4][2];
     tail_partial<NW>(p, b, kvh, tile, m, l, o);
-    if (lane < 4) S.m[wave][lane] = pick4(m[0], m[1], m[2], m[3], lane);
-    __syncthreads();
-    workgroup_max<NW>(S, lane, Mwg);
+    if (lane < 4) { S.m[wave][lane] = pick4(m[0], m[1], m[2], m[3], lane); S.l[wave][lane] = pick4(l[0], l[1], l[2], l[3], lane); }
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
-      const float f = m[h] == -INFINITY ? 0.f : fexp2(m[h] - Mwg[h]);
-      if (lane == 0) S.l[wave][h] = f * l[h];
       float* so = S.o(wave, h);
-      so[2 * lane] = f * o[h][0];
-      so[2 * lane + 1] = f * o[h][1];
+      so[2 * lane] = o[h][0];
+      so[2 * lane + 1] = o[h][1];
     }
-    __syncthreads();
   }
+  __syncthreads();
   // ---- workgroup partial: (o[4][128] relative to M, M, L); thread = (head, 2 dims) for the first 4 wavefronts
   float po[2] = {0.f, 0.f}, pm = -INFINITY, pl = 0.f;
   const int oh = wave & 3;           // head of this thread's two outputs
   if (act) {
-    // the sums were scaled by their wavefront's factor when they were stored: lane w fetches wavefront w's
+    // lane w holds wavefront w's maximum and sum of head oh: the workgroup's maximum, every wavefront's factor
+    // 2^(m_w - M) and the scaled sum come from two row reductions
+    const float mw = lane < NW ? S.m[lane][oh] : -INFINITY;
     const float lw = lane < NW ? S.l[lane][oh] : 0.f;
-    pm = pick4(Mwg[0], Mwg[1], Mwg[2], Mwg[3], oh);
-    pl = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_sum16(lw))));
+    pm = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(mw))));
+    const float fw = mw == -INFINITY ? 0.f : fexp2(mw - pm);
+    pl = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_sum16(fw * lw))));
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
+      const float f = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, fw), w));
       const float2 v = *reinterpret_cast<const float2*>(S.o(w, oh) + 2 * lane);
-      po[0] += v.x; po[1] += v.y;
+      po[0] += f * v.x; po[1] += f * v.y;
     }
   }
   if (is_tail && p.vmask != nullptr) {  // the merged sum is rotated back once: bring the tail into the stored basis
@@ -408,13 +406,15 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) {    // every draw of this workgroup precedes its ticket: the last arriver may clear the slot
-      const int prev = __hip_atomic_fetch_add(ctr, dyn ? DRAW_MASK + 1 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int prev = __hip_atomic_fetch_add(ctr, dyn ? DRAW_MASK + 1 : 1, STRICT_MERGE ? __ATOMIC_RELEASE : __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
       S.last = (dyn ? static_cast<int>(static_cast<unsigned>(prev) >> DRAW_BITS) : prev) == tpc * nparts - 1;
       if (S.last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!S.last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if constexpr (STRICT_MERGE) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   } else if (dyn && threadIdx.x == 0) {
     __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // the only workgroup of the slot
   }

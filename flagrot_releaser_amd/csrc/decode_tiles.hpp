@@ -47,11 +47,13 @@ struct Smem {
   int btc[BT_CACHE];
   int next;                                          // next quad of 4 pages nobody has taken yet
   int last;
+  static_assert(STRIP_BYTES >= 2048 && STRIP_BYTES % 16 == 0, "a wavefront's strips must hold its partial outputs");
   DEVI uint8_t* pb(int w) { return work + w * STRIP_BYTES; }
   DEVI const uint8_t* pb(int w) const { return work + w * STRIP_BYTES; }
   DEVI uint8_t* zb(int w) { return work + w * STRIP_BYTES + PB_BYTES; }
   DEVI const uint8_t* zb(int w) const { return work + w * STRIP_BYTES + PB_BYTES; }
-  DEVI float* o(int w, int h) { return reinterpret_cast<float*>(work) + (w * 4 + h) * 128; }
+  // a wavefront's partial outputs [4][128] take the place of its OWN strips (2 KB of them): no other wavefront's strip is touched
+  DEVI float* o(int w, int h) { return reinterpret_cast<float*>(work + w * (STRIP_BYTES > 2048 ? STRIP_BYTES : 2048)) + h * 128; }
 };
 
 // slot of element (isB, i) of a K word / of token r8 of a V word inside the 8-fp16 operand vector

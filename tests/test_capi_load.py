@@ -71,7 +71,8 @@ def test_probe_library_exports_header_symbols():
         build.build("probe", verbose=False)
     L = ctypes.CDLL(str(path))
     names = _declared("flagrot_probe.h")
-    assert set(names) == set(probe.EXPORTS) == {"fr_probe_abi_version", "fr_probe_last_error", "fr_probe_read"}
+    assert set(names) == set(probe.EXPORTS) == {"fr_probe_abi_version", "fr_probe_last_error", "fr_probe_read",
+                                                      "fr_probe_mfma", "fr_probe_mfma_flops"}
     for n in names:
         assert hasattr(L, n), n
     L.fr_probe_abi_version.restype = ctypes.c_int

@@ -39,3 +39,13 @@ def test_probe_rejects_bad_arguments():
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     with pytest.raises(RuntimeError):
         probe.read_pages(pool, bt, seq, sink, 16)          # chunk bytes not a multiple of 16
+
+
+def test_mfma_probe_runs_and_reports_a_plausible_rate():
+    """the matrix-pipe probe: both modes launch, finish, and land between 5 % and 110 % of the nominal dense fp16 rate"""
+    import bench
+    dev = torch.device("cuda:0")
+    r = bench.mfma_probe(torch, dev, iters=800)
+    print(f"\nmfma probe: {r}", flush=True)
+    for key in ("registers_TFLOPs", "lds_operand_TFLOPs"):
+        assert 0.05 * r["nominal_TFLOPs"] < r[key] < 1.1 * r["nominal_TFLOPs"], r
