@@ -324,6 +324,9 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
         name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
                 "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
     HKV, DH, G = globals()["HKV"], globals()["DH"], globals()["G"]
+    if getattr(args, "gqa", 4) != 4:              # not a configuration of the baseline: GQA groups of 8 (Qwen-32B's 64q/8kv) on the same pages
+        G = int(args.gqa)
+        name = name.replace("32q/8kv", f"{G * HKV}q/{HKV}kv") + f" [GQA {G}: not a baseline configuration]"
     if getattr(args, "head_dim", 128) == 256:     # not a configuration of the baseline: the head dim 256 kernels, same page bytes
         HKV, DH, G = 4, 256, 6
         name = (f"{'INT4' if workload == 'int4' else 'INT2'} FlagRot {kind} paged decode at head dim 256, GQA 24q/4kv, B={B} "
@@ -360,7 +363,7 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
         else:      # "reference": the reference front end's cost model fed with this library's occupancy answer
             occ = K.lib().fr_cb_occupancy(K.CB_KINDS[kind], 0, K.STAGES, P)
             ns, ch = reference_plan(B, Lpages, HKV, max(1, occ) * cus)
-        if DH == 128:
+        if DH == 128 and G == 4:
             ws = K.Workspace(B, HKV, B * HKV * (ns + 1), dev)
         else:
             hv = K.vheads(HKV, G, DH, kind)
@@ -667,6 +670,7 @@ def main():
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
     ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="256 = the head dim 256 kernels (GQA 24q/4kv, the reference's test shape class); not a baseline configuration")
+    ap.add_argument("--gqa", type=int, default=4, help="int4 / int2 workloads: query heads per KV head (8 = tiles of 8 heads; not a baseline configuration)")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", action="store_true", help="the chosen workload only (no extra legs)")

@@ -30,7 +30,7 @@ if os.environ.get("FLAGROT_STRICT_MERGE", "0") not in ("", "0"):
 
 # library -> [(source, extra flags)]
 LIBS = {
-    "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_wide.hip", []), ("decode_wide_mma.hip", []), ("capi.hip", [])]),
+    "kernels": ("libflagrot_kernels.so", [("writer.hip", STRICT), ("decode.hip", []), ("decode_gqa8.hip", []), ("decode_wide.hip", []), ("decode_wide_mma.hip", []), ("capi.hip", [])]),
     "kivi": ("libflagrot_kivi.so", [("kivi_write.hip", STRICT), ("kivi_wide.hip", STRICT), ("kivi_attn.hip", []), ("kivi_decode.hip", []), ("kivi_decode_wide.hip", [])]),
     "mq": ("libflagrot_mq.so", [("mq_prefill.hip", []), ("mq_wide.hip", [])]),
     "probe": ("libflagrot_probe.so", [("probe_read.hip", []), ("probe_mfma.hip", [])]),      # measurement aid (bench.py), not a boundary library

@@ -83,12 +83,10 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   p.kmask = (!k2 && qrot) ? kmask : nullptr;
   p.vmask = (!k2 && (vrot || tail != nullptr)) ? vmask : nullptr;
   p.opart = opart; p.mlpart = mlpart; p.counter = counter;
-  const int gt = ((variant & GEN) && (variant & GT8)) ? 8 : 4;
-  const int ntile = (gqa + 3) / 4, nct = (gqa + gt - 1) / gt;
-  // a counter slot must hold a whole number of 4-head tiles: with tiles of 8 and 9..12 heads (3 tiles, 2 slots) the
-  // kernel would index three counter words where the caller sized two
-  if (ntile % nct != 0) return fail(-7, "fr_v2_attn: the 8-head tile variant needs gqa <= 8 (or a multiple of 8)");
-  p.counter_div = ntile / nct;
+  // tiles of 8 query heads (GEN | GT8): one workgroup per (KV head, 8 heads), one counter slot and two 4-head partial
+  // slots per tile -- the layout a caller sizes with tile_of(variant) = 8; heads past gqa are padding
+  p.tile8 = ((variant & GEN) && (variant & GT8)) ? 1 : 0;
+  const int ntile = p.tile8 ? (gqa + 7) / 8 : (gqa + 3) / 4;
   p.out = out; p.o_bs = o_bs;
   p.tail = tail; p.tail_len = tail_len; p.tail_idx = tail_idx; p.tail_bs = tail_bs; p.tail_ts = tail_ts;
   p.gqa = gqa; p.kv_start = kv_start;
@@ -103,7 +101,7 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   static const int env_waves = getenv("FLAGROT_WG_WAVES") != nullptr ? atoi(getenv("FLAGROT_WG_WAVES")) : 0;
   const long long wgs = static_cast<long long>(B) * Hkv * ntile * nsplit;
   const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && wgs <= device_cus());
-  const bool can_draw = !force_static && counter != nullptr && p.counter_div == 1 && nparts <= 1023;
+  const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;
   // the split merge goes through the caller's workspace: partials, their (max, sum) pairs and, at head dim 128, the ticket
   if (nparts > 1 && (opart == nullptr || mlpart == nullptr || (!(variant & HD256) && counter == nullptr)))
     return fail(-3, "fr_v2_attn: more than one partial per (sequence, KV head) needs opart, mlpart and counter");
@@ -272,8 +270,10 @@ int fr_cb_attn_noalloc(const void* q, long long q_bs, const uint8_t* pool, const
   const int nctr = static_cast<int>(static_cast<long long>(B) * Hkv * ntile);
   hipLaunchKernelGGL(k_clear_words, dim3((nctr + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), counter, nctr);
   if (hipPeekAtLastError() != hipSuccess) return launched(-1, "fr_cb_attn_noalloc (clear)");
+  // groups of 5 .. 8 heads (and whole multiples of 8) run tiles of 8 heads: same partial slots, half the counter words
+  const int variant = 264 | GEN | (((gqa > 4 && gqa <= 8) || gqa % 8 == 0) ? GT8 : 0);
   return fr_v2_attn(fmt, q, q_bs, pool, block_table, bt_stride, seq_lens, B, Hkv, page, nsplit, chunk, qscale, nullptr,
-                    nullptr, 32, 0, 0, 264 | GEN, 4, opart, mlpart, counter, out, o_bs, tail, tail_len, tail_idx,
+                    nullptr, 32, 0, 0, variant, 4, opart, mlpart, counter, out, o_bs, tail, tail_len, tail_idx,
                     tail_bs, tail_ts, stream, gqa, kv_start);
 }
 

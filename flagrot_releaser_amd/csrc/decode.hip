@@ -48,46 +48,6 @@ using namespace dec;
 namespace {
 constexpr bool STRICT_MERGE = FLAGROT_STRICT_MERGE != 0;
 
-// BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
-template <int NW>
-DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&m)[4], float (&l)[4], float (&o)[4][2]) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = p.tail_len[b];
-  const int row = p.tail_idx != nullptr ? p.tail_idx[b] : b;
-  const uint16_t* base = static_cast<const uint16_t*>(p.tail) + static_cast<long long>(row) * p.tail_bs;
-  float q[4][2];
-#pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int hq = tile * 4 + h;
-    q[h][0] = q[h][1] = 0.f;
-    if (hq < p.gqa) {
-      const uint32_t raw = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
-                                                              (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 2 * lane);
-      q[h][0] = bf16_lo(raw) * p.qscale;
-      q[h][1] = bf16_hi(raw) * p.qscale;
-    }
-    m[h] = -INFINITY; l[h] = 0.f; o[h][0] = o[h][1] = 0.f;
-  }
-  for (int t = wave; t < n; t += NW) {
-    const uint16_t* tr = base + static_cast<long long>(t) * p.tail_ts;
-    const uint32_t kr = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
-    const uint32_t vr = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
-    const float k0 = bf16_lo(kr), k1 = bf16_hi(kr), v0 = bf16_lo(vr), v1 = bf16_hi(vr);
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      float s = q[h][0] * k0 + q[h][1] * k1;
-      s += dpp_xor1(s); s += dpp_xor2(s);
-      s = wave_sum_over_tokens(s);
-      const float mn = fmaxf(m[h], s);
-      const float alpha = fexp2(m[h] - mn), pe = fexp2(s - mn);
-      m[h] = mn;
-      l[h] = l[h] * alpha + pe;
-      o[h][0] = o[h][0] * alpha + pe * v0;
-      o[h][1] = o[h][1] * alpha + pe * v1;
-    }
-  }
-}
-
 template <int QM, bool K2, int P, int NW>
 __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int ntile, int nparts) {
   using L = Lay<QM, P>;
@@ -148,7 +108,11 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
   const bool act = wave < 4;      // the 256 threads that own the workgroup's 4 x 128 outputs
 
   // the (sequence, KV head, q tile)'s counter slot: merge ticket, and in the dynamic mode the quad draw counter
-  const int tpc = p.counter_div;                                 // q tiles that share one counter slot
+  // q tiles per counter slot: always 1.  The value is hidden from the compiler on purpose: folded in as a constant it
+  // turns the final merge into straight-line code, the register allocation of the page loop changes with it, and the
+  // loops of two formats spill (a reload from scratch waits for every page fetch in flight).
+  int tpc = 1;
+  asm volatile("" : "+s"(tpc));
   int* const ctr = p.counter + (static_cast<long long>(b) * p.Hkv + kvh) * (ntile / tpc) + tile / tpc;
   if (!is_tail) {
     const int lo = dyn ? min(p.kv_start, len) : max(split * p.chunk, min(p.kv_start, len));
@@ -504,7 +468,9 @@ int decode_dispatch(int fmt, const DecodeParams& p, hipStream_t st) {
 
 }  // namespace
 
-int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) { return decode_dispatch(fmt, p, st); }
+int decode_launch(int fmt, const DecodeParams& p, hipStream_t st) {
+  return p.tile8 ? decode8_launch(fmt, p, st) : decode_dispatch(fmt, p, st);
+}
 int decode_waves(int chunk_tokens) { return waves_for(chunk_tokens); }
 int decode_big_chunk() {      // FLAGROT_BIG_CHUNK overrides (experiments)
   static const int v = getenv("FLAGROT_BIG_CHUNK") != nullptr ? atoi(getenv("FLAGROT_BIG_CHUNK")) : BIG_CHUNK;

@@ -485,5 +485,323 @@ DEVI float pick4(float v0, float v1, float v2, float v3, int i) {
   return (i & 2) ? hi : lo;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Tiles of 8 query heads (GQA groups of 5 .. 8 heads at head dim 128; the reference's GT = 8 kernels,
+// kernels/csrc/attn_decode_v2g.cuh:5-10): one workgroup serves both 4-head halves of the tile on ONE unpacking of a quad
+// -- the pages are read once.  The key phase runs the score products of both halves against the same masked code
+// words (two sets of query operands), the softmax keeps two (token, head) states per lane, the strips hold p * V-scale
+// for 8 heads per group, and the value phase multiplies the same masked V^T entries with two sets of strip rows into
+// two sets of accumulators.  Everything that depends only on the tokens (unpacking, flags, scale words and their
+// exchange among a token's four lanes, zero points) is done once.
+constexpr int PB8_RSTRIDE = 33;                    // uint4 per row group: 32 (group, head of 8) entries + 1 pad (stays zero)
+template <int QM> struct Strip8 {
+  static constexpr int ROWS = 2 * QBLK<QM>;
+  static constexpr int PB_BYTES = ROWS * PB8_RSTRIDE * 16;     // per wave: [block][c8][group][head of 8][8 fp16]
+  static constexpr int ZB_BYTES = ROWS * ZB_RSTRIDE * 16;
+  static constexpr int BYTES = PB_BYTES + ZB_BYTES;
+};
+template <int QM, int NW>
+struct Smem8 {
+  static constexpr int STRIP_BYTES = Strip8<QM>::BYTES, PB_BYTES = Strip8<QM>::PB_BYTES;
+  static_assert(STRIP_BYTES >= 8 * 128 * 4 && STRIP_BYTES % 16 == 0, "a wavefront's strips must hold its partial outputs");
+  alignas(16) uint4 qhi[2][4][64];                   // [half of the tile][group][lane of the matrix instruction]: as Smem::qhi
+  alignas(16) uint4 qlo[2][4][64];
+  alignas(16) uint4 qz[2][4][64];
+  alignas(16) uint8_t work[NW * STRIP_BYTES];
+  float m[NW][8], l[NW][8];
+  int btc[BT_CACHE];
+  int next;
+  int last;
+  DEVI uint8_t* pb(int w) { return work + w * STRIP_BYTES; }
+  DEVI const uint8_t* pb(int w) const { return work + w * STRIP_BYTES; }
+  DEVI uint8_t* zb(int w) { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI const uint8_t* zb(int w) const { return work + w * STRIP_BYTES + PB_BYTES; }
+  DEVI float* o(int w, int h) { return reinterpret_cast<float*>(work + w * STRIP_BYTES) + h * 128; }   // h: head of 8
+};
+struct WaveState8 {          // WaveState for the two halves of the tile
+  float m[2], l[2];
+  f32x4 ot[2][2];
+  float z[2][2];
+};
+
+// q_prologue for a tile of 8 heads: head hh (0..7) is prepared by wavefront hh (workgroups of fewer wavefronts take
+// several heads in turn) into the operand tables of half hh >> 2, rows of head hh & 3.
+template <int QM, bool K2, int NW, class SM>
+DEVI void q_prologue8(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
+  const int wv = threadIdx.x >> 6, half = (threadIdx.x >> 5) & 1, l32 = threadIdx.x & 31;
+  for (int hh = wv; hh < 8; hh += NW) {
+  const int th = hh >> 2, w = hh & 3;
+  const int hq = tile * 8 + hh;                      // head inside the GQA group
+  float x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (hq < p.gqa) {
+    const uint16_t* qr = static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
+                         (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 4 * l32;
+    const uint2 raw = *reinterpret_cast<const uint2*>(qr);
+    x[0] = bf16_lo(raw.x); x[1] = bf16_hi(raw.x); x[2] = bf16_lo(raw.y); x[3] = bf16_hi(raw.y);
+  }
+  const int g = l32 >> 3, isB = (l32 >> 2) & 1, tg = l32 & 3;
+  float y[4] = {x[0], x[1], x[2], x[3]};
+  if (half == 0) fwht<32>(y, l32); else fwht<128>(y, l32);
+  const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
+  const float fold = QPRE / beta;
+#pragma unroll
+  for (int vi = 0; vi < 2; ++vi) {
+    const int var = 2 * half + vi;
+    float v[4];
+    bool live;
+    if (K2) {
+      live = var < 3;
+      const bool rot = var != 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = rot ? y[i] : x[i];
+    } else {
+      live = var == 0;
+      const uint32_t rot = (p.kmask != nullptr && p.kmask[kvh * 4 + g] != 0) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = __uint_as_float((__float_as_uint(y[i]) & rot) | (__float_as_uint(x[i]) & ~rot));
+    }
+    uint32_t hb[4], lb[4];
+    float qs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = live ? v[i] * fold : 0.f;
+      const _Float16 hi = static_cast<_Float16>(a);
+      const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
+      hb[i] = __builtin_bit_cast(uint16_t, hi);
+      lb[i] = __builtin_bit_cast(uint16_t, lo);
+      qs += (static_cast<float>(hi) + static_cast<float>(lo)) * beta;
+    }
+    const int m = 4 * w + var, ln = m + 16 * tg;
+    uint32_t* dh = reinterpret_cast<uint32_t*>(&S.qhi[th][g][ln]);
+    uint32_t* dl = reinterpret_cast<uint32_t*>(&S.qlo[th][g][ln]);
+    dh[isB] = hb[0] | (hb[2] << 16); dh[2 + isB] = hb[1] | (hb[3] << 16);
+    dl[isB] = lb[0] | (lb[2] << 16); dl[2 + isB] = lb[1] | (lb[3] << 16);
+    if constexpr (QM != QM_SYM4) {
+      qs += hx(qs, 1); qs += hx(qs, 2); qs += hx(qs, 4);
+      if ((l32 & 7) == 0) {
+        const _Float16 zh = static_cast<_Float16>(-qs);
+        const _Float16 zl = static_cast<_Float16>(-qs - static_cast<float>(zh));
+        const int sh = 16 * (g & 1);
+        S.qz[th][g][m] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zh)) << sh, 0u, 0u, 0u);
+        S.qz[th][g][m + 16] = make_uint4(static_cast<uint32_t>(__builtin_bit_cast(uint16_t, zl)) << sh, 0u, 0u, 0u);
+        S.qz[th][g][m + 32] = make_uint4(0u, 0u, 0u, 0u);
+        S.qz[th][g][m + 48] = make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  }
+  }
+}
+
+// scores of the lane's token for heads x and 4 + x (x = lane >> 4), four blocks: the group's masked words are made once
+// and multiplied with the query operands of both halves of the tile
+template <int QM, bool K2, class SM>
+DEVI void key_phase8(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[2][QBLK<QM>]) {
+  constexpr int QB = QBLK<QM>;
+  static_assert(QB == 4, "four blocks per wave iteration");
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  bool full[QB];
+  whole_head_flags<QM, K2>(r, lane, full);
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int b = 0; b < QB; ++b) sc[t][b] = 0.f;
+  const uint32_t zlane = (lane < 32) ? static_cast<uint32_t>(ZM) : 0u;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    half8 kb[QB], kz[QB];
+    float sv[QB];
+    bool h32[QB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      uint32_t x[4];
+      if constexpr (QM == QM_ASYM2) {
+        if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
+      }
+      else UnpackD<QM>::run(r.kc[b][j], x);
+      kb[b] = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+      const uint32_t kw = (j & 2) ? r.ks[b].y : r.ks[b].x;
+      kz[b] = __builtin_bit_cast(half8, make_uint4(kw & (zlane << (16 * (j & 1))), 0u, 0u, 0u));
+      sv[b] = fabsf(word_value(kw, j));
+      h32[b] = (kw >> (16 * (j & 1) + 15)) & 1u;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const half8 qh = __builtin_bit_cast(half8, S.qhi[t][j][lane]), ql = __builtin_bit_cast(half8, S.qlo[t][j][lane]);
+      half8 qz;
+      if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[t][j][lane]);
+      f32x4 acc[QB];
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh, kb[b], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql, kb[b], a, 0, 0, 0);
+        if constexpr (ZM != 0) a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qz, kz[b], a, 0, 0, 0);
+        acc[b] = a;
+      }
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        float pick = acc[b][0];
+        if constexpr (K2) pick = full[b] ? acc[b][2] : (h32[b] ? acc[b][1] : acc[b][0]);
+        sc[t][b] += pick * sv[b];
+      }
+    }
+  }
+}
+
+// softmax step of both halves; the strips take p * V-scale of heads x and 4 + x for all four groups
+template <int QM, class SM>
+DEVI void softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[2][QBLK<QM>], const bool (&valid)[QBLK<QM>],
+                         float qs20, float sc0, int lane, int wave) {
+  constexpr int QB = QBLK<QM>;
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  float mx[2];
+  bool beat = false;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    mx[t] = -INFINITY;
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      sc[t][b] = valid[b] ? sc[t][b] * qs20 + sc0 : -INFINITY;
+      mx[t] = fmaxf(mx[t], sc[t][b]);
+    }
+    beat = beat || mx[t] > st.m[t];
+  }
+  float al[2] = {1.f, 1.f}, az0[2] = {1.f, 1.f}, az1[2] = {1.f, 1.f}, am[2] = {1.f, 1.f};
+  if (__builtin_expect(__any(beat), 0)) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const float mn = fmaxf(st.m[t], row_max16(mx[t]));
+      am[t] = mn == -INFINITY ? 1.f : fexp2(st.m[t] - mn);
+      st.m[t] = mn;
+      const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am[t]), 0));
+      const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am[t]), 16));
+      const float a2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am[t]), 32));
+      const float a3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, am[t]), 48));
+      al[t] = (lane & 2) ? ((lane & 1) ? a3 : a2) : ((lane & 1) ? a1 : a0);
+      az0[t] = (lane & 1) ? a2 : a0;
+      az1[t] = (lane & 1) ? a3 : a1;
+    }
+  }
+  float pe[2][QB];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    st.l[t] *= am[t];
+    st.ot[t][0] *= al[t]; st.ot[t][1] *= al[t];
+    st.z[t][0] *= az0[t]; st.z[t][1] *= az1[t];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      pe[t][b] = fexp2(sc[t][b] - st.m[t]);
+      st.l[t] += pe[t][b];
+    }
+  }
+  // strips: row entry (group g, head of 8) of the token's run; the token's four V scale words are exchanged once
+  const int tk = lane & 15, x = lane >> 4;
+  const int sl = vslot(tk & 7);
+  uint16_t* pb = reinterpret_cast<uint16_t*>(S.pb(wave)) + (tk >> 3) * PB8_RSTRIDE * 8 + sl;
+  uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (tk >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
+  const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;
+  const int c0 = ((x) * 8 + x) * 8, c1 = ((x ^ 1) * 8 + x) * 8, c2 = ((x ^ 2) * 8 + x) * 8, c3 = ((x ^ 3) * 8 + x) * 8;
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    const uint32_t v0 = valid[b] ? (r.vs[b] & 0x7FFFu) : 0u;
+    const uint32_t v1 = lane_from(v0, 4 * (lane ^ 16)), v2 = lane_from(v0, 4 * (lane ^ 32)), v3 = lane_from(v0, 4 * (lane ^ 48));
+    const uint32_t va = (v1 << 16) | v0, vb = (v3 << 16) | v2;
+    uint16_t* row = pb + b * 2 * PB8_RSTRIDE * 8;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe[t][b], pe[t][b]));
+      const uint32_t xa = pk_mul(pp, va), xb = pk_mul(pp, vb);
+      row[c0 + 32 * t] = static_cast<uint16_t>(xa);
+      row[c1 + 32 * t] = static_cast<uint16_t>(xa >> 16);
+      row[c2 + 32 * t] = static_cast<uint16_t>(xb);
+      row[c3 + 32 * t] = static_cast<uint16_t>(xb >> 16);
+    }
+    if constexpr (QM != QM_SYM4) zb[b * 2 * ZB_RSTRIDE * 8] = static_cast<uint16_t>((r.vs[b] & ZM) << zsh);
+  }
+}
+
+template <int QM, class SM>
+DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane, int wave) {
+  // column n = lane & 15 = (group n >> 2, head n & 3 of the half); a masked entry word is multiplied with the strip
+  // rows of both halves (entries 8 g + head and 8 g + 4 + head; lanes of foreign groups read the zero pad entry)
+  const int n = lane & 15, kc = lane >> 4;
+  const uint4* rowg = reinterpret_cast<const uint4*>(S.pb(wave)) + kc * PB8_RSTRIDE;
+#pragma unroll
+  for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {            // strip group g = entries of half eh = g & 1, word pair g >> 1
+      const int eh = g & 1;
+      const uint4* src = rowg + 4 * s2 * PB8_RSTRIDE;
+      const half8 b0 = __builtin_bit_cast(half8, src[(n >> 2) == g ? 8 * g + (n & 3) : 32]);
+      const half8 b1 = __builtin_bit_cast(half8, src[(n >> 2) == g ? 8 * g + 4 + (n & 3) : 32]);
+#pragma unroll
+      for (int y = 0; y < 2; ++y) {
+        const int sub = 2 * (g >> 1) + y;
+        uint32_t x[4];
+        if constexpr (QM == QM_ASYM2) {
+          if (sub & 1) UnpackD<QM>::run_hi(r.vc[2 * s2 + eh][sub >> 1], x); else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub >> 1], x);
+        }
+        else UnpackD<QM>::run(r.vc[2 * s2 + eh][sub], x);
+        const half8 aq = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+        st.ot[0][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq, b0, st.ot[0][y], 0, 0, 0);
+        st.ot[1][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq, b1, st.ot[1][y], 0, 0, 0);
+      }
+    }
+  }
+  if constexpr (QM != QM_SYM4) {   // sum p' zero point: lane = (row group, group, head pair), both halves
+    const int rg = lane >> 3, g = (lane >> 1) & 3, hp = lane & 1;
+    const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
+    const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB8_RSTRIDE + g * 8 + 2 * hp;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const uint4 pq = pp[4 * t + e];
+        float a = st.z[t][e];
+        a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
+        st.z[t][e] = a;
+      }
+  }
+}
+
+// BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
+template <int NW>
+DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&m)[4], float (&l)[4], float (&o)[4][2]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = p.tail_len[b];
+  const int row = p.tail_idx != nullptr ? p.tail_idx[b] : b;
+  const uint16_t* base = static_cast<const uint16_t*>(p.tail) + static_cast<long long>(row) * p.tail_bs;
+  float q[4][2];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int hq = tile * 4 + h;
+    q[h][0] = q[h][1] = 0.f;
+    if (hq < p.gqa) {
+      const uint32_t raw = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
+                                                              (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 2 * lane);
+      q[h][0] = bf16_lo(raw) * p.qscale;
+      q[h][1] = bf16_hi(raw) * p.qscale;
+    }
+    m[h] = -INFINITY; l[h] = 0.f; o[h][0] = o[h][1] = 0.f;
+  }
+  for (int t = wave; t < n; t += NW) {
+    const uint16_t* tr = base + static_cast<long long>(t) * p.tail_ts;
+    const uint32_t kr = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
+    const uint32_t vr = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
+    const float k0 = bf16_lo(kr), k1 = bf16_hi(kr), v0 = bf16_lo(vr), v1 = bf16_hi(vr);
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      float s = q[h][0] * k0 + q[h][1] * k1;
+      s += dpp_xor1(s); s += dpp_xor2(s);
+      s = wave_sum_over_tokens(s);
+      const float mn = fmaxf(m[h], s);
+      const float alpha = fexp2(m[h] - mn), pe = fexp2(s - mn);
+      m[h] = mn;
+      l[h] = l[h] * alpha + pe;
+      o[h][0] = o[h][0] * alpha + pe * v0;
+      o[h][1] = o[h][1] * alpha + pe * v1;
+    }
+  }
+}
+
 }  // namespace dec
 }  // namespace fr

@@ -50,7 +50,7 @@ struct DecodeParams {
   float* opart;
   float* mlpart;
   int* counter;
-  int counter_div;         // q tiles of 4 heads that share one counter slot
+  int tile8;               // 1: a workgroup serves a tile of 8 query heads (both 4-head halves on one unpacking), 0: tiles of 4
   void* out;
   long long o_bs;
   const void* tail;
@@ -64,6 +64,7 @@ struct DecodeParams {
   int wg_waves;            // wavefronts per workgroup: 4, or the large workgroup that fills a CU
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
+int decode8_launch(int fmt, const DecodeParams& p, hipStream_t st);       // tiles of 8 query heads (decode_gqa8.hip)
 int decode_wide_launch(int fmt, const DecodeParams& p, hipStream_t st);   // head dim 256 (decode_wide.hip)
 int decode_big_chunk();                     // tokens per split from which the large workgroup is worth launching
 int decode_waves(int chunk_tokens);          // wavefronts per workgroup the launcher picks for a split of that many tokens

@@ -155,11 +155,15 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
 
 
 def plan_v2(B, Lmax, Hkv, page, nsplit=None, fmt="int4", G=4, Dh=128):
-    """(nsplit, chunk) of a static-format decode: a workgroup per (KV head, tile of 4 query heads)"""
-    tiles = Hkv * ((G + 3) // 4)
+    """(nsplit, chunk) of a static-format decode: a workgroup per (KV head, tile of 4 -- or, for GQA groups of 5 .. 8
+    heads at head dim 128, of 8 -- query heads)"""
+    tile = qtile(G, Dh)
+    tiles = Hkv * ((G + tile - 1) // tile)
     slots = _slots(fmt)
     if Dh == 256:      # workgroups of 4 wavefronts only, two resident per CU (256 registers): one round of them
         return plan_splits(B, Lmax, tiles, page, slots // 2, nsplit, ncu=0)
+    if tile == 8:      # tiles of 8 heads: three small workgroups resident per CU (two for the sign-magnitude INT4 format)
+        slots = slots * (2 if fmt == "int4" else 3) // 4
     return plan_splits(B, Lmax, tiles, page, slots, nsplit, ncu=_NUM_CU)
 
 

@@ -187,6 +187,21 @@ def test_gqa_groups(dev, G, Hkv):
 
 
 @pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
+                                      ("static", "int4a"), ("static", "int2a"), ("static", "int4")])
+def test_tiles_of_8_heads(dev, mode, fmt):
+    """GQA groups of 5 .. 8 heads: one workgroup serves all heads of a KV head on one unpacking of the pages (the
+    reference's GT = 8 kernels, kernels/csrc/attn_decode_v2g.cuh:5-10).  Ragged lengths, groups that do not fill the
+    tile (heads past the group are padding), splits with BF16 rows and a masked sink range, the large workgroup, and
+    32-token pages."""
+    run_case(dev, mode, LENS, fmt, seed=60, G=8, Hkv=2)
+    run_case(dev, mode, [700, 120, 2300], fmt, seed=61, G=7, Hkv=2, nsplit=3, win=(40, 5), kv_start=4)
+    ns, ch = run_case(dev, mode, [2300, 2100], fmt, seed=62, G=8, Hkv=1, nsplit=1)
+    assert (ns, ch) == (1, 2304)
+    run_case(dev, mode, [200, 1000, 33], fmt, seed=63, G=5, Hkv=2, P=32)
+    run_case(dev, mode, [4500, 2049], fmt, seed=64, G=6, Hkv=1, nsplit=2, win=(24, 3), P=32)
+
+
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("codebook", "konly"),
                                       ("static", "int4a"), ("static", "int2a")])
 def test_pages_of_32_tokens(dev, mode, fmt):
     """32-token pages: a quad is two pages of four 8-token runs each; ragged lengths, splits, the large workgroup,
