@@ -324,6 +324,13 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
         name = ("configs[2]: INT2 FlagRot konlya2 paged decode + static key centring + 4 sink / 128 window BF16, "
                 "Qwen3-8B GQA 32q/8kv d=128, B=64 L=16384 page=16")
     HKV, DH, G = globals()["HKV"], globals()["DH"], globals()["G"]
+    if getattr(args, "batch", 0) or getattr(args, "context", 0) or getattr(args, "window", -1) >= 0:
+        # shape overrides for experiments: not a baseline configuration
+        B, L = getattr(args, "batch", 0) or B, getattr(args, "context", 0) or L
+        if getattr(args, "window", -1) >= 0:
+            W = args.window
+            S = S if W else 0
+        name += f" [shape override: B={B} L={L} sink={S} window={W}: not a baseline configuration]"
     if getattr(args, "gqa", 4) != 4:              # not a configuration of the baseline: GQA groups of 8 (Qwen-32B's 64q/8kv) on the same pages
         G = int(args.gqa)
         name = name.replace("32q/8kv", f"{G * HKV}q/{HKV}kv") + f" [GQA {G}: not a baseline configuration]"
@@ -670,6 +677,9 @@ def main():
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
     ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="256 = the head dim 256 kernels (GQA 24q/4kv, the reference's test shape class); not a baseline configuration")
+    ap.add_argument("--batch", type=int, default=0, help="int4 / int2 workloads: another batch size (not a baseline configuration)")
+    ap.add_argument("--context", type=int, default=0, help="int4 / int2 workloads: another context length (not a baseline configuration)")
+    ap.add_argument("--window", type=int, default=-1, help="int4 / int2 workloads: BF16 window tokens (0: no BF16 rows and no sinks; not a baseline configuration)")
     ap.add_argument("--gqa", type=int, default=4, help="int4 / int2 workloads: query heads per KV head (8 = tiles of 8 heads; not a baseline configuration)")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

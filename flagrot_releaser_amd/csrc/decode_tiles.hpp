@@ -172,7 +172,9 @@ template <int QM> struct VRegs {
 };
 
 // lane offsets of the key-side loads inside a chunk (block 0 of a page; a 32-token page's second block adds constants)
-template <int QM, int P> struct KOffs { int k, ks, vs; };
+// (unsigned 32-bit lane offsets on a wave-uniform chunk address: the loads then take the chunk address from scalar
+// registers and the offset from one vector register -- no 64-bit vector additions per load)
+template <int QM, int P> struct KOffs { uint32_t k, ks, vs; };
 template <int QM, int P>
 DEVI KOffs<QM, P> key_offsets(int lane) {
   using L = Lay<QM, P>;
@@ -186,20 +188,24 @@ DEVI KOffs<QM, P> key_offsets(int lane) {
 // chunk[b]: the chunk of block b's page (wave uniform); 32-token pages: blocks 2 s, 2 s + 1 are the halves of page s
 // STREAM = false: ordinary loads, for the kernels whose q tiles of one KV head count on finding each other's lines in L2
 template <int QM, int P, bool STREAM = true>
-DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], const KOffs<QM, P>& o) {
+DEVI void load_k(KRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], const KOffs<QM, P>& o0) {
+  // (the offsets are made opaque at the point of use: hoisted out of the page loop as 64-bit values they would be added
+  // to the chunk address by vector instructions, one 64-bit addition per load)
+  KOffs<QM, P> o = o0;
+  asm volatile("" : "+v"(o.k), "+v"(o.ks), "+v"(o.vs));
 #pragma unroll
   for (int b = 0; b < QBLK<QM>; ++b) {
     const int hp = P == 32 ? (b & 1) : 0;            // second half of a 32-token page: 16 tokens further
     const uint8_t* ch = chunk[b];
     if constexpr (QM == QM_ASYM2) {
-      const u32x2 k = gload_stream<u32x2, STREAM>(ch + o.k + hp * 16 * 32);
+      const u32x2 k = gload_stream<u32x2, STREAM>(ch + static_cast<size_t>(o.k + hp * 16 * 32));
       r.kc[b][0] = k.x; r.kc[b][1] = k.y;
     } else {
-      const u32x4 k = gload_stream<u32x4, STREAM>(ch + o.k + hp * 16 * 64);
+      const u32x4 k = gload_stream<u32x4, STREAM>(ch + static_cast<size_t>(o.k + hp * 16 * 64));
       r.kc[b][0] = k.x; r.kc[b][1] = k.y; r.kc[b][2] = k.z; r.kc[b][3] = k.w;
     }
-    { const u32x2 t2 = gload_stream<u32x2, STREAM>(ch + o.ks + hp * 16 * 8); r.ks[b] = make_uint2(t2.x, t2.y); }
-    r.vs[b] = gload_stream<uint16_t, STREAM>(ch + o.vs + hp * 16 * 2);
+    { const u32x2 t2 = gload_stream<u32x2, STREAM>(ch + static_cast<size_t>(o.ks + hp * 16 * 8)); r.ks[b] = make_uint2(t2.x, t2.y); }
+    r.vs[b] = gload_stream<uint16_t, STREAM>(ch + static_cast<size_t>(o.vs + hp * 16 * 2));
   }
 }
 
@@ -783,22 +789,46 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&
     }
     m[h] = -INFINITY; l[h] = 0.f; o[h][0] = o[h][1] = 0.f;
   }
-  for (int t = wave; t < n; t += NW) {
-    const uint16_t* tr = base + static_cast<long long>(t) * p.tail_ts;
-    const uint32_t kr = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
-    const uint32_t vr = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
-    const float k0 = bf16_lo(kr), k1 = bf16_hi(kr), v0 = bf16_lo(vr), v1 = bf16_hi(vr);
+  // TR rows per wavefront and step: their loads go out together and their 4 x TR reductions interleave (a row at a time
+  // is one memory latency and one chain of cross-lane steps per row)
+  constexpr int TR = 4;
+  for (int t0 = wave * TR; t0 < n; t0 += NW * TR) {
+    uint32_t kr[TR], vr[TR];
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      float s = q[h][0] * k0 + q[h][1] * k1;
-      s += dpp_xor1(s); s += dpp_xor2(s);
-      s = wave_sum_over_tokens(s);
-      const float mn = fmaxf(m[h], s);
-      const float alpha = fexp2(m[h] - mn), pe = fexp2(s - mn);
-      m[h] = mn;
-      l[h] = l[h] * alpha + pe;
-      o[h][0] = o[h][0] * alpha + pe * v0;
-      o[h][1] = o[h][1] * alpha + pe * v1;
+    for (int r = 0; r < TR; ++r) {
+      const uint16_t* tr = base + static_cast<long long>(min(t0 + r, n - 1)) * p.tail_ts;
+      kr[r] = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
+      vr[r] = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
+    }
+    float s[TR][4];
+#pragma unroll
+    for (int r = 0; r < TR; ++r) {
+      const float k0 = bf16_lo(kr[r]), k1 = bf16_hi(kr[r]);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        float a = q[h][0] * k0 + q[h][1] * k1;
+        a += dpp_xor1(a); a += dpp_xor2(a);
+        s[r][h] = a;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < TR; ++r)
+#pragma unroll
+      for (int h = 0; h < 4; ++h) s[r][h] = wave_sum_over_tokens(s[r][h]);
+#pragma unroll
+    for (int r = 0; r < TR; ++r) {
+      const bool in = t0 + r < n;
+      const float v0 = bf16_lo(vr[r]), v1 = bf16_hi(vr[r]);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const float sc = in ? s[r][h] : -INFINITY;
+        const float mn = fmaxf(m[h], sc);
+        const float alpha = mn == -INFINITY ? 1.f : fexp2(m[h] - mn), pe = mn == -INFINITY ? 0.f : fexp2(sc - mn);
+        m[h] = mn;
+        l[h] = l[h] * alpha + pe;
+        o[h][0] = o[h][0] * alpha + pe * v0;
+        o[h][1] = o[h][1] * alpha + pe * v1;
+      }
     }
   }
 }
