@@ -282,10 +282,11 @@ DEVI void whole_head_flags(const KRegs<QM>& r, int lane, bool (&full)[QBLK<QM>])
     // union over the four lanes names it
     full[b] = false;
     if constexpr (K2) {
-      uint32_t f = r.vs[b] & 0x8000u;
-      f |= lane_from(f, 4 * (lane ^ 16));
-      f |= lane_from(f, 4 * (lane ^ 32));
-      full[b] = f != 0u;
+      // as a lane mask in scalar registers: the four lanes of token t are bits t, t + 16, t + 32, t + 48 -- folded onto
+      // 16 bits and spread again by scalar instructions, no lane exchange and no vector work beyond the bit test
+      unsigned long long m = __builtin_amdgcn_ballot_w64((r.vs[b] & 0x8000u) != 0u);
+      m |= m >> 32; m |= m >> 16; m &= 0xFFFFull; m |= m << 16; m |= m << 32;
+      full[b] = __builtin_amdgcn_inverse_ballot_w64(m);
     }
   }
 }
