@@ -33,13 +33,28 @@ __global__ void __launch_bounds__(64 * PROBE_WAVES) k_probe_mfma(int iters, uint
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
   const uint4* row = &tile[wave][lane];
-  for (int it = 0; it < iters; ++it) {
-    if constexpr (MODE == 1) asm volatile("" : "+v"(row));      // the reads stay inside the loop
+  if constexpr (MODE == 0) {
+    for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int k = 0; k < PROBE_CHAINS; ++k) {
-      half8 x = a;
-      if constexpr (MODE == 1) x = __builtin_bit_cast(half8, row[k * 64]);
-      acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, b, acc[k], 0, 0, 0);
+      for (int k = 0; k < PROBE_CHAINS; ++k) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[k], 0, 0, 0);
+    }
+  } else {
+    // software-pipelined as a real kernel would be: the operands of step it + 1 are requested before the products of
+    // step it are issued, so that what is measured is the LDS feed and not the latency of one read
+    half8 x[PROBE_CHAINS], y[PROBE_CHAINS];
+#pragma unroll
+    for (int k = 0; k < PROBE_CHAINS; ++k) x[k] = __builtin_bit_cast(half8, row[k * 64]);
+    for (int it = 0; it < iters; it += 2) {
+      asm volatile("" : "+v"(row));      // the reads stay inside the loop
+#pragma unroll
+      for (int k = 0; k < PROBE_CHAINS; ++k) y[k] = __builtin_bit_cast(half8, row[k * 64]);
+#pragma unroll
+      for (int k = 0; k < PROBE_CHAINS; ++k) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[k], b, acc[k], 0, 0, 0);
+      asm volatile("" : "+v"(row));
+#pragma unroll
+      for (int k = 0; k < PROBE_CHAINS; ++k) x[k] = __builtin_bit_cast(half8, row[k * 64]);
+#pragma unroll
+      for (int k = 0; k < PROBE_CHAINS; ++k) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(y[k], b, acc[k], 0, 0, 0);
     }
   }
   float s = 0.f;
@@ -55,11 +70,13 @@ __global__ void __launch_bounds__(64 * PROBE_WAVES) k_probe_mfma(int iters, uint
 extern "C" {
 
 long long fr_probe_mfma_flops(int iters, int workgroups) {
+  iters += iters & 1;
   return 2LL * 32 * 32 * 16 * PROBE_CHAINS * PROBE_WAVES * static_cast<long long>(iters) * workgroups;
 }
 
 int fr_probe_mfma(int mode, int iters, int workgroups, uint32_t* sink, void* stream) {
   if (iters <= 0 || workgroups <= 0) return 0;
+  iters += iters & 1;      // mode 1 works through the steps in pairs
   if (mode != 0 && mode != 1) return -2;
   if (mode == 0) hipLaunchKernelGGL(k_probe_mfma<0>, dim3(workgroups), dim3(64 * PROBE_WAVES), 0, static_cast<hipStream_t>(stream), iters, sink);
   else hipLaunchKernelGGL(k_probe_mfma<1>, dim3(workgroups), dim3(64 * PROBE_WAVES), 0, static_cast<hipStream_t>(stream), iters, sink);

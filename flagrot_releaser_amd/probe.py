@@ -30,4 +30,4 @@ def read_pages(pool, block_table, seq_lens, sink, page=16):
 def mfma_burst(mode: int, iters: int, workgroups: int, sink):
     """launches the matrix-pipe probe (mode 0: register operands, 1: one LDS operand per instruction); returns its flops"""
     NATIVE.run("fr_probe_mfma", mode, iters, workgroups, sink, current_stream())
-    return 2 * 32 * 32 * 16 * 4 * 8 * iters * workgroups
+    return 2 * 32 * 32 * 16 * 4 * 8 * (iters + (iters & 1)) * workgroups
