@@ -28,7 +28,7 @@ int fr_abi_version(void);
  * nsplit counts the body splits; with a tail the workspace must hold B*Hkv*ceil(gqa/GT)*(nsplit+1) partials of
  * GT*128 floats (GT = 8 when variant has bits 1024|2048, else 4); counter int32 [B*Hkv*ceil(gqa/GT)] zeroed once by the
  * caller (merge tickets and, when the body workgroups of a sequence share its page range, their page draws; the last
- * arriving workgroup leaves the word at 0).  If B*Hkv*ceil(gqa/4)*nsplit fits the CUs and chunk >= 1024, split s owns
+ * arriving workgroup leaves the word at 0).  If B*Hkv*ceil(gqa/GT)*nsplit fits the CUs and chunk >= 1024, split s owns
  * tokens [s, s+1)*chunk and one large workgroup per CU runs it; otherwise nsplit only counts the workgroups per
  * (sequence, KV head, q tile); nsplit*chunk must cover the longest sequence either way.
  * variant bit 4096 (kernels/csrc/attn_decode_v2g.cuh:11-25, 276): head dim 256 -- q, out and tail rows have 256 channels,
