@@ -382,6 +382,8 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
     for plan in plans:
         if plan == "own":
             ns, ch = K.plan_cb(B, Lpages, HKV, P, kind, nsplit=args.nsplit or None, G=G, Dh=DH)
+            if getattr(args, "chunk", 0):
+                ns, ch = math.ceil(Lpages / args.chunk), args.chunk
         else:      # "reference": the reference front end's cost model fed with this library's occupancy answer
             occ = K.lib().fr_cb_occupancy(K.CB_KINDS[kind], 0, K.STAGES, P)
             ns, ch = reference_plan(B, Lpages, HKV, max(1, occ) * cus)
@@ -403,7 +405,7 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
         out.zero_()
         step(0)
         torch.cuda.synchronize()
-        rows = sorted({0, B // 2 + 1, B - 1})
+        rows = sorted({0, min(B // 2 + 1, B - 1), B - 1})   # every index < B, also for a batch override of 1 or 2
         idx = bt[rows].long().reshape(-1)
         mp = pools[0].index_select(0, idx).cpu().numpy()
         mbt = np.arange(idx.numel(), dtype=np.int32).reshape(len(rows), -1)
@@ -714,6 +716,7 @@ def main():
     ap.add_argument("--window", type=int, default=-1, help="int4 / int2 workloads: BF16 window tokens (0: no BF16 rows and no sinks; not a baseline configuration)")
     ap.add_argument("--gqa", type=int, default=4, help="int4 / int2 workloads: query heads per KV head (8 = tiles of 8 heads; not a baseline configuration)")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
+    ap.add_argument("--chunk", type=int, default=0, help="int4 / int2 workloads: tokens per split, overriding the planner (experiments)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", action="store_true", help="the chosen workload only (no extra legs)")
     args = ap.parse_args()

@@ -392,22 +392,32 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
     for (int ps = 0; ps < 2; ++ps) {
       // value strips: lane = (token l32, half hh) serves sub-vectors 2 hh, 2 hh + 1 of the pass.  Scale and min go to the
       // strip of the token's class (0 in the other two; tokens outside the range have no class), the code bytes to byte rows.
+      // Passes that hold a value scale above WIDE_SCALE (wave uniform) keep their scales times 2^-8 in the strips and
+      // run a second set of value products (below, where the reason is given).
+      bool wide_scales;
       {
         const int pos = gi * 32 + l32;
         const bool vF = cur.vf != 0;
+        uint32_t w2[2];                                  // fp16 scale (bit 15 = H32) | fp16 min << 16 of sub-vectors 2 hh, 2 hh + 1 of the pass
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
-          uint32_t w;                                    // fp16 scale (bit 15 = H32) | fp16 min << 16
           if (F8) {
             const uint32_t b2 = jj ? cur.vm[ps].x >> 16 : cur.vm[ps].x;                // s8 | m8 << 8
-            w = pk_mul(((b2 & 0x7Fu) << 7) | ((b2 & 0x7F00u) << 15) | ((b2 & 0x8000u) << 16), X256) | ((b2 & 0x80u) << 8);
-          } else w = jj ? cur.vm[ps].y : cur.vm[ps].x;
+            w2[jj] = pk_mul(((b2 & 0x7Fu) << 7) | ((b2 & 0x7F00u) << 15) | ((b2 & 0x8000u) << 16), X256) | ((b2 & 0x80u) << 8);
+          } else w2[jj] = jj ? cur.vm[ps].y : cur.vm[ps].x;
+        }
+        wide_scales = __any(max(w2[0] & 0x7FFFu, w2[1] & 0x7FFFu) > WIDE_SCALE);
+        const uint32_t sfold = wide_scales ? 0x1C00u : 0x3C00u;                          // fp16 2^-8 or 1
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const uint32_t w = w2[jj];
           const int j = 2 * hh + jj;
           int cls = vF ? 2 : static_cast<int>((w >> 15) & 1u);
           if (!full) cls = (pos >= t0 && pos < t1) ? cls : 3;
+          const uint16_t sc16 = static_cast<uint16_t>(pk_mul(w & 0x7FFFu, sfold));
 #pragma unroll
           for (int c = 0; c < 3; ++c) {
-            W.vsm[c][32 * j + l32] = cls == c ? static_cast<uint16_t>(w & 0x7FFFu) : static_cast<uint16_t>(0);
+            W.vsm[c][32 * j + l32] = cls == c ? sc16 : static_cast<uint16_t>(0);
             W.vmm[c][32 * j + l32] = cls == c ? static_cast<uint16_t>(w >> 16) : static_cast<uint16_t>(0);
           }
           const uint32_t c0 = jj ? cur.vc[ps].z : cur.vc[ps].x, c1 = jj ? cur.vc[ps].w : cur.vc[ps].y;
@@ -437,6 +447,37 @@ __global__ void __launch_bounds__(256, 2) k_attn_pages256(const uint16_t* __rest
           const u32x4 bo = u32x4{pk_mul(pr.x, sv.x), pk_mul(pr.y, sv.y), pk_mul(pr.z, sv.z), pk_mul(pr.w, sv.w)};
           const u32x4 ao = u32x4{by.x & vmask, by.y & vmask, by.z & vmask, by.w & vmask};
           accv[4 * ps + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, ao), __builtin_bit_cast(half8, bo), accv[4 * ps + j], 0, 0, 0);
+        }
+      }
+      // The matrix pipe aligns the addends of an instruction to the largest NOMINAL exponent (a denormal code operand
+      // counts as 2^-14) and keeps 24 bits from there; a token whose p * scale is hundreds of times its neighbours'
+      // lifts that window for all of them and for the accumulator.  In such passes the strips hold scale * 2^-8: the
+      // products above came to 1/256 of their value, the other 255/256 follow here with the code operands times 255
+      // (exact), and what the fp16 rounding of p * scale dropped with the code operands times 256.
+      if (__builtin_expect(wide_scales, 0)) {
+        // (read again through an offset the compiler cannot see through: recognised as the reads of the products
+        // above, they would keep every operand of those in registers until here)
+        int again = 0;
+        asm volatile("" : "+s"(again));
+        constexpr uint32_t X255 = 0x5BF85BF8u;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const int tk = 16 * s + 8 * hh + again;
+          const u32x4 pr = *reinterpret_cast<const u32x4*>(&W.pst[vh][tk]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x4 sv = *reinterpret_cast<const u32x4*>(&W.vsm[vcl][32 * j + tk]);
+            const u32x4 by = *reinterpret_cast<const u32x4*>(&W.vt[j][(l32 >> 2) * PROW + tk]);
+            const u32x4 bo = u32x4{pk_mul(pr.x, sv.x), pk_mul(pr.y, sv.y), pk_mul(pr.z, sv.z), pk_mul(pr.w, sv.w)};
+            const u32x4 br = u32x4{pk_fma(pr.x, sv.x, bo.x ^ 0x80008000u), pk_fma(pr.y, sv.y, bo.y ^ 0x80008000u),
+                                   pk_fma(pr.z, sv.z, bo.z ^ 0x80008000u), pk_fma(pr.w, sv.w, bo.w ^ 0x80008000u)};
+            const u32x4 ao = u32x4{by.x & vmask, by.y & vmask, by.z & vmask, by.w & vmask};
+            const u32x4 a255 = u32x4{pk_mul(ao.x, X255), pk_mul(ao.y, X255), pk_mul(ao.z, X255), pk_mul(ao.w, X255)};
+            const u32x4 a256 = u32x4{pk_mul(ao.x, X256), pk_mul(ao.y, X256), pk_mul(ao.z, X256), pk_mul(ao.w, X256)};
+            accv[4 * ps + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a255), __builtin_bit_cast(half8, bo), accv[4 * ps + j], 0, 0, 0);
+            accv[4 * ps + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a256), __builtin_bit_cast(half8, br), accv[4 * ps + j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);      // one step's operands at a time: this path is rare and must not claim registers
+          }
         }
       }
       wave_lds_sync();

@@ -37,6 +37,10 @@ template <class T> DEVI T gload(const uint8_t* p) {
   return __builtin_nontemporal_load((gp)(p));
 }
 constexpr uint32_t X256 = 0x5C005C00u;                                         // fp16 pair (256, 256)
+// fp16 pattern of the value scale (8.0) above which a 32-token group takes the rescaled form of its value products: up
+// to there the plain form loses at most 2^-13 * 8 = 1e-3 of a token's weight per instruction, which is what the rescaled
+// form leaves at a scale of 700 (unit-variance data has scales around 1.4 and reaches 2.5 in a few per cent of the groups)
+constexpr uint32_t WIDE_SCALE = 0x4800u;
 constexpr int GT = 8;                           // query heads per workgroup (a whole GQA group of up to 8)
 constexpr int QROW = 68;                        // words per row of the query strips and tables: 64 + 4 pad (conflict-free 128-bit rows)
 constexpr int PROW = 40;                        // fp16 per row of the p and code-byte strips: 32 + 8 pad

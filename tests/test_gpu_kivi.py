@@ -7,7 +7,12 @@ Bars:
              mismatches, integrations/vllm_flagrot/tests/test_kivi.py:139-140); `ident` and `fix` modes are bit-pinned
              on the whole pool;
   attention  |out - ref| <= 1e-2 max|ref| against fp64 attention over the oracle's dequantised pages + BF16 tail
-             (the reference's bar, tests/test_kivi.py:243);
+             (the reference's bar, tests/test_kivi.py:243), and element-wise |out - ref| <= 2e-3 + 1e-2 |ref| on the
+             committed cases.  Every sequence of 8 tokens or more holds a row scaled x200 next to ordinary rows: where
+             that row takes the softmax weight and the exact output is near zero, what decides is the 24-bit window of
+             the matrix pipe's accumulation (about 1e-3 absolute on accumulators of 2000); the x200 cases at the end
+             are held to three times the element-wise bar (randomised shapes reach 2.5; 16 before the value products
+             of such groups were rescaled);
   dequant    fp32 within 2e-6 max|ref| of the fp64 oracle; bf16 = round of it within one ulp;
   lse_merge  bf16 patterns equal to the oracle's, up to one ulp on at most 0.1 % (library exp).
 Every page test runs on both meta formats: FP16 scale / min (1552-byte chunks) and FP8 E4M3 (1280-byte chunks, codes
@@ -309,6 +314,16 @@ CASES = [
     ([2049, 2047], 2, 8, 1, None, [1, 127]),
     ([65, 64, 63], 3, 1, 33, (1, 256), [0, 0, 0]),
 ]
+# shapes on which randomised runs had the x200 row's weight meet near-zero outputs (5 to 15 times the element-wise bar
+# before the value products of groups with large scales were rescaled): held to 3 times the bar
+X200_CASES = [
+    ([96, 97, 32], 4, 8, 0, (1, 256), [64, 0, 0]),
+    ([200, 64, 333, 96], 2, 4, 0, (7, 256), [9, 128, 64, 64]),
+    ([97], 4, 8, 0, (3, 256), [1]),
+    ([1000, 64, 32], 4, 6, 0, (2, 512), [64, 127, 9]),
+]
+N_PLAIN = len(CASES)
+CASES = CASES + X200_CASES
 
 
 @F8
@@ -354,6 +369,7 @@ def test_attn_against_fp64(dev, case, f8):
             assert err.max() <= tol, (case, rep, b, err.max(), tol)
     print(f"\ncase {case} f8={f8}: worst max |err| / max |ref| = {worst_mx:.2e} (bar 1e-2); element-wise "
           f"|err| / (2e-3 + 1e-2 |ref|) = {worst_el:.2f} (the data holds rows scaled x200 and x1e-4)", flush=True)
+    assert worst_el <= (1.0 if case < N_PLAIN else 3.0), (case, f8, worst_el)
     assert (outbuf[:, Hq * D:] == 7.0).all()
 
 
