@@ -28,6 +28,7 @@
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
 #include "kivi_quant.hpp"
+#include "kivi_vrow.hpp"
 
 namespace frkv {
 using namespace fr;
@@ -64,164 +65,62 @@ template <bool F8> DEVI bool value_whole(const uint8_t* chunk, int cell) {
 }
 
 // ------------------------------------------------------------------------------------------------ value writer
-// WMAT: the selection weighs the error vectors by a full matrix per head (e^T M e; kivi.cu:213-287) as the 128-d
-// writer's matrix form does: the diagonal 32-block for a sub-vector's choice, all of M for the whole-head candidate and
-// for the combination.  The three error vectors of a row sit in an LDS strip per half wave; a lane forms the products
-// of its eight rows of M.
+// Half wave per (token, KV head), the row as two halves of 128 channels: the three trials, the picks, the stores
+// (kivi_vrow.hpp has the per-row work).  WMAT: picks by a full 256 x 256 matrix per head (kivi.cu:213-287) through an
+// LDS strip per half wave; `vfix` bits 0..7: H32 per sub-vector, bit 16: whole head.
 template <bool F8, bool WMAT>
 __global__ void __launch_bounds__(256) k_v_write256(const uint16_t* __restrict__ kv, long long kv_rs, int n, int Hkv,
                                                     const long long* __restrict__ slots, const float* __restrict__ co,
                                                     const float* __restrict__ M, uint8_t* __restrict__ pool, int ident,
                                                     const int* __restrict__ vfix) {
-  constexpr int EW = WMAT ? D2 : 1;                       // the strips exist only in the matrix-weighted kernel
-  __shared__ float esh[WMAT ? 8 : 1][3][EW];
+  __shared__ float strips[WMAT ? 8 : 1][WMAT ? 3 * D2 : 1];
   const int l32 = threadIdx.x & 31;
   const long long item = static_cast<long long>(blockIdx.x) * 8 + (threadIdx.x >> 5);
   if (item >= static_cast<long long>(n) * Hkv) return;
   const int t = static_cast<int>(item / Hkv), h = static_cast<int>(item % Hkv);
   const long long slot = slots[t];
   if (slot < 0) return;
-  float x[2][4], cw[2][4];
+  float x[2][4];
   load_row(kv + static_cast<long long>(t) * kv_rs + static_cast<long long>(Hkv + h) * D2, l32, x);
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const float4 c4 = *reinterpret_cast<const float4*>(co + h * D2 + 128 * s + 4 * l32);
-    cw[s][0] = c4.x; cw[s][1] = c4.y; cw[s][2] = c4.z; cw[s][3] = c4.w;
-  }
-  float sc[3][2], mnv[3][2], err[3][2], dv[3][2][4];
-  int code[3][2][4];
-#pragma unroll
-  for (int c = 0; c < 3; ++c) {
-    float y[2][4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) y[s][i] = x[s][i];
-    if (c == 1) to_basis2<1>(y, l32);
-    if (c == 2) to_basis2<2>(y, l32);
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      float mn = fminf(fminf(y[s][0], y[s][1]), fminf(y[s][2], y[s][3])), mx = fmaxf(fmaxf(y[s][0], y[s][1]), fmaxf(y[s][2], y[s][3]));
-      mn = gmin8(mn); mx = gmax8(mx);
-      float sv = kv_scale(mn, mx);
-      kv_params<F8>(mn, sv);
-      sc[c][s] = sv; mnv[c][s] = mn;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) { code[c][s][i] = kv_code(y[s][i], mn, sv); y[s][i] = kv_rec(code[c][s][i], mn, sv); }
-    }
-    if (c == 1) to_basis2<1>(y, l32);
-    if (c == 2) to_basis2<2>(y, l32);
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      float e = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) { const float d = y[s][i] - x[s][i]; dv[c][s][i] = d; e += d * d * cw[s][i]; }
-      err[c][s] = e;
-    }
-  }
+  vrow::Trial<2> tr[3];
+  vrow::trial_in_basis<2, vrow::AS_STORED, F8>(x, l32, tr[0]);
+  vrow::trial_in_basis<2, vrow::BLOCK32, F8>(x, l32, tr[1]);
+  vrow::trial_in_basis<2, vrow::WHOLE, F8>(x, l32, tr[2]);
   const int j = l32 >> 3;
-  bool useH0, useH1, useF;
-  if (ident) { useH0 = useH1 = useF = false; }
-  else if (vfix != nullptr) { useF = (vfix[h] >> 16) & 1; useH0 = (vfix[h] >> j) & 1; useH1 = (vfix[h] >> (4 + j)) & 1; }
-  else if constexpr (WMAT) {
-    float (*E)[EW] = esh[threadIdx.x >> 5];
-    const float* Mh = M + static_cast<long long>(h) * D2 * D2;
-#pragma unroll
-    for (int c = 0; c < 3; ++c)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) E[c][128 * s + 4 * l32 + i] = dv[c][s][i];
-    wave_lds_sync();
-    float eI[2] = {0.f, 0.f}, eH[2] = {0.f, 0.f}, eF = 0.f;
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
-        const int k0 = 128 * s + 32 * j;
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-        // (the sums keep their order; unrolled whole, the 256-term loops spilled some 400 registers)
-#pragma unroll 8
-        for (int k = k0; k < k0 + 32; ++k) { const float m = row[k]; a0 += m * E[0][k]; a1 += m * E[1][k]; }
-#pragma unroll 8
-        for (int k = 0; k < D2; ++k) a2 += row[k] * E[2][k];
-        eI[s] += dv[0][s][i] * a0; eH[s] += dv[1][s][i] * a1; eF += dv[2][s][i] * a2;
-      }
+  vrow::Picks pk{0u, false};
+  if (ident) {
+  } else if (vfix != nullptr) {
+    pk.whole = (vfix[h] >> 16) & 1;
+    pk.block32 = ((vfix[h] >> j) & 1u) | (((vfix[h] >> (4 + j)) & 1u) << 1);
+  } else if constexpr (WMAT) {
+    pk = vrow::pick_matrix<2>(tr, M + static_cast<long long>(h) * D2 * D2, strips[threadIdx.x >> 5], l32);
+  } else {
+    float w[2][4];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      eI[s] += hx(eI[s], 1); eI[s] += hx(eI[s], 2); eI[s] += hx(eI[s], 4);
-      eH[s] += hx(eH[s], 1); eH[s] += hx(eH[s], 2); eH[s] += hx(eH[s], 4);
+      const float4 c4 = *reinterpret_cast<const float4*>(co + h * D2 + 128 * s + 4 * l32);
+      w[s][0] = c4.x; w[s][1] = c4.y; w[s][2] = c4.z; w[s][3] = c4.w;
     }
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
-    useH0 = eH[0] < eI[0]; useH1 = eH[1] < eI[1];          // identity on ties
-    wave_lds_sync();                                       // every lane has read the strips
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-      if (s ? useH1 : useH0)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) E[0][128 * s + 4 * l32 + i] = dv[1][s][i];
-    wave_lds_sync();
-    float eB = 0.f;
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float* row = Mh + static_cast<long long>(128 * s + 4 * l32 + i) * D2;
-        float a = 0.f;
-#pragma unroll 8
-        for (int k = 0; k < D2; ++k) a += row[k] * E[0][k];
-        eB += ((s ? useH1 : useH0) ? dv[1][s][i] : dv[0][s][i]) * a;
-      }
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
-    useF = eF < eB;                                        // base on ties
-  } else {
-    float eI0 = err[0][0], eI1 = err[0][1], eH0 = err[1][0], eH1 = err[1][1], eF = err[2][0] + err[2][1];
-    eI0 += hx(eI0, 1); eI0 += hx(eI0, 2); eI0 += hx(eI0, 4);
-    eI1 += hx(eI1, 1); eI1 += hx(eI1, 2); eI1 += hx(eI1, 4);
-    eH0 += hx(eH0, 1); eH0 += hx(eH0, 2); eH0 += hx(eH0, 4);
-    eH1 += hx(eH1, 1); eH1 += hx(eH1, 2); eH1 += hx(eH1, 4);
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
-    useH0 = eH0 < eI0; useH1 = eH1 < eI1;                  // identity on ties
-    float eB = (l32 & 7) == 0 ? (useH0 ? eH0 : eI0) + (useH1 ? eH1 : eI1) : 0.f;
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
-    useF = eF < eB;                                        // base on ties
+    pk = vrow::pick_diagonal<2>(tr, w, l32);
   }
   uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * CHUNK2<F8>;
   const int off = static_cast<int>(slot % 16);
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    const int cand = useF ? 2 : ((s ? useH1 : useH0) ? 1 : 0);
-    uint32_t byte = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int cd = cand == 0 ? code[0][s][i] : cand == 1 ? code[1][s][i] : code[2][s][i];
-      byte |= static_cast<uint32_t>(cd & 3) << (2 * i);
-    }
-    chunk[VC2<F8> + off * 64 + 32 * s + l32] = static_cast<uint8_t>(byte);
+    const int basis = vrow::basis_of<2>(pk, s);
+    chunk[VC2<F8> + off * 64 + 32 * s + l32] = static_cast<uint8_t>(vrow::chosen_byte<2>(tr, basis, s));
     if ((l32 & 7) == 0) {
-      const float sv = cand == 0 ? sc[0][s] : cand == 1 ? sc[1][s] : sc[2][s];
-      const float m0 = cand == 0 ? mnv[0][s] : cand == 1 ? mnv[1][s] : mnv[2][s];
+      const uint32_t meta = vrow::chosen_meta<2, F8>(tr, basis, s);
       const int jj = 4 * s + j;
-      if (F8) {
-        const uint32_t sb = e4m3_bits(sv) | (cand == 1 ? 0x80u : 0u);
-        *reinterpret_cast<uint16_t*>(chunk + VM2<true> + off * 16 + 2 * jj) = static_cast<uint16_t>(sb | (e4m3_bits(m0) << 8));
-      } else {
-        uint32_t sb = f16_bits_rn(sv) & 0x7FFFu;
-        if (cand == 1) sb |= 0x8000u;
-        *reinterpret_cast<uint32_t*>(chunk + VM2<false> + off * 32 + 4 * jj) = sb | (f16_bits_rn(m0) << 16);
-      }
+      if (F8) *reinterpret_cast<uint16_t*>(chunk + VM2<true> + off * 16 + 2 * jj) = static_cast<uint16_t>(meta);
+      else *reinterpret_cast<uint32_t*>(chunk + VM2<false> + off * 32 + 4 * jj) = meta;
     }
   }
   if (l32 == 0) {
     if (F8) {                                              // bit 7 of the key scale byte in slot 7 of this token's cell
       uint8_t* kb = chunk + KM2 + off * 16 + 14;
-      *kb = static_cast<uint8_t>((*kb & 0x7Fu) | (useF ? 0x80u : 0u));
-    } else chunk[VF2 + off] = useF ? 1 : 0;
+      *kb = static_cast<uint8_t>((*kb & 0x7Fu) | (pk.whole ? 0x80u : 0u));
+    } else chunk[VF2 + off] = pk.whole ? 1 : 0;
   }
 }
 

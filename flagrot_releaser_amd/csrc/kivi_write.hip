@@ -19,6 +19,7 @@
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
 #include "kivi_quant.hpp"
+#include "kivi_vrow.hpp"
 
 namespace frkv {
 using namespace fr;
@@ -27,23 +28,18 @@ namespace {
 template <bool F8> constexpr long long CHUNK = F8 ? 1280 : 1552;
 template <bool F8> constexpr int VC_AT = F8 ? 640 : 768;
 template <bool F8> constexpr int VM_AT = F8 ? 1152 : 1280;
-template <int C> DEVI void to_basis(float (&y)[4], int l32) {   // candidate 0 identity, 1 H32, 2 H128
-  if (C == 1) fwht<32>(y, l32);
-  if (C == 2) fwht<128>(y, l32);
-}
 
 // ------------------------------------------------------------------------------------------------ value writer
-// WMAT: the selection weighs the reconstruction error e (original basis) by a full matrix per head, e^T M e, instead of
-// the diagonal sum co . e^2 (kivi.cu:213-287): per sub-vector only the diagonal 32-block of M counts, the whole-head
-// candidate and the combination of the chosen sub-vector candidates use all of M.  The error vectors of a row sit in
-// LDS (one strip per half wave) and every lane forms the products of its four rows of M.
+// Half wave per (token, KV head): the three trials, the picks, the stores (kivi_vrow.hpp has the per-row work; the
+// kernel loads the row and knows where the chunk keeps what).  WMAT: the picks weigh the miss vectors by a full matrix
+// per head (kivi.cu:213-287) and need an LDS strip per half wave; `ident` stores the row as it is, `vfix` takes the
+// picks from a word per head (bits 0..3: H32 per sub-vector, bit 16: whole head).
 template <bool F8, bool WMAT>
 __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv, long long kv_rs, int n, int Hkv,
                                                  const long long* __restrict__ slots, const float* __restrict__ co,
                                                  const float* __restrict__ M, uint8_t* __restrict__ pool, int ident,
                                                  const int* __restrict__ vfix) {
-  constexpr int EW = WMAT ? 128 : 1;                    // the strips exist only in the matrix-weighted kernel
-  __shared__ float esh[WMAT ? 8 : 1][3][EW];
+  __shared__ float strips[WMAT ? 8 : 1][WMAT ? 3 * 128 : 1];
   const int l32 = threadIdx.x & 31;
   const long long item = static_cast<long long>(blockIdx.x) * 8 + (threadIdx.x >> 5);
   if (item >= static_cast<long long>(n) * Hkv) return;
@@ -51,105 +47,38 @@ __global__ void __launch_bounds__(256) k_v_write(const uint16_t* __restrict__ kv
   const long long slot = slots[t];
   if (slot < 0) return;
   const uint2 raw = *reinterpret_cast<const uint2*>(kv + static_cast<long long>(t) * kv_rs + (Hkv + h) * 128 + 4 * l32);
-  const float x[4] = {bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)};
-  const float4 cw = *reinterpret_cast<const float4*>(co + h * 128 + 4 * l32);
-  const float cwv[4] = {cw.x, cw.y, cw.z, cw.w};
-  float sc[3], mnv[3], err[3], dv[3][4];
-  int code[3][4];
-#pragma unroll
-  for (int c = 0; c < 3; ++c) {
-    float y[4] = {x[0], x[1], x[2], x[3]};
-    if (c == 1) fwht<32>(y, l32);
-    if (c == 2) fwht<128>(y, l32);
-    float mn = fminf(fminf(y[0], y[1]), fminf(y[2], y[3])), mx = fmaxf(fmaxf(y[0], y[1]), fmaxf(y[2], y[3]));
-    mn = gmin8(mn); mx = gmax8(mx);
-    float s = kv_scale(mn, mx);
-    kv_params<F8>(mn, s);
-    sc[c] = s; mnv[c] = mn;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { code[c][i] = kv_code(y[i], mn, s); y[i] = kv_rec(code[c][i], mn, s); }
-    if (c == 1) fwht<32>(y, l32);
-    if (c == 2) fwht<128>(y, l32);
-    float e = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { const float d = y[i] - x[i]; dv[c][i] = d; e += d * d * cwv[i]; }
-    err[c] = e;
-  }
+  const float x[1][4] = {{bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)}};
+  vrow::Trial<1> tr[3];
+  vrow::trial_in_basis<1, vrow::AS_STORED, F8>(x, l32, tr[0]);
+  vrow::trial_in_basis<1, vrow::BLOCK32, F8>(x, l32, tr[1]);
+  vrow::trial_in_basis<1, vrow::WHOLE, F8>(x, l32, tr[2]);
   const int j = l32 >> 3;
-  bool useH, useF;
-  if (ident) { useH = false; useF = false; }
-  else if (vfix != nullptr) { useF = (vfix[h] >> 16) & 1; useH = (vfix[h] >> j) & 1; }
-  else if constexpr (WMAT) {
-    float (*E)[EW] = esh[threadIdx.x >> 5];
-    const float* Mh = M + static_cast<long long>(h) * 128 * 128;
-#pragma unroll
-    for (int c = 0; c < 3; ++c)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) E[c][4 * l32 + i] = dv[c][i];
-    wave_lds_sync();
-    float eI = 0.f, eH = 0.f, eF = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float* row = Mh + (4 * l32 + i) * 128;
-      float a0 = 0.f, a1 = 0.f, a2 = 0.f;
-      for (int k = 32 * j; k < 32 * j + 32; ++k) { const float m = row[k]; a0 += m * E[0][k]; a1 += m * E[1][k]; }
-      for (int k = 0; k < 128; ++k) a2 += row[k] * E[2][k];
-      eI += dv[0][i] * a0; eH += dv[1][i] * a1; eF += dv[2][i] * a2;
-    }
-    eI += hx(eI, 1); eI += hx(eI, 2); eI += hx(eI, 4);
-    eH += hx(eH, 1); eH += hx(eH, 2); eH += hx(eH, 4);
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
-    useH = eH < eI;                                      // identity on ties
-    wave_lds_sync();                                     // every lane has read the strips
-    if (useH)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) E[0][4 * l32 + i] = dv[1][i];
-    wave_lds_sync();
-    float eB = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float* row = Mh + (4 * l32 + i) * 128;
-      float a = 0.f;
-      for (int k = 0; k < 128; ++k) a += row[k] * E[0][k];
-      eB += (useH ? dv[1][i] : dv[0][i]) * a;
-    }
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
-    useF = eF < eB;                                      // base on ties
+  vrow::Picks pk{0u, false};
+  if (ident) {
+  } else if (vfix != nullptr) {
+    pk.whole = (vfix[h] >> 16) & 1;
+    pk.block32 = (vfix[h] >> j) & 1u;
+  } else if constexpr (WMAT) {
+    pk = vrow::pick_matrix<1>(tr, M + static_cast<long long>(h) * 128 * 128, strips[threadIdx.x >> 5], l32);
   } else {
-    float eI = err[0], eH = err[1], eF = err[2];
-    eI += hx(eI, 1); eI += hx(eI, 2); eI += hx(eI, 4);
-    eH += hx(eH, 1); eH += hx(eH, 2); eH += hx(eH, 4);
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eF += hx(eF, m);
-    useH = eH < eI;                                      // identity on ties
-    float eB = (l32 & 7) == 0 ? (useH ? eH : eI) : 0.f;
-#pragma unroll
-    for (int m = 1; m < 32; m <<= 1) eB += hx(eB, m);
-    useF = eF < eB;                                      // base on ties
+    const float4 c4 = *reinterpret_cast<const float4*>(co + h * 128 + 4 * l32);
+    const float w[1][4] = {{c4.x, c4.y, c4.z, c4.w}};
+    pk = vrow::pick_diagonal<1>(tr, w, l32);
   }
-  const int cand = useF ? 2 : (useH ? 1 : 0);
-  const int* cd = cand == 0 ? code[0] : cand == 1 ? code[1] : code[2];
+  const int basis = vrow::basis_of<1>(pk, 0);
   uint8_t* chunk = pool + ((slot / 16) * Hkv + h) * CHUNK<F8>;
   const int off = static_cast<int>(slot % 16);
-  chunk[VC_AT<F8> + off * 32 + l32] = static_cast<uint8_t>((cd[0] & 3) | ((cd[1] & 3) << 2) | ((cd[2] & 3) << 4) | ((cd[3] & 3) << 6));
+  chunk[VC_AT<F8> + off * 32 + l32] = static_cast<uint8_t>(vrow::chosen_byte<1>(tr, basis, 0));
   if ((l32 & 7) == 0) {
-    const float s = cand == 0 ? sc[0] : cand == 1 ? sc[1] : sc[2], m0 = cand == 0 ? mnv[0] : cand == 1 ? mnv[1] : mnv[2];
-    if (F8) {
-      const uint32_t sb = e4m3_bits(s) | (cand == 1 ? 0x80u : 0u);
-      *reinterpret_cast<uint16_t*>(chunk + VM_AT<true> + off * 8 + 2 * j) = static_cast<uint16_t>(sb | (e4m3_bits(m0) << 8));
-    } else {
-      uint32_t sb = f16_bits_rn(s) & 0x7FFFu;
-      if (cand == 1) sb |= 0x8000u;
-      *reinterpret_cast<uint32_t*>(chunk + VM_AT<false> + off * 16 + 4 * j) = sb | (f16_bits_rn(m0) << 16);
-    }
+    const uint32_t meta = vrow::chosen_meta<1, F8>(tr, basis, 0);
+    if (F8) *reinterpret_cast<uint16_t*>(chunk + VM_AT<true> + off * 8 + 2 * j) = static_cast<uint16_t>(meta);
+    else *reinterpret_cast<uint32_t*>(chunk + VM_AT<false> + off * 16 + 4 * j) = meta;
   }
   if (l32 == 0) {
     if (F8) {                                            // bit 7 of the key scale byte in slot 3 of this token's cell
       uint8_t* kb = chunk + 512 + off * 8 + 6;
-      *kb = static_cast<uint8_t>((*kb & 0x7Fu) | (useF ? 0x80u : 0u));
-    } else chunk[1536 + off] = useF ? 1 : 0;
+      *kb = static_cast<uint8_t>((*kb & 0x7Fu) | (pk.whole ? 0x80u : 0u));
+    } else chunk[1536 + off] = pk.whole ? 1 : 0;
   }
 }
 
