@@ -238,7 +238,7 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
         }
         float sc[QB];
         key_phase<QM, K2>(S, cur, lane, sc);
-        softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
+        const bool wide = softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
         // path (past the range chunks_of names the range's last page again, a cache hit nobody uses): were they inside
         // a branch, the wait counts after the join would be those of the path without them, and the value phase
@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
           __builtin_amdgcn_s_setprio(0);
         }
         wave_lds_sync();
-        value_phase<QM>(S, st, vr, lane, wave);
+        value_phase<QM>(S, st, vr, lane, wave, wide);
         wave_lds_sync();
         qi = qn;
       }

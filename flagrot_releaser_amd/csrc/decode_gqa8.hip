@@ -224,7 +224,7 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
         }
         float sc[2][QB];
         key_phase8<QM, K2>(S, cur, lane, sc);
-        softmax_phase8<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
+        const bool wide = softmax_phase8<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
       
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
         // path (past the range chunks_of names the range's last page again, a cache hit nobody uses): were they inside
@@ -244,7 +244,7 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
           __builtin_amdgcn_s_setprio(0);
         }
         wave_lds_sync();
-        value_phase8<QM>(S, st, vr, lane, wave);
+        value_phase8<QM>(S, st, vr, lane, wave, wide);
         wave_lds_sync();
         qi = qn;
       }

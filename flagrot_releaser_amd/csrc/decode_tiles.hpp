@@ -32,6 +32,7 @@ template <int QM> struct Strip {
 constexpr int DRAW_BATCH = 2;                      // quads per draw from the shared (device-scope) counter
 constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
 constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
+constexpr uint32_t WIDE_VSCALE = 0x4800u;          // fp16 pattern of the V scale (8.0) above which a quad's value products are rescaled (value_phase)
 constexpr float QPRE = 16.f;                       // the query operands carry 2^4 (fp16 range: |q| up to 127 in any rotation)
 
 template <int QM, int NW>
@@ -354,9 +355,20 @@ DEVI void key_phase(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[QBLK<
 
 // p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order (vs: the lane's
 // V scale words of its group x per block).
+// Whether the quad holds a V scale above WIDE_VSCALE (wave uniform; slots outside the range count too, which at worst
+// sends a quad through the second set of products for nothing): the strips then hold p * scale * 2^-8 and the value
+// phase runs a second set of products (value_phase, where the reason is given).
+template <int QM>
+DEVI bool quad_is_wide(const uint16_t (&vs)[QBLK<QM>]) {
+  uint32_t top = 0u;
+#pragma unroll
+  for (int b = 0; b < QBLK<QM>; ++b) top = max(top, static_cast<uint32_t>(vs[b]) & 0x7FFFu);
+  return __any(top > WIDE_VSCALE);
+}
+
 template <int QM, class SM>
 DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
-                       int lane, int wave) {
+                       int lane, int wave, bool wide) {
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   constexpr int QB = QBLK<QM>;
   // Odd tokens are unpacked from the V^T words with the factor 2^SH (UnpackD): their scores were lowered by SH (p
@@ -367,12 +379,13 @@ DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[
   uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (t >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
   const int c0 = ((x) * 4 + x) * 8, c1 = ((x ^ 1) * 4 + x) * 8, c2 = ((x ^ 2) * 4 + x) * 8, c3 = ((x ^ 3) * 4 + x) * 8;
+  const uint32_t sfold = wide ? 0x1C00u : 0x3C00u;      // fp16 2^-8 or 1
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
     const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe[b], pe[b]));
     // the token's four V scale words, sign bits stripped: own group x, then the lanes 16, 32, 48 further (groups
     // x ^ 1, x ^ 2, x ^ 3); unwritten slots may hold any pattern: masked
-    const uint32_t v0 = valid[b] ? (vs[b] & 0x7FFFu) : 0u;
+    const uint32_t v0 = pk_mul(valid[b] ? (vs[b] & 0x7FFFu) : 0u, sfold);
     const uint32_t v1 = lane_from(v0, 4 * (lane ^ 16)), v2 = lane_from(v0, 4 * (lane ^ 32)), v3 = lane_from(v0, 4 * (lane ^ 48));
     const uint32_t xa = pk_mul(pp, (v1 << 16) | v0), xb = pk_mul(pp, (v3 << 16) | v2);
     uint16_t* row = pb + b * 2 * PB_RSTRIDE * 8;
@@ -388,7 +401,7 @@ DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[
 // beats it; then p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order.
 // qs20 = qscale * 2^20 (the factor the raw score sums lack); sc0 lowers the scores of odd tokens by SH (below).
 template <int QM, class SM>
-DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
+DEVI bool softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
                         float qs20, float sc0, int lane, int wave) {
   constexpr int QB = QBLK<QM>;
   bool beat = false;
@@ -424,11 +437,13 @@ DEVI void softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QB
     pe[b] = fexp2(sc[b] - st.m);       // masked tokens: 2^-inf = 0 (the maximum is finite once a quad has been seen)
     st.l += pe[b];
   }
-  write_strips<QM>(S, r.vs, pe, valid, lane, wave);
+  const bool wide = quad_is_wide<QM>(r.vs);
+  write_strips<QM>(S, r.vs, pe, valid, lane, wave, wide);
+  return wide;
 }
 
 template <int QM, class SM>
-DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave) {
+DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, int wave, bool wide) {
   // An entry word (entry half eh, word sub) holds channels of group 2 (sub >> 1) + eh only.  The products of all
   // four groups share one accumulator per word parity: the B operand of a group is the strip row with the columns of
   // the other groups zero (those lanes read the row group's pad entry, which nobody writes and which is zeroed once),
@@ -469,6 +484,63 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
       a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
       st.z[e] = a;
     }
+    }
+  }
+  // The code fields enter the matrix pipe as fp16 denormals, and the pipe aligns the addends of an instruction --
+  // products and accumulator -- to the largest NOMINAL exponent (a denormal counts as 2^-14 whatever its leading zeros)
+  // and keeps 24 bits from there.  A token whose p * V-scale is hundreds of times its neighbours' lifts that window for
+  // its whole instruction: neighbours and accumulator lose up to 2^-13 of ITS p * scale each, which shows where the exact
+  // output is near zero (measured with equal weights: 0.05 on sums of 500 beside a group scaled x300, nothing without
+  // it).  In a quad that holds such a scale the strips carry p * scale * 2^-8 (write_strips): the products above came to
+  // 1/256 of their value with the window 8 bits lower, and here the other 255/256 follow: the code operands times 256
+  // (exact) against the strips, minus the plain product once more.  The zero-point sums are vector sums: times 255.
+  if (__builtin_expect(wide, 0)) {
+    // (strips and entry words go through values the compiler cannot see through: recognised as the operands of the
+    // products above, those would all stay in registers until here)
+    // (... and the lane's own indices likewise: as loop invariants their derived addresses are computed ahead of the
+    // page loop and, used here only, parked in scratch memory -- a kernel that uses scratch starts its workgroups late)
+    int again = 0;
+    asm volatile("" : "+s"(again));
+    const int n2 = (lane + again) & 15, kc2 = (lane + again) >> 4;
+    const uint4* rowg2 = reinterpret_cast<const uint4*>(S.pb(wave)) + kc2 * PB_RSTRIDE;
+#pragma unroll
+    for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {
+#pragma unroll
+      for (int eh = 0; eh < 2; ++eh)
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+          const int g = 2 * (sub >> 1) + eh;
+          const uint4 bq = (rowg2 + ((n2 >> 2) == g ? n2 : 16))[4 * s2 * PB_RSTRIDE];
+          uint32_t w = QM == QM_ASYM2 ? r.vc[2 * s2 + eh][sub >> 1] : r.vc[2 * s2 + eh][sub];
+          asm volatile("" : "+v"(w));
+          uint32_t x[4];
+          if constexpr (QM == QM_ASYM2) {
+            if (sub & 1) UnpackD<QM>::run_hi(w, x); else UnpackD<QM>::run(w, x);
+          }
+          else UnpackD<QM>::run(w, x);
+          const uint4 aq = make_uint4(x[0], x[1], x[2], x[3]);
+          const uint4 a256 = make_uint4(pk_mul(x[0], 0x5C005C00u), pk_mul(x[1], 0x5C005C00u), pk_mul(x[2], 0x5C005C00u), pk_mul(x[3], 0x5C005C00u));
+          const uint4 nb = make_uint4(bq.x ^ 0x80008000u, bq.y ^ 0x80008000u, bq.z ^ 0x80008000u, bq.w ^ 0x80008000u);
+          st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a256), __builtin_bit_cast(half8, bq), st.ot[sub & 1], 0, 0, 0);
+          st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aq), __builtin_bit_cast(half8, nb), st.ot[sub & 1], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);      // one step's operands at a time: this path is rare and must not claim registers
+        }
+    }
+    if constexpr (QM != QM_SYM4) {
+#pragma unroll
+      for (int r8 = 0; r8 < Strip<QM>::ROWS; r8 += 8) {
+        const int l2 = lane + again;
+        const int rg = r8 + (l2 >> 3), g = (l2 >> 1) & 3, hp = l2 & 1;
+        const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
+        const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB_RSTRIDE + g * 4 + 2 * hp;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const uint4 pq = pp[e];
+          float a = dot2(zq.x, pq.x, 0.f);
+          a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
+          st.z[e] += 255.f * a;
+        }
+      }
     }
   }
 }
@@ -656,7 +728,7 @@ DEVI void key_phase8(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[2][Q
 
 // softmax step of both halves; the strips take p * V-scale of heads x and 4 + x for all four groups
 template <int QM, class SM>
-DEVI void softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[2][QBLK<QM>], const bool (&valid)[QBLK<QM>],
+DEVI bool softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[2][QBLK<QM>], const bool (&valid)[QBLK<QM>],
                          float qs20, float sc0, int lane, int wave) {
   constexpr int QB = QBLK<QM>;
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
@@ -707,9 +779,11 @@ DEVI void softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[
   uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (tk >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;
   const int c0 = ((x) * 8 + x) * 8, c1 = ((x ^ 1) * 8 + x) * 8, c2 = ((x ^ 2) * 8 + x) * 8, c3 = ((x ^ 3) * 8 + x) * 8;
+  const bool wide = quad_is_wide<QM>(r.vs);      // its strips then keep p * scale * 2^-8 (value_phase has the reason)
+  const uint32_t sfold = wide ? 0x1C00u : 0x3C00u;      // fp16 2^-8 or 1
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
-    const uint32_t v0 = valid[b] ? (r.vs[b] & 0x7FFFu) : 0u;
+    const uint32_t v0 = pk_mul(valid[b] ? (r.vs[b] & 0x7FFFu) : 0u, sfold);
     const uint32_t v1 = lane_from(v0, 4 * (lane ^ 16)), v2 = lane_from(v0, 4 * (lane ^ 32)), v3 = lane_from(v0, 4 * (lane ^ 48));
     const uint32_t va = (v1 << 16) | v0, vb = (v3 << 16) | v2;
     uint16_t* row = pb + b * 2 * PB8_RSTRIDE * 8;
@@ -724,10 +798,11 @@ DEVI void softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[
     }
     if constexpr (QM != QM_SYM4) zb[b * 2 * ZB_RSTRIDE * 8] = static_cast<uint16_t>((r.vs[b] & ZM) << zsh);
   }
+  return wide;
 }
 
 template <int QM, class SM>
-DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane, int wave) {
+DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane, int wave, bool wide) {
   // column n = lane & 15 = (group n >> 2, head n & 3 of the half); a masked entry word is multiplied with the strip
   // rows of both halves (entries 8 g + head and 8 g + 4 + head; lanes of foreign groups read the zero pad entry)
   const int n = lane & 15, kc = lane >> 4;
@@ -767,6 +842,57 @@ DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane
         a = dot2(zq.x, pq.x, a); a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
         st.z[t][e] = a;
       }
+  }
+  // quads with a wide V scale: the other 255/256 of the value products and of the zero-point sums (value_phase)
+  if (__builtin_expect(wide, 0)) {
+    int again = 0;
+    asm volatile("" : "+s"(again));
+    const int n2 = (lane + again) & 15, kc2 = (lane + again) >> 4;
+    const uint4* rowg2 = reinterpret_cast<const uint4*>(S.pb(wave)) + kc2 * PB8_RSTRIDE;
+#pragma unroll
+    for (int s2 = 0; s2 < QBLK<QM> / 2; ++s2) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int eh = g & 1;
+        const uint4* src = rowg2 + 4 * s2 * PB8_RSTRIDE;
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+          const int sub = 2 * (g >> 1) + y;
+          uint32_t w = QM == QM_ASYM2 ? r.vc[2 * s2 + eh][sub >> 1] : r.vc[2 * s2 + eh][sub];
+          asm volatile("" : "+v"(w));
+          uint32_t x[4];
+          if constexpr (QM == QM_ASYM2) {
+            if (sub & 1) UnpackD<QM>::run_hi(w, x); else UnpackD<QM>::run(w, x);
+          }
+          else UnpackD<QM>::run(w, x);
+          const half8 aq = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+          const half8 a256 = __builtin_bit_cast(half8, make_uint4(pk_mul(x[0], 0x5C005C00u), pk_mul(x[1], 0x5C005C00u), pk_mul(x[2], 0x5C005C00u), pk_mul(x[3], 0x5C005C00u)));
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            uint4 bq = src[(n2 >> 2) == g ? 8 * g + 4 * t + (n2 & 3) : 32];
+            st.ot[t][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a256, __builtin_bit_cast(half8, bq), st.ot[t][y], 0, 0, 0);
+            bq = make_uint4(bq.x ^ 0x80008000u, bq.y ^ 0x80008000u, bq.z ^ 0x80008000u, bq.w ^ 0x80008000u);
+            st.ot[t][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq, __builtin_bit_cast(half8, bq), st.ot[t][y], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);      // one step's operands at a time: this path is rare and must not claim registers
+          }
+        }
+      }
+    }
+    if constexpr (QM != QM_SYM4) {
+      const int l2 = lane + again;
+      const int rg = l2 >> 3, g = (l2 >> 1) & 3, hp = l2 & 1;
+      const uint4 zq = (reinterpret_cast<const uint4*>(S.zb(wave)) + rg * ZB_RSTRIDE)[g];
+      const uint4* pp = reinterpret_cast<const uint4*>(S.pb(wave)) + rg * PB8_RSTRIDE + g * 8 + 2 * hp;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const uint4 pq = pp[4 * t + e];
+          float a = dot2(zq.x, pq.x, 0.f);
+          a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
+          st.z[t][e] += 255.f * a;
+        }
+    }
   }
 }
 

@@ -343,13 +343,15 @@ __global__ void __launch_bounds__(64 * NWW, 2) k_wide_parts_mma(const DecodePara
     load_k<QM, P, false>(k0, ch0, koff);
     load_k<QM, P, false>(k1, ch1, koff);
     // ---- values, half by half through the same strips
-    write_strips<QM>(H0, vs0, pe, valid, lane, wave);
+    const bool wide0 = quad_is_wide<QM>(vs0);
+    write_strips<QM>(H0, vs0, pe, valid, lane, wave, wide0);
     wave_lds_sync();
-    value_phase<QM>(H0, st0, v0, lane, wave);
+    value_phase<QM>(H0, st0, v0, lane, wave, wide0);
     wave_lds_sync();
-    write_strips<QM>(H1, vs1, pe, valid, lane, wave);
+    const bool wide1 = quad_is_wide<QM>(vs1);
+    write_strips<QM>(H1, vs1, pe, valid, lane, wave, wide1);
     wave_lds_sync();
-    value_phase<QM>(H1, st1, v1, lane, wave);
+    value_phase<QM>(H1, st1, v1, lane, wave, wide1);
     wave_lds_sync();
     qi = qn;
   }

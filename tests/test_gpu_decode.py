@@ -6,7 +6,10 @@ Bar (floating point, the tolerance of the build's north star: max-abs 2e-3 / rel
     adversarial groups (values x300, x1e-5, constants, one-hots: log2 scores of +-1000, outputs of several hundred, so
     that a 1e-5 relative change of one score moves a weight by percents): |out - ref| <= 2e-3 + 1e-2 * max |ref[row]|
     (the reference's own tests measure every row against the global max |ref| with a 4e-3 floor,
-    test_kernels.py:173).  The query variants enter the score products as fp16 value + fp16 remainder (22 bits).
+    test_kernels.py:173), AND element-wise within TWICE the bar of the ordinary rows (measured: at most 1.32 times; up
+    to 15 times before the value products of quads with large V scales were rescaled -- beside a group scaled x300 the
+    matrix pipe's 24-bit window cut its neighbours short).  The query variants enter the score products as fp16 value
+    + fp16 remainder (22 bits).
 Every case prints its worst element-wise ratio |err| / (2e-3 + 1e-2 |ref|), ordinary and adversarial rows apart.
 ref = fp64 softmax attention over the pages parsed by the oracle's independent layout parser (the cache bytes are
 written by the HIP writers, whose bit-exactness tests/test_gpu_writers.py establishes)."""
@@ -23,6 +26,7 @@ from tests.gpu_util import P as P16, alloc_tables, bits, make_kv, slots_of, spd_
 pytestmark = pytest.mark.gpu
 LOG2E = 1.4426950408889634
 ATOL, RTOL = 2e-3, 1e-2
+HARD_ROWS = 2.0      # element-wise bound of the rows that read the adversarial tokens, in units of the ordinary bar
 
 
 def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None, P=P16):
@@ -110,6 +114,7 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
               f"adversarial tokens ({(err / lim)[hard].max():.3f} of their row-max bar)", flush=True)
         assert (err <= lim).all(), (f"{fmt} {lens} ns={ns} ch={ch} worst(b,head,d)={tuple(int(i) for i in worst)} "
                                     f"got={got[worst]:.5f} ref={ref[worst]:.5f} limit={lim[worst]:.5f}")
+        assert strict[hard].max() <= HARD_ROWS, (fmt, lens, ns, float(strict[hard].max()))
     assert int(ws.counter.abs().sum()) == 0
     return ns, ch
 
