@@ -3,6 +3,8 @@
 import ctypes
 import os
 import re
+import shutil
+import subprocess
 
 import pytest
 
@@ -77,6 +79,29 @@ def test_probe_library_exports_header_symbols():
         assert hasattr(L, n), n
     L.fr_probe_abi_version.restype = ctypes.c_int
     assert L.fr_probe_abi_version() == probe.ABI
+
+
+def test_c_caller_compiles_links_and_runs(tmp_path):
+    """tests/c_abi/abi_check.c, a plain C99 caller: the headers compile as C (-Wall -Wextra -Werror -pedantic), every
+    declared entry point of the three boundary libraries resolves at link time, and the calls that need no GPU
+    (versions, sizes, argument checks that return before any launch) give the documented answers"""
+    from flagrot_releaser_amd import build
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    libdir = build.lib_path("kernels").parent
+    for lib in ("kernels", "kivi", "mq"):
+        if not build.lib_path(lib).exists():
+            build.build(lib, verbose=False)
+    exe = tmp_path / "abi_check"
+    cmd = [gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "c_abi", "abi_check.c"), "-o", str(exe), "-L", str(libdir), "-lflagrot_kernels",
+           "-lflagrot_kivi", "-lflagrot_mq", f"-Wl,-rpath,{libdir}", "-Wl,-rpath-link,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.returncode, r.stderr[-500:])
+    assert "all checks passed" in r.stdout
 
 
 def test_host_planner_invariants():
