@@ -7,6 +7,7 @@
 #include "../../include/flagrot_kivi.h"
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
+#include "kivi_merge.hpp"
 
 namespace frkv {
 using namespace fr;
@@ -16,42 +17,6 @@ char g_err[512] = "";
 int bad(const char* msg) {
   std::strncpy(g_err, msg, sizeof(g_err) - 1);
   return 2;
-}
-
-__global__ void __launch_bounds__(128) k_merge(const float* __restrict__ opart, const float* __restrict__ ml, int Hkv, int G,
-                                               int NS, uint16_t* __restrict__ out, long long out_rs) {
-  const int b = blockIdx.x, hq = blockIdx.y, h = hq / G, g = hq % G;
-  const long long p0 = (static_cast<long long>(b) * Hkv + h) * (NS + 1);
-  // eight partials at a time: their loads are issued together (one after the other in a plain loop, each iteration
-  // would wait for its own)
-  float M = -INFINITY;
-  for (int s0 = 0; s0 <= NS; s0 += 8) {
-    float m8[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) m8[i] = ml[((p0 + min(s0 + i, NS)) * G + g) * 2];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) M = fmaxf(M, m8[i]);
-  }
-  float o = 0.f, L = 0.f;
-  if (M != -INFINITY) {
-    for (int s0 = 0; s0 <= NS; s0 += 8) {
-      float m8[8], l8[8], o8[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const long long at = (p0 + min(s0 + i, NS)) * G + g;
-        m8[i] = ml[at * 2]; l8[i] = ml[at * 2 + 1]; o8[i] = opart[at * 128 + threadIdx.x];
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (s0 + i > NS || m8[i] == -INFINITY) continue;
-        const float f = exp2f(m8[i] - M);
-        L += f * l8[i];
-        o += f * o8[i];
-      }
-    }
-  }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  out[static_cast<long long>(b) * out_rs + static_cast<long long>(hq) * 128 + threadIdx.x] = static_cast<uint16_t>(bf16_rn(o * inv));
 }
 
 int launched(int rc, const char* what) {
@@ -114,7 +79,7 @@ int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, lon
   const int rc = attn_splits_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
                                     tail_idx, T, opart, ml, f8 & 1, st);
   if (rc) return launched(rc, "kv_attn");
-  hipLaunchKernelGGL(k_merge, dim3(B, Hkv * G), dim3(128), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
+  hipLaunchKernelGGL(k_merge_parts<128>, dim3(B, Hkv * G), dim3(128), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
                      Hkv, G, NS, static_cast<uint16_t*>(out), out_rs);
   return launched(hipPeekAtLastError() == hipSuccess ? 0 : 1, "kv_attn (merge)");
 }

@@ -27,6 +27,7 @@
 
 #include "fr_common.hpp"
 #include "kivi_launch.hpp"
+#include "kivi_merge.hpp"
 #include "kivi_quant.hpp"
 #include "kivi_vrow.hpp"
 
@@ -646,42 +647,6 @@ __global__ void __launch_bounds__(256) k_attn256(const uint16_t* __restrict__ q,
   if (l32 == 0 && hw < G) { mlp[2 * hw] = m_run; mlp[2 * hw + 1] = l_run; }
 }
 
-__global__ void __launch_bounds__(256) k_merge256(const float* __restrict__ opart, const float* __restrict__ ml, int Hkv, int G,
-                                                  int NS, uint16_t* __restrict__ out, long long out_rs) {
-  const int b = blockIdx.x, hq = blockIdx.y, h = hq / G, g = hq % G;
-  const long long p0 = (static_cast<long long>(b) * Hkv + h) * (NS + 1);
-  // eight partials at a time: their loads are issued together (one after the other in a plain loop, each iteration
-  // would wait for its own)
-  float M = -INFINITY;
-  for (int s0 = 0; s0 <= NS; s0 += 8) {
-    float m8[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) m8[i] = ml[((p0 + min(s0 + i, NS)) * G + g) * 2];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) M = fmaxf(M, m8[i]);
-  }
-  float o = 0.f, L = 0.f;
-  if (M != -INFINITY) {
-    for (int s0 = 0; s0 <= NS; s0 += 8) {
-      float m8[8], l8[8], o8[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const long long at = (p0 + min(s0 + i, NS)) * G + g;
-        m8[i] = ml[at * 2]; l8[i] = ml[at * 2 + 1]; o8[i] = opart[at * D2 + threadIdx.x];
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (s0 + i > NS || m8[i] == -INFINITY) continue;
-        const float f = exp2f(m8[i] - M);
-        L += f * l8[i];
-        o += f * o8[i];
-      }
-    }
-  }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  out[static_cast<long long>(b) * out_rs + static_cast<long long>(hq) * D2 + threadIdx.x] = static_cast<uint16_t>(bf16_rn(o * inv));
-}
-
 template <typename K> bool carve(K kern, size_t bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                              static_cast<int>(bytes)) == hipSuccess;
@@ -751,7 +716,7 @@ int attn256_launch(int G, const void* q, long long q_rs, const void* pool, const
                                         tail_idx, T, opart, ml, f8, st);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(k_merge256, dim3(B, Hkv * G), dim3(256), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
+  hipLaunchKernelGGL(k_merge_parts<D2>, dim3(B, Hkv * G), dim3(256), 0, st, static_cast<const float*>(opart), static_cast<const float*>(ml),
                      Hkv, G, NS, static_cast<uint16_t*>(out), out_rs);
   return hipPeekAtLastError() == hipSuccess ? 0 : 1;
 }
