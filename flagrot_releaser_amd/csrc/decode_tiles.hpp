@@ -33,6 +33,15 @@ constexpr int DRAW_BATCH = 2;                      // quads per draw from the sh
 constexpr int DRAW_BITS = 21, DRAW_MASK = (1 << DRAW_BITS) - 1;   // counter slot: quad draws below, merge tickets above
 constexpr int BT_CACHE = 1024;                     // block-table entries of the workgroup's page range kept in LDS
 constexpr uint32_t WIDE_VSCALE = 0x4800u;          // fp16 pattern of the V scale (8.0) above which a quad's value products are rescaled (value_phase)
+// ... by 2^-8, or by 2^-4 where the odd tokens' p already carries 2^-4 (the 4-bit fields with zero points): p * scale
+// must stay a NORMAL fp16 number for ordinary scales, or the strips themselves lose what the rescaling is there to keep
+// (measured with 2^-8 on those pages: 3e-3 on sums of 25 with equal weights).  fold: fp16 pattern of the factor; up: its
+// inverse as an fp16 pair; rest: inverse - 1, what the zero-point sums (plain vector sums) still lack.
+template <int QM> struct WideFold {
+  static constexpr uint32_t fold = QM == QM_ASYM4 ? 0x2C00u : 0x1C00u;
+  static constexpr uint32_t up = QM == QM_ASYM4 ? 0x4C004C00u : 0x5C005C00u;
+  static constexpr float rest = QM == QM_ASYM4 ? 15.f : 255.f;
+};
 constexpr float QPRE = 16.f;                       // the query operands carry 2^4 (fp16 range: |q| up to 127 in any rotation)
 
 template <int QM, int NW>
@@ -379,7 +388,7 @@ DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[
   uint16_t* zb = reinterpret_cast<uint16_t*>(S.zb(wave)) + (t >> 3) * ZB_RSTRIDE * 8 + x * 8 + sl;
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;      // odd position inside the page
   const int c0 = ((x) * 4 + x) * 8, c1 = ((x ^ 1) * 4 + x) * 8, c2 = ((x ^ 2) * 4 + x) * 8, c3 = ((x ^ 3) * 4 + x) * 8;
-  const uint32_t sfold = wide ? 0x1C00u : 0x3C00u;      // fp16 2^-8 or 1
+  const uint32_t sfold = wide ? WideFold<QM>::fold : 0x3C00u;      // fp16 2^-8 (2^-4) or 1
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
     const uint32_t pp = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pe[b], pe[b]));
@@ -519,7 +528,7 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
           }
           else UnpackD<QM>::run(w, x);
           const uint4 aq = make_uint4(x[0], x[1], x[2], x[3]);
-          const uint4 a256 = make_uint4(pk_mul(x[0], 0x5C005C00u), pk_mul(x[1], 0x5C005C00u), pk_mul(x[2], 0x5C005C00u), pk_mul(x[3], 0x5C005C00u));
+          const uint4 a256 = make_uint4(pk_mul(x[0], WideFold<QM>::up), pk_mul(x[1], WideFold<QM>::up), pk_mul(x[2], WideFold<QM>::up), pk_mul(x[3], WideFold<QM>::up));
           const uint4 nb = make_uint4(bq.x ^ 0x80008000u, bq.y ^ 0x80008000u, bq.z ^ 0x80008000u, bq.w ^ 0x80008000u);
           st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a256), __builtin_bit_cast(half8, bq), st.ot[sub & 1], 0, 0, 0);
           st.ot[sub & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aq), __builtin_bit_cast(half8, nb), st.ot[sub & 1], 0, 0, 0);
@@ -538,7 +547,7 @@ DEVI void value_phase(const SM& S, WaveState& st, const VRegs<QM>& r, int lane, 
           const uint4 pq = pp[e];
           float a = dot2(zq.x, pq.x, 0.f);
           a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
-          st.z[e] += 255.f * a;
+          st.z[e] += WideFold<QM>::rest * a;
         }
       }
     }
@@ -780,7 +789,7 @@ DEVI bool softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[
   const int zsh = (lane & 1) ? UnpackD<QM>::SH : 0;
   const int c0 = ((x) * 8 + x) * 8, c1 = ((x ^ 1) * 8 + x) * 8, c2 = ((x ^ 2) * 8 + x) * 8, c3 = ((x ^ 3) * 8 + x) * 8;
   const bool wide = quad_is_wide<QM>(r.vs);      // its strips then keep p * scale * 2^-8 (value_phase has the reason)
-  const uint32_t sfold = wide ? 0x1C00u : 0x3C00u;      // fp16 2^-8 or 1
+  const uint32_t sfold = wide ? WideFold<QM>::fold : 0x3C00u;      // fp16 2^-8 (2^-4) or 1
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
     const uint32_t v0 = pk_mul(valid[b] ? (r.vs[b] & 0x7FFFu) : 0u, sfold);
@@ -866,7 +875,7 @@ DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane
           }
           else UnpackD<QM>::run(w, x);
           const half8 aq = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
-          const half8 a256 = __builtin_bit_cast(half8, make_uint4(pk_mul(x[0], 0x5C005C00u), pk_mul(x[1], 0x5C005C00u), pk_mul(x[2], 0x5C005C00u), pk_mul(x[3], 0x5C005C00u)));
+          const half8 a256 = __builtin_bit_cast(half8, make_uint4(pk_mul(x[0], WideFold<QM>::up), pk_mul(x[1], WideFold<QM>::up), pk_mul(x[2], WideFold<QM>::up), pk_mul(x[3], WideFold<QM>::up)));
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
             uint4 bq = src[(n2 >> 2) == g ? 8 * g + 4 * t + (n2 & 3) : 32];
@@ -890,7 +899,7 @@ DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane
           const uint4 pq = pp[4 * t + e];
           float a = dot2(zq.x, pq.x, 0.f);
           a = dot2(zq.y, pq.y, a); a = dot2(zq.z, pq.z, a); a = dot2(zq.w, pq.w, a);
-          st.z[t][e] += 255.f * a;
+          st.z[t][e] += WideFold<QM>::rest * a;
         }
     }
   }
