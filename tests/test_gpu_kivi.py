@@ -131,7 +131,6 @@ def test_v_write_matrix_weight(dev, f8):
         badF = useF != enc["useF"]
         badH = (useH != enc["useH"]) & ~useF[..., None] & ~enc["useF"][..., None]
         assert (enc["marginF"][badF] < 1e-3).all() and (enc["marginH"][badH] < 1e-3).all(), name
-        if T >= 64:      # a rate needs rows to be a rate of: with a dozen rows one tie on the zero or constant row is 10 %
         assert badF.mean() < 0.02 and badH.mean() < 0.02
         if name == "diagonal":
             ref = torch.zeros_like(pool)
