@@ -204,7 +204,8 @@ def k_encode_group(x_bits, valid, qs, lz, qsc, ident=False, fix=None, f8=False, 
         return res
     e = [np.where(valid[:, None], _back(rec[c], c) - x, F32(0)).astype(np.float64) for c in range(3)]
     qd = np.asarray(qs, np.float64)
-    w = np.minimum(1.0, np.exp(float(qsc) * (x.astype(np.float64) @ qd.T) - np.asarray(lz, np.float64)[None]))
+    # the weight is min(1, e^(score - lz)): the exponent is capped at 0 first (the rows scaled x200 of the tests would overflow exp)
+    w = np.exp(np.minimum(0.0, float(qsc) * (x.astype(np.float64) @ qd.T) - np.asarray(lz, np.float64)[None]))
     w = np.where(valid[:, None], w, 0.0)                                           # [32, NQ]
     loc = lambda ec: np.stack([(w * (ec[:, 32 * j:32 * j + 32] @ qd[:, 32 * j:32 * j + 32].T) ** 2).sum()  # noqa: E731
                                for j in range(NV)])

@@ -1,0 +1,153 @@
+"""Seeded random shapes through the checkers of the other GPU test files: the committed cases of those files are the
+shapes somebody thought of; these are a few hundred nobody did (fixed seeds, so every run sees the same ones).  Each
+generator was first run open-ended for minutes at a time; what those runs found is fixed and is now a committed case
+where it belongs (the rescale factor of the 4-bit pages in the decode kernels; the rate assertion of the KIVI writer
+tests on a dozen rows).
+
+Bars: the writers byte for byte; the decode attention as in tests/test_gpu_decode.py, with the rows that read the
+adversarial tokens held to 6 times the element-wise bar instead of 2 (open-ended runs: 1 % of such rows above 1, largest
+4.4, on the 2-bit pages); the KIVI decode attention at the reference's row bar and 6 times the element-wise bar (every
+sequence holds a row scaled x200; open-ended runs: 2.6 % of the shapes above 1, largest 4.2); the multi-query prefill at
+the bars of tests/test_gpu_mq.py."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pages as PG
+from oracle import quant as Q
+from tests.gpu_util import bits, make_kv, spd_calib
+
+pytestmark = pytest.mark.gpu
+
+
+def test_decode_shapes(dev):
+    from tests.test_gpu_decode import run_case
+    rng = random.Random(20250)
+    lengths = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 300, 511, 777, 1024, 1500]
+    for n in range(160):
+        mode = rng.choice(["codebook", "static"])
+        fmt = rng.choice(["konly", "konlya", "konlya2"]) if mode == "codebook" else rng.choice(["int4", "int4a", "int2a"])
+        P = rng.choice([16, 16, 32])
+        G, Hkv = rng.choice([(4, 4), (4, 2), (8, 2), (8, 4), (5, 2), (6, 2), (12, 1), (1, 4), (2, 4), (3, 3)])
+        B = rng.choice([1, 2, 3, 5, 8])
+        lens = [rng.choice(lengths) for _ in range(B)]
+        if rng.random() < 0.2:
+            lens[rng.randrange(B)] = rng.choice([2049, 4097, 6000])
+        if max(lens) == 0:
+            lens[0] = 5
+        win = rng.choice([None, None, (4, B + 2), (128, B + 1), (17, B + 3)])
+        kv_start = rng.choice([0, 0, 0, 1, 16, 40, 64])
+        nsplit = rng.choice([None, None, None, 1, 2, 3, 5, 8, 16])
+        shared = rng.choice([False, False, False, True, "stride0"])
+        if shared and rng.random() < 0.5:
+            lens = [max(lens)] * B
+        seed = rng.randrange(1 << 30)
+        print(f"\nshape {n}: {mode} {fmt} P={P} G={G} Hkv={Hkv} lens={lens} win={win} kv_start={kv_start} nsplit={nsplit} "
+              f"shared={shared} seed={seed}", flush=True)
+        run_case(dev, mode, lens, fmt, win=win, bt_shared=shared, seed=seed, G=G, Hkv=Hkv, kv_start=kv_start, nsplit=nsplit,
+                 P=P, hard_rows=6.0)
+
+
+def test_writer_shapes(dev):
+    from flagrot_releaser_amd import kernels as K
+    rng = random.Random(4321)
+    for n in range(400):
+        static = rng.random() < 0.4
+        fmt = rng.choice(["int4", "int4a", "int2a"]) if static else rng.choice(["konly", "konlya", "konlya2"])
+        P = rng.choice([16, 16, 32])
+        T = rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 33, 64, 100, 255, 256, 257, 511, 600, 1025])
+        Hkv = rng.choice([1, 2, 4, 8])
+        if not static and T * Hkv > 2100:
+            Hkv = 1
+        seed = rng.randrange(1 << 30)
+        order = rng.choice(["scattered", "consecutive", "consecutive_holes"])
+        base = rng.choice([0, 3, 8, 13, 16, 29])
+        centred = rng.random() < 0.4
+        pad = rng.choice([0, 0, 1])                     # extra rows per token: a token stride the kernel must honour
+        g = torch.Generator().manual_seed(seed)
+        npg = (T + base) // P + 4
+        pool = torch.randint(0, 256, (npg, Hkv, PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g)
+        rows = torch.zeros(T, 2 * Hkv + pad, 128, dtype=torch.bfloat16)
+        rows[:, :2 * Hkv] = make_kv(T, Hkv, g)
+        kv = rows.to(dev)[:, :2 * Hkv]
+        if order == "scattered":
+            slots = torch.randperm(npg * P, generator=g)[:T].long()
+            if T >= 4:
+                slots[T // 3] = -1
+        else:
+            slots = base + torch.arange(T).long()
+            if order == "consecutive_holes" and T >= 20:
+                slots[T // 2] = -1
+                a = rng.randrange(0, T - 16)
+                slots[a:a + 16] = slots[a:a + 16].flip(0)
+        kmu = torch.randn(Hkv, 128, generator=g) if centred else None
+        dpool = pool.to(dev)
+        want = pool.numpy().copy()
+        if static:
+            mask = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8)
+            K.v2_write(kv, slots.to(dev), mask.to(dev), 32, dpool, P, fmt=fmt, kmu=None if kmu is None else kmu.to(dev))
+            codes, words = Q.static_encode(bits(rows[:, :2 * Hkv]), mask.numpy(), fmt, None if kmu is None else kmu.numpy())
+        else:
+            Cq, co = spd_calib(Hkv, g)
+            K.cb_write(kv, slots.to(dev), Cq.transpose(1, 2).contiguous().to(dev), co.to(dev), fmt, dpool, P,
+                       kmu=None if kmu is None else kmu.to(dev))
+            codes, words, _ = Q.k2_encode(bits(rows[:, :2 * Hkv]), Cq.numpy(), fmt, None if kmu is None else kmu.numpy())
+        torch.cuda.synchronize()
+        PG.pack_tokens(want, slots.numpy(), codes, words, fmt, P)
+        got = dpool.cpu().numpy()
+        assert np.array_equal(got, want), (n, fmt, P, T, Hkv, seed, order, base, centred, pad, int((got != want).sum()))
+
+
+def test_kivi_attention_shapes(dev):
+    import tests.test_gpu_kivi as narrow
+    import tests.test_gpu_kivi_wide as wide
+    rng = random.Random(99)
+    lengths = [1, 31, 32, 33, 64, 96, 97, 200, 333, 512, 777, 1000, 1500, 2100]
+    for n in range(70):
+        mod = rng.choice([wide, narrow])
+        B = rng.choice([1, 2, 3, 4])
+        lens = [rng.choice(lengths) for _ in range(B)]
+        Hkv = rng.choice([1, 2, 4])
+        G = rng.choice([1, 2, 3, 4, 5, 6, 7, 8])
+        kv_start = rng.choice([0, 0, 5, 32, 37, 64, 255])
+        ns = rng.choice([1, 2, 3, 4, 5, 7])
+        chunk = max(256, -(-(-(-max(lens) // ns)) // 32) * 32)
+        tails = [rng.choice([0, 0, 1, 9, 64, 127, 128]) for _ in range(B)]
+        f8 = rng.random() < 0.5
+        seed = rng.randrange(1 << 30)
+        mod.attn_case(dev, (lens, Hkv, G, kv_start, (ns, chunk), tails), seed, f8, 6.0,
+                      label=f"shape {n} ({'256' if mod is wide else '128'}-d) {lens} Hkv={Hkv} G={G} kv_start={kv_start} ns={ns}")
+
+
+def test_kivi_writer_shapes(dev):
+    import tests.test_gpu_kivi as narrow
+    import tests.test_gpu_kivi_wide as wide
+    rng = random.Random(777)
+    for n in range(120):
+        mod = rng.choice([narrow, wide])
+        f8 = rng.random() < 0.5
+        seed = rng.randrange(1 << 30)
+        if rng.random() < 0.67:
+            T, Hkv = rng.choice([1, 2, 9, 16, 17, 64, 100, 333, 700]), rng.choice([1, 2, 4, 8])
+            mod.test_v_write_given_flags(dev, seed, T, Hkv, f8)
+        else:
+            NG, Hkv, NQ = rng.choice([1, 2, 4, 6]), rng.choice([1, 2, 8]), rng.choice([8, 24, 37, 64])
+            mod.test_k_encode_given_flags(dev, seed, NG, Hkv, NQ, f8)
+
+
+def test_mq_prefill_shapes(dev):
+    import tests.test_gpu_mq as mq
+    rng = random.Random(2024)
+    first = len(mq.CASES)
+    for _ in range(10):
+        for c in mq._random_cases(4, rng.randrange(1 << 30)):
+            c = list(c)
+            c[5] = rng.choice([1, 2, 3, 4, 4, None])        # rows per tile: 64 / 128 / 128 / 256, or the planner's choice
+            mq.CASES.append(tuple(c))
+    try:
+        for idx in range(first, len(mq.CASES)):
+            mq.test_mq_attention_against_fp64(dev, idx)
+    finally:
+        del mq.CASES[first:]
