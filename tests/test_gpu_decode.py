@@ -257,12 +257,12 @@ def test_head_dim_256_groups(dev, fmt, G, Hkv):
     _head_dim_256(dev, fmt, 16, G, Hkv)
 
 
-def _head_dim_256(dev, fmt, P, G, Hkv):
+def _head_dim_256(dev, fmt, P, G, Hkv, lens=None, seed=None):
     from flagrot_releaser_amd import kernels as K
     Dh = 256
     static = fmt in ("int4", "int4a", "int2a")
-    g = torch.Generator().manual_seed(600 + len(fmt) + P)
-    lens = [1, 17, 64, 65, 333, 700, 0]
+    g = torch.Generator().manual_seed(600 + len(fmt) + P if seed is None else seed)
+    lens = [1, 17, 64, 65, 333, 700, 0] if lens is None else list(lens) + [0]      # the last sequence is empty
     B, HQ = len(lens), G * Hkv
     num_pages = sum((n + P - 1) // P for n in lens) + 5
     pool = torch.randint(0, 256, (num_pages, Hkv, 2 * PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g).to(dev)

@@ -50,6 +50,20 @@ def test_decode_shapes(dev):
                  P=P, hard_rows=6.0)
 
 
+def test_decode_shapes_head_dim_256(dev):
+    from tests.test_gpu_decode import _head_dim_256
+    rng = random.Random(256)
+    lengths = [1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 127, 129, 255, 300, 511, 777, 1024, 1500, 2100]
+    for n in range(24):
+        fmt = rng.choice(["konly", "konlya", "konlya2", "int4", "int4a", "int2a"])
+        P = rng.choice([16, 16, 32])
+        G, Hkv = rng.choice([(6, 4), (1, 4), (4, 2), (8, 2), (12, 1), (5, 8), (3, 3)])
+        lens = [rng.choice(lengths) for _ in range(rng.choice([1, 2, 4, 6]))]
+        seed = rng.randrange(1 << 30)
+        print(f"\nshape {n}: {fmt} P={P} G={G} Hkv={Hkv} lens={lens} seed={seed}", flush=True)
+        _head_dim_256(dev, fmt, P, G, Hkv, lens=lens, seed=seed)
+
+
 def test_writer_shapes(dev):
     from flagrot_releaser_amd import kernels as K
     rng = random.Random(4321)
