@@ -172,6 +172,25 @@ def ring_slot(p, S: int, W: int):
     return RingGeometry(S, W).slot(p)
 
 
+def chunk_key_groups(geo: RingGeometry, start: int, n: int, ring_row0: int, table_row, page: int = PAGE):
+    """The 32-token key groups that a prompt chunk of n tokens at positions [start, start + n) completes, as the
+    (sources, page slots) pair the key group encoder takes: int64 [N, 32] each, or None when the chunk completes no
+    group.  A position of such a group comes from the chunk (its row index), from the BF16 ring of the request when an
+    earlier chunk brought it (encoded -2 - ring row; ring_row0 = the request's first row of the flattened ring), or is
+    a sink that stays BF16 only (-1).  A group that straddles the chunk's start has at most 31 earlier positions, all
+    still in a window of W >= 32 slots -- so the groups must be encoded BEFORE the chunk's own rows go into the ring.
+    table_row: the request's block-table row (int tensor).  Reference: attention/backend.py:1327-1371."""
+    g0, g1 = start // GROUP, (start + n) // GROUP
+    if g1 <= g0:
+        return None
+    dev = table_row.device
+    pos = torch.arange(g0 * GROUP, g1 * GROUP, device=dev).view(g1 - g0, GROUP)
+    from_ring = -2 - (ring_row0 + geo.slot(pos))
+    src = torch.where(pos < geo.S, torch.full_like(pos, -1), torch.where(pos >= start, pos - start, from_ring))
+    dst = table_row[pos // page].long() * page + pos % page
+    return src.contiguous(), dst.contiguous()
+
+
 @dataclass
 class StepPlan:
     """what one decode step of a batch needs on the device (views of the planner's persistent buffers)"""
@@ -321,6 +340,16 @@ class DecodeLayer:
             keep, where = self.geo.kept(kv.shape[0], kv.device)
             self.ring[req].index_copy_(0, where, self.center_rows(kv[keep]))
 
+    def prefill_chunk(self, kv, slots, req: int, start: int):
+        """the next n tokens of request row `req`'s prompt, positions [start, start + n): every token to its page; the
+        sinks among them and the newest W of the prompt so far also to the BF16 row"""
+        self.write_pages(kv, slots)
+        if self.ring is not None:
+            n = kv.shape[0]
+            pos = start + torch.arange(n, device=kv.device)
+            keep = (pos < self.geo.S) | (pos >= start + n - self.geo.W)
+            self.ring[req].index_copy_(0, self.geo.slot(pos[keep]), self.center_rows(kv[keep]))
+
     def update(self, kv, sp: StepPlan):
         """cache update of a decode step: the new tokens to their pages and to their BF16 slots"""
         self.write_pages(kv, sp.slots)
@@ -381,6 +410,21 @@ class KiviDecodeLayer:
             src = torch.where(pos < self.geo.S, torch.full_like(pos, -1), pos).contiguous()     # sinks stay BF16 only
             KIVI.k_encode(kv, src, slots[:whole * GROUP].view(whole, GROUP).contiguous(), self.qs, self.lz, self.scale,
                           self.pool, self.Hkv, D, f8=self.f8)
+
+    def prefill_chunk(self, kv, slots, req: int, start: int, table_row):
+        """the next n tokens of request `req`'s prompt, positions [start, start + n): values of every token, the key
+        groups the chunk completes (their earlier positions read from the ring, which therefore takes the chunk's own
+        rows only afterwards), then the sinks and the newest W rows of the prompt so far in BF16"""
+        n = kv.shape[0]
+        KIVI.v_write(kv, slots, self.co, None, self.pool, self.Hkv, D, f8=self.f8)
+        flat = self.ring.view(-1, 2 * self.Hkv, D)
+        groups = chunk_key_groups(self.geo, start, n, req * self.geo.slots, table_row)
+        if groups is not None:
+            KIVI.k_encode(kv, groups[0], groups[1], self.qs, self.lz, self.scale, self.pool, self.Hkv, D, src2=flat,
+                          f8=self.f8)
+        pos = start + torch.arange(n, device=kv.device)
+        keep = (pos < self.geo.S) | (pos >= start + n - self.geo.W)
+        flat.index_copy_(0, req * self.geo.slots + self.geo.slot(pos[keep]), kv[keep])
 
     def update(self, kv, sp: StepPlan):
         KIVI.v_write(kv, sp.slots, self.co, None, self.pool, self.Hkv, D, f8=self.f8)

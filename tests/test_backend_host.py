@@ -73,3 +73,34 @@ def test_kivi_decode_groups():
             p = L - 32 + j
             assert int(md.group_dst[i, j]) == int(bt[i, p // 16]) * 16 + p % 16
             assert int(md.group_src[i, j]) == (-1 if p < S else int(req[i]) * T + BK.ring_slot(p, S, W))
+
+
+@pytest.mark.parametrize("S,W", [(4, 32), (0, 64), (4, 128)])
+def test_chunk_key_groups_against_a_position_walk(S, W):
+    """the key groups a prompt chunk completes: every position's source (chunk row, ring row of an earlier chunk, or
+    sink) and page slot, against a walk over positions with a model of which chunk brought which position"""
+    geo = BK.RingGeometry(S, W)
+    T = S + W
+    rng = np.random.default_rng(5 + S + W)
+    bt = torch.from_numpy(rng.permutation(64).astype(np.int32))
+    for req, cuts in ((0, [0, 150]), (2, [0, 50, 87, 150]), (1, [0, 31, 32, 33, 97, 128, 129]), (3, [0, 64, 65, 200, 201, 233])):
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            got = BK.chunk_key_groups(geo, a, b - a, req * T, bt)
+            groups = [g for g in range(b // 32) if 32 * g + 31 >= a]          # completed by [a, b): last position inside it
+            if not groups:
+                assert got is None
+                continue
+            src, dst = got
+            assert src.shape == dst.shape == (len(groups), 32) and src.dtype == dst.dtype == torch.int64
+            for i, g in enumerate(groups):
+                for j in range(32):
+                    p = 32 * g + j
+                    assert int(dst[i, j]) == int(bt[p // 16]) * 16 + p % 16
+                    if p < S:
+                        want = -1
+                    elif p >= a:
+                        want = p - a
+                    else:
+                        assert a - p <= W, "an earlier position must still be in the window"
+                        want = -2 - (req * T + S + (p - S) % W)
+                    assert int(src[i, j]) == want, (req, a, b, g, j)

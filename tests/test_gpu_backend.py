@@ -190,3 +190,66 @@ def test_kivi_decode_steps_in_graph(dev, f8, big):
             assert np.abs(got[b] - ref).max() <= tol, (step, b, float(np.abs(got[b] - ref).max()), tol)
     print(f"\nkivi backend steps (f8={f8}, large row x{big:g}): worst max |err| / (1e-2 max |ref|) = {worst:.3f}", flush=True)
     assert encoded == 2                                               # lengths 64 and 96 were reached
+
+
+@pytest.mark.parametrize("kind,S,W,center", [("konlya2", 4, 16, True), ("int4a", 0, 8, False), ("konly", 2, 0, False)])
+def test_chunked_prefill_equals_whole_prompt(dev, kind, S, W, center):
+    """a prompt that arrives in chunks leaves the same page bytes and the same BF16 rows as the prompt in one piece"""
+    from flagrot_releaser_amd import backend as BK
+    Hkv, G, R, n, cuts = 2, 4, 2, 150, [0, 50, 87, 88, 150]
+    g = torch.Generator().manual_seed(51)
+    nblk = (n + P - 1) // P
+    init = torch.randint(0, 256, (nblk + 3, Hkv, PG.chunk_bytes(kind, P)), dtype=torch.uint8, generator=g)
+    row = torch.randperm(nblk + 3, generator=g)[:nblk].int()
+    slots = (row.long()[torch.arange(n) // P] * P + torch.arange(n) % P).to(dev)
+    kw = {}
+    if BK.is_static(kind):
+        kw["wmask"] = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8).to(dev)
+    else:
+        Cq, co = spd_calib(Hkv, g)
+        kw.update(CT=Cq.transpose(1, 2).contiguous().to(dev), co=co.to(dev))
+    if center:
+        kw["kmu"] = (1.5 * torch.randn(Hkv, 128, generator=g)).to(dev)
+    kv = make_kv(n, Hkv, g, edge=True).to(dev)
+    layers = []
+    for _ in range(2):
+        planner = BK.StepPlanner(kind, Hkv, G, n + 8, 4, R, S, W, dev)
+        layers.append(BK.DecodeLayer(kind, Hkv, G, init.clone().to(dev), planner, **kw))
+    whole, chunked = layers
+    whole.prefill(kv, slots, 1)
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        chunked.prefill_chunk(kv[a:b], slots[a:b], 1, a)
+    torch.cuda.synchronize()
+    assert torch.equal(whole.pool, chunked.pool)
+    if S + W:
+        assert torch.equal(whole.ring, chunked.ring)
+
+
+@pytest.mark.parametrize("f8", [False, True], ids=["f16meta", "f8meta"])
+def test_kivi_chunked_prefill_equals_whole_prompt(dev, f8):
+    """KIVI-style pages: a prompt in chunks -- a chunk may start inside a 32-token key group, whose earlier positions
+    the encoder then reads from the BF16 ring -- leaves the same page bytes (values, key codes, key meta, flags) and the
+    same BF16 rows as the prompt in one piece"""
+    from flagrot_releaser_amd import backend as BK
+    from flagrot_releaser_amd import kivi as KV
+    from tests.test_gpu_kivi import _calib, _kv
+    Hkv, G, R, S, W, n = 2, 4, 2, 4, 32, 150
+    g = torch.Generator().manual_seed(52)
+    nblk = (n + P - 1) // P
+    row = torch.randperm(nblk + 3, generator=g)[:nblk].int()
+    slots = (row.long()[torch.arange(n) // P] * P + torch.arange(n) % P).to(dev)
+    qs, lz, co = _calib(Hkv, 24, g)
+    kv = _kv(n, Hkv, g, big=20.0).to(dev)
+    for cuts in ([0, 50, 87, 88, 150], [0, 31, 33, 64, 97, 150], [0, 150]):
+        layers = []
+        for _ in range(2):
+            pool = torch.zeros(nblk + 3, Hkv, KV.chunk_bytes(128, f8), dtype=torch.uint8, device=dev)
+            planner = BK.StepPlanner("kivi2", Hkv, G, n + 8, 4, R, S, W, dev)
+            layers.append(BK.KiviDecodeLayer(Hkv, G, pool, planner, qs.to(dev), lz.to(dev), co.to(dev), f8=f8))
+        whole, chunked = layers
+        whole.prefill(kv, slots, 1)
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            chunked.prefill_chunk(kv[a:b], slots[a:b], 1, a, row.to(dev))
+        torch.cuda.synchronize()
+        assert torch.equal(whole.pool, chunked.pool), cuts
+        assert torch.equal(whole.ring, chunked.ring), cuts
