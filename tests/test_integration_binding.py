@@ -1,5 +1,5 @@
-"""The binding tables a maintainer of the reference plugin is told to use, taken literally out of INTEGRATION.md:
-every `L.<entry point>.argtypes = [...]` line is parsed from the document, compared type by type with the declaration
+"""The binding tables a maintainer of the reference plugin is told to use, taken literally out of the integration
+notes at the repository root (NOTES below): every `L.<entry point>.argtypes = [...]` line is parsed from the document, compared type by type with the declaration
 in include/*.h (CPU), and used -- on a fresh ctypes handle, without this package's own loader -- for one writer call
 and one decode call checked against the oracle (GPU).  A typo in the document fails here."""
 import ctypes
@@ -13,10 +13,11 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CT = {"P": ctypes.c_void_p, "I": ctypes.c_int, "LL": ctypes.c_longlong, "F": ctypes.c_float}
 LIB_OF_PREFIX = {"fr": "kernels", "kv": "kivi", "frmq": "mq"}
+NOTES = "INTEGRATION.md"
 
 
 def documented_tables():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, NOTES)).read()
     out = {}
     for name, body in re.findall(r"L\.(\w+)\.argtypes\s*=\s*\[([^\]]*)\]", text):
         out[name] = [t.strip() for t in body.split(",") if t.strip()]
@@ -59,7 +60,7 @@ def test_documented_tables_match_the_headers():
     for name, types in tables.items():
         assert name in decl, f"{name} is documented but not declared in include/"
         assert all(t in CT for t in types), (name, types)
-        assert types == decl[name], f"{name}: INTEGRATION.md says {types}, the header declares {decl[name]}"
+        assert types == decl[name], f"{name}: the notes say {types}, the header declares {decl[name]}"
 
 
 def test_documented_tables_match_the_front_ends():
