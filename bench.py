@@ -455,6 +455,36 @@ def run_flagrot(args, torch, dev, workload, steps, warmup, plans=("own",)):
     first["writer"] = {"decode_step_us": round(e0.elapsed_time(e1) / 20 * 1e3, 2), "decode_step_tokens": B,
                        "prefill_fill_s": round(fill_s, 3), "prefill_tokens": B * L,
                        "note": "prefill_fill_s includes synthetic input generation"}
+    # one prefill-sized call (a sequence's first n_pre tokens, consecutive slots of its pages) on resident inputs: the
+    # exact selecting writer and, at head dim 128, the screened one (same bytes); into the last cache copy, after
+    # everything that reads the caches
+    n_pre = min(L, 8192)
+    kv_pre = synth_kv(n_pre, g, dev, torch, mu=kmu, hkv=HKV, dh=DH)
+    pos = torch.arange(n_pre, device=dev)
+    slots_pre = (bt[0].long()[pos // P] * P + pos % P).contiguous()
+
+    def writer_us(call, reps=10):
+        for _ in range(2):
+            call()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            call()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3
+
+    token_bytes = 2 * HKV * DH * 2 + HKV * cell                # bf16 K and V rows in, one page cell per KV head out
+    legs = {"exact": lambda: K.cb_write(kv_pre, slots_pre, CT, co, kind, pools[-1], P, kmu=kmu)}
+    if DH == 128:
+        legs["screened"] = lambda: K.cb_write3(kv_pre, slots_pre, CT, co, None, None, kind, pools[-1], P, split=False, kmu=kmu)
+    pre = {"tokens": n_pre, "kv_heads": HKV, "bytes_per_token_in_plus_out": token_bytes}
+    for leg, call in legs.items():
+        us_w = writer_us(call)
+        pre[leg] = {"us": round(us_w, 1), "Mtokens_per_s": round(n_pre / us_w, 2),
+                    "GBps_in_plus_out": round(n_pre * token_bytes / (us_w * 1e-6) / 1e9, 1)}
+    first["writer"]["prefill_call"] = pre
     return results
 
 
