@@ -238,7 +238,18 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
         }
         float sc[QB];
         key_phase<QM, K2>(S, cur, lane, sc);
-        const bool wide = softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
+        const bool wide = softmax_phase<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave, [&](float (&raw)[QB]) {
+          // (the quad's page ids are read again, behind an opaque value, and each chunk address is formed when its
+          // block's turn comes: kept from the loads they would occupy eight scalar registers across the key phase)
+          int quad = __builtin_amdgcn_readfirstlane(qi);
+          asm volatile("" : "+s"(quad));
+          const int i = min(PPQ * quad + (lane & (PPQ - 1)), npg - 1);
+          int entry = i < BT_CACHE ? S.btc[min(i, BT_CACHE - 1)] : bt[pg0 + i];
+          rescore_fine<QM, K2, P, 1>(S, cur.vs, lane, raw, [&](int blk) {
+            const int page = __builtin_amdgcn_readlane(entry, P == 16 ? blk : blk >> 1);
+            return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
+          });
+        });
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
         // path (past the range chunks_of names the range's last page again, a cache hit nobody uses): were they inside
         // a branch, the wait counts after the join would be those of the path without them, and the value phase

@@ -224,7 +224,17 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
         }
         float sc[2][QB];
         key_phase8<QM, K2>(S, cur, lane, sc);
-        const bool wide = softmax_phase8<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave);
+        const bool wide = softmax_phase8<QM>(S, st, cur, sc, valid, qs20, sc0, lane, wave, [&](float (&raw)[2 * QB]) {
+          // (as in k_decode: page ids read again behind an opaque value, a chunk address per block when its turn comes)
+          int quad = __builtin_amdgcn_readfirstlane(qi);
+          asm volatile("" : "+s"(quad));
+          const int i = min(PPQ * quad + (lane & (PPQ - 1)), npg - 1);
+          int entry = i < BT_CACHE ? S.btc[min(i, BT_CACHE - 1)] : bt[pg0 + i];
+          rescore_fine<QM, K2, P, 2>(S, cur.vs, lane, raw, [&](int blk) {
+            const int page = __builtin_amdgcn_readlane(entry, P == 16 ? blk : blk >> 1);
+            return (const uint8_t*)(pool + (static_cast<long long>(page) * p.Hkv + kvh) * L::CHUNK);
+          });
+        });
       
         // The key registers are free: the next quad's keys fly during the value phase.  The loads are issued on every
         // path (past the range chunks_of names the range's last page again, a cache hit nobody uses): were they inside

@@ -406,12 +406,99 @@ DEVI void write_strips(SM& S, const uint16_t (&vs)[QBLK<QM>], const float (&pe)[
   }
 }
 
+// The raw score sums of key_scores keep about 14.6 bits below the largest query x code product of an instruction (the
+// code fields are fp16 denormals with up to 10 leading zeros, and the matrix pipe keeps 24 bits below the largest NOMINAL
+// exponent; value_phase has the mechanism), and the key scale multiplies what is lost: nothing on ordinary scores, but
+// 0.03-0.1 log2 units on a score of a thousand, which moves per cent of the weight where two such tokens compete.  A quad
+// that holds a score above FINE_SCORE (softmax_phase: one compare on the maximum it forms anyway) is scored again with
+// the code operands times 2^8, which the scale multiplication takes back: the fields sit 8 bits higher in their fp16
+// words, the window 8 bits lower.  Block by block, one group at a time, codes and scale words fetched again and the
+// query operands read again, all behind a value the compiler cannot see through: nothing of the ordinary pass stays in
+// registers for this one, and this pass needs fewer registers than the ordinary one.
+// chunk_of(b): the chunk address of block b's page (wave uniform), formed when block b's turn comes: four addresses
+// at once are eight scalar registers, and those are as short as the vector ones in these kernels.
+constexpr float FINE_SCORE = 64.f;       // log2 units
+// NT: q tiles of 4 heads that share the unpacked words (k_decode: 1, raw[block]; k_decode8: 2, raw[tile][block])
+template <int QM, bool K2, int P, int NT, class SM, class ChunkOf>
+DEVI void rescore_fine(const SM& S, const uint16_t (&vs)[QBLK<QM>], int lane, float (&raw)[NT * QBLK<QM>], ChunkOf&& chunk_of) {
+  constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
+  int again = 0;
+  asm volatile("" : "+s"(again));
+  const int lane2 = lane + again;
+  const KOffs<QM, P> o0 = key_offsets<QM, P>(lane2);
+  uint32_t ok = o0.k, oks = o0.ks;
+  asm volatile("" : "+v"(ok), "+v"(oks));
+  const uint32_t zlane = (lane2 < 32) ? static_cast<uint32_t>(ZM) : 0u;
+#pragma unroll
+  for (int b = 0; b < QBLK<QM>; ++b) {
+    const int hp = P == 32 ? (b & 1) : 0;
+    uint32_t kc[KRegs<QM>::NW];
+    const uint8_t* chunk = chunk_of(b);
+    if constexpr (QM == QM_ASYM2) {
+      const u32x2 k = gload<u32x2>(chunk + static_cast<size_t>(ok + hp * 16 * 32));
+      kc[0] = k.x; kc[1] = k.y;
+    } else {
+      const u32x4 k = gload<u32x4>(chunk + static_cast<size_t>(ok + hp * 16 * 64));
+      kc[0] = k.x; kc[1] = k.y; kc[2] = k.z; kc[3] = k.w;
+    }
+    const u32x2 ks = gload<u32x2>(chunk + static_cast<size_t>(oks + hp * 16 * 8));
+    bool full = false;
+    if constexpr (K2) {      // whole_head_flags
+      unsigned long long m = __builtin_amdgcn_ballot_w64((vs[b] & 0x8000u) != 0u);
+      m |= m >> 32; m |= m >> 16; m &= 0xFFFFull; m |= m << 16; m |= m << 32;
+      full = __builtin_amdgcn_inverse_ballot_w64(m);
+    }
+    float sum[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) sum[t] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t x[4];
+      if constexpr (QM == QM_ASYM2) {
+        if (j & 1) UnpackD<QM>::run_hi(kc[j >> 1], x); else UnpackD<QM>::run(kc[j >> 1], x);
+      }
+      else UnpackD<QM>::run(kc[j], x);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = pk_mul(x[i], 0x5C005C00u);       // times 2^8: exact, the fields have at most 10 bits
+      const half8 kb = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
+      const uint32_t kw = (j & 2) ? ks.y : ks.x;
+      const uint32_t zz = pk_mul(kw & (zlane << (16 * (j & 1))), 0x5C005C00u);
+      const float scale = fabsf(word_value(kw, j)) * 0.00390625f;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        half8 qh, ql, qz;
+        if constexpr (NT == 1) {
+          qh = __builtin_bit_cast(half8, S.qhi[j][lane2]); ql = __builtin_bit_cast(half8, S.qlo[j][lane2]);
+          if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[j][lane2]);
+        } else {
+          qh = __builtin_bit_cast(half8, S.qhi[t][j][lane2]); ql = __builtin_bit_cast(half8, S.qlo[t][j][lane2]);
+          if constexpr (ZM != 0) qz = __builtin_bit_cast(half8, S.qz[t][j][lane2]);
+        }
+        f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh, kb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql, kb, a, 0, 0, 0);
+        if constexpr (ZM != 0)
+          a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qz, __builtin_bit_cast(half8, make_uint4(zz, 0u, 0u, 0u)), a, 0, 0, 0);
+        float pick = a[0];
+        if constexpr (K2) {
+          const bool h32 = (kw >> (16 * (j & 1) + 15)) & 1u;
+          pick = full ? a[2] : (h32 ? a[1] : a[0]);
+        }
+        sum[t] += pick * scale;
+        __builtin_amdgcn_sched_barrier(0);     // in program order: scheduled freely, several steps' operands are formed ahead
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) raw[t * QBLK<QM> + b] = sum[t];
+  }
+}
+
 // online softmax step for the quad, lane = (token, head x): the running maximum is only re-reduced when some lane
 // beats it; then p' = p * V scale per group as fp16 and the zero points go to the wave's strips in V^T token order.
 // qs20 = qscale * 2^20 (the factor the raw score sums lack); sc0 lowers the scores of odd tokens by SH (below).
-template <int QM, class SM>
+// rescore(raw): the quad's raw score sums again through rescore_fine (the caller knows the quad's chunk addresses)
+template <int QM, class SM, class Rescore>
 DEVI bool softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QBLK<QM>], const bool (&valid)[QBLK<QM>],
-                        float qs20, float sc0, int lane, int wave) {
+                        float qs20, float sc0, int lane, int wave, Rescore&& rescore) {
   constexpr int QB = QBLK<QM>;
   bool beat = false;
   float mx = -INFINITY;
@@ -419,6 +506,18 @@ DEVI bool softmax_phase(SM& S, WaveState& st, const KRegs<QM>& r, float (&sc)[QB
   for (int b = 0; b < QB; ++b) {
     sc[b] = valid[b] ? sc[b] * qs20 + sc0 : -INFINITY;
     mx = fmaxf(mx, sc[b]);
+  }
+  if constexpr (QM == QM_ASYM2) {      // rescore_fine has the reason, and why the 2-bit pages only
+    if (__builtin_expect(__any(mx > FINE_SCORE), 0)) {
+      float raw[QB];
+      rescore(raw);
+      mx = -INFINITY;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        sc[b] = valid[b] ? raw[b] * qs20 + sc0 : -INFINITY;
+        mx = fmaxf(mx, sc[b]);
+      }
+    }
   }
   beat = mx > st.m;
   // The state is multiplied every time (by 1 unless the maxima moved): modifying it only inside the rare branch makes
@@ -736,9 +835,9 @@ DEVI void key_phase8(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[2][Q
 }
 
 // softmax step of both halves; the strips take p * V-scale of heads x and 4 + x for all four groups
-template <int QM, class SM>
+template <int QM, class SM, class Rescore>
 DEVI bool softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[2][QBLK<QM>], const bool (&valid)[QBLK<QM>],
-                         float qs20, float sc0, int lane, int wave) {
+                         float qs20, float sc0, int lane, int wave, Rescore&& rescore) {
   constexpr int QB = QBLK<QM>;
   constexpr int ZM = QM == QM_ASYM4 ? 15 : QM == QM_ASYM2 ? 3 : 0;
   float mx[2];
@@ -751,8 +850,24 @@ DEVI bool softmax_phase8(SM& S, WaveState8& st, const KRegs<QM>& r, float (&sc)[
       sc[t][b] = valid[b] ? sc[t][b] * qs20 + sc0 : -INFINITY;
       mx[t] = fmaxf(mx[t], sc[t][b]);
     }
-    beat = beat || mx[t] > st.m[t];
   }
+  if constexpr (QM == QM_ASYM2) {      // as in softmax_phase
+    if (__builtin_expect(__any(fmaxf(mx[0], mx[1]) > FINE_SCORE), 0)) {
+      float raw[2 * QB];
+      rescore(raw);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        mx[t] = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+          sc[t][b] = valid[b] ? raw[t * QB + b] * qs20 + sc0 : -INFINITY;
+          mx[t] = fmaxf(mx[t], sc[t][b]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t) beat = beat || mx[t] > st.m[t];
   float al[2] = {1.f, 1.f}, az0[2] = {1.f, 1.f}, az1[2] = {1.f, 1.f}, am[2] = {1.f, 1.f};
   if (__builtin_expect(__any(beat), 0)) {
 #pragma unroll

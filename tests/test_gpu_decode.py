@@ -31,7 +31,7 @@ HARD_ROWS = 2.0      # element-wise bound of the rows that read the adversarial 
 
 
 def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None, P=P16,
-             hard_rows=None):
+             hard_rows=None, twin=None):
     from flagrot_releaser_amd import kernels as K
     g = torch.Generator().manual_seed(seed)
     B = len(lens)
@@ -40,7 +40,10 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
     pool = torch.randint(0, 256, (num_pages, Hkv, PG.chunk_bytes(fmt, P)), dtype=torch.uint8, generator=g).to(dev)
     bt = alloc_tables(lens, num_pages, g, P)
     if bt_shared:
-        bt = bt[:1].expand(B, -1)
+        # every sequence reads the table row of the longest one (a shorter row would name page 0 for the positions past
+        # its end, and the writer below would be handed the same slot several times)
+        first = max(range(B), key=lambda b: lens[b])
+        bt = bt[first:first + 1].expand(B, -1)
         if bt_shared != "stride0":
             bt = bt.contiguous()
     mask = (torch.rand(2 * Hkv, 4, generator=g) < 0.5).to(torch.uint8)
@@ -51,7 +54,15 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
         n = max(lens) if bt_shared else lens[b]
         if n == 0:
             continue
-        kv = make_kv(n, Hkv, g, edge=(b == 0)).to(dev)
+        kv = make_kv(n, Hkv, g, edge=(b == 0))
+        if twin is not None and b == 0:
+            # a second token with token 4's key (x 300 group included) up to a small change in another group, and values of
+            # its own: two keys whose scores are in the hundreds and a few hundredths apart, so the weights between the
+            # two value rows hang on the last bits of those scores
+            kv[twin] = kv[4]
+            kv[twin, :Hkv, 64:96] += (0.05 * torch.randn(Hkv, 32, generator=g)).bfloat16()
+            kv[twin, Hkv:] = torch.randn(Hkv, 128, generator=g).bfloat16()
+        kv = kv.to(dev)
         sl = slots_of(bt, b, n, P).to(dev)
         if mode == "static":
             K.v2_write(kv, sl, mask.to(dev), 32, pool, P, fmt=fmt)
@@ -122,6 +133,18 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
 
 
 LENS = [1, 15, 16, 17, 63, 64, 65, 200, 1000, 3, 511]
+
+
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya2"), ("static", "int2a"), ("codebook", "konlya"), ("static", "int4a")])
+def test_two_keys_with_very_large_scores(dev, mode, fmt):
+    """Two tokens share a key group scaled x 300: their scores are in the hundreds of log2 units and a few units apart.
+    On the 2-bit pages the ordinary score products are 0.03-0.1 units off there (the key scale multiplies what the
+    products lose), which moves per cent of the weight between the two; the quads that hold such scores are scored
+    again with the code operands eight bits higher (decode_tiles.hpp: rescore_fine).  4- and 8-head tiles, pages of 16
+    and 32, one and several splits."""
+    for seed, (G, Hkv), P, nsplit, twin in ((31, (4, 2), 16, None, 21), (32, (8, 2), 16, 2, 70), (33, (4, 4), 32, None, 40),
+                                           (34, (6, 2), 16, None, 9), (35, (4, 2), 16, 3, 130)):
+        run_case(dev, mode, [300, 40], fmt, seed=seed, G=G, Hkv=Hkv, P=P, nsplit=nsplit, twin=twin)
 
 
 @pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])

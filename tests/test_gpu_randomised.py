@@ -5,8 +5,8 @@ where it belongs (the rescale factor of the 4-bit pages in the decode kernels; t
 tests on a dozen rows).
 
 Bars: the writers byte for byte; the decode attention as in tests/test_gpu_decode.py, with the rows that read the
-adversarial tokens held to 6 times the element-wise bar instead of 2 (open-ended runs: 1 % of such rows above 1, largest
-4.4, on the 2-bit pages); the KIVI decode attention at the reference's row bar and 6 times the element-wise bar (every
+adversarial tokens held to 6 times the element-wise bar instead of 2 (open-ended runs: 0.3-0.5 % of such rows above 1,
+all on the 2-bit pages, largest 1.8 apart from one shape of the static 2-bit format at 17 in a single channel); the KIVI decode attention at the reference's row bar and 6 times the element-wise bar (every
 sequence holds a row scaled x200; open-ended runs: 2.6 % of the shapes above 1, largest 4.2); the multi-query prefill at
 the bars of tests/test_gpu_mq.py."""
 import random
