@@ -137,11 +137,12 @@ LENS = [1, 15, 16, 17, 63, 64, 65, 200, 1000, 3, 511]
 
 @pytest.mark.parametrize("mode,fmt", [("codebook", "konlya2"), ("static", "int2a"), ("codebook", "konlya"), ("static", "int4a")])
 def test_two_keys_with_very_large_scores(dev, mode, fmt):
-    """Two tokens share a key group scaled x 300: their scores are in the hundreds of log2 units and a few units apart.
-    On the 2-bit pages the ordinary score products are 0.03-0.1 units off there (the key scale multiplies what the
-    products lose), which moves per cent of the weight between the two; the quads that hold such scores are scored
-    again with the code operands eight bits higher (decode_tiles.hpp: rescore_fine).  4- and 8-head tiles, pages of 16
-    and 32, one and several splits."""
+    """Two tokens share a key group scaled x 300 and differ a little in another group: scores in the hundreds of log2
+    units, a few hundredths apart, value rows of their own.  On the 2-bit pages every quad that holds such a score is
+    scored a second time with the code operands eight bits higher (decode_tiles.hpp: rescore_fine); this test runs that
+    pass in 4- and 8-head tiles, on pages of 16 and 32, with one and several splits, and holds its rows to the bars of
+    the other adversarial rows.  (It does not by itself show what the second pass gains: two tokens with the same codes
+    in the scaled group lose the same bits.  The randomised runs do.)"""
     for seed, (G, Hkv), P, nsplit, twin in ((31, (4, 2), 16, None, 21), (32, (8, 2), 16, 2, 70), (33, (4, 4), 32, None, 40),
                                            (34, (6, 2), 16, None, 9), (35, (4, 2), 16, 3, 130)):
         run_case(dev, mode, [300, 40], fmt, seed=seed, G=G, Hkv=Hkv, P=P, nsplit=nsplit, twin=twin)
