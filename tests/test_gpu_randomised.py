@@ -5,10 +5,11 @@ where it belongs (the rescale factor of the 4-bit pages in the decode kernels; t
 tests on a dozen rows).
 
 Bars: the writers byte for byte; the decode attention as in tests/test_gpu_decode.py, with the rows that read the
-adversarial tokens held to 6 times the element-wise bar instead of 2 (open-ended runs: 0.3-0.5 % of such rows above 1,
-all on the 2-bit pages, largest 1.8 apart from one shape of the static 2-bit format at 17 in a single channel); the KIVI decode attention at the reference's row bar and 6 times the element-wise bar (every
-sequence holds a row scaled x200; open-ended runs: 2.6 % of the shapes above 1, largest 4.2); the multi-query prefill at
-the bars of tests/test_gpu_mq.py."""
+adversarial tokens held to 3 times the element-wise bar where that file's own cases hold them to 2 (largest on these
+seeds: 0.99; open-ended runs: 0.3-0.5 % of such rows above 1, largest 1.8 apart from a few shapes of the static 2-bit
+format at 8-17 in a single channel); the KIVI decode attention at the reference's row bar and 6 times the element-wise
+bar (every sequence holds a row scaled x200; open-ended runs: 2.6 % of the shapes above 1, largest 4.2); the
+multi-query prefill at the bars of tests/test_gpu_mq.py."""
 import random
 
 import numpy as np
@@ -47,7 +48,7 @@ def test_decode_shapes(dev):
         print(f"\nshape {n}: {mode} {fmt} P={P} G={G} Hkv={Hkv} lens={lens} win={win} kv_start={kv_start} nsplit={nsplit} "
               f"shared={shared} seed={seed}", flush=True)
         run_case(dev, mode, lens, fmt, win=win, bt_shared=shared, seed=seed, G=G, Hkv=Hkv, kv_start=kv_start, nsplit=nsplit,
-                 P=P, hard_rows=6.0)
+                 P=P, hard_rows=3.0)
 
 
 def test_decode_shapes_head_dim_256(dev):
