@@ -96,11 +96,46 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   // body workgroups of a (sequence, KV head, q tile) share its whole page range and draw quads from the slot's
   // counter: the split plan then only says how many workgroups there are.  FLAGROT_DECODE_STATIC=1 keeps fixed
   // ranges, FLAGROT_WG_WAVES=4 | 16 forces a workgroup size (above 4: the large one).
-  const int nparts = nsplit + (tail != nullptr ? 1 : 0);
   static const bool force_static = getenv("FLAGROT_DECODE_STATIC") != nullptr && getenv("FLAGROT_DECODE_STATIC")[0] == '1';
   static const int env_waves = getenv("FLAGROT_WG_WAVES") != nullptr ? atoi(getenv("FLAGROT_WG_WAVES")) : 0;
-  const long long wgs = static_cast<long long>(B) * Hkv * ntile * nsplit;
-  const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && wgs <= device_cus());
+  static const bool replan = !(getenv("FLAGROT_REPLAN") != nullptr && getenv("FLAGROT_REPLAN")[0] == '0');
+  // A plan of more workgroups than CUs is run as fewer, longer splits where shape (a) then applies.  The reference front
+  // end caps a chunk at 8192 tokens (vllm_flagrot/kernels.py:74, MAX_CHUNK), so a context beyond 8192 tokens always
+  // arrives as two or more splits per (sequence, KV head, q tile) pair -- also where 256 pairs fill the CUs by
+  // themselves (B = 32, 8 KV heads), the case in which one large workgroup per CU streaming the whole sequence is the
+  // fastest shape there is (B = 32, L = 16 k ... 64 k on the 4-bit pages: 0.59-0.65 -> 0.76-0.79 of the bandwidth).
+  //  * pairs <= CUs: CUs / pairs splits per pair, one round of large workgroups (every format);
+  //  * pairs > CUs, 4-bit pages (launches bound by memory; the 2-bit ones are bound by vector issue and gain nothing):
+  //    the fewest splits (the longest chunks, >= 4096 tokens) whose large workgroups fill their last round of CUs to
+  //    90 % -- B = 64, L = 8 k ... 32 k: 0.61-0.67 -> 0.72-0.79; a round and a quarter of them would be slower than the
+  //    small workgroups (B = 40: 82 -> 89 us), so such plans stay as they are.
+  // The splits that are run are the first `nsplit` of the caller's layout: never more than the caller planned, so
+  // partials and tickets stay inside what the caller sized.  FLAGROT_REPLAN=0 switches this off (experiments).
+  const long long pairs = static_cast<long long>(B) * Hkv * ntile;
+  const long long cus = device_cus();
+  bool rounds = false;                       // large workgroups although there are more of them than CUs
+  if (replan && env_waves == 0 && !(variant & HD256) && pairs * nsplit > cus) {
+    const long long span = static_cast<long long>(nsplit) * chunk;
+    auto chunk_for = [&](long long ns) { return static_cast<int>(((span + ns - 1) / ns + 63) / 64 * 64); };   // a multiple of both page sizes
+    int fewer = 0;
+    if (span < (1ll << 30)) {
+      if (pairs <= cus) {
+        if (chunk_for(cus / pairs) >= decode_big_chunk()) fewer = static_cast<int>(cus / pairs);   // >= 1 and < nsplit
+      } else if (!fmt_int2(fmt)) {
+        for (int ns = 1; ns <= nsplit && ns <= 8 && chunk_for(ns) >= 4096; ++ns) {
+          const long long wg = pairs * ns, full = (wg + cus - 1) / cus * cus;
+          if (wg * 10 >= full * 9) { fewer = ns; rounds = true; break; }
+        }
+      }
+    }
+    if (fewer > 0) {
+      chunk = chunk_for(fewer); nsplit = fewer;
+      p.nsplit = nsplit; p.chunk = chunk;
+    }
+  }
+  const int nparts = nsplit + (tail != nullptr ? 1 : 0);
+  const long long wgs = pairs * nsplit;
+  const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
   const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;
   // the split merge goes through the caller's workspace: partials, their (max, sum) pairs and, at head dim 128, the ticket
   if (nparts > 1 && (opart == nullptr || mlpart == nullptr || (!(variant & HD256) && counter == nullptr)))

@@ -148,6 +148,27 @@ def test_two_keys_with_very_large_scores(dev, mode, fmt):
         run_case(dev, mode, [300, 40], fmt, seed=seed, G=G, Hkv=Hkv, P=P, nsplit=nsplit, twin=twin)
 
 
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("static", "int2a")])
+def test_plans_the_library_runs_as_fewer_longer_splits(dev, mode, fmt):
+    """A plan of more workgroups than CUs whose (sequence, KV head, q tile) pairs fit the CUs by themselves (256 pairs
+    here) is run as one large workgroup per pair over the whole sequence (csrc/capi.hip: fr_v2_attn) -- the reference
+    front end never plans chunks beyond 8192 tokens, so every longer context reaches the library like this.  Ragged
+    lengths, an empty and a one-page sequence, BF16 rows, kv_start; the caller's workspace is sized for ITS plan."""
+    lens = [2300 - 37 * (b % 9) for b in range(32)]
+    lens[5], lens[17] = 0, 9
+    ns, ch = run_case(dev, mode, lens, fmt, seed=41, G=4, Hkv=8, nsplit=3, win=(20, 33), kv_start=4)
+    assert (ns, ch) == (3, 768)
+
+
+def test_large_workgroups_in_full_rounds(dev):
+    """4-bit pages, more pairs than CUs (40 sequences x 4 KV heads x 3 q tiles = 480), sequences of >= 4096 tokens: the
+    library runs large workgroups in rounds that fill the CUs to >= 90 % (here one split per pair, 480 of 512) instead
+    of the plan's small ones"""
+    lens = [4200 - 11 * (b % 7) for b in range(40)]
+    ns, ch = run_case(dev, "codebook", lens, "konlya", seed=42, G=12, Hkv=4)
+    assert ns * 480 > 256 and ns * ch >= 4200
+
+
 @pytest.mark.parametrize("kind", ["konly", "konlya", "konlya2"])
 def test_codebook_decode(dev, kind):
     run_case(dev, "codebook", LENS, kind, seed=1)
