@@ -505,6 +505,12 @@ def run_kivi(args, torch, dev, steps, warmup):
         B, L, Gq, HKV, DH = 16, 8192 + W, 6, 4, 256
         name = ("KIVI-style FlagRot INT2 paged decode at head dim 256" + (", FP8 meta" if f8 else "") +
                 f", 128-token BF16 residual, GQA 24q/4kv d=256, B={B} L={L} page=16 (no baseline configuration)")
+    elif getattr(args, "batch", 0) or getattr(args, "context", 0) or getattr(args, "gqa", 4) != 4:
+        # shape overrides for experiments (the reference micro-benchmark sweeps B and L at 32q/8kv): not a baseline configuration
+        B, L = getattr(args, "batch", 0) or B, (getattr(args, "context", 0) or L - W) + W
+        Gq = int(args.gqa) if (getattr(args, "batch", 0) or getattr(args, "context", 0)) else Gq
+        name = ("KIVI-style FlagRot INT2 paged decode" + (", FP8 meta" if f8 else "") + f", 128-token BF16 residual, GQA "
+                f"{Gq * HKV}q/{HKV}kv d=128, B={B} L={L} page=16 [shape override: not a baseline configuration]")
     CB = KV.chunk_bytes(DH, f8)
     g = torch.Generator(device=dev).manual_seed(3)
     Lp = L - W
@@ -741,8 +747,8 @@ def main():
     ap.add_argument("--mq-fmt", default="konlya", choices=["konlya", "int4a"])
     ap.add_argument("--f8", action="store_true", help="kivi: FP8-meta pages")
     ap.add_argument("--head-dim", type=int, default=128, choices=[128, 256], help="256 = the head dim 256 kernels (GQA 24q/4kv, the reference's test shape class); not a baseline configuration")
-    ap.add_argument("--batch", type=int, default=0, help="int4 / int2 workloads: another batch size (not a baseline configuration)")
-    ap.add_argument("--context", type=int, default=0, help="int4 / int2 workloads: another context length (not a baseline configuration)")
+    ap.add_argument("--batch", type=int, default=0, help="int4 / int2 / kivi workloads: another batch size (not a baseline configuration)")
+    ap.add_argument("--context", type=int, default=0, help="int4 / int2 / kivi workloads: another context length (kivi: cached tokens besides the 128 BF16 rows; not a baseline configuration)")
     ap.add_argument("--window", type=int, default=-1, help="int4 / int2 workloads: BF16 window tokens (0: no BF16 rows and no sinks; not a baseline configuration)")
     ap.add_argument("--gqa", type=int, default=4, help="int4 / int2 workloads: query heads per KV head (8 = tiles of 8 heads; not a baseline configuration)")
     ap.add_argument("--nsplit", type=int, default=0, help="override the planner's split count")
