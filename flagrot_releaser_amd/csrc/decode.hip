@@ -400,17 +400,7 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
     float M = pm, Lsum = pl, o0 = po[0], o1 = po[1];
     if (nparts > 1 && act) {
       const long long base = ((static_cast<long long>(b) * p.Hkv + kvh) * ntile + tt) * nparts;
-      M = -INFINITY;
-      for (int s = 0; s < nparts; ++s) M = fmaxf(M, __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      Lsum = 0.f; o0 = 0.f; o1 = 0.f;
-      for (int s = 0; s < nparts; ++s) {
-        const float ms = __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float ls = __hip_atomic_load(p.mlpart + (base + s) * 8 + 2 * oh + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float f = ms == -INFINITY ? 0.f : fexp2(ms - M);
-        Lsum += f * ls;
-        o0 += f * __hip_atomic_load(p.opart + (base + s) * 512 + oh * 128 + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        o1 += f * __hip_atomic_load(p.opart + (base + s) * 512 + oh * 128 + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      merge_parts(p.mlpart, p.opart, base, nparts, oh, lane, M, Lsum, o0, o1);
     }
     const float inv = Lsum > 0.f ? 1.f / Lsum : 0.f;
     o0 *= inv; o1 *= inv;
