@@ -244,23 +244,16 @@ DEVI void load_v(VRegs<QM>& r, const uint8_t* const (&chunk)[QBLK<QM>], int lane
 }
 
 // The split merge of one output thread (head oh, channels 2 lane and 2 lane + 1) over the nparts partials of its
-// (sequence, KV head, q tile): maxima first, then the weighted sums, the partials in their order.  Eight partials at a
-// time, every load of a batch in flight before the first is used and none under a condition (the batch's last
-// partial is read again in place of those past the end, with weight 0): one partial per turn of a loop waits a memory
-// latency per turn, and 32 splits then took 20 of the 28 us of a single-sequence launch.
+// (sequence, KV head, q tile), in their order.  Eight partials at a time, every load of a batch -- maxima, sums and
+// channels alike -- in flight before the first is used and none under a condition (the batch's last partial is read
+// again in place of those past the end, with weight 0); the running maximum moves from batch to batch and what was
+// summed so far is rescaled with it.  One partial per turn of a loop waits a memory latency per turn (32 splits then
+// took 20 of the 28 us of a single-sequence launch), and a pass for the maxima ahead of the sums is one latency more.
 DEVI void merge_parts(const float* mlpart, const float* opart, long long base, int nparts, int oh, int lane,
                       float& M, float& Lsum, float& o0, float& o1) {
   constexpr int NB = 8;
   auto ld = [](const float* q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-  M = -INFINITY;
-  for (int s0 = 0; s0 < nparts; s0 += NB) {
-    float m[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) m[k] = ld(mlpart + (base + min(s0 + k, nparts - 1)) * 8 + 2 * oh);
-#pragma unroll
-    for (int k = 0; k < NB; ++k) M = fmaxf(M, m[k]);
-  }
-  Lsum = 0.f; o0 = 0.f; o1 = 0.f;
+  M = -INFINITY; Lsum = 0.f; o0 = 0.f; o1 = 0.f;
   for (int s0 = 0; s0 < nparts; s0 += NB) {
     float m[NB], l[NB], a[NB], c[NB];
 #pragma unroll
@@ -271,6 +264,12 @@ DEVI void merge_parts(const float* mlpart, const float* opart, long long base, i
       a[k] = ld(opart + part * 512 + oh * 128 + 2 * lane);
       c[k] = ld(opart + part * 512 + oh * 128 + 2 * lane + 1);
     }
+    float top = M;
+#pragma unroll
+    for (int k = 0; k < NB; ++k) top = fmaxf(top, m[k]);          // (a partial read twice changes no maximum)
+    const float keep = M == -INFINITY ? 0.f : fexp2(M - top);      // nothing summed yet, or top is finite
+    M = top;
+    Lsum *= keep; o0 *= keep; o1 *= keep;
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
       const float f = (s0 + k < nparts && m[k] != -INFINITY) ? fexp2(m[k] - M) : 0.f;
