@@ -48,6 +48,9 @@ def test_kivi_library_exports_header_symbols():
     assert L.kv_abi_version() == 9
     assert L.kv_chunk_bytes(128) == 1552 and L.kv_chunk_bytes8(128) == 1280
     assert kivi.plan(16, 32768, 8, sms=256) == (6, 5472) and kivi.plan(1, 100, 8, sms=256)[1] == 256
+    # few pairs or short contexts: half the slots, 24 splits at most, 1024 tokens per split at least
+    assert kivi.plan(1, 32640, 8, sms=256) == (24, 1376) and kivi.plan(8, 8064, 8, sms=256) == (7, 1152)
+    assert kivi.plan(64, 2048, 8, sms=256) == (2, 1024)
     assert kivi.plan(16, 8192, 4, sms=256, D=256) == (7, 1184)         # two workgroups per CU at head dim 256, one of the 8 slots for the ring rows
 
 
