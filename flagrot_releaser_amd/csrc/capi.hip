@@ -133,9 +133,13 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
       p.nsplit = nsplit; p.chunk = chunk;
     }
   }
-  const int nparts = nsplit + (tail != nullptr ? 1 : 0);
   const long long wgs = pairs * nsplit;
   const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
+  // BF16 rows beside ONE split of large workgroups (4-head tiles, key-only formats: no rotation of the rows into a
+  // stored basis): the body's wavefronts take them themselves -- no second partial, no ticket, no merge
+  static const bool fuse_ok = !(getenv("FLAGROT_FUSE_TAIL") != nullptr && getenv("FLAGROT_FUSE_TAIL")[0] == '0');
+  p.fuse_tail = (fuse_ok && tail != nullptr && big && env_waves == 0 && nsplit == 1 && k2 && !p.tile8 && !(variant & HD256)) ? 1 : 0;
+  const int nparts = nsplit + ((tail != nullptr && !p.fuse_tail) ? 1 : 0);
   const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;
   // the split merge goes through the caller's workspace: partials, their (max, sum) pairs and, at head dim 128, the ticket
   if (nparts > 1 && (opart == nullptr || mlpart == nullptr || (!(variant & HD256) && counter == nullptr)))

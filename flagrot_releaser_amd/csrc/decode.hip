@@ -313,6 +313,27 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
         *reinterpret_cast<float4*>(o + d) = make_float4(st.ot[y][0], st.ot[y][1], st.ot[y][2], st.ot[y][3]);
       }
     }
+    if (p.fuse_tail) {      // uniform over the launch
+      // The BF16 rows of the sequence, this wavefront's share, folded into what it has just left in LDS: a workgroup
+      // of their own costs its whole life -- arguments, rows, epilogue, partial, ticket, merge: 10 us behind the 43-53 us
+      // of the body at B = 32 x 8 k -- where these rows are a few hundred KB per sequence.
+      // (more rows per step -- nine, so that 144 rows are one step of 16 wavefronts -- measured no better: 62.1 against
+      // 60.4 us)
+      float m[4], l[4], o[4][2];
+      tail_partial<NW>(p, b, kvh, tile, m, l, o);
+      wave_lds_sync();
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const float mp = S.m[wave][h], lp = S.l[wave][h];
+        float2* slot = reinterpret_cast<float2*>(S.o(wave, h)) + lane;
+        const float2 op = *slot;
+        const float top = fmaxf(mp, m[h]);
+        const float fp = mp == -INFINITY ? 0.f : fexp2(mp - top), ft = m[h] == -INFINITY ? 0.f : fexp2(m[h] - top);
+        *slot = make_float2(op.x * fp + o[h][0] * ft, op.y * fp + o[h][1] * ft);
+        wave_lds_sync();      // every lane has read the pair before lane 0 replaces it
+        if (lane == 0) { S.m[wave][h] = top; S.l[wave][h] = lp * fp + l[h] * ft; }
+      }
+    }
   } else {
     float m[4], l[4], o[4][2];
     tail_partial<NW>(p, b, kvh, tile, m, l, o);
@@ -444,7 +465,7 @@ template <int QM, bool K2>
 int launch_qm(const DecodeParams& p, hipStream_t st) {
   if (p.page != 16 && p.page != 32) return -5;
   const int ntile = (p.gqa + 3) / 4;
-  const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
+  const int nparts = p.nsplit + ((p.tail != nullptr && !p.fuse_tail) ? 1 : 0);
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
   if (p.page == 32) {
