@@ -313,10 +313,11 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
         *reinterpret_cast<float4*>(o + d) = make_float4(st.ot[y][0], st.ot[y][1], st.ot[y][2], st.ot[y][3]);
       }
     }
-    if (p.fuse_tail) {      // uniform over the launch
-      // The BF16 rows of the sequence, this wavefront's share, folded into what it has just left in LDS: a workgroup
-      // of their own costs its whole life -- arguments, rows, epilogue, partial, ticket, merge: 10 us behind the 43-53 us
-      // of the body at B = 32 x 8 k -- where these rows are a few hundred KB per sequence.
+    if (p.fuse_tail && split == 0) {      // uniform over the workgroup
+      // The BF16 rows of the sequence, this wavefront's share, folded into what it has just left in LDS (the first
+      // split's workgroup takes them): a workgroup of their own costs its whole life -- arguments, rows, epilogue,
+      // partial, ticket, merge: 10 us behind the 43-53 us of the body at B = 32 x 8 k -- where these rows are a few
+      // hundred KB per sequence.
       // (more rows per step -- nine, so that 144 rows are one step of 16 wavefronts -- measured no better: 62.1 against
       // 60.4 us)
       float m[4], l[4], o[4][2];

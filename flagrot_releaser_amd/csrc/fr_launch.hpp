@@ -62,7 +62,7 @@ struct DecodeParams {
   int dyn;                 // 1: the nsplit body workgroups of a (sequence, KV head, q tile) share its whole page range and
                            //    draw quads of 4 pages from the slot's counter; 0: split s owns tokens [s, s + 1) * chunk
   int wg_waves;            // wavefronts per workgroup: 4, or the large workgroup that fills a CU
-  int fuse_tail;           // 1: no workgroup of their own for the BF16 rows -- the wavefronts of the (only) body split take
+  int fuse_tail;           // 1: no workgroup of their own for the BF16 rows -- the wavefronts of the first body split take
                            //    them after their pages and fold them into their own partials (k_decode; key-only formats)
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
