@@ -207,6 +207,8 @@ def test_large_workgroup_shape(dev, mode, fmt):
     # (an empty sequence that has rows only, one of five tokens behind kv_start = 4, padding heads in the q tile)
     run_case(dev, mode, [2300, 0, 5, 2100], fmt, seed=25, G=3, Hkv=2, nsplit=1, win=(132, 6), kv_start=4)
     run_case(dev, mode, [2049, 2049], fmt, seed=26, Hkv=2, nsplit=1, win=(7, 3), bt_shared=True)
+    # two splits of 4544 tokens: the first split's workgroup takes the rows, its partial and the second split's are merged
+    run_case(dev, mode, [9000, 4200, 0], fmt, seed=27, Hkv=2, nsplit=2, win=(40, 5), kv_start=4)
 
 
 def test_block_table_beyond_the_lds_cache(dev):
