@@ -135,14 +135,14 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   }
   const long long wgs = pairs * nsplit;
   const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
-  // BF16 rows beside large workgroups (4-head tiles, key-only formats: no rotation of the rows into a stored basis):
+  // BF16 rows beside large workgroups (key-only formats: no rotation of the rows into a stored basis):
   // the wavefronts of the first split take them themselves -- one partial less, and with a single split no ticket and
   // no merge at all
   static const bool fuse_ok = !(getenv("FLAGROT_FUSE_TAIL") != nullptr && getenv("FLAGROT_FUSE_TAIL")[0] == '0');
   // (several splits: only where a split is long -- 4096 tokens measured: B = 8, L = 16 k 40.0 -> 38.4 us, B = 4, L = 32 k
   // 36.3 -> 33.6 -- since the first split's workgroup then ends later than the others; with 32 splits of 1024 tokens
   // of one sequence the rows' own workgroups were faster, 18.9 against 23.4 us)
-  p.fuse_tail = (fuse_ok && tail != nullptr && big && env_waves == 0 && k2 && !p.tile8 && !(variant & HD256) &&
+  p.fuse_tail = (fuse_ok && tail != nullptr && big && env_waves == 0 && k2 && !(variant & HD256) &&
                  (nsplit == 1 || chunk >= 4096)) ? 1 : 0;
   const int nparts = nsplit + ((tail != nullptr && !p.fuse_tail) ? 1 : 0);
   const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;

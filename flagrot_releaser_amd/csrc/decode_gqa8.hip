@@ -299,7 +299,25 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
                                                         (st.ot[t][y][2] - zg[t]) * 16777216.f, (st.ot[t][y][3] - zg[t]) * 16777216.f);
       }
     }
-  
+    if (p.fuse_tail && split == 0) {      // uniform over the workgroup: as in k_decode, half by half
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        float m[4], l[4], o[4][2];
+        tail_partial<NW>(p, b, kvh, tile * NT + t, m, l, o);
+        wave_lds_sync();
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const float mp = S.m[wave][4 * t + h], lp = S.l[wave][4 * t + h];
+          float2* slot = reinterpret_cast<float2*>(S.o(wave, 4 * t + h)) + lane;
+          const float2 op = *slot;
+          const float top = fmaxf(mp, m[h]);
+          const float fp = mp == -INFINITY ? 0.f : fexp2(mp - top), ft = m[h] == -INFINITY ? 0.f : fexp2(m[h] - top);
+          *slot = make_float2(op.x * fp + o[h][0] * ft, op.y * fp + o[h][1] * ft);
+          wave_lds_sync();
+          if (lane == 0) { S.m[wave][4 * t + h] = top; S.l[wave][4 * t + h] = lp * fp + l[h] * ft; }
+        }
+      }
+    }
   } else {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -429,7 +447,7 @@ template <int QM, bool K2>
 int launch_qm(const DecodeParams& p, hipStream_t st) {
   if (p.page != 16 && p.page != 32) return -5;
   const int ntile = (p.gqa + 7) / 8;
-  const int nparts = p.nsplit + (p.tail != nullptr ? 1 : 0);
+  const int nparts = p.nsplit + ((p.tail != nullptr && !p.fuse_tail) ? 1 : 0);
   if (nparts <= 0 || p.B <= 0) return 0;
   dim3 grid(p.Hkv * ntile, nparts, p.B);
   if (p.page == 32) launch_shape<QM, K2, 32>(p, grid, ntile, nparts, st);

@@ -63,7 +63,7 @@ struct DecodeParams {
                            //    draw quads of 4 pages from the slot's counter; 0: split s owns tokens [s, s + 1) * chunk
   int wg_waves;            // wavefronts per workgroup: 4, or the large workgroup that fills a CU
   int fuse_tail;           // 1: no workgroup of their own for the BF16 rows -- the wavefronts of the first body split take
-                           //    them after their pages and fold them into their own partials (k_decode; key-only formats)
+                           //    them after their pages and fold them into their own partials (k_decode, k_decode8; key-only formats)
 };
 int decode_launch(int fmt, const DecodeParams& p, hipStream_t st);
 int decode8_launch(int fmt, const DecodeParams& p, hipStream_t st);       // tiles of 8 query heads (decode_gqa8.hip)
