@@ -267,6 +267,9 @@ def v2_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kmas
     Hkv = pool.shape[1]
     G = Hq // Hkv
     assert G * Hkv == Hq and q.stride(2) == 1 and q.stride(1) == Dh and out.stride(1) == 1
+    # (a pool of pages of another size read with this `page` sends the kernel past the ends of the block-table rows)
+    assert pool.shape[-1] == v2_chunk_bytes(page, Dh, fmt), \
+        f"the pool's chunks hold {pool.shape[-1]} bytes: not pages of {page} tokens of format {fmt} at head dim {Dh}"
     variant = v2_variant(fmt, G, Dh)
     splits = nsplit + (tail is not None)
     assert ws.fits(B, vheads(Hkv, G, Dh, fmt), splits, tile_of(variant), Dh), "split-K workspace too small"
@@ -365,6 +368,8 @@ def cb_attn(q, pool, block_table, seq_lens, out, nsplit, chunk, ws, qscale, kind
                        bound=bound)
     assert (Hq, Dh) == (4 * Hkv, D), f"codebook {kind}: GQA 4, head dim 128 only"
     assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
+    assert pool.shape[-1] == cb_chunk_bytes(kind, page), \
+        f"the pool's chunks hold {pool.shape[-1]} bytes: not pages of {page} tokens of kind {kind}"
     assert ws.fits(B, Hkv, nsplit + (tail is not None)), "split-K workspace too small"
     args = (q, q.stride(0), pool, block_table, block_table.stride(0), seq_lens, B, Hkv, page, nsplit, chunk, qscale,
             sign_words(), CB_KINDS[kind], 0, STAGES, ws.opart, ws.mlpart, ws.counter, out, out.stride(0),
@@ -382,6 +387,8 @@ def cb_attn_noalloc(q, pool, block_table, seq_lens, out, nsplit, chunk, qscale, 
     G = Hq // Hkv
     assert kind in K2 and Hq == G * Hkv and Dh == D, f"{kind}: key-only 2x2 kinds, head dim 128 only"
     assert q.stride(2) == 1 and q.stride(1) == D and out.stride(1) == 1
+    assert pool.shape[-1] == cb_chunk_bytes(kind, page), \
+        f"the pool's chunks hold {pool.shape[-1]} bytes: not pages of {page} tokens of kind {kind}"
     args = (q, q.stride(0), pool, block_table, block_table.stride(0), seq_lens, B, Hkv, page, nsplit, chunk, qscale,
             CB_KINDS[kind], out, out.stride(0), *_tail_args(tail, tail_len, tail_idx, tail_bs, tail_ts), current_stream(),
             G, int(kv_start))

@@ -142,3 +142,21 @@ def test_key_loops_keep_their_registers():
                 seen += 1
                 assert n == 0, (kernel, n)
     assert seen >= 40
+
+
+def test_decode_front_end_rejects_a_pool_of_another_page_size():
+    """a pool of 32-token pages read with page = 16 would send the kernels past the ends of the block-table rows: the
+    front end compares the chunk size with (format, page, head dim) before anything is launched"""
+    import torch
+    from flagrot_releaser_amd import kernels as K
+    q = torch.zeros(2, 32, 128, dtype=torch.bfloat16)
+    out = torch.zeros(2, 32 * 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 4, dtype=torch.int32)
+    lens = torch.zeros(2, dtype=torch.int32)
+    pool32 = torch.zeros(8, 8, K.cb_chunk_bytes("konlya", 32), dtype=torch.uint8)
+    with pytest.raises(AssertionError, match="not pages of 16 tokens"):
+        K.cb_attn(q, pool32, bt, lens, out, 1, 64, None, 1.0, "konlya")
+    with pytest.raises(AssertionError, match="not pages of 16 tokens"):
+        K.v2_attn(q, pool32, bt, lens, out, 1, 64, None, 1.0, fmt="int4a")
+    with pytest.raises(AssertionError, match="not pages of 16 tokens"):
+        K.cb_attn_noalloc(q, pool32, bt, lens, out, 1, 64, 1.0, "konlya")
