@@ -77,13 +77,14 @@ template <> struct UnpackD<QM_ASYM2> {   // fields at bits 0, 2, 8, 10 (+16) of 
     x[0] = w & 0x00300030u; x[1] = w & 0x00C000C0u; x[2] = t & 0x00300030u; x[3] = t & 0x00C000C0u;
   }
 };
-template <> struct UnpackD<QM_SYM4> {    // sign-magnitude bytes s0000mmm -> signed denormals (no extra factor)
+template <> struct UnpackD<QM_SYM4> {    // sign-magnitude bytes s....mmm -> signed denormals (no extra factor)
   static constexpr int SH = 0;
-  static DEVI uint32_t pair(uint32_t bytes02) { return (bytes02 & 0x00070007u) | ((bytes02 & 0x00800080u) << 8); }
+  // A byte doubled into both bytes of an fp16 half has its magnitude bits in the mantissa (low copy) and its sign bit
+  // on the sign (high copy): one byte permute and one mask per pair.
+  static DEVI uint32_t pair(uint32_t w, uint32_t sel) { return __builtin_amdgcn_perm(w, w, sel) & 0x80078007u; }
   static DEVI void run(uint32_t w, uint32_t (&x)[4]) {
-    const uint32_t a = w & 0x87878787u;                                   // A_i in byte i
-    const uint32_t b = ((w << 4) | (w >> 28)) & 0x87878787u;              // B_i in byte i
-    x[0] = pair(a); x[1] = pair(b); x[2] = pair(a >> 8); x[3] = pair(b >> 8);
+    const uint32_t b = __builtin_amdgcn_alignbit(w, w, 28);               // B_i (magnitude, sign) in byte i like A_i
+    x[0] = pair(w, 0x02020000u); x[1] = pair(b, 0x02020000u); x[2] = pair(w, 0x03030101u); x[3] = pair(b, 0x03030101u);
   }
 };
 // fp16 pattern of -(1024 + z)
