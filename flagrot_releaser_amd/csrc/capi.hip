@@ -90,6 +90,10 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   p.out = out; p.o_bs = o_bs;
   p.tail = tail; p.tail_len = tail_len; p.tail_idx = tail_idx; p.tail_bs = tail_bs; p.tail_ts = tail_ts;
   p.gqa = gqa; p.kv_start = kv_start;
+  // the head-dim-128 kernels read q and the BF16 rows 16 bytes at a time (operands of the matrix instructions)
+  if (tail != nullptr && !(variant & HD256) &&
+      (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(tail)) & 15u) != 0 || ((q_bs | tail_bs | tail_ts) & 7) != 0))
+    return fail(-3, "fr_v2_attn: with BF16 rows, q and the rows must be 16-byte aligned and their strides multiples of 8 elements");
   // Two launch shapes.  (a) The split plan fills the CUs at most once with long chunks: one large workgroup per CU, each
   // owning its chunk, its wavefronts drawing quads of pages from a counter in LDS.  (b) Otherwise workgroups of 4
   // wavefronts, and where the slot's counter word can hold both (one q tile per slot, tickets above the draw bits) the
@@ -135,14 +139,14 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   }
   const long long wgs = pairs * nsplit;
   const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
-  // BF16 rows beside large workgroups (key-only formats: no rotation of the rows into a stored basis):
-  // the wavefronts of the first split take them themselves -- one partial less, and with a single split no ticket and
-  // no merge at all
+  // BF16 rows (key-only formats: no rotation of the rows into a stored basis): the wavefronts of the first split take
+  // them themselves -- one partial less, and with a single split no ticket and no merge at all.  Their cost is small
+  // (scores on the matrix pipe, tail_partial), a workgroup of their own costs its whole life: arguments, rows, epilogue,
+  // partial, ticket, merge.
   static const bool fuse_ok = !(getenv("FLAGROT_FUSE_TAIL") != nullptr && getenv("FLAGROT_FUSE_TAIL")[0] == '0');
-  // (several splits: only where a split is long -- 4096 tokens measured: B = 8, L = 16 k 40.0 -> 38.4 us, B = 4, L = 32 k
-  // 36.3 -> 33.6 -- since the first split's workgroup then ends later than the others; with 32 splits of 1024 tokens
-  // of one sequence the rows' own workgroups were faster, 18.9 against 23.4 us)
-  p.fuse_tail = (fuse_ok && tail != nullptr && big && env_waves == 0 && k2 && !(variant & HD256) &&
+  // (several splits: only where a split is long -- 4096 tokens -- since the first split's workgroup ends later than
+  // the others; with 32 splits of 1024 tokens of one sequence the rows' own workgroups were faster)
+  p.fuse_tail = (fuse_ok && tail != nullptr && env_waves == 0 && k2 && !(variant & HD256) &&
                  (nsplit == 1 || chunk >= 4096)) ? 1 : 0;
   const int nparts = nsplit + ((tail != nullptr && !p.fuse_tail) ? 1 : 0);
   const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;

@@ -321,7 +321,7 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
       // (more rows per step -- nine, so that 144 rows are one step of 16 wavefronts -- measured no better: 62.1 against
       // 60.4 us)
       float m[4], l[4], o[4][2];
-      tail_partial<NW>(p, b, kvh, tile, m, l, o);
+      tail_partial<NW>(p, b, kvh, tile, S.tailw[wave], m, l, o);
       wave_lds_sync();
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
@@ -337,7 +337,7 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
     }
   } else {
     float m[4], l[4], o[4][2];
-    tail_partial<NW>(p, b, kvh, tile, m, l, o);
+    tail_partial<NW>(p, b, kvh, tile, S.tailw[wave], m, l, o);
     if (lane < 4) { S.m[wave][lane] = pick4(m[0], m[1], m[2], m[3], lane); S.l[wave][lane] = pick4(l[0], l[1], l[2], l[3], lane); }
 #pragma unroll
     for (int h = 0; h < 4; ++h) {

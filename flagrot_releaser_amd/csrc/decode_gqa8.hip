@@ -303,7 +303,7 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         float m[4], l[4], o[4][2];
-        tail_partial<NW>(p, b, kvh, tile * NT + t, m, l, o);
+        tail_partial<NW>(p, b, kvh, tile * NT + t, S.tailw[wave], m, l, o);
         wave_lds_sync();
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
@@ -322,7 +322,7 @@ __global__ void __launch_bounds__(64 * NW, (MINW8<QM, K2, P>)) k_decode8(const D
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       float m[4], l[4], o[4][2];
-      tail_partial<NW>(p, b, kvh, tile * NT + t, m, l, o);
+      tail_partial<NW>(p, b, kvh, tile * NT + t, S.tailw[wave], m, l, o);
       if (lane < 4) { S.m[wave][4 * t + lane] = pick4(m[0], m[1], m[2], m[3], lane); S.l[wave][4 * t + lane] = pick4(l[0], l[1], l[2], l[3], lane); }
 #pragma unroll
       for (int h = 0; h < 4; ++h) {

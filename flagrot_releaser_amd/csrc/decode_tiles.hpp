@@ -54,6 +54,7 @@ struct Smem {
   // per-wave strips during the page loop; the waves' partial outputs o[NW][4][128] (fp32) afterwards
   alignas(16) uint8_t work[NW * STRIP_BYTES > NW * 2048 ? NW * STRIP_BYTES : NW * 2048];
   float m[NW][4], l[NW][4];
+  alignas(16) float tailw[NW][64];                   // tail_partial: a wavefront's weights of 16 BF16 rows x 4 heads
   int btc[BT_CACHE];
   int next;                                          // next quad of 4 pages nobody has taken yet
   int last;
@@ -733,6 +734,7 @@ struct Smem8 {
   alignas(16) uint4 qz[2][4][64];
   alignas(16) uint8_t work[NW * STRIP_BYTES];
   float m[NW][8], l[NW][8];
+  alignas(16) float tailw[NW][64];                   // tail_partial: a wavefront's weights of 16 BF16 rows x 4 heads
   int btc[BT_CACHE];
   int next;
   int last;
@@ -1057,68 +1059,80 @@ DEVI void value_phase8(const SM& S, WaveState8& st, const VRegs<QM>& r, int lane
   }
 }
 
-// BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims.
+// BF16 sink / window rows of one sequence: partial softmax over tail_len rows, lanes own 2 dims of the outputs.
+// A wavefront takes 16 rows per step.  Scores on the matrix pipe: A = the tile's four query rows (rows 4..15 of the
+// operand are zero), B = the 16 key rows as they lie in memory (a lane's 16 bytes are 8 channels of row lane & 15),
+// four products of 32 channels -- lanes 0..15 then hold the four heads' scores of row `lane`, with no cross-lane sum.
+// One maximum per head and step (a row reduction), one exponential per (row, head), column sums kept per lane until
+// the end.  The weights pass through 256 bytes of LDS (`pw`, this wavefront's own) and come back as broadcast reads,
+// one per row, for the value products on the vector pipe: 8 multiply-adds and 2 conversions per row.
+// q and the rows are read 16 bytes at a time: the caller has checked their alignment (fr_v2_attn).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 template <int NW>
-DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float (&m)[4], float (&l)[4], float (&o)[4][2]) {
+DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float* pw, float (&m)[4], float (&l)[4], float (&o)[4][2]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, kb = lane >> 4;
   const int n = p.tail_len[b];
   const int row = p.tail_idx != nullptr ? p.tail_idx[b] : b;
   const uint16_t* base = static_cast<const uint16_t*>(p.tail) + static_cast<long long>(row) * p.tail_bs;
-  float q[4][2];
+  uint4 qa[4];
+  {
+    const int hq = tile * 4 + col;
+    const bool live = col < 4 && hq < p.gqa;
+    const uint16_t* qr = static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
+                         (static_cast<long long>(kvh) * p.gqa + (live ? hq : 0)) * 128 + 8 * kb;
 #pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int hq = tile * 4 + h;
-    q[h][0] = q[h][1] = 0.f;
-    if (hq < p.gqa) {
-      const uint32_t raw = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p.q) + static_cast<long long>(b) * p.q_bs +
-                                                              (static_cast<long long>(kvh) * p.gqa + hq) * 128 + 2 * lane);
-      q[h][0] = bf16_lo(raw) * p.qscale;
-      q[h][1] = bf16_hi(raw) * p.qscale;
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(qr + 32 * s);
+      qa[s] = live ? v : make_uint4(0u, 0u, 0u, 0u);
     }
-    m[h] = -INFINITY; l[h] = 0.f; o[h][0] = o[h][1] = 0.f;
   }
-  // TR rows per wavefront and step: their loads go out together and their 4 x TR reductions interleave (a row at a time
-  // is one memory latency and one chain of cross-lane steps per row)
-  constexpr int TR = 4;
-  for (int t0 = wave * TR; t0 < n; t0 += NW * TR) {
-    uint32_t kr[TR], vr[TR];
+  float lp[4];
 #pragma unroll
-    for (int r = 0; r < TR; ++r) {
-      const uint16_t* tr = base + static_cast<long long>(min(t0 + r, n - 1)) * p.tail_ts;
-      kr[r] = *reinterpret_cast<const uint32_t*>(tr + kvh * 128 + 2 * lane);
-      vr[r] = *reinterpret_cast<const uint32_t*>(tr + (p.Hkv + kvh) * 128 + 2 * lane);
+  for (int h = 0; h < 4; ++h) { m[h] = -INFINITY; lp[h] = 0.f; o[h][0] = o[h][1] = 0.f; }
+  for (int t0 = wave * 16; t0 < n; t0 += NW * 16) {
+    const uint16_t* kr = base + static_cast<long long>(min(t0 + col, n - 1)) * p.tail_ts + kvh * 128 + 8 * kb;
+    uint4 kk[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kk[s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
+    uint32_t vr[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      vr[r] = *reinterpret_cast<const uint32_t*>(base + static_cast<long long>(min(t0 + r, n - 1)) * p.tail_ts + (p.Hkv + kvh) * 128 + 2 * lane);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, qa[s]), __builtin_bit_cast(bf16x8, kk[s]), acc, 0, 0, 0);
+    const bool in = t0 + col < n;
+    float pe[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const float sc = in ? acc[h] * p.qscale : -INFINITY;
+      // (lane 0 is in the row of the scores; row t0 exists, so the maximum is a number)
+      const float mx = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_max16(sc))));
+      const float mn = fmaxf(m[h], mx);
+      const float alpha = fexp2(m[h] - mn);
+      pe[h] = fexp2(sc - mn);
+      m[h] = mn;
+      lp[h] = lp[h] * alpha + pe[h];
+      o[h][0] *= alpha; o[h][1] *= alpha;
     }
-    float s[TR][4];
+    if (lane < 16) *reinterpret_cast<float4*>(pw + 4 * lane) = make_float4(pe[0], pe[1], pe[2], pe[3]);
+    wave_lds_sync();
 #pragma unroll
-    for (int r = 0; r < TR; ++r) {
-      const float k0 = bf16_lo(kr[r]), k1 = bf16_hi(kr[r]);
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        float a = q[h][0] * k0 + q[h][1] * k1;
-        a += dpp_xor1(a); a += dpp_xor2(a);
-        s[r][h] = a;
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < TR; ++r)
-#pragma unroll
-      for (int h = 0; h < 4; ++h) s[r][h] = wave_sum_over_tokens(s[r][h]);
-#pragma unroll
-    for (int r = 0; r < TR; ++r) {
-      const bool in = t0 + r < n;
+    for (int r = 0; r < 16; ++r) {
+      const float4 w = *reinterpret_cast<const float4*>(pw + 4 * r);
       const float v0 = bf16_lo(vr[r]), v1 = bf16_hi(vr[r]);
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const float sc = in ? s[r][h] : -INFINITY;
-        const float mn = fmaxf(m[h], sc);
-        const float alpha = mn == -INFINITY ? 1.f : fexp2(m[h] - mn), pe = mn == -INFINITY ? 0.f : fexp2(sc - mn);
-        m[h] = mn;
-        l[h] = l[h] * alpha + pe;
-        o[h][0] = o[h][0] * alpha + pe * v0;
-        o[h][1] = o[h][1] * alpha + pe * v1;
-      }
+      o[0][0] += w.x * v0; o[0][1] += w.x * v1;
+      o[1][0] += w.y * v0; o[1][1] += w.y * v1;
+      o[2][0] += w.z * v0; o[2][1] += w.z * v1;
+      o[3][0] += w.w * v0; o[3][1] += w.w * v1;
     }
+    wave_lds_sync();      // the weights have been read before the next step replaces them
   }
+#pragma unroll
+  for (int h = 0; h < 4; ++h)
+    l[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_sum16(lp[h]))));
 }
 
 }  // namespace dec

@@ -25,6 +25,8 @@ int fr_abi_version(void);
  * block_table int32 [B, bt_stride] (bt_stride may be 0); seq_lens int32 [B]; out bf16 [B, gqa*Hkv*128] (row stride
  * o_bs); kmask / vmask uint8 [Hkv, 4] or null (honoured if qrot / if vrot or tail); tail bf16
  * [rows, W, 2*Hkv, 128] (strides tail_bs / tail_ts elements) + tail_len int32 [B] (+ tail_idx int32 [B]) or null.
+ * With a tail at head dim 128, q and tail must be 16-byte aligned and q_bs, tail_bs, tail_ts multiples of 8 elements
+ * (the rows are operands of matrix instructions, read 16 bytes at a time; contiguous torch tensors always are): -3 if not.
  * nsplit counts the body splits; with a tail the workspace must hold B*Hkv*ceil(gqa/GT)*(nsplit+1) partials of
  * GT*128 floats (GT = 8 when variant has bits 1024|2048, else 4); counter int32 [B*Hkv*ceil(gqa/GT)] zeroed once by the
  * caller (merge tickets and, when the body workgroups of a sequence share its page range, their page draws; the last

@@ -286,6 +286,10 @@ def test_decode_error_codes(dev):
     assert L.fr_v2_attn(5, *no_ctr, 4, 0) == -3
     hd = list(base); hd[17] = 264 | 1024 | 2048 | 4096
     assert L.fr_v2_attn(5, *hd, 4, 0) == -3              # head dim 256 takes q tiles of 4 heads, not 8
+    odd = list(base); odd[24] = zp + 2; odd[25] = zp; odd[27] = 2048; odd[28] = 2048     # BF16 rows off a 16-byte boundary
+    assert L.fr_v2_attn(5, *odd, 4, 0) == -3 and b"16-byte" in L.fr_last_error()
+    odd[24] = zp; odd[28] = 2052                                                         # ... or a row stride that leaves it
+    assert L.fr_v2_attn(5, *odd, 4, 0) == -3 and b"16-byte" in L.fr_last_error()
     assert L.fr_cb_attn(zp, 512, zp, zp, 1, zp, 1, 1, 16, 1, 64, 1.0, K.sign_words(), 3, 0, 4, zp, zp, zp, zp, 512, None,
                         None, None, 0, 0, None, 0) == -4
     assert L.fr_v2_attn(5, *(base[:6] + [0] + base[7:]), 4, 0) == 0     # B = 0: nothing to do
