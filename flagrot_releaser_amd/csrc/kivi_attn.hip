@@ -73,6 +73,10 @@ int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, lon
   if (G > 8 || G < 1 || chunk % 32 || chunk <= 0) { std::snprintf(g_err, sizeof(g_err), "kv_attn: G %d chunk %d", G, chunk); return 2; }
   if (D != 128 && D != 256) return bad("kv_attn: head dim 128 or 256");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // the head-dim-128 kernel reads q and the ring rows 16 bytes at a time (operands of matrix instructions)
+  if (D == 128 && ring != nullptr &&
+      (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(ring)) & 15u) != 0 || (q_rs & 7) != 0))
+    return bad("kv_attn: with ring rows, q and the ring must be 16-byte aligned and q_rs a multiple of 8 elements");
   if (D == 256)
     return launched(attn256_launch(G, q, q_rs, pool, bt, bt_rs, cached, kv_start, B, Hkv, NS, chunk, qscale, ring, tail_len,
                                    tail_idx, T, opart, ml, out, out_rs, f8 & 1, st), "kv_attn");

@@ -95,44 +95,108 @@ DEVI void load_group(GroupRegs& r, const uint8_t* chA, const uint8_t* chB, int l
   }
 }
 
+// all-reduce over the 16 lanes of a row (DPP: quad permutes, then the mirrors of 8 and of 16 lanes)
+DEVI float row16_max(float v) {
+  v = fmaxf(v, dpp_xor1(v)); v = fmaxf(v, dpp_xor2(v));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true)));
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true)));
+}
+DEVI float row16_sum(float v) {
+  v += dpp_xor1(v); v += dpp_xor2(v);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+DEVI float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
 // The BF16 ring rows of one sequence (split index NS): rows [0, tail_len) of ring block tail_idx, K row h, V row Hkv + h,
-// original basis.  A wavefront takes every fourth row, lanes own 2 dims; same partial format as the page splits.
+// original basis; same partial format as the page splits.  A wavefront takes 16 rows per step.  Scores on the matrix
+// pipe: A = the GQA group's query rows as BF16 (rows G..15 of the operand zero), B = the 16 key rows as they lie in
+// memory (a lane's 16 bytes are 8 channels of row lane & 15), four products of 32 channels: lanes 0..15 then hold the
+// scores of heads 0..3 for row `lane`, lanes 16..31 those of heads 4..7 -- no cross-lane sums.  One maximum per head
+// and step, one exponential per (row, head); the weights pass through LDS (the wavefront's own scratch block, idle in
+// this split) and come back as broadcast reads for the value products on the vector pipe, lanes owning 2 dims.
+// q and the ring are read 16 bytes at a time (kv_attn checks their alignment).
 template <int G>
 DEVI void tail_split(Smem& S, const uint16_t* __restrict__ q, long long q_rs, const uint16_t* __restrict__ ring,
                      const int* __restrict__ tail_len, const int* __restrict__ tail_idx, int T, int Hkv, int Gq, int b, int h,
                      int g0, float qscale, float* __restrict__ op, float* __restrict__ mlp) {
+  static_assert(G == 8, "two rows of 16 lanes carry the heads");
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
   const int n = tail_len != nullptr ? tail_len[b] : 0;
   if (n <= 0) {
     if (tid < G && g0 + tid < Gq) { mlp[2 * tid] = -INFINITY; mlp[2 * tid + 1] = 0.f; }
     return;
   }
-  float qa[G], qb[G], m[G], l[G], oa[G], ob[G];
+  const int col = lane & 15, kb = lane >> 4;
+  uint4 qa[4];
+  {
+    const bool live = col < G && g0 + col < Gq;
+    const uint16_t* qr = q + static_cast<long long>(b) * q_rs + (static_cast<long long>(h) * Gq + (live ? g0 + col : 0)) * 128 + 8 * kb;
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    qa[g] = qb[g] = 0.f;
-    if (g0 + g < Gq) {
-      const uint32_t raw = *reinterpret_cast<const uint32_t*>(q + static_cast<long long>(b) * q_rs + (static_cast<long long>(h) * Gq + g0 + g) * 128 + 2 * lane);
-      qa[g] = bf16_lo(raw) * qscale; qb[g] = bf16_hi(raw) * qscale;
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(qr + 32 * s);
+      qa[s] = live ? v : make_uint4(0u, 0u, 0u, 0u);
     }
-    m[g] = -INFINITY; l[g] = 0.f; oa[g] = ob[g] = 0.f;
   }
+  // the lane's four heads 4 kb + i (kb < 2; the other lanes carry the operand's zero rows): maxima (alike over the
+  // lane's row of 16), column sums of the weights
+  float mr[4], lp[4], oa[G], ob[G];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { mr[i] = -INFINITY; lp[i] = 0.f; }
+#pragma unroll
+  for (int g = 0; g < G; ++g) oa[g] = ob[g] = 0.f;
+  float* pw = reinterpret_cast<float*>(&S.w[wv]);            // [head quad kb][row][4]
   const uint16_t* rbase = ring + static_cast<long long>(tail_idx != nullptr ? tail_idx[b] : 0) * T * 2 * Hkv * 128;
-  for (int t = wv; t < n; t += 4) {
-    const uint16_t* row = rbase + static_cast<long long>(t) * 2 * Hkv * 128;
-    const uint32_t kr = *reinterpret_cast<const uint32_t*>(row + h * 128 + 2 * lane);
-    const uint32_t vr = *reinterpret_cast<const uint32_t*>(row + (Hkv + h) * 128 + 2 * lane);
-    const float k0 = bf16_lo(kr), k1 = bf16_hi(kr), v0 = bf16_lo(vr), v1 = bf16_hi(vr);
+  const long long rs = 2ll * Hkv * 128;
+  for (int t0 = wv * 16; t0 < n; t0 += 64) {
+    const uint16_t* kr = rbase + min(t0 + col, n - 1) * rs + h * 128 + 8 * kb;
+    uint4 kk[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kk[s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
+    uint32_t vr[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      vr[r] = *reinterpret_cast<const uint32_t*>(rbase + min(t0 + r, n - 1) * rs + (Hkv + h) * 128 + 2 * lane);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, qa[s]), __builtin_bit_cast(bf16x8, kk[s]), acc, 0, 0, 0);
+    const bool in = t0 + col < n;
+    float pe[4], al[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float sc = in ? acc[i] * qscale : -INFINITY;
+      const float mn = fmaxf(mr[i], row16_max(sc));          // a number: row t0 exists
+      al[i] = fexp2(mr[i] - mn);
+      pe[i] = fexp2(sc - mn);
+      mr[i] = mn;
+      lp[i] = lp[i] * al[i] + pe[i];
+    }
+    if (lane < 32) *reinterpret_cast<float4*>(pw + 4 * lane) = make_float4(pe[0], pe[1], pe[2], pe[3]);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const float sc = wave_sum64(qa[g] * k0 + qb[g] * k1);
-      const float mn = fmaxf(m[g], sc);
-      const float alpha = m[g] == -INFINITY ? 0.f : fexp2(m[g] - mn), p = fexp2(sc - mn);
-      l[g] = l[g] * alpha + p;
-      oa[g] = oa[g] * alpha + p * v0;
-      ob[g] = ob[g] * alpha + p * v1;
-      m[g] = mn;
+      const float a = lane_value(al[g & 3], 16 * (g >> 2));
+      oa[g] *= a; ob[g] *= a;
     }
+    wave_lds_sync();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float4 w0 = *reinterpret_cast<const float4*>(pw + 4 * r);
+      const float4 w1 = *reinterpret_cast<const float4*>(pw + 64 + 4 * r);
+      const float v0 = bf16_lo(vr[r]), v1 = bf16_hi(vr[r]);
+      oa[0] += w0.x * v0; ob[0] += w0.x * v1; oa[1] += w0.y * v0; ob[1] += w0.y * v1;
+      oa[2] += w0.z * v0; ob[2] += w0.z * v1; oa[3] += w0.w * v0; ob[3] += w0.w * v1;
+      oa[4] += w1.x * v0; ob[4] += w1.x * v1; oa[5] += w1.y * v0; ob[5] += w1.y * v1;
+      oa[6] += w1.z * v0; ob[6] += w1.z * v1; oa[7] += w1.w * v0; ob[7] += w1.w * v1;
+    }
+    wave_lds_sync();      // the weights have been read before the next step replaces them
+  }
+  float m[G], l[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = lane_value(mr[g & 3], 16 * (g >> 2));
+    l[g] = lane_value(row16_sum(lp[g & 3]), 16 * (g >> 2));
   }
   if (lane == 0) {
 #pragma unroll

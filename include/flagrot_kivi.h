@@ -41,7 +41,9 @@ int kv_k_encode(const void* src, long long src_rs, const void* src2, long long s
 /* kivi.cu:1987-2039.  q bf16 [B, Hkv*G, D] (row stride q_rs); bt int32 [B, bt_rs]; cached int32 [B] (page tokens
  * [kv_start, cached[b]) are attended); ring bf16 [(R+1)*T, 2*Hkv, D] with tail_len / tail_idx int32 [B]; opart fp32
  * [B*Hkv*(NS+1)*G*D], ml fp32 [B*Hkv*(NS+1)*G*2]; out bf16 [B, Hkv*G*D] (row stride out_rs).  G <= 8, chunk % 32 == 0.
- * f8 bit 1 (the reference's fast variant) is accepted and ignored. */
+ * f8 bit 1 (the reference's fast variant) is accepted and ignored.  At D = 128 with ring rows, q and ring must be
+ * 16-byte aligned and q_rs a multiple of 8 elements (the rows are operands of matrix instructions; contiguous torch
+ * tensors are): 2 if not. */
 int kv_attn(const void* q, long long q_rs, const void* pool, const void* bt, long long bt_rs, const void* cached,
             int kv_start, int B, int Hkv, int G, int D, int NS, int chunk, float qscale, const void* ring,
             const void* tail_len, const void* tail_idx, int T, void* opart, void* ml, void* out, long long out_rs, int f8,

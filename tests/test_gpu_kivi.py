@@ -401,6 +401,12 @@ def test_attn_without_tail_and_rejects(dev):
     with pytest.raises(RuntimeError, match="head dim"):
         KV.v_write(torch.zeros(1, 2 * Hkv, 64, dtype=torch.bfloat16, device=dev), torch.zeros(1, dtype=torch.int64, device=dev),
                    torch.ones(Hkv, 64, device=dev), None, pool, Hkv, 64)
+    # ring rows are read 16 bytes at a time: a q that starts 4 bytes off such a boundary is refused, not mis-read
+    ring = torch.zeros(2 * 32, 2 * Hkv, D, dtype=torch.bfloat16, device=dev)
+    one = torch.ones(1, dtype=torch.int32, device=dev)
+    q_off = torch.zeros(Hkv * G * D + 8, dtype=torch.bfloat16, device=dev)[2:2 + Hkv * G * D].view(1, Hkv * G, D)
+    with pytest.raises(RuntimeError, match="16-byte"):
+        KV.attn(q_off, pool, bt.to(dev), cached, out, 2, 256, ws, 0.1, 0, G, ring=ring, tail_len=one, tail_idx=one, T=32)
 
 
 @F8
