@@ -102,7 +102,9 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   // ranges, FLAGROT_WG_WAVES=4 | 16 forces a workgroup size (above 4: the large one).
   static const bool force_static = getenv("FLAGROT_DECODE_STATIC") != nullptr && getenv("FLAGROT_DECODE_STATIC")[0] == '1';
   static const int env_waves = getenv("FLAGROT_WG_WAVES") != nullptr ? atoi(getenv("FLAGROT_WG_WAVES")) : 0;
-  static const bool replan = !(getenv("FLAGROT_REPLAN") != nullptr && getenv("FLAGROT_REPLAN")[0] == '0');
+  // (read at every call, unlike the others: the tests run the same cases with and without it in one process)
+  const char* const replan_env = getenv("FLAGROT_REPLAN");
+  const bool replan = !(replan_env != nullptr && replan_env[0] == '0');
   // A plan of more workgroups than CUs is run as fewer, longer splits where shape (a) then applies.  The reference front
   // end caps a chunk at 8192 tokens (vllm_flagrot/kernels.py:74, MAX_CHUNK), so a context beyond 8192 tokens always
   // arrives as two or more splits per (sequence, KV head, q tile) pair -- also where 256 pairs fill the CUs by
@@ -137,8 +139,27 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
       p.nsplit = nsplit; p.chunk = chunk;
     }
   }
+  // Short splits (below the large workgroups' threshold; the reference planner makes them for short contexts on few
+  // pairs: one sequence of 2048 tokens arrives as 6 x 384) are run as large workgroups too where those fit the CUs once:
+  // a single one up to 1024 tokens, splits of 512 tokens beyond -- these launches are chains of latencies, and a
+  // workgroup whose 16 wavefronts take one quad each has the shortest one (one sequence: 512 tokens 10.3 -> 9.6 us,
+  // 1536 14.5 -> 11.8, 2048 15.0 -> 11.9; 32 sequences of 512 14.7 -> 11.0; tiles of 8 heads, one sequence of 2048
+  // 20.8 -> 15.3).  From 512 tokens: below, the four wavefronts of a small workgroup are as fast or faster (256 tokens:
+  // 7.9 against 8.8 us).  Never more splits than the caller's.
+  bool short_big = false;
+  if (replan && env_waves == 0 && !(variant & HD256) && chunk < decode_big_chunk()) {
+    const long long span = static_cast<long long>(nsplit) * chunk;
+    if (span >= 512 && span < (1ll << 30)) {
+      const int ns = span <= 1024 ? 1 : static_cast<int>((span + 511) / 512);
+      const int ch = span <= 1024 ? static_cast<int>(span) : 512;
+      if (ns <= nsplit && pairs * ns <= cus) {
+        nsplit = ns; chunk = ch; short_big = true;
+        p.nsplit = nsplit; p.chunk = chunk;
+      }
+    }
+  }
   const long long wgs = pairs * nsplit;
-  const bool big = env_waves > 4 || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
+  const bool big = env_waves > 4 || short_big || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
   // BF16 rows (key-only formats: no rotation of the rows into a stored basis): the wavefronts of the first split take
   // them themselves -- one partial less, and with a single split no ticket and no merge at all.  Their cost is small
   // (scores on the matrix pipe, tail_partial), a workgroup of their own costs its whole life: arguments, rows, epilogue,

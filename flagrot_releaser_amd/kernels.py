@@ -149,6 +149,13 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
         ns, chunk = plan(min(ncu // pairs, Lmax // BIG_CHUNK))     # even when they fill only part of the CUs)
         if chunk >= BIG_CHUNK and 24 <= pairs * ns <= ncu:
             return ns, chunk
+    # short contexts on few pairs: large workgroups as well -- one up to 1024 tokens, splits of 512 tokens beyond (the
+    # library runs such plans that way whoever made them; one sequence of 2048 tokens: 4 x 512 11.9 us, 6 x 384 in
+    # workgroups of 4 wavefronts 15.0)
+    if ncu and 512 <= Lmax < 4 * BIG_CHUNK:
+        ns = 1 if Lmax <= 2 * 512 else math.ceil(Lmax / 512)
+        if pairs * ns <= ncu:
+            return plan(ns)
     # small workgroups: one round at most; a short job is a trade of pages per wavefront against partials to merge
     quads = math.ceil(Lmax / 64)
     return plan(min(max(1, slots // pairs), max(1, quads // 4), max(1, round(math.sqrt(quads)))))

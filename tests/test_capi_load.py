@@ -119,8 +119,15 @@ def test_host_planner_invariants():
     assert K.plan_splits(8, 32768, 8, 16, 1024, ncu=256) == (4, 8192)
     assert K.plan_splits(64, 16256, 8, 16, 1024, ncu=256) == (2, 8128)
     assert K.plan_splits(2, 4097, 8, 16, 1024, ncu=256) == (4, 1088)
-    assert K.plan_splits(1, 1024, 8, 16, 1024, ncu=256) == (4, 256)
-    assert K.plan_splits(1, 2048, 8, 16, 1024, ncu=256) == (6, 384)
+    # short contexts on few pairs: one large workgroup up to 1024 tokens, splits of 512 tokens beyond; below 512 tokens
+    # (and where such splits would not fit the CUs) the small workgroups' plan
+    assert K.plan_splits(1, 1024, 8, 16, 1024, ncu=256) == (1, 1024)
+    assert K.plan_splits(1, 2048, 8, 16, 1024, ncu=256) == (4, 512)
+    assert K.plan_splits(2, 1500, 8, 16, 1024, ncu=256) == (3, 512)
+    assert K.plan_splits(1, 300, 8, 16, 1024, ncu=256) == (1, 320)
+    assert K.plan_splits(32, 2000, 8, 16, 1024, ncu=256) == (1, 2048)
+    assert K.plan_splits(40, 800, 8, 16, 1024, ncu=256) == (3, 320)
+    assert K.plan_splits(1, 2048, 8, 16, 512, ncu=0) == (6, 384)                     # head dim 256: small workgroups only
     assert K.plan_splits(1, 32768, 8, 16, 1024, ncu=256) == (32, 1024)
     assert K.plan_splits(64, 2048, 8, 16, 1024, ncu=256) == (2, 1024)
     assert K.v2_variant("int4a", 4) == 264 and K.tile_of(K.v2_variant("konlya", 8)) == 8

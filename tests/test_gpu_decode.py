@@ -14,7 +14,9 @@ Bar (floating point, the tolerance of the build's north star: max-abs 2e-3 / rel
 Every case prints its worst element-wise ratio |err| / (2e-3 + 1e-2 |ref|), ordinary and adversarial rows apart.
 ref = fp64 softmax attention over the pages parsed by the oracle's independent layout parser (the cache bytes are
 written by the HIP writers, whose bit-exactness tests/test_gpu_writers.py establishes)."""
+import contextlib
 import math
+import os
 
 import numpy as np
 import pytest
@@ -28,6 +30,22 @@ pytestmark = pytest.mark.gpu
 LOG2E = 1.4426950408889634
 ATOL, RTOL = 2e-3, 1e-2
 HARD_ROWS = 2.0      # element-wise bound of the rows that read the adversarial tokens, in units of the ordinary bar
+
+
+@contextlib.contextmanager
+def as_planned(on):
+    """the library runs the caller's split plan unchanged inside this block (if `on`)"""
+    before = os.environ.get("FLAGROT_REPLAN")
+    if on:
+        os.environ["FLAGROT_REPLAN"] = "0"
+    try:
+        yield
+    finally:
+        if on:
+            if before is None:
+                del os.environ["FLAGROT_REPLAN"]
+            else:
+                os.environ["FLAGROT_REPLAN"] = before
 
 
 def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4, kv_start=0, nsplit=None, P=P16,
@@ -100,13 +118,17 @@ def run_case(dev, mode, lens, fmt, win=None, bt_shared=False, seed=0, G=4, Hkv=4
         dt = tail.to(dev)
         tkw = dict(tail=dt, tail_len=tail_len.to(dev), tail_idx=tail_idx.to(dev), tail_bs=dt.stride(0), tail_ts=dt.stride(1))
     dq, dbt, dseq = q.to(dev), bt.to(dev) if bt_shared != "stride0" else bt.to(dev)[:1].expand(B, -1), seq.to(dev)
-    for rep in range(2):      # second call: the self-resetting tickets must be back at zero
+    # Two calls: the second finds the self-resetting tickets back at zero.  The first runs the plan as the library
+    # re-shapes it (fewer, longer splits; short splits as large workgroups), the second exactly as the caller planned it
+    # (FLAGROT_REPLAN=0, read at every call): both launch shapes of every case.
+    for rep in range(2):
         out.fill_(float("nan"))
-        if mode == "static":
-            K.v2_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, kmask=mask[:Hkv].to(dev),
-                      vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, page=P, **tkw)
-        else:
-            K.cb_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start, page=P, **tkw)
+        with as_planned(rep == 1):
+            if mode == "static":
+                K.v2_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, kmask=mask[:Hkv].to(dev),
+                          vmask=mask[Hkv:].to(dev), fmt=fmt, kv_start=kv_start, page=P, **tkw)
+            else:
+                K.cb_attn(dq, pool, dbt, dseq, out, ns, ch, ws, scale * LOG2E, fmt, kv_start=kv_start, page=P, **tkw)
         torch.cuda.synchronize()
         got = out.view(B, HQ, 128).float().cpu().numpy().astype(np.float64)
         valid = np.array([min(kv_start, lens[b]) < lens[b] or (tail is not None and int(tail_len[b]) > 0) for b in range(B)])
@@ -158,6 +180,20 @@ def test_plans_the_library_runs_as_fewer_longer_splits(dev, mode, fmt):
     lens[5], lens[17] = 0, 9
     ns, ch = run_case(dev, mode, lens, fmt, seed=41, G=4, Hkv=8, nsplit=3, win=(20, 33), kv_start=4)
     assert (ns, ch) == (3, 768)
+
+
+@pytest.mark.parametrize("mode,fmt", [("codebook", "konlya"), ("codebook", "konlya2"), ("static", "int4a")])
+def test_short_splits_run_as_large_workgroups(dev, mode, fmt):
+    """Plans of short splits (the reference planner's answer to short contexts: 6 x 384 tokens for one sequence of
+    2048) are run as large workgroups where those fit the CUs once (csrc/capi.hip: fr_v2_attn): one of them up to 1024
+    tokens, splits of 512 tokens beyond, never more splits than planned.  Ragged and empty sequences, BF16 rows,
+    kv_start, tiles of 8 heads; the second call of every case runs the plan as given (run_case)."""
+    ns, ch = run_case(dev, mode, [2040, 1300, 0, 7], fmt, seed=71, Hkv=2, nsplit=6, win=(40, 6), kv_start=4)
+    assert ch < 512 and ns * ch >= 2040                 # 6 x 352 -> run as 5 x 512
+    ns, ch = run_case(dev, mode, [1000, 513, 1], fmt, seed=72, Hkv=2, nsplit=4)
+    assert ch == 256                                    # 4 x 256 -> run as 1 x 1024
+    run_case(dev, mode, [520, 100], fmt, seed=73, Hkv=1, G=8, nsplit=2, win=(17, 3))
+    run_case(dev, mode, [1500], fmt, seed=74, Hkv=4, nsplit=5, P=32)
 
 
 def test_large_workgroups_in_full_rounds(dev):
