@@ -145,17 +145,18 @@ def plan_splits(B: int, Lmax: int, HV: int, page: int, slots: int, nsplit=None, 
     if nsplit is not None:
         return plan(nsplit)
     pairs = B * HV
+    # short contexts on few pairs: large workgroups, one up to 1024 tokens, splits of 512 tokens up to 4096 tokens where
+    # they fit the CUs once (these launches are chains of latencies: one sequence of 2048 tokens 4 x 512 11.9 us, 6 x 384
+    # in workgroups of 4 wavefronts 15.0; of 4096 tokens 8 x 512 12.5 us, 4 x 1024 13.4; the library runs plans of
+    # short splits as large workgroups whoever made them)
+    if ncu and 512 <= Lmax <= 4 * BIG_CHUNK:
+        ns = 1 if Lmax <= 2 * 512 else math.ceil(Lmax / 512)
+        if pairs * ns <= ncu:
+            return plan(ns)
     if pairs <= ncu and Lmax >= BIG_CHUNK:          # as many large workgroups as keep >= 1024 tokens each (measured best
         ns, chunk = plan(min(ncu // pairs, Lmax // BIG_CHUNK))     # even when they fill only part of the CUs)
         if chunk >= BIG_CHUNK and 24 <= pairs * ns <= ncu:
             return ns, chunk
-    # short contexts on few pairs: large workgroups as well -- one up to 1024 tokens, splits of 512 tokens beyond (the
-    # library runs such plans that way whoever made them; one sequence of 2048 tokens: 4 x 512 11.9 us, 6 x 384 in
-    # workgroups of 4 wavefronts 15.0)
-    if ncu and 512 <= Lmax < 4 * BIG_CHUNK:
-        ns = 1 if Lmax <= 2 * 512 else math.ceil(Lmax / 512)
-        if pairs * ns <= ncu:
-            return plan(ns)
     # small workgroups: one round at most; a short job is a trade of pages per wavefront against partials to merge
     quads = math.ceil(Lmax / 64)
     return plan(min(max(1, slots // pairs), max(1, quads // 4), max(1, round(math.sqrt(quads)))))

@@ -124,6 +124,9 @@ def test_host_planner_invariants():
     assert K.plan_splits(1, 1024, 8, 16, 1024, ncu=256) == (1, 1024)
     assert K.plan_splits(1, 2048, 8, 16, 1024, ncu=256) == (4, 512)
     assert K.plan_splits(2, 1500, 8, 16, 1024, ncu=256) == (3, 512)
+    assert K.plan_splits(1, 4096, 8, 16, 1024, ncu=256) == (8, 512)
+    assert K.plan_splits(8, 2048, 8, 16, 1024, ncu=256) == (4, 512)
+    assert K.plan_splits(8, 4096, 8, 16, 1024, ncu=256) == (4, 1024)
     assert K.plan_splits(1, 300, 8, 16, 1024, ncu=256) == (1, 320)
     assert K.plan_splits(32, 2000, 8, 16, 1024, ncu=256) == (1, 2048)
     assert K.plan_splits(40, 800, 8, 16, 1024, ncu=256) == (3, 320)
