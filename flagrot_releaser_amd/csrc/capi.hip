@@ -160,14 +160,14 @@ int fr_v2_attn(int fmt, const void* q, long long q_bs, const uint8_t* pool, cons
   }
   const long long wgs = pairs * nsplit;
   const bool big = env_waves > 4 || short_big || (env_waves == 0 && chunk >= decode_big_chunk() && (wgs <= cus || rounds));
-  // BF16 rows (key-only formats: no rotation of the rows into a stored basis): the wavefronts of the first split take
-  // them themselves -- one partial less, and with a single split no ticket and no merge at all.  Their cost is small
+  // BF16 rows: the wavefronts of the first split take them themselves (static formats: rotated into the stored basis
+  // wavefront by wavefront) -- one partial less, and with a single split no ticket and no merge at all.  Their cost is small
   // (scores on the matrix pipe, tail_partial), a workgroup of their own costs its whole life: arguments, rows, epilogue,
   // partial, ticket, merge.
   static const bool fuse_ok = !(getenv("FLAGROT_FUSE_TAIL") != nullptr && getenv("FLAGROT_FUSE_TAIL")[0] == '0');
   // (several splits: only where a split is long -- 4096 tokens -- since the first split's workgroup ends later than
   // the others; with 32 splits of 1024 tokens of one sequence the rows' own workgroups were faster)
-  p.fuse_tail = (fuse_ok && tail != nullptr && env_waves == 0 && k2 && !(variant & HD256) &&
+  p.fuse_tail = (fuse_ok && tail != nullptr && env_waves == 0 && !(variant & HD256) &&
                  (nsplit == 1 || chunk >= 4096)) ? 1 : 0;
   const int nparts = nsplit + ((tail != nullptr && !p.fuse_tail) ? 1 : 0);
   const bool can_draw = !force_static && counter != nullptr && nparts <= 1023;

@@ -322,6 +322,10 @@ __global__ void __launch_bounds__(64 * NW, 4) k_decode(const DecodeParams p, int
       // 60.4 us)
       float m[4], l[4], o[4][2];
       tail_partial<NW>(p, b, kvh, tile, S.tailw[wave], m, l, o);
+      // static formats merge in the stored basis: the rows' share is rotated on the groups the writer rotated
+      if constexpr (!K2) {
+        if (p.vmask != nullptr) tail_to_stored_basis(o, p.vmask[kvh * 4 + (lane >> 4)] != 0, lane);
+      }
       wave_lds_sync();
 #pragma unroll
       for (int h = 0; h < 4; ++h) {

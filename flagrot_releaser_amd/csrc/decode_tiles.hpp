@@ -1135,5 +1135,26 @@ DEVI void tail_partial(const DecodeParams& p, int b, int kvh, int tile, float* p
     l[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_sum16(lp[h]))));
 }
 
+// H32 (Sylvester order, factor 1/sqrt(32)) over the 32 channels of a group held two per lane by a row of 16 lanes
+// (channel 2 (lane & 15) + e): what brings a share of the BF16 rows into the basis the static formats store V in
+DEVI void h32_row16(float& a, float& b, int lane) {
+  float y0 = a + b, y1 = a - b;
+  { const float p0 = dpp_xor1(y0), p1 = dpp_xor1(y1); y0 = (lane & 1) ? p0 - y0 : y0 + p0; y1 = (lane & 1) ? p1 - y1 : y1 + p1; }
+  { const float p0 = dpp_xor2(y0), p1 = dpp_xor2(y1); y0 = (lane & 2) ? p0 - y0 : y0 + p0; y1 = (lane & 2) ? p1 - y1 : y1 + p1; }
+  { const float p0 = swz_xor<4>(y0), p1 = swz_xor<4>(y1); y0 = (lane & 4) ? p0 - y0 : y0 + p0; y1 = (lane & 4) ? p1 - y1 : y1 + p1; }
+  { const float p0 = swz_xor<8>(y0), p1 = swz_xor<8>(y1); y0 = (lane & 8) ? p0 - y0 : y0 + p0; y1 = (lane & 8) ? p1 - y1 : y1 + p1; }
+  a = y0 * kC32; b = y1 * kC32;
+}
+// ... for the lane's four heads where the group's mask asks for it (every lane runs the exchanges)
+DEVI void tail_to_stored_basis(float (&o)[4][2], bool rotated, int lane) {
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    float a = o[h][0], b = o[h][1];
+    h32_row16(a, b, lane);
+    o[h][0] = rotated ? a : o[h][0];
+    o[h][1] = rotated ? b : o[h][1];
+  }
+}
+
 }  // namespace dec
 }  // namespace fr

@@ -239,7 +239,7 @@ def test_large_workgroup_shape(dev, mode, fmt):
     assert (ns, ch) == (1, 2304)
     run_case(dev, mode, [4500, 2049, 70], fmt, seed=21, Hkv=2, nsplit=2, win=(40, 5), kv_start=4)
     run_case(dev, mode, [2200], fmt, seed=22, Hkv=1, G=8, nsplit=1)
-    # one split of large workgroups with BF16 rows: on the key-only formats the body's wavefronts take the rows themselves
+    # one split of large workgroups with BF16 rows: the body's wavefronts take the rows themselves
     # (an empty sequence that has rows only, one of five tokens behind kv_start = 4, padding heads in the q tile)
     run_case(dev, mode, [2300, 0, 5, 2100], fmt, seed=25, G=3, Hkv=2, nsplit=1, win=(132, 6), kv_start=4)
     run_case(dev, mode, [2049, 2049], fmt, seed=26, Hkv=2, nsplit=1, win=(7, 3), bt_shared=True)
