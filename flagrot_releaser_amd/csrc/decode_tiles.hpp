@@ -94,7 +94,6 @@ DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
   if (half == 0) fwht<32>(y, l32); else fwht<128>(y, l32);
   // factor of the lane's code fields after the unpacking (the operand is divided by it)
   const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
-  const float fold = QPRE / beta;
 #pragma unroll
   for (int vi = 0; vi < 2; ++vi) {
     const int var = 2 * half + vi;
@@ -117,7 +116,7 @@ DEVI void q_prologue(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
     float qs = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float a = live ? v[i] * fold : 0.f;
+      const float a = live ? v[i] * (QPRE / key_field_factor<QM>(isB, g, i)) : 0.f;
       const _Float16 hi = static_cast<_Float16>(a);
       const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
       hb[i] = __builtin_bit_cast(uint16_t, hi);
@@ -364,7 +363,7 @@ DEVI void key_scores(const SM& S, const KRegs<QM>& r, int lane, const bool (&ful
       if constexpr (QM == QM_ASYM2) {     // two groups per word: the odd one 4 bits higher (2^4 is in its query operand)
         if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
       }
-      else UnpackD<QM>::run(r.kc[b][j], x);
+      else unpack_key<QM>(r.kc[b][j], x);
       const half8 kb = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
       f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh, kb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
       a = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql, kb, a, 0, 0, 0);
@@ -769,7 +768,6 @@ DEVI void q_prologue8(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
   float y[4] = {x[0], x[1], x[2], x[3]};
   if (half == 0) fwht<32>(y, l32); else fwht<128>(y, l32);
   const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
-  const float fold = QPRE / beta;
 #pragma unroll
   for (int vi = 0; vi < 2; ++vi) {
     const int var = 2 * half + vi;
@@ -790,7 +788,7 @@ DEVI void q_prologue8(SM& S, const DecodeParams& p, int b, int kvh, int tile) {
     float qs = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float a = live ? v[i] * fold : 0.f;
+      const float a = live ? v[i] * (QPRE / key_field_factor<QM>(isB, g, i)) : 0.f;
       const _Float16 hi = static_cast<_Float16>(a);
       const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
       hb[i] = __builtin_bit_cast(uint16_t, hi);
@@ -843,7 +841,7 @@ DEVI void key_phase8(const SM& S, const KRegs<QM>& r, int lane, float (&sc)[2][Q
       if constexpr (QM == QM_ASYM2) {
         if (j & 1) UnpackD<QM>::run_hi(r.kc[b][j >> 1], x); else UnpackD<QM>::run(r.kc[b][j >> 1], x);
       }
-      else UnpackD<QM>::run(r.kc[b][j], x);
+      else unpack_key<QM>(r.kc[b][j], x);
       kb[b] = __builtin_bit_cast(half8, make_uint4(x[0], x[1], x[2], x[3]));
       const uint32_t kw = (j & 2) ? r.ks[b].y : r.ks[b].x;
       kz[b] = __builtin_bit_cast(half8, make_uint4(kw & (zlane << (16 * (j & 1))), 0u, 0u, 0u));

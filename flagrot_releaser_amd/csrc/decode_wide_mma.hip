@@ -66,7 +66,6 @@ DEVI void q_prologue_wide(WideMma<QM>& S, const DecodeParams& p, int b, int kvh,
     for (int i = 0; i < 4; ++i) y[s][i] = x[s][i];
   if (half == 0) { fwht<32>(y[0], l32); fwht<32>(y[1], l32); } else h256(y, l32);
   const float beta = (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
-  const float fold = QPRE / beta;
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
 #pragma unroll
@@ -89,7 +88,7 @@ DEVI void q_prologue_wide(WideMma<QM>& S, const DecodeParams& p, int b, int kvh,
       float qs = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float a = live ? v[i] * fold : 0.f;
+        const float a = live ? v[i] * (QPRE / key_field_factor<QM>(isB, g, i)) : 0.f;
         const _Float16 hi = static_cast<_Float16>(a);
         const _Float16 lo = static_cast<_Float16>(a - static_cast<float>(hi));
         hb[i] = __builtin_bit_cast(uint16_t, hi);

@@ -86,7 +86,24 @@ template <> struct UnpackD<QM_SYM4> {    // sign-magnitude bytes s....mmm -> sig
     const uint32_t b = __builtin_amdgcn_alignbit(w, w, 28);               // B_i (magnitude, sign) in byte i like A_i
     x[0] = pair(w, 0x02020000u); x[1] = pair(b, 0x02020000u); x[2] = pair(w, 0x03030101u); x[3] = pair(b, 0x03030101u);
   }
+  // Key side: the odd bytes are left where they are.  Bits 8..10 of an fp16 half are the top two mantissa bits and the
+  // lowest exponent bit, and a pattern below 2^11 still reads code * 2^(position - 24) (exponent field 0 and 1 share one
+  // scale), the byte's bit 7 is the half's sign already: one mask per pair, the pairs carrying 2^8 (KODD) that the query
+  // operand is divided by.  7 instructions per word.  (Not for the value side: there the factor would sit on p.)
+  static constexpr int KODD = 8;
+  static DEVI void run_k(uint32_t w, uint32_t (&x)[4]) {
+    const uint32_t b = __builtin_amdgcn_alignbit(w, w, 28);
+    x[0] = pair(w, 0x02020000u); x[1] = pair(b, 0x02020000u); x[2] = w & 0x87008700u; x[3] = b & 0x87008700u;
+  }
 };
+// the key words of a format, and the power of two element (isB, i) of a lane's four comes out of them with (group g)
+template <int QM> DEVI void unpack_key(uint32_t w, uint32_t (&x)[4]) {
+  if constexpr (QM == QM_SYM4) UnpackD<QM>::run_k(w, x); else UnpackD<QM>::run(w, x);
+}
+template <int QM> DEVI float key_field_factor(int isB, int g, int i) {
+  if constexpr (QM == QM_SYM4) return (i & 1) ? static_cast<float>(1 << UnpackD<QM>::KODD) : 1.f;
+  else return (isB ? static_cast<float>(1 << UnpackD<QM>::SH) : 1.f) * ((QM == QM_ASYM2 && (g & 1)) ? 16.f : 1.f);
+}
 // fp16 pattern of -(1024 + z)
 DEVI uint32_t negz16(uint32_t z) { return 0xE400u | z; }
 
